@@ -1,0 +1,148 @@
+/*
+ * relax_amd_wq.h — C ABI of the MI355X (gfx950) weight-only quantized linear library.
+ *
+ * Plain pointers and sizes only.  All tensor pointers are DEVICE pointers unless
+ * a parameter says "host".  fp16 tensors are passed as uint16_t bit patterns.
+ * Every launch is asynchronous on `stream` (a hipStream_t; NULL = the default
+ * stream); no entry point synchronises, allocates device memory or keeps a
+ * pointer after it returns, so all of them may be captured into a HIP graph.
+ *
+ * Return value: 0 on success, a negative WQ_E* code on failure; the message is
+ * available from wq_last_error() on the calling thread.  Nothing calls exit().
+ *
+ * Paths in the comments are relative to the reference tree (mlc-ai/relax).
+ */
+#ifndef RELAX_AMD_WQ_H_
+#define RELAX_AMD_WQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Every entry point below is exported with default visibility. */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+#define WQ_OK 0
+#define WQ_EINVAL (-1)   /* bad shape / pointer / enum */
+#define WQ_EDEVICE (-2)  /* a HIP call failed */
+#define WQ_EUNSUPPORTED (-3)
+
+typedef void* wq_stream_t; /* hipStream_t */
+
+/* activation / binary_op / unary_op selectors of the mixed-input GEMM epilogue;
+ * the strings the reference passes ("identity", "relu", "silu", "gelu",
+ * "plus", "multiply": python/tvm/contrib/cutlass/build.py:742-775) map onto these. */
+enum { WQ_ACT_IDENTITY = 0, WQ_ACT_RELU = 1, WQ_ACT_SILU = 2, WQ_ACT_GELU = 3 };
+enum { WQ_BIN_NONE = 0, WQ_BIN_PLUS = 1, WQ_BIN_MULTIPLY = 2 };
+enum { WQ_UN_IDENTITY = 0, WQ_UN_RELU = 1 };
+
+const char* wq_last_error(void);
+int wq_abi_version(void);
+/* Name of the device architecture the kernels were built for ("gfx950"). */
+const char* wq_target_arch(void);
+
+/* ------------------------------------------------------------------------- *
+ * Format A — q4f16_1 group quantization.
+ *   W  uint32 [N, K/8]   element k of row n = bits 4*(k%8).. of word k/8, code 0..15
+ *   S  fp16   [N, K/32]  one scale per 32 consecutive k
+ *   w[n,k] = (fp16(q) - 7) * S[n, k/32]      (fp16, one rounding)
+ *   y[m,n] = sum_k x[m,k] * w[n,k]           (fp32 accumulate, fp16 out)
+ * Replaces the generated kernels of the TIR functions in
+ *   tests/python/dlight/test_gpu_reduction.py:33-51, 400-424     (M = 1)
+ *   tests/python/dlight/test_gpu_low_batch_gemv.py:30-57         (small batch)
+ *   tests/python/dlight/test_gpu_matmul.py:352-401               (prefill + epilogue)
+ * which the reference schedules with python/tvm/dlight/gpu/{gemv,low_batch_gemv,matmul}.py.
+ * Requirements: K % 32 == 0; W, S rows 16-byte aligned (true for K % 32 == 0
+ * and 16-byte aligned bases).
+ * ------------------------------------------------------------------------- */
+
+/* q[n,k] = code (uint8 [N,K]); test_gpu_gemv.py:198 */
+int wq_q4_unpack(const uint32_t* W, uint8_t* q, int64_t N, int64_t K, wq_stream_t stream);
+
+/* out[n,k] = dequantized weight (fp16 [N,K]); the "decode" block, test_gpu_reduction.py:37-42.
+ * Uses the same device function as the fused kernels below. */
+int wq_q4g32_dequantize(const uint32_t* W, const uint16_t* S, uint16_t* out, int64_t N, int64_t K,
+                        wq_stream_t stream);
+
+/* y = x @ dequant(W,S)^T (+ bias[n] in fp32, then fp16, then + residual[m,n] in fp16).
+ * x fp16 [M,K], y fp16 [M,N]; bias / residual may be NULL.  Chooses the decode
+ * GEMV (M <= WQ_GEMV_MAX_M) or the MFMA GEMM from M. */
+int wq_q4g32_linear(const uint32_t* W, const uint16_t* S, const uint16_t* x, const uint16_t* bias,
+                    const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
+                    wq_stream_t stream);
+
+/* The two kernels behind wq_q4g32_linear, selectable for tests and measurement. */
+#define WQ_GEMV_MAX_M 8
+int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x, const uint16_t* bias,
+                  const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
+                  wq_stream_t stream);
+int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x, const uint16_t* bias,
+                  const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
+                  wq_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * Format B — fp16 activations x int8 / int4 weights (per-channel or group-64 scales).
+ *   packed weight  int8 [K, N]   or  int4 as int8 [K, N/2] (two's complement
+ *                  nibbles, low nibble = even n)
+ *   w[k,n] = fp16(q) * scale            (tests/python/relax/test_codegen_cutlass.py:1371-1389, 1628, 2041)
+ *   C[m,n] = act(sum_k A[m,k] w[k,n] + bias)                  fp32 accumulate, fp16 out
+ * ------------------------------------------------------------------------- */
+
+/* cutlass.ft_preprocess_weight (src/runtime/contrib/cutlass/weight_preprocess.cc:38-59):
+ * reorders a packed weight into the layout the GEMM kernels read.  `rows` = K,
+ * `cols` = N in ELEMENTS (the caller doubles the packed column count for int4,
+ * as weight_preprocess.cc:48-50 does).  Output has the same byte size as the
+ * input.  sm selects the layout family; only 75 <= sm < 90 is supported.
+ * Requires rows % 64 == 0 and cols % 64 == 0.
+ * _host works on host memory (what the reference does); the other one runs a
+ * device kernel on device memory and never leaves the GPU. */
+int wq_ft_preprocess_weight_host(int8_t* out_host, const int8_t* in_host, int64_t num_experts,
+                                 int64_t rows, int64_t cols, int is_int4, int sm);
+int wq_ft_preprocess_weight(int8_t* out, const int8_t* in, int64_t num_experts, int64_t rows,
+                            int64_t cols, int is_int4, int sm, wq_stream_t stream);
+
+/* Dequantized weight fp16 [K,N] from the PREPROCESSED layout (the decode
+ * PrimFunc of test_codegen_cutlass.py:1359-1389 composed with the inverse of the
+ * reordering).  group_size <= 0: scales [N]; group_size == 64: scales [K/64, N]. */
+int wq_intb_dequantize(const int8_t* B, const uint16_t* scales, uint16_t* out, int64_t K, int64_t N,
+                       int weight_nbit, int64_t group_size, wq_stream_t stream);
+
+/* fastertransformer::gemm_fp16_int_bias_act<WeightType, QuantOp>(A, B, scales, bias, C,
+ *   activation, m, n, k, group_size, bias_stride, workspace, workspace_bytes, stream)
+ * — call site python/tvm/contrib/cutlass/gemm_operation.py:441-447.  Same argument
+ * order; the two template parameters become weight_nbit (8 | 4) and the sign of
+ * group_size (per-column when group_size <= 0 or == k, else fine-grained, 64).
+ * B is the preprocessed weight.  bias may be NULL; bias_stride == 0 broadcasts
+ * bias[n] over rows, otherwise bias[m*bias_stride + n].  workspace is unused. */
+int wq_fpA_intB_gemm(const uint16_t* A, const int8_t* B, const uint16_t* scales,
+                     const uint16_t* bias, uint16_t* C, int activation, int64_t m, int64_t n,
+                     int64_t k, int64_t group_size, int64_t bias_stride, int weight_nbit,
+                     void* workspace, size_t workspace_bytes, wq_stream_t stream);
+
+/* fastertransformer::gemm_fp16_int_bias_act_residual<...>(A, B, scales, bias, residual, C,
+ *   activation, binary_op, unary_op, m, n, k, group_size, workspace, workspace_bytes, stream)
+ * — call site gemm_operation.py:452-458.  C = unary(binary(act(A w + bias), residual)). */
+int wq_fpA_intB_gemm_residual(const uint16_t* A, const int8_t* B, const uint16_t* scales,
+                              const uint16_t* bias, const uint16_t* residual, uint16_t* C,
+                              int activation, int binary_op, int unary_op, int64_t m, int64_t n,
+                              int64_t k, int64_t group_size, int weight_nbit, void* workspace,
+                              size_t workspace_bytes, wq_stream_t stream);
+
+/* Maps the reference's epilogue strings onto the enums above; -1 if unknown. */
+int wq_activation_from_string(const char* name);
+int wq_binary_op_from_string(const char* name);
+int wq_unary_op_from_string(const char* name);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RELAX_AMD_WQ_H_ */

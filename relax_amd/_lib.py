@@ -1,0 +1,64 @@
+"""Loads ``librelax_amd_wq.so`` and declares the C ABI of ``include/relax_amd_wq.h``.
+
+There is no fallback: if the library is missing or a symbol is absent the import
+fails with an error that says how to build it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "librelax_amd_wq.so")
+
+_i64, _int, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+
+# name -> argument types (all return int unless listed in _RESTYPES)
+SIGNATURES = {
+    "wq_last_error": [],
+    "wq_abi_version": [],
+    "wq_target_arch": [],
+    "wq_q4_unpack": [_vp, _vp, _i64, _i64, _vp],
+    "wq_q4g32_dequantize": [_vp, _vp, _vp, _i64, _i64, _vp],
+    "wq_q4g32_linear": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "wq_q4g32_gemv": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "wq_q4g32_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    #TODO "wq_ft_preprocess_weight_host": [_vp, _vp, _i64, _i64, _i64, _int, _int],
+    #TODO "wq_ft_preprocess_weight": [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp],
+    #TODO "wq_intb_dequantize": [_vp, _vp, _vp, _i64, _i64, _int, _i64, _vp],
+    #TODO "wq_fpA_intB_gemm": [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
+    #TODO "wq_fpA_intB_gemm_residual": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
+    "wq_activation_from_string": [ctypes.c_char_p],
+    "wq_binary_op_from_string": [ctypes.c_char_p],
+    "wq_unary_op_from_string": [ctypes.c_char_p],
+}
+_RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p}
+
+_lib = None
+
+
+class WqError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m relax_amd.build` "
+                "(hipcc, --offload-arch=gfx950). There is no CPU fallback."
+            )
+        l = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(l, name)  # AttributeError if the symbol is not exported
+            fn.argtypes = argtypes
+            fn.restype = _RESTYPES.get(name, ctypes.c_int)
+        _lib = l
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().wq_last_error()
+        raise WqError(f"{what} failed ({rc}): {msg.decode() if msg else ''}")

@@ -1,0 +1,109 @@
+// Device-side building blocks shared by every kernel of the quantized linear path.
+// gfx950 only: 64-wide wavefronts, packed fp16 VALU, v_dot2_f32_f16, MFMA.
+#ifndef RELAX_AMD_CSRC_WQ_DEVICE_H_
+#define RELAX_AMD_CSRC_WQ_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace wq {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+__device__ __forceinline__ half_t as_half(uint16_t u) { return __builtin_bit_cast(half_t, u); }
+__device__ __forceinline__ uint16_t as_u16(half_t h) { return __builtin_bit_cast(uint16_t, h); }
+
+// ---------------------------------------------------------------------------
+// Format A: one uint32 holds 8 codes, code i in bits 4i..4i+3.
+// (w >> 4i) & 0x000F000F isolates code i in the low half-word and code i+4 in the
+// high half-word.  OR-ing 0x6400 into each half-word makes the fp16 number
+// 1024 + code (exact), and subtracting 1031 leaves code - 7 exactly.  So
+// pair i of the result is (code_i - 7, code_{i+4} - 7): the PAIRING IS (i, i+4),
+// not (2i, 2i+1).  Every caller arranges its activations to match.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void q4_word_minus7(uint32_t w, half2_t out[4]) {
+  const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t t = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+    out[i] = as_half2(t) - off;
+  }
+}
+
+// The reference's dequantized weight, bit for bit: (fp16(code) - 7) * s with a single
+// fp16 rounding in the multiply.  s2 holds the group's scale in both halves.
+__device__ __forceinline__ void q4_word_dequant(uint32_t w, half2_t s2, half2_t out[4]) {
+  half2_t d[4];
+  q4_word_minus7(w, d);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) out[i] = d[i] * s2;
+}
+
+// fp32 += a.x*b.x + a.y*b.y with exact fp16 products (v_dot2_f32_f16).
+__device__ __forceinline__ float dot2(half2_t a, half2_t b, float c) {
+  return __builtin_amdgcn_fdot2(a, b, c, false);
+}
+
+// Rearranges 8 consecutive halves (4 dwords, natural order) into the (i, i+4)
+// pairing q4_word_minus7 produces: out[i] = (h[i], h[i+4]).
+__device__ __forceinline__ void pair_i_i4(const uint32_t in[4], uint32_t out[4]) {
+  // v_perm_b32(hi_src, lo_src, sel): byte k of the result = byte sel[k] of {hi_src:lo_src}
+  // (bytes 0-3 from lo_src, 4-7 from hi_src).
+  out[0] = __builtin_amdgcn_perm(in[2], in[0], 0x05040100u);  // (h0, h4)
+  out[1] = __builtin_amdgcn_perm(in[2], in[0], 0x07060302u);  // (h1, h5)
+  out[2] = __builtin_amdgcn_perm(in[3], in[1], 0x05040100u);  // (h2, h6)
+  out[3] = __builtin_amdgcn_perm(in[3], in[1], 0x07060302u);  // (h3, h7)
+}
+
+// Sum over the 64 lanes of a wavefront; every lane receives the total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// ---------------------------------------------------------------------------
+// Format B helpers.  After preprocessing, every stored code is unsigned
+// (int8: q + 128, int4: q + 8).
+// ---------------------------------------------------------------------------
+
+// Two bytes of `w` (selected by the v_perm selector `sel`, whose bytes 1 and 3
+// must pick the constant 0x64) -> (q_a, q_b) as exact fp16 integers.
+// sel examples: 0x04020400 -> bytes (0, 2);  0x04030401 -> bytes (1, 3).
+__device__ __forceinline__ half2_t u8x2_to_half2(uint32_t w, uint32_t sel) {
+  uint32_t t = __builtin_amdgcn_perm(0x64646464u, w, sel);  // (1024 + u_a, 1024 + u_b)
+  const half2_t off = {(half_t)1152.0f, (half_t)1152.0f};    // 1024 + 128
+  return as_half2(t) - off;
+}
+
+// Eight unsigned nibbles of `w` -> pairs (nibble i, nibble i+4) minus 8, exact.
+__device__ __forceinline__ void u4_word_minus8(uint32_t w, half2_t out[4]) {
+  const half2_t off = {(half_t)1032.0f, (half_t)1032.0f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint32_t t = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+    out[i] = as_half2(t) - off;
+  }
+}
+
+__device__ __forceinline__ float apply_activation(float v, int act) {
+  switch (act) {
+    case 1: return v > 0.0f ? v : 0.0f;
+    case 2: return v / (1.0f + __expf(-v));
+    case 3: return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    default: return v;
+  }
+}
+
+}  // namespace wq
+#endif  // RELAX_AMD_CSRC_WQ_DEVICE_H_

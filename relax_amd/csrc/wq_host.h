@@ -1,0 +1,43 @@
+// Host-side helpers shared by the entry points: error reporting and argument checks.
+#ifndef RELAX_AMD_CSRC_WQ_HOST_H_
+#define RELAX_AMD_CSRC_WQ_HOST_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/relax_amd_wq.h"
+
+namespace wq {
+
+// Stores a printf-style message for wq_last_error() on this thread and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace wq
+
+#define WQ_REQUIRE(cond, ...)                                  \
+  do {                                                         \
+    if (!(cond)) return ::wq::fail(WQ_EINVAL, __VA_ARGS__);    \
+  } while (0)
+
+// Checks the launch that was just enqueued (hipGetLastError catches bad grids /
+// missing code objects without synchronising).
+#define WQ_CHECK_LAUNCH(what)                                                              \
+  do {                                                                                     \
+    hipError_t e_ = hipGetLastError();                                                     \
+    if (e_ != hipSuccess)                                                                  \
+      return ::wq::fail(WQ_EDEVICE, "%s: launch failed: %s", what, hipGetErrorString(e_)); \
+  } while (0)
+
+#define WQ_HIP(call)                                                                        \
+  do {                                                                                      \
+    hipError_t e_ = (call);                                                                 \
+    if (e_ != hipSuccess)                                                                   \
+      return ::wq::fail(WQ_EDEVICE, "%s failed: %s", #call, hipGetErrorString(e_));         \
+  } while (0)
+
+#endif  // RELAX_AMD_CSRC_WQ_HOST_H_

@@ -1,0 +1,113 @@
+"""torch-tensor front end of the C ABI.
+
+torch is used for device memory and streams only: every function validates its
+arguments, takes ``data_ptr()`` of each tensor and calls the C entry point on
+torch's current stream.  Argument names and orders follow the reference's
+PrimFuncs / PackedFuncs:
+
+* format A: ``(W uint32[N,K/8], S fp16[N,K/32], x fp16[...,K]) -> y fp16[...,N]``
+  (tests/python/dlight/test_gpu_gemv.py:189, test_gpu_low_batch_gemv.py:30-34)
+* format B: ``(x, w_preprocessed, scales, [bias], [residual]) -> out``
+  (tests/python/relax/test_codegen_cutlass.py:1474-1520)
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import check
+
+ACTIVATIONS = {"identity": 0, "relu": 1, "silu": 2, "gelu": 3}
+BINARY_OPS = {"none": 0, "plus": 1, "multiply": 2}
+UNARY_OPS = {"identity": 0, "relu": 1}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, dtype, name: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise ValueError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must have dtype {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be compact (contiguous)")
+    return t
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+# torch has no uint32 arithmetic; packed weights may arrive as int32 or uint32 (same bytes)
+def _w32(W: torch.Tensor) -> torch.Tensor:
+    if W.dtype not in (torch.int32, torch.uint32):
+        raise ValueError(f"packed weight must be 32-bit integers, got {W.dtype}")
+    return _dev(W, W.dtype, "W")
+
+
+# ----------------------------------------------------------------- format A
+
+
+def q4_unpack(W: torch.Tensor) -> torch.Tensor:
+    """codes uint8 [N, K] of a packed ``uint32 [N, K/8]`` weight."""
+    W = _w32(W)
+    N, kw = W.shape
+    q = torch.empty((N, kw * 8), dtype=torch.uint8, device=W.device)
+    check(_lib.lib().wq_q4_unpack(_ptr(W), _ptr(q), N, kw * 8, _stream()), "wq_q4_unpack")
+    return q
+
+
+def q4g32_dequantize(W: torch.Tensor, S: torch.Tensor) -> torch.Tensor:
+    """fp16 [N, K] dequantized weight, bit-identical to the reference's ``decode`` block."""
+    W = _w32(W)
+    S = _dev(S, torch.float16, "S")
+    N, kw = W.shape
+    K = kw * 8
+    if tuple(S.shape) != (N, K // 32) or K % 32:
+        raise ValueError(f"S must be [N, K/32] = [{N}, {K // 32}], got {tuple(S.shape)}")
+    out = torch.empty((N, K), dtype=torch.float16, device=W.device)
+    check(_lib.lib().wq_q4g32_dequantize(_ptr(W), _ptr(S), _ptr(out), N, K, _stream()), "wq_q4g32_dequantize")
+    return out
+
+
+def q4g32_linear(W: torch.Tensor, S: torch.Tensor, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                 residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                 kernel: str = "auto") -> torch.Tensor:
+    """``y[..., n] = sum_k x[..., k] * dequant(W, S)[n, k]`` (+bias, +residual), fp32 accumulate.
+
+    ``kernel``: "auto" (by M), "gemv" or "gemm".  ``out`` makes the call destination-passing.
+    """
+    W = _w32(W)
+    S = _dev(S, torch.float16, "S")
+    x = _dev(x, torch.float16, "x")
+    N, kw = W.shape
+    K = kw * 8
+    if x.shape[-1] != K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {K}")
+    if K % 32 or tuple(S.shape) != (N, K // 32):
+        raise ValueError(f"S must be [N, K/32] = [{N}, {K // 32}], got {tuple(S.shape)}")
+    M = x.numel() // K if K else 0
+    oshape = tuple(x.shape[:-1]) + (N,)
+    if bias is not None:
+        bias = _dev(bias, torch.float16, "bias")
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
+    if residual is not None:
+        residual = _dev(residual, torch.float16, "residual")
+        if residual.numel() != M * N:
+            raise ValueError("residual must have M*N elements")
+    if out is None:
+        out = torch.empty(oshape, dtype=torch.float16, device=x.device)
+    else:
+        out = _dev(out, torch.float16, "out")
+        if out.numel() != M * N:
+            raise ValueError("out must have M*N elements")
+    fn = {"auto": _lib.lib().wq_q4g32_linear, "gemv": _lib.lib().wq_q4g32_gemv,
+          "gemm": _lib.lib().wq_q4g32_gemm}[kernel]
+    check(fn(_ptr(W), _ptr(S), _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), M, N, K, _stream()),
+          f"wq_q4g32_{kernel}")
+    return out

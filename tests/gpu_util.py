@@ -1,0 +1,37 @@
+"""Helpers shared by the GPU parity tests."""
+import numpy as np
+import torch
+
+
+def dev(a: np.ndarray) -> torch.Tensor:
+    """numpy -> device tensor (uint32 travels as int32: same bytes)."""
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)
+    return torch.from_numpy(a).cuda()
+
+
+def host(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().numpy()
+
+
+# Tolerance of the fused kernels against the fp32-accumulated oracle.  The
+# requirement is a maximum relative error of 1e-2; the reference's own tests use
+# assert_allclose(rtol=1e-2, atol=1e-2) (tests/python/relax/test_codegen_cutlass.py:1609).
+# Both kernels accumulate in fp32 and differ from the oracle only in summation
+# order, so a 10x tighter normalised bound is asserted as well.
+RTOL = 1e-2
+ATOL = 1e-2
+NORM_TOL = 1e-3
+
+
+def assert_close(got: np.ndarray, ref: np.ndarray, what: str = ""):
+    g = got.astype(np.float64)
+    r = ref.astype(np.float64)
+    assert g.shape == r.shape, (what, g.shape, r.shape)
+    assert np.all(np.isfinite(g)), what
+    err = np.abs(g - r)
+    bad = err > RTOL * np.abs(r) + ATOL
+    assert not bad.any(), f"{what}: {bad.sum()} elements outside rtol={RTOL} atol={ATOL}; max err {err.max()}"
+    scale = max(np.abs(r).max(), 1e-6)
+    assert err.max() / scale <= NORM_TOL, f"{what}: normalised max error {err.max() / scale:.3e} > {NORM_TOL}"
