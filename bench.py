@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Benchmark of the weight-only quantized linear path on one MI355X.
+
+One step = one pass of the four Llama-2-7B-shaped decode linears at batch M=1
+(int4 codes packed 8 per uint32 along K, group 32, fp16 scales, zero point 7):
+4096->12288 (fused QKV), 4096->4096 (o_proj), 4096->22016 (gate/up), 11008->4096 (down).
+Inputs are synthetic and resident in HBM before the timed region.  Each step
+reads a different copy of the weights (a ring of copies larger than the
+256 MB last-level cache), so the reported GB/s is HBM traffic, not cache hits.
+
+Prints ONE JSON line.  `value` is algorithmic bytes per second over the whole
+step; `roofline` describes the decode GEMV kernel, `gemm` the M=2048 prefill
+GEMM of the same quantization scheme, `cpu_baseline` the CPU restatement of the
+reference's path timed on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "int4 GEMV HBM GB/s (M=1, %peak); int4 GEMM TFLOPS (M=2048, %MFMA peak)"
+DECODE_SHAPES = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]  # (N, K)
+PREFILL_SHAPES = [(11008, 4096), (4096, 11008)]
+PREFILL_M = 2048
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def gemv_bytes(M, N, K):
+    """Algorithmic bytes of one format-A linear: codes + scales + x + y."""
+    return N * K // 2 + N * (K // 32) * 2 + M * K * 2 + M * N * 2
+
+
+def make_device_set(torch, seed):
+    """Random codes / scales for the four decode linears, generated on the device."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    out = []
+    for N, K in DECODE_SHAPES:
+        W = torch.randint(-2**31, 2**31 - 1, (N, K // 8), dtype=torch.int32, device="cuda", generator=g)
+        S = (torch.rand((N, K // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+        out.append((W, S))
+    return out
+
+
+def cpu_baseline(budget_s=8.0):
+    """Times the CPU oracle (the reference's llvm-target semantics: decode pass +
+    naive fp32-accumulate loop nest, one thread) on the same four linears."""
+    from oracle import wq_oracle as o
+
+    o.build()
+    rng = np.random.default_rng(0)
+    sets = []
+    for N, K in DECODE_SHAPES:
+        x, W, S = o.make_q4g32_inputs(1, N, K, seed=int(rng.integers(1 << 30)))
+        sets.append((W, S, x))
+    nbytes = sum(gemv_bytes(1, N, K) for N, K in DECODE_SHAPES)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        for W, S, x in sets:
+            o.q4g32_linear(W, S, x, nthreads=1)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s and reps >= 2:
+            break
+    return {
+        "value": round(nbytes * reps / dt / 1e9, 4),
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"{reps} full steps (the same four M=1 linears), {dt:.1f} s, single thread, "
+                  f"{dt / reps * 1e3:.1f} ms per step",
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--copies", type=int, default=16, help="distinct weight copies in the ring")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM measurement")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of through a HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from relax_amd import ops
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    copies = [make_device_set(torch, 1000 + i) for i in range(args.copies)]
+    xs = [torch.randn((1, K), device="cuda", dtype=torch.float16) for _, K in DECODE_SHAPES]
+    ys = [torch.empty((1, N), device="cuda", dtype=torch.float16) for N, _ in DECODE_SHAPES]
+    step_bytes = sum(gemv_bytes(1, N, K) for N, K in DECODE_SHAPES)
+    launches_per_step = len(DECODE_SHAPES)
+
+    def step(i):
+        for (W, S), x, y in zip(copies[i % args.copies], xs, ys):
+            ops.q4g32_linear(W, S, x, out=y, kernel="gemv")
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(args.warmup):
+            step(i)
+        stream.synchronize()
+        graph = None
+        if not args.no_graph:
+            # one graph holds all timed steps: the host only issues a single launch
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(args.steps):
+                    step(i)
+            graph.replay()  # untimed replay (graph upload)
+            stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(args.steps):
+                step(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        total_ms = e0.elapsed_time(e1)
+
+    ms_per_step = total_ms / args.steps
+    gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
+    # the GEMV kernel is the only kernel in the timed region: its average launch
+    # duration (launch gaps included, so a slight under-estimate of the kernel) is
+    avg_launch_us = total_ms * 1e3 / (args.steps * launches_per_step)
+    bytes_per_launch = step_bytes / launches_per_step
+    achieved = bytes_per_launch / (avg_launch_us * 1e-6) / 1e9
+
+    out = {
+        "metric": METRIC,
+        "value": round(gbs, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "Llama-2-7B-shaped decode linears at M=1, int4 group-32 (q4f16_1): "
+                        "4096->12288, 4096->4096, 4096->22016, 11008->4096",
+            "weight_copies_in_ring": args.copies,
+            "ring_bytes": step_bytes * args.copies,
+            "launch": "eager" if graph is None else "hip_graph",
+            "bytes_per_step": step_bytes,
+        },
+        "roofline": {
+            "kernel": "q4g32_gemv_kernel",
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "avg_launch_us": round(avg_launch_us, 3),
+            "bytes_per_launch": bytes_per_launch,
+        },
+    }
+
+    if not args.no_gemm:
+        gem = []
+        tot_flops, tot_ms = 0.0, 0.0
+        reps = 10
+        for N, K in PREFILL_SHAPES:
+            g = torch.Generator(device="cuda")
+            g.manual_seed(N)
+            W = torch.randint(-2**31, 2**31 - 1, (N, K // 8), dtype=torch.int32, device="cuda", generator=g)
+            S = (torch.rand((N, K // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+            x = torch.randn((PREFILL_M, K), device="cuda", dtype=torch.float16)
+            y = torch.empty((PREFILL_M, N), device="cuda", dtype=torch.float16)
+            for _ in range(3):
+                ops.q4g32_linear(W, S, x, out=y, kernel="gemm")
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                ops.q4g32_linear(W, S, x, out=y, kernel="gemm")
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b) / reps
+            fl = 2.0 * PREFILL_M * N * K
+            gem.append({"M": PREFILL_M, "N": N, "K": K, "us": round(ms * 1e3, 2), "tflops": round(fl / ms / 1e9, 1)})
+            tot_flops += fl
+            tot_ms += ms
+            del W, S, x, y
+        tf = tot_flops / tot_ms / 1e9
+        out["gemm"] = {
+            "kernel": "q4g32_gemm_kernel",
+            "value": round(tf, 1),
+            "unit": "TFLOP/s",
+            "shapes": gem,
+            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+        }
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -49,6 +49,11 @@ def lib() -> ctypes.CDLL:
                 f"{LIB_PATH} is missing: build it with `python -m relax_amd.build` "
                 "(hipcc, --offload-arch=gfx950). There is no CPU fallback."
             )
+        # torch goes first: it ships its own HIP runtime (same soname as the system
+        # one), and whichever copy is mapped first serves the whole process.  The
+        # tensors this package receives live in torch's runtime, so the kernels must too.
+        import torch  # noqa: F401
+
         l = ctypes.CDLL(LIB_PATH)
         for name, argtypes in SIGNATURES.items():
             fn = getattr(l, name)  # AttributeError if the symbol is not exported

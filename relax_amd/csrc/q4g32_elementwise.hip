@@ -60,9 +60,8 @@ extern "C" int wq_q4_unpack(const uint32_t* W, uint8_t* q, int64_t N, int64_t K,
   WQ_REQUIRE(((uintptr_t)q & 7u) == 0, "wq_q4_unpack: output must be 8-byte aligned");
   int64_t blocks = (nwords + 255) / 256;
   WQ_REQUIRE(blocks < (1ll << 31), "wq_q4_unpack: tensor too large");
-  hipLaunchKernelGGL(wq::q4_unpack_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                     (hipStream_t)stream, W, (wq::uint2_t*)q, nwords);
-  WQ_CHECK_LAUNCH("wq_q4_unpack");
+  WQ_LAUNCH("wq_q4_unpack", wq::q4_unpack_kernel, dim3((unsigned)blocks), dim3(256), 0,
+            (hipStream_t)stream, W, (wq::uint2_t*)q, nwords);
   return WQ_OK;
 }
 
@@ -77,9 +76,8 @@ extern "C" int wq_q4g32_dequantize(const uint32_t* W, const uint16_t* S, uint16_
              "wq_q4g32_dequantize: W and out must be 16-byte aligned");
   int64_t blocks = (ngroups + 255) / 256;
   WQ_REQUIRE(blocks < (1ll << 31), "wq_q4g32_dequantize: tensor too large");
-  hipLaunchKernelGGL(wq::q4g32_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                     (hipStream_t)stream, (const wq::uint4_t*)W, (const wq::half_t*)S,
-                     (wq::uint4_t*)out, ngroups);
-  WQ_CHECK_LAUNCH("wq_q4g32_dequantize");
+  WQ_LAUNCH("wq_q4g32_dequantize", wq::q4g32_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0,
+            (hipStream_t)stream, (const wq::uint4_t*)W, (const wq::half_t*)S, (wq::uint4_t*)out,
+            ngroups);
   return WQ_OK;
 }

@@ -214,11 +214,9 @@ static int launch_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x,
     WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(Cfg::kThreads),
-                     Cfg::kLdsBytes, stream, W, (const half_t*)S, (const half_t*)x,
-                     (const half_t*)bias, (const half_t*)residual, (half_t*)y, (int)M, (int)N,
-                     (int)K, tiles_m, tiles_n);
-  WQ_CHECK_LAUNCH("wq_q4g32_gemm");
+  WQ_LAUNCH("wq_q4g32_gemm", kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(Cfg::kThreads),
+            Cfg::kLdsBytes, stream, W, (const half_t*)S, (const half_t*)x, (const half_t*)bias,
+            (const half_t*)residual, (half_t*)y, (int)M, (int)N, (int)K, tiles_m, tiles_n);
   return WQ_OK;
 }
 

@@ -1,132 +1,349 @@
 // Format A decode GEMV: y[m,n] = sum_k x[m,k] * ((code[n,k] - 7) * S[n,k/32]), M <= 8.
 //
-// The kernel is a weight stream.  One wavefront owns R consecutive output rows;
-// lane l walks the row in 16-byte steps (4 words = 32 codes = exactly one scale
-// group), so a wavefront-wide load is 1 KiB of contiguous weights per row and the
-// matching scales are one contiguous 128-byte load.  The activations are staged
-// once per workgroup in LDS, already rearranged to the (i, i+4) pairing the
-// in-register unpack produces, 16-byte chunk c of group g at ((c*G + g) * 16) so
-// that the 64 lanes of a wavefront read 64 consecutive chunks (no bank conflicts).
-// Partial sums stay in fp32 registers and are combined with wavefront shuffles.
+// The kernel is a weight stream bounded by HBM bandwidth, so the design goal is
+// to keep many 16-byte loads in flight per CU, to put nothing (no LDS staging, no
+// barrier) between the start of a workgroup and its first weight loads, and to
+// spend as few VALU instructions per weight word as possible.
+//
+// Work split.  A row set is ROWS consecutive output rows and belongs to one
+// wavefront (or to `parts` wavefronts when K > 64*32*GPL); lane l of wavefront
+// `part` owns the scale groups g = (j*parts + part)*64 + l, j < GPL, of every row
+// of the set: 16 bytes of W (4 words = 32 codes) and one scale per group, so a
+// wavefront-wide load is 1 KiB of contiguous weights (128 bytes of scales).
+// All ROWS*GPL weight loads of a lane are independent and issued back to back.
+//
+// Activations.  The workgroup (4 wavefronts, 4 row sets) first issues one pass of
+// coalesced loads over x, THEN its weight loads: vector loads complete in issue
+// order, so x can be processed while the weights are still in flight.  Each
+// thread rearranges its 8 activations to the pairing of the unpack, folds the
+// zero point into the group constant c_g (below) and writes the result to LDS;
+// after one barrier every lane copies the activations of its own groups into
+// registers, where they stay for all rows.  x is therefore read from L2 once per
+// workgroup instead of once per wavefront, and its rearrangement costs a dozen
+// VALU instructions per thread.
+//
+// Reduction.  DPP row shifts inside a wavefront (total in lane 63); only when
+// parts > 1 do partial sums cross wavefronts, through a few LDS words.
+//
+// Arithmetic.  With t = 1024 + code (the fp16 number obtained by OR-ing the code
+// into the mantissa of 0x6400) the group's contribution is
+//     s * ( sum_k x_k * t_k  -  c_g ),    c_g = sum_k x_k * 1031
+// so the subtraction of the zero point and the multiplication by the scale are
+// done once per group instead of once per weight; c_g depends only on x.  Codes
+// in odd nibble positions are taken without a shift as 1024 + 16*code and meet
+// activations pre-multiplied by 1/16; their share of c_g uses 64 + 7 = 71 instead
+// of 1031.  Products are exact in fp32 (v_dot2_f32_f16), accumulation is fp32.
+// The result differs from the reference's "round each weight to fp16 first" only
+// by those roundings, far inside the 1e-2 tolerance; a one-hot x still reproduces
+// a dequantized column bit for bit.  The bit-exact dequantization itself is
+// q4_word_dequant, used by the dequantize entry point and by the MFMA GEMM.
 #include "wq_device.h"
 #include "wq_host.h"
 
 namespace wq {
 
-constexpr int kGemvThreads = 256;
-constexpr int kGemvWaves = kGemvThreads / 64;
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_shift(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
+}
 
-template <int R, int MB>
-__global__ __launch_bounds__(kGemvThreads) void q4g32_gemv_kernel(
+// Sum over the wavefront; the total is valid in lane 63.
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v += dpp_shift<0x111, 0xf>(v);  // row_shr:1
+  v += dpp_shift<0x112, 0xf>(v);  // row_shr:2
+  v += dpp_shift<0x114, 0xf>(v);  // row_shr:4
+  v += dpp_shift<0x118, 0xf>(v);  // row_shr:8   -> lane 15 of each row holds the row sum
+  v += dpp_shift<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_shift<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+constexpr int kGemvMaxWaves = 16;
+
+// Few groups per lane means more wavefronts share a row: allow larger workgroups there.
+template <int GPL>
+constexpr int gemv_max_threads() {
+  return GPL == 1 ? 1024 : GPL == 2 ? 512 : 256;
+}
+
+template <int ROWS, int GPL>
+struct GemvFrag {
+  uint4_t w[ROWS][GPL];
+  half_t s[ROWS][GPL];
+};
+
+template <int ROWS, int MB, int GPL>
+__global__ __launch_bounds__(gemv_max_threads<GPL>()) void q4g32_gemv_kernel(
     const uint4_t* __restrict__ W, const half_t* __restrict__ S, const half_t* __restrict__ x,
     const half_t* __restrict__ bias, const half_t* __restrict__ residual, half_t* __restrict__ y,
-    int N, int K) {
-  extern __shared__ uint4_t xs[];  // [MB][4][G] chunks of 16 bytes
-  const int G = K >> 5;            // scale groups per row == 16-byte chunks of W per row
+    int N, int K, int parts, int nsets) {
+  extern __shared__ uint4_t smem[];
+  __shared__ float red[2][kGemvMaxWaves][ROWS * MB];
+  const int G = K >> 5;
+  uint4_t* xs = smem;                                       // [MB][4][G] rearranged chunks
+  float* cs = reinterpret_cast<float*>(smem + MB * 4 * G);  // [MB][G]    -c_g
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nthreads = blockDim.x;
+  const int sets_per_block = (nthreads >> 6) / parts;
+  const int part = wave % parts;
+  const int set_in_block = wave / parts;
+  const int stride = gridDim.x * sets_per_block;  // row sets between two turns of this workgroup
+  int base = blockIdx.x * sets_per_block;         // first row set of the workgroup's current turn
 
-  // ---- stage x: word wi = 8 halves, stored in the (i, i+4) pairing ----
-  const int nwords = K >> 3;
+  int g[GPL];
+  bool active[GPL];
 #pragma unroll
-  for (int m = 0; m < MB; ++m) {
-    const uint4_t* xrow = reinterpret_cast<const uint4_t*>(x + (int64_t)m * K);
-    for (int wi = tid; wi < nwords; wi += kGemvThreads) {
-      uint4_t v = xrow[wi];
-      uint32_t in[4] = {v.x, v.y, v.z, v.w}, o[4];
-      pair_i_i4(in, o);
-      uint4_t p = {o[0], o[1], o[2], o[3]};
-      xs[(m * 4 + (wi & 3)) * G + (wi >> 2)] = p;
-    }
+  for (int j = 0; j < GPL; ++j) {
+    const int gj = (j * parts + part) * 64 + lane;
+    active[j] = gj < G;
+    g[j] = active[j] ? gj : G - 1;  // idle lanes shadow a real group and get a zero scale
   }
-  __syncthreads();
 
-  const int n0 = (blockIdx.x * kGemvWaves + wave) * R;
-  if (n0 >= N) return;
-
-  float acc[R][MB];
+  // All loads of one row set: independent, issued back to back.  Row sets and
+  // rows past the end are clamped here and dropped at the store; the row base is
+  // wave-uniform.
+  auto load = [&](GemvFrag<ROWS, GPL>& f, int base_) {
+    const int n0_ = min(base_ + set_in_block, nsets - 1) * ROWS;
 #pragma unroll
-  for (int r = 0; r < R; ++r)
+    for (int r = 0; r < ROWS; ++r) {
+      const uint4_t* wrow = W + (int64_t)min(n0_ + r, N - 1) * G;
+      const half_t* srow = S + (int64_t)min(n0_ + r, N - 1) * G;
 #pragma unroll
-    for (int m = 0; m < MB; ++m) acc[r][m] = 0.0f;
-
-  // rows past the end are clamped for the loads and dropped at the store
-  int64_t rowoff[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) rowoff[r] = (int64_t)min(n0 + r, N - 1) * G;
-
-  for (int g = lane; g < G; g += 64) {
-    uint4_t wv[R];
-    half_t sv[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      wv[r] = __builtin_nontemporal_load(&W[rowoff[r] + g]);
-      sv[r] = __builtin_nontemporal_load(&S[rowoff[r] + g]);
-    }
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      uint4_t xv[MB];
-#pragma unroll
-      for (int m = 0; m < MB; ++m) xv[m] = xs[(m * 4 + c) * G + g];
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const uint32_t word = c == 0 ? wv[r].x : c == 1 ? wv[r].y : c == 2 ? wv[r].z : wv[r].w;
-        const half2_t s2 = {sv[r], sv[r]};
-        half2_t d[4];
-        q4_word_dequant(word, s2, d);
-#pragma unroll
-        for (int m = 0; m < MB; ++m) {
-          acc[r][m] = dot2(d[0], as_half2(xv[m].x), acc[r][m]);
-          acc[r][m] = dot2(d[1], as_half2(xv[m].y), acc[r][m]);
-          acc[r][m] = dot2(d[2], as_half2(xv[m].z), acc[r][m]);
-          acc[r][m] = dot2(d[3], as_half2(xv[m].w), acc[r][m]);
-        }
+      for (int j = 0; j < GPL; ++j) {
+        f.w[r][j] = __builtin_nontemporal_load(&wrow[g[j]]);
+        f.s[r][j] = __builtin_nontemporal_load(&srow[g[j]]);
       }
     }
-  }
+  };
 
+  // ---- 1. activations: thread t takes words t, t + nthreads, ... (8 halves each) ----
+  constexpr int kMaxXW = 8;  // words of x per thread and batch row: K <= 8*8*nthreads
+  const int nwords = K >> 3;
+  uint4_t xraw[MB][kMaxXW];
 #pragma unroll
-  for (int r = 0; r < R; ++r)
+  for (int m = 0; m < MB; ++m)
 #pragma unroll
-    for (int m = 0; m < MB; ++m) acc[r][m] = wave_sum(acc[r][m]);
+    for (int i = 0; i < kMaxXW; ++i) {
+      const int wi = tid + i * nthreads;
+      if (wi < nwords) xraw[m][i] = reinterpret_cast<const uint4_t*>(x + (int64_t)m * K)[wi];
+    }
 
-  if (lane == 0) {
+  // ---- 2. weights and scales of the first row set: issued now, consumed last ----
+  GemvFrag<ROWS, GPL> fa, fb;
+  load(fa, base);
+
+  // ---- 3. rearrange x, fold the zero point into c_g, publish through LDS ----
+  const half2_t k1031 = {(half_t)1031.0f, (half_t)1031.0f};
+  const half2_t k71 = {(half_t)71.0f, (half_t)71.0f};
+  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
+  for (int m = 0; m < MB; ++m)
+#pragma unroll
+    for (int i = 0; i < kMaxXW; ++i) {
+      const int wi = tid + i * nthreads;
+      if (wi < nwords) {  // nwords % 4 == 0 and nthreads % 4 == 0: a quad is in or out together
+        const uint4_t v = xraw[m][i];
+        const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+        pair_i_i4(in, o);  // o[i] = (x_i, x_{i+4})
+        float c = dot2(as_half2(o[0]), k1031, 0.0f);
+        c = dot2(as_half2(o[1]), k71, c);
+        c = dot2(as_half2(o[2]), k1031, c);
+        c = dot2(as_half2(o[3]), k71, c);
+        // the 4 words of a group sit in 4 adjacent lanes
+        c += dpp_shift<0xb1, 0xf>(c);  // quad_perm [1,0,3,2]
+        c += dpp_shift<0x4e, 0xf>(c);  // quad_perm [2,3,0,1]
+        const int grp = wi >> 2, ch = wi & 3;
+        xs[(m * 4 + ch) * G + grp] = uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2],
+                                             as_u32(as_half2(o[3]) * sixteenth)};
+        if (ch == 0) cs[m * G + grp] = -c;
+      }
+    }
+  __syncthreads();
+
+  // ---- 4. this lane's activations -> registers, for the whole kernel ----
+  uint4_t xv[MB][GPL][4];
+  float cg[MB][GPL];
+#pragma unroll
+  for (int m = 0; m < MB; ++m)
+#pragma unroll
+    for (int j = 0; j < GPL; ++j) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) xv[m][j][c] = xs[(m * 4 + c) * G + g[j]];
+      cg[m][j] = cs[m * G + g[j]];
+    }
+
+  const uint32_t magic = 0x64006400u;
+  int turn = 0;
+
+  // ---- 5. one row set: 1 shift + 4 and_or + 4 dot2 per word, reduce, store ----
+  auto process = [&](const GemvFrag<ROWS, GPL>& f, int base_) {
+    const int set = base_ + set_in_block;
+    const bool set_ok = set < nsets;  // uniform per wavefront
+    const int n0 = min(set, nsets - 1) * ROWS;
+    float acc[ROWS][MB];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[r][m] = 0.0f;
+#pragma unroll
+      for (int j = 0; j < GPL; ++j) {
+        float grp[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) grp[m] = cg[m][j];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint4_t w4 = f.w[r][j];
+          const uint32_t word = c == 0 ? w4.x : c == 1 ? w4.y : c == 2 ? w4.z : w4.w;
+          const uint32_t w8 = word >> 8;
+          const half2_t t0 = as_half2(and_or(word, 0x000F000Fu, magic));  // 1024 + (q0, q4)
+          const half2_t t1 = as_half2(and_or(word, 0x00F000F0u, magic));  // 1024 + 16*(q1, q5)
+          const half2_t t2 = as_half2(and_or(w8, 0x000F000Fu, magic));    // 1024 + (q2, q6)
+          const half2_t t3 = as_half2(and_or(w8, 0x00F000F0u, magic));    // 1024 + 16*(q3, q7)
+#pragma unroll
+          for (int m = 0; m < MB; ++m) {
+            float d = grp[m];
+            d = dot2(t0, as_half2(xv[m][j][c].x), d);
+            d = dot2(t1, as_half2(xv[m][j][c].y), d);
+            d = dot2(t2, as_half2(xv[m][j][c].z), d);
+            d = dot2(t3, as_half2(xv[m][j][c].w), d);
+            grp[m] = d;
+          }
+        }
+        const float sf = active[j] ? (float)f.s[r][j] : 0.0f;
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[r][m] = fmaf(sf, grp[m], acc[r][m]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+      for (int m = 0; m < MB; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
+
+    auto finish = [&](float v, int r, int m) {
       const int n = n0 + r;
-      if (n >= N) break;
-#pragma unroll
-      for (int m = 0; m < MB; ++m) {
-        float v = acc[r][m];
+      if (n < N) {
         if (bias) v += (float)bias[n];
         half_t h = (half_t)v;
         if (residual) h = h + residual[(int64_t)m * N + n];
         y[(int64_t)m * N + n] = h;
       }
+    };
+    if (parts == 1) {
+      if (lane == 63 && set_ok) {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+          for (int m = 0; m < MB; ++m) finish(acc[r][m], r, m);
+      }
+    } else {
+      // partial sums cross wavefronts through LDS; the buffer alternates between
+      // turns so that one barrier per turn is enough
+      float(*rb)[ROWS * MB] = red[turn & 1];
+      if (lane == 63) {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+          for (int m = 0; m < MB; ++m) rb[wave][r * MB + m] = acc[r][m];
+      }
+      __syncthreads();
+      if (part == 0 && lane < ROWS * MB && set_ok) {
+        float v = 0.0f;
+        for (int w = 0; w < parts; ++w) v += rb[wave + w][lane];
+        finish(v, lane / MB, lane % MB);
+      }
     }
+    ++turn;
+  };
+
+  // ---- 6. the workgroup's turns, loads of the next turn in flight during this one ----
+  // `base` is uniform over the workgroup, so every wavefront takes the same number of turns.
+  while (true) {
+    if (base >= nsets) break;
+    if (base + stride < nsets) load(fb, base + stride);
+    process(fa, base);
+    base += stride;
+    if (base >= nsets) break;
+    if (base + stride < nsets) load(fa, base + stride);
+    process(fb, base);
+    base += stride;
   }
 }
 
-template <int R, int MB>
+static int g_gemv_rows = 0;  // 0 = choose from the shape
+static int g_gemv_gpl = 0;
+static int g_gemv_blocks_per_cu = 0;
+
+static int cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+template <int ROWS, int MB, int GPL>
 static int launch_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                        const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t N,
                        int64_t K, hipStream_t stream) {
-  const size_t lds = (size_t)MB * K * 2;
-  const int64_t blocks = (N + kGemvWaves * R - 1) / (kGemvWaves * R);
-  auto kern = q4g32_gemv_kernel<R, MB>;
-  if (lds > 64 * 1024) {
+  const int G = (int)(K / 32);
+  const int parts = (G + 64 * GPL - 1) / (64 * GPL);
+  const int sets_per_block = parts >= 4 ? 1 : 4 / parts;
+  const int threads = 64 * parts * sets_per_block;
+  if (parts > kGemvMaxWaves || threads > gemv_max_threads<GPL>())
+    return fail(WQ_EUNSUPPORTED, "wq_q4g32_gemv: K=%lld needs %d threads per row set", (long long)K,
+                threads);
+  const int64_t nsets = (N + ROWS - 1) / ROWS;
+  int64_t blocks = (nsets + sets_per_block - 1) / sets_per_block;
+  // Very tall matrices run persistent workgroups that take several turns, with the
+  // loads of the next turn in flight during the current one; for the usual sizes
+  // every workgroup takes a single turn (measured to be slightly faster).
+  const int64_t cap = (int64_t)cu_count() * (g_gemv_blocks_per_cu ? g_gemv_blocks_per_cu : 32);
+  if (blocks > cap) blocks = cap;
+  if (K > 8 * 8 * (int64_t)threads)
+    return fail(WQ_EUNSUPPORTED, "wq_q4g32_gemv: K=%lld too large for %d threads", (long long)K,
+                threads);
+  const size_t lds = (size_t)MB * K * 2 + (size_t)MB * G * 4;
+  auto kern = q4g32_gemv_kernel<ROWS, MB, GPL>;
+  if (lds > 60 * 1024) {
     WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kGemvThreads), lds, stream,
-                     (const uint4_t*)W, (const half_t*)S, (const half_t*)x, (const half_t*)bias,
-                     (const half_t*)residual, (half_t*)y, (int)N, (int)K);
-  WQ_CHECK_LAUNCH("wq_q4g32_gemv");
+  WQ_LAUNCH("wq_q4g32_gemv", kern, dim3((unsigned)blocks), dim3(threads), lds, stream, (const uint4_t*)W, (const half_t*)S, (const half_t*)x,
+            (const half_t*)bias, (const half_t*)residual, (half_t*)y, (int)N, (int)K, parts,
+            (int)nsets);
   return WQ_OK;
 }
 
+template <int MB, int GPL>
+static int launch_gemv_rows(int rows, const uint32_t* W, const uint16_t* S, const uint16_t* x,
+                            const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t N,
+                            int64_t K, hipStream_t stream) {
+  switch (rows) {
+    case 1: return launch_gemv<1, MB, GPL>(W, S, x, bias, residual, y, N, K, stream);
+    case 2: return launch_gemv<2, MB, GPL>(W, S, x, bias, residual, y, N, K, stream);
+    default: return launch_gemv<4, MB, GPL>(W, S, x, bias, residual, y, N, K, stream);
+  }
+}
+
 }  // namespace wq
+
+// Launch-shape overrides for measurement: rows per row set, groups per lane and
+// resident workgroups per CU (0 = automatic).
+extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemv_config(int rows, int gpl) {
+  wq::g_gemv_rows = rows;
+  wq::g_gemv_gpl = gpl;
+}
+extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemv_blocks_per_cu(int n) {
+  wq::g_gemv_blocks_per_cu = n;
+}
 
 extern "C" int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                              const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M,
@@ -140,25 +357,35 @@ extern "C" int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_
   WQ_REQUIRE(K > 0, "wq_q4g32_gemv: K must be positive");
   WQ_REQUIRE(W && S && x && y, "wq_q4g32_gemv: null pointer");
   WQ_REQUIRE(aligned16(W) && aligned16(x), "wq_q4g32_gemv: W and x must be 16-byte aligned");
-  WQ_REQUIRE(N < (1ll << 31) && K <= 32768,
+  WQ_REQUIRE(N < (1ll << 30) && K <= 32768,
              "wq_q4g32_gemv: N=%lld K=%lld outside the supported range (K <= 32768)",
              (long long)N, (long long)K);
-  // batches of up to 4 rows share one pass over the weights
+  const int G = (int)(K / 32);
+  // groups per lane: one wavefront covers a whole row when K <= 64*32*GPL
+  // (rows longer than 256 groups are split over several wavefronts)
+  int gpl = g_gemv_gpl ? g_gemv_gpl
+                       : (G <= 64 ? 1 : G <= 128 ? 2 : G <= 192 ? 3 : G <= 256 ? 4 : G <= 384 ? 3 : 2);
+  const int rows = g_gemv_rows ? g_gemv_rows : 2;
+  // batches of up to 4 rows of x share one pass over the weights
   for (int64_t m0 = 0; m0 < M;) {
     const int64_t left = M - m0;
     const uint16_t* xp = x + m0 * K;
     const uint16_t* rp = residual ? residual + m0 * N : nullptr;
     uint16_t* yp = y + m0 * N;
     int rc;
-    if (left >= 4 && K <= 16384) {
-      rc = launch_gemv<2, 4>(W, S, xp, bias, rp, yp, N, K, stream);
+    if (left >= 4) {
+      rc = launch_gemv_rows<4, 1>(rows > 2 ? 2 : rows, W, S, xp, bias, rp, yp, N, K, stream);
       m0 += 4;
     } else if (left >= 2) {
-      rc = launch_gemv<2, 2>(W, S, xp, bias, rp, yp, N, K, stream);
+      rc = gpl >= 2 ? launch_gemv_rows<2, 2>(rows, W, S, xp, bias, rp, yp, N, K, stream)
+                    : launch_gemv_rows<2, 1>(rows, W, S, xp, bias, rp, yp, N, K, stream);
       m0 += 2;
     } else {
-      rc = N >= 8192 ? launch_gemv<4, 1>(W, S, xp, bias, rp, yp, N, K, stream)
-                     : launch_gemv<2, 1>(W, S, xp, bias, rp, yp, N, K, stream);
+      rc = gpl == 1   ? launch_gemv_rows<1, 1>(rows, W, S, xp, bias, rp, yp, N, K, stream)
+           : gpl == 2 ? launch_gemv_rows<1, 2>(rows, W, S, xp, bias, rp, yp, N, K, stream)
+           : gpl == 3 ? launch_gemv_rows<1, 3>(rows, W, S, xp, bias, rp, yp, N, K, stream)
+           : gpl == 4 ? launch_gemv_rows<1, 4>(rows, W, S, xp, bias, rp, yp, N, K, stream)
+                      : launch_gemv_rows<1, 6>(rows, W, S, xp, bias, rp, yp, N, K, stream);
       m0 += 1;
     }
     if (rc != WQ_OK) return rc;

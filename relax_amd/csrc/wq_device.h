@@ -23,6 +23,15 @@ __device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cas
 __device__ __forceinline__ half_t as_half(uint16_t u) { return __builtin_bit_cast(half_t, u); }
 __device__ __forceinline__ uint16_t as_u16(half_t h) { return __builtin_bit_cast(uint16_t, h); }
 
+// (a & mask) | bits in one VALU instruction.  The compiler prefers two VOP2
+// instructions with literal operands; v_and_or_b32 (VOP3, no literals on gfx9)
+// needs the constants in registers: `mask` in an SGPR, `bits` in a VGPR.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(bits));
+  return r;
+}
+
 // ---------------------------------------------------------------------------
 // Format A: one uint32 holds 8 codes, code i in bits 4i..4i+3.
 // (w >> 4i) & 0x000F000F isolates code i in the low half-word and code i+4 in the
@@ -35,7 +44,7 @@ __device__ __forceinline__ void q4_word_minus7(uint32_t w, half2_t out[4]) {
   const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    uint32_t t = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+    uint32_t t = and_or(w >> (4 * i), 0x000F000Fu, 0x64006400u);
     out[i] = as_half2(t) - off;
   }
 }

@@ -24,10 +24,13 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
     if (!(cond)) return ::wq::fail(WQ_EINVAL, __VA_ARGS__);    \
   } while (0)
 
-// Checks the launch that was just enqueued (hipGetLastError catches bad grids /
-// missing code objects without synchronising).
-#define WQ_CHECK_LAUNCH(what)                                                              \
+// Launches `kernel` and reports a failed launch (bad grid, missing code object)
+// without synchronising.  The thread's sticky error is cleared first so that an
+// error left behind by an unrelated earlier HIP call is not blamed on this launch.
+#define WQ_LAUNCH(what, kernel, grid, block, lds, stream, ...)                              \
   do {                                                                                     \
+    (void)hipGetLastError();                                                               \
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                     \
     hipError_t e_ = hipGetLastError();                                                     \
     if (e_ != hipSuccess)                                                                  \
       return ::wq::fail(WQ_EDEVICE, "%s: launch failed: %s", what, hipGetErrorString(e_)); \
