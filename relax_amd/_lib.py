@@ -23,11 +23,11 @@ SIGNATURES = {
     "wq_q4g32_linear": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_gemv": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
-    #TODO "wq_ft_preprocess_weight_host": [_vp, _vp, _i64, _i64, _i64, _int, _int],
-    #TODO "wq_ft_preprocess_weight": [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp],
-    #TODO "wq_intb_dequantize": [_vp, _vp, _vp, _i64, _i64, _int, _i64, _vp],
-    #TODO "wq_fpA_intB_gemm": [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
-    #TODO "wq_fpA_intB_gemm_residual": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
+    "wq_ft_preprocess_weight_host": [_vp, _vp, _i64, _i64, _i64, _int, _int],
+    "wq_ft_preprocess_weight": [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp],
+    "wq_intb_dequantize": [_vp, _vp, _vp, _i64, _i64, _int, _i64, _vp],
+    "wq_fpA_intB_gemm": [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
+    "wq_fpA_intB_gemm_residual": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
     "wq_activation_from_string": [ctypes.c_char_p],
     "wq_binary_op_from_string": [ctypes.c_char_p],
     "wq_unary_op_from_string": [ctypes.c_char_p],

@@ -1,0 +1,158 @@
+// Format B GEMM entry points: fp16 activations x preprocessed int8 / int4 weights,
+// the MI355X-native counterpart of fastertransformer::gemm_fp16_int_bias_act and
+// gemm_fp16_int_bias_act_residual (call sites python/tvm/contrib/cutlass/gemm_operation.py:441-458).
+// m <= 4 goes to the streaming GEMV (intb_gemv.hip); larger m to the shared MFMA
+// GEMM (mfma_gemm.h) with the weight loaders below.
+#include "intb_common.h"
+#include "mfma_gemm.h"
+
+int wq_gemm_cfg_override();
+
+namespace wq {
+
+// Per K-step (one 64-row tile) lane (j, h) needs k = 32h..32h+31 of column n.
+// int8: two 16-byte pieces (16 k each) at ((n/2)*(K/64) + ks)*8 + (n%2)*4 + 2h (16-byte units);
+// int4: one 16-byte piece (32 k) at ((n/4)*(K/64) + ks)*8 + (n%4)*2 + h.
+// Both come out in natural k order, so the activations are stored unpermuted.
+template <int NBIT>
+struct IntbLoader {
+  static constexpr bool kPairA = false;
+  static constexpr int kPieces = NBIT == 8 ? 2 : 1;
+  struct Args {
+    const uint4_t* B;
+    const half_t* scales;
+    int group;  // 0 = per column, 64 = one scale per K-step
+  };
+  struct Lane {
+    const uint4_t* w;
+    const half_t* s;  // per column: &scales[n]; fine-grained: &scales[n] with row stride N
+    int N;
+  };
+  struct Frag {
+    uint4_t w[kPieces];
+    half_t s;
+  };
+  __device__ static void init(Lane& l, const Args& a, int n, int lh, int K, int N) {
+    constexpr int I = NBIT == 8 ? 2 : 4;
+    l.w = a.B + ((int64_t)(n / I) * (K >> 6)) * 8 + (n % I) * (8 / I) + lh * kPieces;
+    l.s = a.scales + n;
+    l.N = N;
+  }
+  __device__ static void load(Frag& f, const Lane& l, const Args& a, int ks, int, int, bool) {
+#pragma unroll
+    for (int p = 0; p < kPieces; ++p) f.w[p] = l.w[(int64_t)ks * 8 + p];
+    f.s = a.group ? l.s[(int64_t)ks * l.N] : l.s[0];
+  }
+  __device__ static void dequant(const Frag& f, half8_t out[4]) {
+    const half2_t s2 = {f.s, f.s};
+    if (NBIT == 8) {
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const uint32_t w[4] = {f.w[p].x, f.w[p].y, f.w[p].z, f.w[p].w};
+        half2_t lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          lo[j] = u8x2_to_half2(w[j], 0x04020400u) * s2;  // k = 2j, 2j+1
+          hi[j] = u8x2_to_half2(w[j], 0x04030401u) * s2;  // k = 2j+8, 2j+9
+        }
+        out[2 * p] = half8_t{lo[0].x, lo[0].y, lo[1].x, lo[1].y, lo[2].x, lo[2].y, lo[3].x, lo[3].y};
+        out[2 * p + 1] = half8_t{hi[0].x, hi[0].y, hi[1].x, hi[1].y, hi[2].x, hi[2].y, hi[3].x, hi[3].y};
+      }
+    } else {
+      const uint32_t w[4] = {f.w[0].x, f.w[0].y, f.w[0].z, f.w[0].w};
+      half2_t d[4][4];  // d[j][i] = (k = 2j+8i, 2j+8i+1)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u4_word_minus8(w[j], d[j]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) d[j][i] = d[j][i] * s2;
+      }
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+        out[kk] = half8_t{d[0][kk].x, d[0][kk].y, d[1][kk].x, d[1][kk].y,
+                          d[2][kk].x, d[2][kk].y, d[3][kk].x, d[3][kk].y};
+    }
+  }
+};
+
+// act(acc + bias) [binary residual] [unary], all in fp32, one rounding at the store
+struct IntbGemmEpilogue {
+  IntbEpilogue e;
+  int N;
+  __device__ half_t operator()(float v, int m, int n) const {
+    if (e.bias) v += (float)e.bias[e.bias_stride ? (int64_t)m * e.bias_stride + n : n];
+    v = apply_activation(v, e.activation);
+    if (e.residual) {
+      const float r = (float)e.residual[(int64_t)m * N + n];
+      if (e.binary_op == 1) v += r;
+      if (e.binary_op == 2) v *= r;
+    }
+    if (e.unary_op == 1) v = v > 0.0f ? v : 0.0f;
+    return (half_t)v;
+  }
+};
+
+static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
+                            const uint16_t* scales, const uint16_t* bias, const uint16_t* residual,
+                            uint16_t* C, int activation, int binary_op, int unary_op, int64_t m,
+                            int64_t n, int64_t k, int64_t group_size, int64_t bias_stride,
+                            int nbit, hipStream_t stream) {
+  WQ_REQUIRE(nbit == 8 || nbit == 4, "%s: weight_nbit must be 8 or 4, got %d", who, nbit);
+  WQ_REQUIRE(m >= 0 && n >= 0 && k >= 0, "%s: negative dimension", who);
+  WQ_REQUIRE(k % 64 == 0 && n % 64 == 0, "%s: k=%lld and n=%lld must be multiples of 64", who,
+             (long long)k, (long long)n);
+  WQ_REQUIRE(activation >= 0 && activation <= 3, "%s: unknown activation %d", who, activation);
+  WQ_REQUIRE(binary_op >= 0 && binary_op <= 2 && unary_op >= 0 && unary_op <= 1,
+             "%s: unknown binary_op %d / unary_op %d", who, binary_op, unary_op);
+  WQ_REQUIRE(group_size <= 0 || group_size == 64 || group_size == k,
+             "%s: group_size must be 64 (fine-grained) or <= 0 / k (per column), got %lld", who,
+             (long long)group_size);
+  WQ_REQUIRE(bias_stride == 0 || bias_stride >= n, "%s: bias_stride %lld smaller than n", who,
+             (long long)bias_stride);
+  if (m == 0 || n == 0) return WQ_OK;
+  WQ_REQUIRE(k > 0, "%s: k must be positive", who);
+  WQ_REQUIRE(A && B && scales && C, "%s: null pointer", who);
+  WQ_REQUIRE(binary_op == 0 || residual, "%s: binary_op needs a residual tensor", who);
+  WQ_REQUIRE(aligned16(A) && aligned16(B), "%s: A and B must be 16-byte aligned", who);
+  WQ_REQUIRE(m < (1ll << 30) && n < (1ll << 30) && k < (1ll << 30), "%s: too large", who);
+  const int group = (group_size > 0 && group_size != k) ? 64 : 0;
+  const IntbEpilogue ep{(const half_t*)bias, binary_op ? (const half_t*)residual : nullptr,
+                        bias_stride, activation, binary_op, unary_op};
+  if (m <= 4 && wq_gemm_cfg_override() == 0)
+    return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
+  const int cfg = wq_gemm_cfg_override() ? wq_gemm_cfg_override() : choose_gemm_cfg(m, n);
+  const IntbGemmEpilogue gep{ep, (int)n};
+  if (nbit == 8) {
+    const IntbLoader<8>::Args bargs{(const uint4_t*)B, (const half_t*)scales, group};
+    return launch_mfma_gemm_cfg<IntbLoader<8>, IntbGemmEpilogue>(cfg, who, bargs, A, C, gep, m, n, k, stream);
+  }
+  const IntbLoader<4>::Args bargs{(const uint4_t*)B, (const half_t*)scales, group};
+  return launch_mfma_gemm_cfg<IntbLoader<4>, IntbGemmEpilogue>(cfg, who, bargs, A, C, gep, m, n, k, stream);
+}
+
+}  // namespace wq
+
+extern "C" int wq_fpA_intB_gemm(const uint16_t* A, const int8_t* B, const uint16_t* scales,
+                                const uint16_t* bias, uint16_t* C, int activation, int64_t m,
+                                int64_t n, int64_t k, int64_t group_size, int64_t bias_stride,
+                                int weight_nbit, void* /*workspace*/, size_t /*workspace_bytes*/,
+                                wq_stream_t stream) {
+  return wq::intb_gemm_common("wq_fpA_intB_gemm", A, B, scales, bias, nullptr, C, activation,
+                              WQ_BIN_NONE, WQ_UN_IDENTITY, m, n, k, group_size, bias_stride,
+                              weight_nbit, (hipStream_t)stream);
+}
+
+extern "C" int wq_fpA_intB_gemm_residual(const uint16_t* A, const int8_t* B, const uint16_t* scales,
+                                         const uint16_t* bias, const uint16_t* residual,
+                                         uint16_t* C, int activation, int binary_op, int unary_op,
+                                         int64_t m, int64_t n, int64_t k, int64_t group_size,
+                                         int weight_nbit, void* /*workspace*/,
+                                         size_t /*workspace_bytes*/, wq_stream_t stream) {
+  if (!residual)
+    return wq::fail(WQ_EINVAL, "wq_fpA_intB_gemm_residual: residual must not be null");
+  if (binary_op != WQ_BIN_PLUS && binary_op != WQ_BIN_MULTIPLY)
+    return wq::fail(WQ_EINVAL, "wq_fpA_intB_gemm_residual: binary_op must be plus or multiply");
+  return wq::intb_gemm_common("wq_fpA_intB_gemm_residual", A, B, scales, bias, residual, C,
+                              activation, binary_op, unary_op, m, n, k, group_size, 0, weight_nbit,
+                              (hipStream_t)stream);
+}

@@ -42,23 +42,6 @@
 
 namespace wq {
 
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_shift(float v) {
-  return __builtin_bit_cast(
-      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
-}
-
-// Sum over the wavefront; the total is valid in lane 63.
-__device__ __forceinline__ float wave_sum_to_lane63(float v) {
-  v += dpp_shift<0x111, 0xf>(v);  // row_shr:1
-  v += dpp_shift<0x112, 0xf>(v);  // row_shr:2
-  v += dpp_shift<0x114, 0xf>(v);  // row_shr:4
-  v += dpp_shift<0x118, 0xf>(v);  // row_shr:8   -> lane 15 of each row holds the row sum
-  v += dpp_shift<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-  v += dpp_shift<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-  return v;
-}
-
 constexpr int kGemvMaxWaves = 16;
 
 // Few groups per lane means more wavefronts share a row: allow larger workgroups there.

@@ -74,6 +74,29 @@ __device__ __forceinline__ void pair_i_i4(const uint32_t in[4], uint32_t out[4])
   out[3] = __builtin_amdgcn_perm(in[3], in[1], 0x07060302u);  // (h3, h7)
 }
 
+// v shifted / permuted across lanes by a DPP control word; lanes without a source get 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_shift(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
+}
+// quad_perm: 0xb1 = [1,0,3,2] (xor 1), 0x4e = [2,3,0,1] (xor 2)
+template <int CTRL>
+__device__ __forceinline__ float dpp_quad(float v) {
+  return dpp_shift<CTRL, 0xf>(v);
+}
+
+// Sum over the wavefront; the total is valid in lane 63.
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v += dpp_shift<0x111, 0xf>(v);  // row_shr:1
+  v += dpp_shift<0x112, 0xf>(v);  // row_shr:2
+  v += dpp_shift<0x114, 0xf>(v);  // row_shr:4
+  v += dpp_shift<0x118, 0xf>(v);  // row_shr:8   -> lane 15 of each row holds the row sum
+  v += dpp_shift<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_shift<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Sum over the 64 lanes of a wavefront; every lane receives the total.
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -111,3 +111,106 @@ def q4g32_linear(W: torch.Tensor, S: torch.Tensor, x: torch.Tensor, bias: Option
     check(fn(_ptr(W), _ptr(S), _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), M, N, K, _stream()),
           f"wq_q4g32_{kernel}")
     return out
+
+
+# ----------------------------------------------------------------- format B
+
+
+def ft_preprocess_weight(packed_weight: torch.Tensor, sm: int, is_int4: bool) -> torch.Tensor:
+    """``cutlass.ft_preprocess_weight(packed_weight, sm, is_int4)``
+    (src/runtime/contrib/cutlass/weight_preprocess.cc:38-59): returns a new tensor of the same
+    shape, dtype and device holding the reordered weight.  ``packed_weight`` is int8 ``[K, N]``,
+    ``[K, N/2]`` (int4) or ``[E, K, N(/2)]``.  Host tensors are reordered on the host, device
+    tensors by a device kernel (no round trip through host memory)."""
+    w = packed_weight
+    if not isinstance(w, torch.Tensor) or w.dtype != torch.int8:
+        raise ValueError("packed_weight must be an int8 tensor")
+    if w.dim() not in (2, 3):
+        raise ValueError("packed_weight must be [K, N] or [E, K, N]")
+    if not w.is_contiguous():
+        raise ValueError("packed_weight must be compact (contiguous)")
+    E = 1 if w.dim() == 2 else w.shape[0]
+    rows, cols = w.shape[-2], w.shape[-1] * (2 if is_int4 else 1)
+    out = torch.empty_like(w)
+    if w.is_cuda:
+        check(_lib.lib().wq_ft_preprocess_weight(_ptr(out), _ptr(w), E, rows, cols, int(bool(is_int4)), int(sm),
+                                                 _stream()), "wq_ft_preprocess_weight")
+    else:
+        check(_lib.lib().wq_ft_preprocess_weight_host(_ptr(out), _ptr(w), E, rows, cols, int(bool(is_int4)),
+                                                      int(sm)), "wq_ft_preprocess_weight_host")
+    return out
+
+
+def _intb_dims(B: torch.Tensor, nbit: int):
+    if nbit not in (4, 8):
+        raise ValueError("weight_nbit must be 4 or 8")
+    B = _dev(B, torch.int8, "B")
+    if B.dim() != 2:
+        raise ValueError("B must be [K, N] or [K, N/2]")
+    K, c = B.shape
+    return B, K, c * (2 if nbit == 4 else 1)
+
+
+def intb_dequantize(B: torch.Tensor, scales: torch.Tensor, weight_nbit: int, group_size: int = -1) -> torch.Tensor:
+    """fp16 ``[K, N]`` dequantized weight from the PREPROCESSED layout, bit-identical to the
+    reference's ``decode`` PrimFunc applied to the original packed weight."""
+    B, K, N = _intb_dims(B, weight_nbit)
+    scales = _dev(scales, torch.float16, "scales")
+    want = N if group_size <= 0 or group_size == K else (K // group_size) * N
+    if scales.numel() != want:
+        raise ValueError(f"scales must have {want} elements, got {scales.numel()}")
+    out = torch.empty((K, N), dtype=torch.float16, device=B.device)
+    check(_lib.lib().wq_intb_dequantize(_ptr(B), _ptr(scales), _ptr(out), K, N, weight_nbit, group_size, _stream()),
+          "wq_intb_dequantize")
+    return out
+
+
+def fpA_intB_gemm(x: torch.Tensor, B: torch.Tensor, scales: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                  residual: Optional[torch.Tensor] = None, *, weight_nbit: int, activation: str = "identity",
+                  binary_op: str = "plus", unary_op: str = "identity", group_size: int = -1,
+                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The fused ``decode -> matmul [-> bias] [-> activation] [-> residual op [-> relu]]`` composite
+    (python/tvm/relax/backend/contrib/cutlass.py:271-314, 344-372), arguments in the composite's
+    order ``(x, w_preprocessed, scales, [bias], [residual])``.  ``m = prod(x.shape[:-1])``,
+    ``bias_stride = 0`` for a bias that only varies along N, else ``bias.shape[-1]``
+    (python/tvm/contrib/cutlass/build.py:722-734)."""
+    B, K, N = _intb_dims(B, weight_nbit)
+    x = _dev(x, torch.float16, "x")
+    scales = _dev(scales, torch.float16, "scales")
+    if x.shape[-1] != K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {K}")
+    M = x.numel() // K
+    want = N if group_size <= 0 or group_size == K else (K // group_size) * N
+    if scales.numel() != want:
+        raise ValueError(f"scales must have {want} elements, got {scales.numel()}")
+    bias_stride = 0
+    if bias is not None:
+        bias = _dev(bias, torch.float16, "bias")
+        if bias.shape[-1] != N:
+            raise ValueError("bias last dim must be N")
+        if bias.numel() != N:
+            if bias.numel() != M * N:
+                raise ValueError("bias must have N or M*N elements")
+            bias_stride = N
+    if residual is not None:
+        residual = _dev(residual, torch.float16, "residual")
+        if residual.numel() != M * N:
+            raise ValueError("residual must have M*N elements")
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (N,), dtype=torch.float16, device=x.device)
+    else:
+        out = _dev(out, torch.float16, "out")
+        if out.numel() != M * N:
+            raise ValueError("out must have M*N elements")
+    L = _lib.lib()
+    if residual is None:
+        check(L.wq_fpA_intB_gemm(_ptr(x), _ptr(B), _ptr(scales), _ptr(bias), _ptr(out), ACTIVATIONS[activation],
+                                 M, N, K, group_size, bias_stride, weight_nbit, 0, 0, _stream()), "wq_fpA_intB_gemm")
+    else:
+        if bias_stride:
+            raise ValueError("the residual form takes a bias that only varies along N")
+        check(L.wq_fpA_intB_gemm_residual(_ptr(x), _ptr(B), _ptr(scales), _ptr(bias), _ptr(residual), _ptr(out),
+                                          ACTIVATIONS[activation], BINARY_OPS[binary_op], UNARY_OPS[unary_op],
+                                          M, N, K, group_size, weight_nbit, 0, 0, _stream()),
+              "wq_fpA_intB_gemm_residual")
+    return out

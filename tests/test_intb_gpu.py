@@ -1,0 +1,186 @@
+"""GPU parity of the format-B (fp16 x int8/int4) path against the CPU oracle, through the C ABI."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "ft_layout_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need a GPU"
+    from relax_amd import ops as _ops
+
+    return _ops
+
+
+@pytest.fixture(scope="module")
+def u():
+    from tests import gpu_util
+
+    return gpu_util
+
+
+@pytest.mark.parametrize("case", ["int8_64x64", "int8_128x192", "int8_256x64", "int4_64x64", "int4_128x192", "int4_256x128"])
+def test_device_preprocess_matches_golden(ops, u, case):
+    g = np.load(GOLD)
+    a, want = g[case + "_in"], g[case + "_out"]
+    got = u.host(ops.ft_preprocess_weight(u.dev(a), 80, case.startswith("int4")))
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("is_int4", [False, True])
+def test_device_preprocess_large_and_experts(ops, u, oracle, is_int4):
+    rng = np.random.default_rng(17)
+    a = rng.integers(-128, 128, size=(2, 512, 320)).astype(np.int8)
+    got = u.host(ops.ft_preprocess_weight(u.dev(a), 80, is_int4))
+    assert np.array_equal(got, oracle.ft_preprocess(a, is_int4, 80))
+    a = rng.integers(-128, 128, size=(8192, 1024 if not is_int4 else 512)).astype(np.int8)
+    got = u.host(ops.ft_preprocess_weight(u.dev(a), 80, is_int4))
+    assert np.array_equal(got, oracle.ft_preprocess(a, is_int4, 80))
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_dequant_exhaustive_bit_exact(ops, u, oracle, nbit):
+    """every code x every fp16 scale bit pattern, through preprocess + device dequantize."""
+    all_s = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(np.float16)
+    ncode = 256 if nbit == 8 else 16
+    lo = -128 if nbit == 8 else -8
+    K = 256  # codes repeat down the rows; K must be a multiple of 64
+    codes = (np.arange(K) % ncode + lo).astype(np.int64)
+    for start in range(0, 65536, 16384):
+        s = all_s[start:start + 16384]
+        N = s.size
+        q = np.repeat(codes[:, None], N, axis=1)
+        if nbit == 8:
+            A = q.astype(np.int8)
+        else:
+            A = ((q[:, 0::2] & 15) | ((q[:, 1::2] & 15) << 4)).astype(np.uint8).view(np.int8)
+        want = oracle.intb_dequant(A, s, nbit)
+        P = ops.ft_preprocess_weight(u.dev(A), 80, nbit == 4)
+        got = u.host(ops.intb_dequantize(P, u.dev(s), nbit))
+        nan = np.isnan(want)
+        assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+        assert np.all(np.isnan(got[nan]))
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_dequant_finegrained(ops, u, oracle, nbit):
+    _, A, s = oracle.make_intb_inputs(1, 128, 256, nbit, seed=4, group_size=64)
+    P = ops.ft_preprocess_weight(u.dev(A), 80, nbit == 4)
+    got = u.host(ops.intb_dequantize(P, u.dev(s), nbit, group_size=64))
+    assert np.array_equal(got.view(np.uint16), oracle.intb_dequant(A, s, nbit, 64).view(np.uint16))
+
+
+def _run(ops, u, oracle, M, N, K, nbit, seed, group_size=-1, **ep):
+    x, A, s = oracle.make_intb_inputs(M, N, K, nbit, seed=seed, group_size=group_size)
+    rng = np.random.default_rng(seed + 1)
+    kw, okw = {}, {}
+    if ep.get("bias") == "row":
+        b = rng.standard_normal(N).astype(np.float16)
+        kw["bias"], okw["bias"] = u.dev(b), b
+    elif ep.get("bias") == "full":
+        b = rng.standard_normal((M, N)).astype(np.float16)
+        kw["bias"], okw["bias"], okw["bias_stride"] = u.dev(b), b, N
+    if ep.get("residual"):
+        r = rng.standard_normal((M, N)).astype(np.float16)
+        kw["residual"], okw["residual"] = u.dev(r), r
+        kw["binary_op"] = okw["binary_op"] = ep.get("binary_op", "plus")
+        kw["unary_op"] = okw["unary_op"] = ep.get("unary_op", "identity")
+    act = ep.get("activation", "identity")
+    P = ops.ft_preprocess_weight(u.dev(A), 80, nbit == 4)
+    got = u.host(ops.fpA_intB_gemm(u.dev(x), P, u.dev(s), weight_nbit=nbit, activation=act, group_size=group_size, **kw))
+    ref = oracle.intb_linear(x, A, s, nbit, group_size=group_size, activation=act, nthreads=8, **okw)
+    u.assert_close(got, ref, f"intb nbit={nbit} M={M} N={N} K={K} g={group_size} {ep}")
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 16, 33, 128, 300])
+def test_gemm_vs_oracle_shapes(ops, u, oracle, nbit, M):
+    print(f"intb nbit={nbit} M={M}", flush=True)
+    _run(ops, u, oracle, M, 256, 512, nbit, seed=M)
+    _run(ops, u, oracle, M, 64, 64, nbit, seed=M + 50)
+    _run(ops, u, oracle, M, 192, 4096, nbit, seed=M + 100)
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+@pytest.mark.parametrize("M", [1, 4, 64])
+def test_gemm_finegrained(ops, u, oracle, nbit, M):
+    _run(ops, u, oracle, M, 128, 512, nbit, seed=M + 7, group_size=64)
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+@pytest.mark.parametrize("M", [2, 48])
+@pytest.mark.parametrize("ep", [
+    dict(bias="row"), dict(bias="full"), dict(bias="row", activation="relu"), dict(bias="row", activation="silu"),
+    dict(bias="row", activation="gelu"), dict(residual=True), dict(bias="row", residual=True, binary_op="plus"),
+    dict(bias="row", residual=True, binary_op="multiply", unary_op="relu"),
+    dict(bias="row", activation="silu", residual=True, binary_op="plus", unary_op="relu"),
+], ids=lambda d: "-".join(f"{k}={v}" for k, v in d.items()))
+def test_gemm_epilogues(ops, u, oracle, nbit, M, ep):
+    _run(ops, u, oracle, M, 128, 256, nbit, seed=M + 3, **ep)
+
+
+@pytest.mark.parametrize("M", [1, 16, 128, 512])
+def test_int8_full_size_sampled(ops, u, oracle, M):
+    """K=8192, N=28672 int8 per-channel.  The oracle checks a sample of output columns
+    (columns are independent given x), the one-hot test checks the layout end to end."""
+    import torch
+
+    K, N = 8192, 28672
+    rng = np.random.default_rng(M)
+    x = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+    dA = torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda")
+    s = rng.uniform(0.001, 0.01, size=N).astype(np.float16)
+    print(f"int8 full size M={M}", flush=True)
+    P = ops.ft_preprocess_weight(dA, 80, False)
+    got = u.host(ops.fpA_intB_gemm(u.dev(x), P, u.dev(s), weight_nbit=8))
+    cols = np.concatenate([np.arange(0, 64), np.arange(14000, 14064), np.arange(N - 64, N)])
+    A_cols = u.host(dA[:, torch.from_numpy(cols).cuda()].contiguous())
+    ref = oracle.intb_linear(x[: min(M, 8)], A_cols, s[cols], 8, nthreads=8)
+    u.assert_close(got[: min(M, 8)][:, cols], ref, f"int8 full M={M}")
+    if M == 1:
+        xh = np.zeros((1, K), np.float16)
+        xh[0, 4321] = 1
+        y = u.host(ops.fpA_intB_gemm(u.dev(xh), P, u.dev(s), weight_nbit=8))
+        want = (u.host(dA[4321]).astype(np.float16) * s)
+        assert np.array_equal(y[0].view(np.uint16), want.view(np.uint16))
+
+
+def test_reference_fixture_chain(ops, u, oracle):
+    """The reference's own small test case (tests/python/relax/test_codegen_cutlass.py:1559-1609):
+    np.random.seed(0); x = randn(64,64); y = normal(0, 0.002, (128,64)); bias = randn(1,128);
+    residual = randn(64,128); encode -> preprocess -> fused GEMM, compared with the UNQUANTIZED
+    np.dot(x, y.T) + bias (+ residual) at the reference's rtol = atol = 1e-2."""
+    np.random.seed(0)
+    x = np.random.randn(64, 64).astype("float16")
+    y = np.random.normal(0, 0.002, size=(128, 64)).astype("float16")
+    bias = np.random.randn(1, 128).astype("float16")
+    residual = np.random.randn(64, 128).astype("float16")
+    for nbit, tol in ((4, 1e-2), (8, 1e-2)):
+        w, s = oracle.intb_encode(y, nbit)
+        P = ops.ft_preprocess_weight(u.dev(w), 80, nbit == 4)
+        out = u.host(ops.fpA_intB_gemm(u.dev(x), P, u.dev(s), bias=u.dev(bias), weight_nbit=nbit))
+        ref = np.dot(x, y.transpose()) + bias
+        np.testing.assert_allclose(out, ref, rtol=tol, atol=tol)
+        out = u.host(ops.fpA_intB_gemm(u.dev(x), P, u.dev(s), bias=u.dev(bias), residual=u.dev(residual),
+                                       weight_nbit=nbit, binary_op="plus"))
+        np.testing.assert_allclose(out, ref + residual, rtol=tol, atol=tol)
+
+
+def test_argument_errors(ops, u, oracle):
+    from relax_amd._lib import WqError
+
+    x, A, s = oracle.make_intb_inputs(2, 64, 64, 8, seed=0)
+    P = ops.ft_preprocess_weight(u.dev(A), 80, False)
+    with pytest.raises(WqError, match="group_size"):
+        ops.fpA_intB_gemm(u.dev(x), P, u.dev(np.tile(s, 2)), weight_nbit=8, group_size=32)
+    with pytest.raises(ValueError):
+        ops.fpA_intB_gemm(u.dev(x[:, :32].copy()), P, u.dev(s), weight_nbit=8)
+    with pytest.raises(ValueError):
+        ops.fpA_intB_gemm(u.dev(x), P, u.dev(s[:10].copy()), weight_nbit=8)
