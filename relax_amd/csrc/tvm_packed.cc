@@ -1,0 +1,509 @@
+// PackedFunc layer: the symbols a Relax VM resolves by name (imported module
+// first, then the global registry: src/runtime/relax_vm/vm.cc:669-681) and calls
+// with TVMValue / type-code arrays.  Each one validates its DLTensors and
+// forwards plain pointers to the C ABI of relax_amd_wq.h.
+#include <dlfcn.h>
+
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/relax_amd_tvm.h"
+#include "wq_host.h"
+
+namespace wq {
+namespace {
+
+// ---- optional services of a host TVM runtime, looked up once with dlsym ----
+struct HostRuntime {
+  void (*set_last_error)(const char*) = nullptr;
+  int (*func_create)(TVMPackedCFunc, void*, TVMPackedCFuncFinalizer, TVMFunctionHandle*) = nullptr;
+  int (*func_register)(const char*, TVMFunctionHandle, int) = nullptr;
+  int (*func_get_global)(const char*, TVMFunctionHandle*) = nullptr;
+  int (*func_call)(TVMFunctionHandle, TVMValue*, int*, int, TVMValue*, int*) = nullptr;
+  int (*set_return)(TVMRetValueHandle, TVMValue*, int*, int) = nullptr;
+  int (*array_alloc)(const tvm_index_t*, int, int, int, int, int, int, TVMArrayHandle*) = nullptr;
+  bool present = false;
+};
+
+HostRuntime& host() {
+  static HostRuntime h = [] {
+    HostRuntime r;
+    auto sym = [](const char* n) { return dlsym(RTLD_DEFAULT, n); };
+    r.set_last_error = reinterpret_cast<decltype(r.set_last_error)>(sym("TVMAPISetLastError"));
+    r.func_create = reinterpret_cast<decltype(r.func_create)>(sym("TVMFuncCreateFromCFunc"));
+    r.func_register = reinterpret_cast<decltype(r.func_register)>(sym("TVMFuncRegisterGlobal"));
+    r.func_get_global = reinterpret_cast<decltype(r.func_get_global)>(sym("TVMFuncGetGlobal"));
+    r.func_call = reinterpret_cast<decltype(r.func_call)>(sym("TVMFuncCall"));
+    r.set_return = reinterpret_cast<decltype(r.set_return)>(sym("TVMCFuncSetReturn"));
+    r.array_alloc = reinterpret_cast<decltype(r.array_alloc)>(sym("TVMArrayAlloc"));
+    r.present = r.func_create && r.func_register;
+    return r;
+  }();
+  return h;
+}
+
+wq_stream_getter_t g_stream_getter = nullptr;
+
+// The stream a PackedFunc call enqueues on.
+void* current_stream() {
+  if (g_stream_getter) return g_stream_getter();
+  HostRuntime& h = host();
+  if (h.func_get_global && h.func_call) {
+    static TVMFunctionHandle getter = [&h]() -> TVMFunctionHandle {
+      TVMFunctionHandle f = nullptr;
+      if (h.func_get_global("runtime.get_rocm_stream", &f) != 0) return nullptr;
+      return f;
+    }();
+    if (getter) {
+      TVMValue ret;
+      int tcode = kTVMNullptr;
+      ret.v_handle = nullptr;
+      if (h.func_call(getter, nullptr, nullptr, 0, &ret, &tcode) == 0 && tcode != kTVMNullptr)
+        return ret.v_handle;
+    }
+  }
+  return nullptr;  // the null stream
+}
+
+// Reports an error the way a PackedFunc must: message to the runtime, -1 to the caller.
+int packed_fail() {
+  HostRuntime& h = host();
+  if (h.set_last_error) h.set_last_error(wq_last_error());
+  return -1;
+}
+
+struct Tensor {
+  const DLTensor* t = nullptr;
+  void* ptr = nullptr;  // data + byte_offset
+  int64_t numel = 1;
+};
+
+bool is_compact(const DLTensor* t) {
+  if (!t->strides) return true;
+  int64_t expect = 1;
+  for (int i = t->ndim - 1; i >= 0; --i) {
+    if (t->shape[i] != 1 && t->strides[i] != expect) return false;
+    expect *= t->shape[i];
+  }
+  return true;
+}
+
+// Fetches argument i as a tensor of the given dtype; returns false with the error set.
+bool get_tensor(const char* who, TVMValue* args, int* tcodes, int num_args, int i, int code, int bits,
+                const char* what, Tensor* out, bool allow_host = false) {
+  if (i >= num_args) {
+    fail(WQ_EINVAL, "%s: missing argument %d (%s)", who, i, what);
+    return false;
+  }
+  if (tcodes[i] != kTVMDLTensorHandle && tcodes[i] != kTVMNDArrayHandle) {
+    fail(WQ_EINVAL, "%s: argument %d (%s) is not a tensor (type code %d)", who, i, what, tcodes[i]);
+    return false;
+  }
+  const DLTensor* t = static_cast<const DLTensor*>(args[i].v_handle);
+  if (!t) {
+    fail(WQ_EINVAL, "%s: argument %d (%s) is null", who, i, what);
+    return false;
+  }
+  if (t->dtype.code != code || t->dtype.bits != bits || t->dtype.lanes != 1) {
+    fail(WQ_EINVAL, "%s: %s has dtype (code %d, %d bits, %d lanes), expected (code %d, %d bits)", who,
+         what, t->dtype.code, t->dtype.bits, t->dtype.lanes, code, bits);
+    return false;
+  }
+  const bool on_gpu = t->device.device_type == kDLROCM;
+  const bool on_host = t->device.device_type == kDLCPU || t->device.device_type == kDLROCMHost;
+  if (!(on_gpu || (allow_host && on_host))) {
+    fail(WQ_EINVAL, "%s: %s lives on device type %d; expected a ROCm device tensor", who, what,
+         (int)t->device.device_type);
+    return false;
+  }
+  if (!is_compact(t)) {
+    fail(WQ_EINVAL, "%s: %s must be compact (row-major, no strides)", who, what);
+    return false;
+  }
+  out->t = t;
+  out->ptr = static_cast<char*>(t->data) + t->byte_offset;
+  out->numel = 1;
+  for (int d = 0; d < t->ndim; ++d) out->numel *= t->shape[d];
+  return true;
+}
+
+bool get_int(const char* who, TVMValue* args, int* tcodes, int num_args, int i, const char* what,
+             int64_t* out) {
+  if (i >= num_args || tcodes[i] != kTVMArgInt) {
+    fail(WQ_EINVAL, "%s: argument %d (%s) must be an integer", who, i, what);
+    return false;
+  }
+  *out = args[i].v_int64;
+  return true;
+}
+
+int64_t leading(const DLTensor* t) {  // product of all dims but the last
+  int64_t m = 1;
+  for (int d = 0; d + 1 < t->ndim; ++d) m *= t->shape[d];
+  return m;
+}
+
+// ------------------------------------------------------------------ format A
+int q4_matmul(const char* who, TVMValue* args, int* tcodes, int n, bool has_bias, bool has_res) {
+  Tensor W, S, x, bias, res, y;
+  int i = 0;
+  if (n != 4 + (int)has_bias + (int)has_res) {
+    fail(WQ_EINVAL, "%s: expected %d arguments, got %d", who, 4 + (int)has_bias + (int)has_res, n);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, tcodes, n, i++, kDLUInt, 32, "W", &W)) return packed_fail();
+  if (!get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "S", &S)) return packed_fail();
+  if (!get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "x", &x)) return packed_fail();
+  if (has_bias && !get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "bias", &bias)) return packed_fail();
+  if (has_res && !get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "residual", &res)) return packed_fail();
+  if (!get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "out", &y)) return packed_fail();
+  if (W.t->ndim != 2 || S.t->ndim != 2 || x.t->ndim < 1 || y.t->ndim < 1) {
+    fail(WQ_EINVAL, "%s: W and S must be matrices", who);
+    return packed_fail();
+  }
+  const int64_t N = W.t->shape[0], K = W.t->shape[1] * 8;
+  const int64_t M = x.t->ndim ? leading(x.t) : 0;
+  if (S.t->shape[0] != N || S.t->shape[1] * 32 != K || x.t->shape[x.t->ndim - 1] != K ||
+      y.numel != M * N || y.t->shape[y.t->ndim - 1] != N || (has_bias && bias.numel != N) ||
+      (has_res && res.numel != M * N)) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (N=%lld K=%lld M=%lld)", who, (long long)N,
+         (long long)K, (long long)M);
+    return packed_fail();
+  }
+  const int rc = wq_q4g32_linear((const uint32_t*)W.ptr, (const uint16_t*)S.ptr, (const uint16_t*)x.ptr,
+                                 (const uint16_t*)bias.ptr, (const uint16_t*)res.ptr, (uint16_t*)y.ptr,
+                                 M, N, K, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
+// ------------------------------------------------------------------ format B
+// op_type follows python/tvm/contrib/cutlass/build.py:742-775: activation is looked up
+// between "matmul_" and "residual_", the residual postfix gives binary / unary op.
+struct DecodeMatmulOp {
+  bool has_bias, has_residual;
+  int activation, binary_op, unary_op;
+};
+
+DecodeMatmulOp parse_op_type(const std::string& op) {
+  DecodeMatmulOp r{};
+  r.has_bias = op.find("bias") != std::string::npos;
+  const size_t rpos = op.find("residual_");
+  r.has_residual = rpos != std::string::npos;
+  const size_t mpos = op.find("matmul");
+  const std::string head = op.substr(mpos, r.has_residual ? rpos - mpos : std::string::npos);
+  r.activation = WQ_ACT_IDENTITY;
+  for (const char* a : {"relu", "silu", "gelu"})
+    if (head.find(a) != std::string::npos) {
+      r.activation = wq_activation_from_string(a);
+      break;
+    }
+  r.binary_op = WQ_BIN_NONE;
+  r.unary_op = WQ_UN_IDENTITY;
+  if (r.has_residual) {
+    const std::string post = op.substr(rpos + strlen("residual_"));
+    r.binary_op = post.rfind("multiply", 0) == 0 ? WQ_BIN_MULTIPLY : WQ_BIN_PLUS;
+    r.unary_op = post.find("relu") != std::string::npos ? WQ_UN_RELU : WQ_UN_IDENTITY;
+  }
+  return r;
+}
+
+int decode_matmul(const char* op_type, TVMValue* args, int* tcodes, int n) {
+  const DecodeMatmulOp op = parse_op_type(op_type);
+  const char* who = op_type;
+  const int expect = 4 + (int)op.has_bias + (int)op.has_residual;
+  if (n != expect) {
+    fail(WQ_EINVAL, "%s: expected %d arguments (x, w, scales%s%s, out), got %d", who, expect,
+         op.has_bias ? ", bias" : "", op.has_residual ? ", residual" : "", n);
+    return packed_fail();
+  }
+  Tensor x, w, s, bias, res, out;
+  int i = 0;
+  if (!get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "x", &x)) return packed_fail();
+  if (!get_tensor(who, args, tcodes, n, i++, kDLInt, 8, "w_encoded", &w)) return packed_fail();
+  if (!get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "scales", &s)) return packed_fail();
+  if (op.has_bias && !get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "bias", &bias)) return packed_fail();
+  if (op.has_residual && !get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "residual", &res)) return packed_fail();
+  if (!get_tensor(who, args, tcodes, n, i++, kDLFloat, 16, "out", &out)) return packed_fail();
+  if (w.t->ndim != 2 || x.t->ndim < 1 || out.t->ndim < 1 || s.t->ndim < 1 || s.t->ndim > 2) {
+    fail(WQ_EINVAL, "%s: unexpected ranks", who);
+    return packed_fail();
+  }
+  const int64_t k = w.t->shape[0];
+  const int64_t N = out.t->shape[out.t->ndim - 1];
+  int nbit;
+  if (N == w.t->shape[1]) {
+    nbit = 8;
+  } else if (N == 2 * w.t->shape[1]) {
+    nbit = 4;
+  } else {
+    fail(WQ_EINVAL, "%s: output width %lld matches neither int8 nor int4 weight of width %lld", who,
+         (long long)N, (long long)w.t->shape[1]);
+    return packed_fail();
+  }
+  // group size: 64 when the scales are a matrix with more than one row, else per column
+  const int64_t group = (s.t->ndim == 2 && s.t->shape[0] != 1) ? 64 : -1;
+  const int64_t m = leading(x.t);
+  if (x.t->shape[x.t->ndim - 1] != k || out.numel != m * N ||
+      s.numel != (group > 0 ? (k / 64) * N : N) || (op.has_residual && res.numel != m * N)) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (m=%lld n=%lld k=%lld)", who, (long long)m,
+         (long long)N, (long long)k);
+    return packed_fail();
+  }
+  int64_t bias_stride = 0;
+  if (op.has_bias) {
+    if (bias.t->ndim < 1 || bias.t->shape[bias.t->ndim - 1] != N ||
+        (bias.numel != N && bias.numel != m * N)) {
+      fail(WQ_EINVAL, "%s: bias must have n or m*n elements with last dim n", who);
+      return packed_fail();
+    }
+    if (bias.numel != N) bias_stride = N;
+  }
+  void* stream = current_stream();
+  int rc;
+  if (op.has_residual) {
+    if (bias_stride) {
+      fail(WQ_EINVAL, "%s: the residual form takes a bias that only varies along n", who);
+      return packed_fail();
+    }
+    rc = wq_fpA_intB_gemm_residual((const uint16_t*)x.ptr, (const int8_t*)w.ptr, (const uint16_t*)s.ptr,
+                                   (const uint16_t*)bias.ptr, (const uint16_t*)res.ptr,
+                                   (uint16_t*)out.ptr, op.activation, op.binary_op, op.unary_op, m, N,
+                                   k, group, nbit, nullptr, 0, stream);
+  } else {
+    rc = wq_fpA_intB_gemm((const uint16_t*)x.ptr, (const int8_t*)w.ptr, (const uint16_t*)s.ptr,
+                          (const uint16_t*)bias.ptr, (uint16_t*)out.ptr, op.activation, m, N, k, group,
+                          bias_stride, nbit, nullptr, 0, stream);
+  }
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
+// ---------------------------------------------------------- weight reordering
+int preprocess_into(const char* who, const Tensor& in, int64_t sm, int64_t is_int4, void* out_ptr) {
+  const DLTensor* t = in.t;
+  if (t->ndim != 2 && t->ndim != 3) {
+    fail(WQ_EINVAL, "%s: packed_weight must be [K, N] or [E, K, N]", who);
+    return -1;
+  }
+  const bool is_2d = t->ndim == 2;
+  const int64_t experts = is_2d ? 1 : t->shape[0];
+  const int64_t rows = t->shape[is_2d ? 0 : 1];
+  int64_t cols = t->shape[is_2d ? 1 : 2];
+  if (is_int4) cols *= 2;  // "cols" counts unpacked elements (weight_preprocess.cc:48-50)
+  int rc;
+  if (t->device.device_type == kDLROCM)
+    rc = wq_ft_preprocess_weight((int8_t*)out_ptr, (const int8_t*)in.ptr, experts, rows, cols,
+                                 (int)is_int4, (int)sm, current_stream());
+  else
+    rc = wq_ft_preprocess_weight_host((int8_t*)out_ptr, (const int8_t*)in.ptr, experts, rows, cols,
+                                      (int)is_int4, (int)sm);
+  return rc == WQ_OK ? 0 : -1;
+}
+
+}  // namespace
+}  // namespace wq
+
+using namespace wq;
+
+extern "C" {
+
+WQ_PACKED(cutlass_ft_preprocess_weight) {
+  (void)resource_handle;
+  const char* who = "cutlass.ft_preprocess_weight";
+  Tensor in;
+  int64_t sm = 0, is_int4 = 0;
+  if (num_args != 3) {
+    fail(WQ_EINVAL, "%s: expected (packed_weight, sm, is_int4)", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLInt, 8, "packed_weight", &in, true) ||
+      !get_int(who, args, type_codes, num_args, 1, "sm", &sm) ||
+      !get_int(who, args, type_codes, num_args, 2, "is_int4", &is_int4))
+    return packed_fail();
+  HostRuntime& h = host();
+  if (!h.array_alloc) {
+    fail(WQ_EUNSUPPORTED,
+         "%s: no TVM runtime in this process to allocate the result; call "
+         "relax_amd.ft_preprocess_weight_dps(packed_weight, sm, is_int4, out) instead",
+         who);
+    return packed_fail();
+  }
+  TVMArrayHandle out = nullptr;
+  const DLTensor* t = in.t;
+  if (h.array_alloc(t->shape, t->ndim, t->dtype.code, t->dtype.bits, t->dtype.lanes,
+                    (int)t->device.device_type, t->device.device_id, &out) != 0 || !out) {
+    fail(WQ_EDEVICE, "%s: TVMArrayAlloc failed", who);
+    return packed_fail();
+  }
+  if (preprocess_into(who, in, sm, is_int4, static_cast<char*>(out->data) + out->byte_offset) != 0)
+    return packed_fail();
+  // ownership of the new array moves to the caller (packed_func.h:975-982)
+  out_ret_value->v_handle = out;
+  *out_ret_tcode = kTVMNDArrayHandle;
+  return 0;
+}
+
+WQ_PACKED(relax_amd_ft_preprocess_weight_dps) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.ft_preprocess_weight_dps";
+  Tensor in, out;
+  int64_t sm = 0, is_int4 = 0;
+  if (num_args != 4) {
+    fail(WQ_EINVAL, "%s: expected (packed_weight, sm, is_int4, out)", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLInt, 8, "packed_weight", &in, true) ||
+      !get_int(who, args, type_codes, num_args, 1, "sm", &sm) ||
+      !get_int(who, args, type_codes, num_args, 2, "is_int4", &is_int4) ||
+      !get_tensor(who, args, type_codes, num_args, 3, kDLInt, 8, "out", &out, true))
+    return packed_fail();
+  if (out.numel != in.numel || out.t->device.device_type != in.t->device.device_type) {
+    fail(WQ_EINVAL, "%s: out must match packed_weight in size and device", who);
+    return packed_fail();
+  }
+  return preprocess_into(who, in, sm, is_int4, out.ptr) == 0 ? 0 : packed_fail();
+}
+
+WQ_PACKED(relax_amd_q4f16_1_matmul) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  return q4_matmul("relax_amd.q4f16_1_matmul", args, type_codes, num_args, false, false);
+}
+WQ_PACKED(relax_amd_q4f16_1_matmul_bias) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  return q4_matmul("relax_amd.q4f16_1_matmul_bias", args, type_codes, num_args, true, false);
+}
+WQ_PACKED(relax_amd_q4f16_1_matmul_bias_residual) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  return q4_matmul("relax_amd.q4f16_1_matmul_bias_residual", args, type_codes, num_args, true, true);
+}
+WQ_PACKED(relax_amd_q4f16_1_decode) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.q4f16_1_decode";
+  Tensor W, S, out;
+  if (num_args != 3) {
+    fail(WQ_EINVAL, "%s: expected (W, S, out)", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W", &W) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "S", &S) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLFloat, 16, "out", &out))
+    return packed_fail();
+  if (W.t->ndim != 2 || S.t->ndim != 2 || S.t->shape[0] != W.t->shape[0] ||
+      S.t->shape[1] * 4 != W.t->shape[1] || out.numel != W.numel * 8) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes", who);
+    return packed_fail();
+  }
+  const int rc = wq_q4g32_dequantize((const uint32_t*)W.ptr, (const uint16_t*)S.ptr, (uint16_t*)out.ptr,
+                                     W.t->shape[0], W.t->shape[1] * 8, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
+#define WQ_DECODE_MATMUL(sym, op)                                       \
+  WQ_PACKED(sym) {                                                      \
+    (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;    \
+    return decode_matmul(op, args, type_codes, num_args);               \
+  }
+#define WQ_DECODE_MATMUL_LIST(X)                                                                     \
+  X(relax_amd_decode_matmul, "decode_matmul")                                                        \
+  X(relax_amd_decode_matmul_bias, "decode_matmul_bias")                                              \
+  X(relax_amd_decode_matmul_cast, "decode_matmul_cast")                                              \
+  X(relax_amd_decode_matmul_cast_bias, "decode_matmul_cast_bias")                                    \
+  X(relax_amd_decode_matmul_bias_gelu, "decode_matmul_bias_gelu")                                    \
+  X(relax_amd_decode_matmul_cast_bias_gelu, "decode_matmul_cast_bias_gelu")                          \
+  X(relax_amd_decode_matmul_bias_residual_add, "decode_matmul_bias_residual_add")                    \
+  X(relax_amd_decode_matmul_bias_residual_multiply, "decode_matmul_bias_residual_multiply")          \
+  X(relax_amd_decode_matmul_bias_residual_add_relu, "decode_matmul_bias_residual_add_relu")          \
+  X(relax_amd_decode_matmul_bias_residual_multiply_relu, "decode_matmul_bias_residual_multiply_relu") \
+  X(relax_amd_decode_matmul_cast_bias_residual_add, "decode_matmul_cast_bias_residual_add")          \
+  X(relax_amd_decode_matmul_cast_bias_residual_multiply, "decode_matmul_cast_bias_residual_multiply") \
+  X(relax_amd_decode_matmul_cast_bias_residual_add_relu, "decode_matmul_cast_bias_residual_add_relu") \
+  X(relax_amd_decode_matmul_cast_bias_residual_multiply_relu,                                        \
+    "decode_matmul_cast_bias_residual_multiply_relu")                                                \
+  X(relax_amd_decode_matmul_bias_gelu_residual_add, "decode_matmul_bias_gelu_residual_add")          \
+  X(relax_amd_decode_matmul_bias_gelu_residual_multiply, "decode_matmul_bias_gelu_residual_multiply") \
+  X(relax_amd_decode_matmul_bias_gelu_residual_add_relu, "decode_matmul_bias_gelu_residual_add_relu") \
+  X(relax_amd_decode_matmul_bias_gelu_residual_multiply_relu,                                        \
+    "decode_matmul_bias_gelu_residual_multiply_relu")                                                \
+  X(relax_amd_decode_matmul_cast_bias_gelu_residual_add, "decode_matmul_cast_bias_gelu_residual_add") \
+  X(relax_amd_decode_matmul_cast_bias_gelu_residual_multiply,                                        \
+    "decode_matmul_cast_bias_gelu_residual_multiply")                                                \
+  X(relax_amd_decode_matmul_cast_bias_gelu_residual_add_relu,                                        \
+    "decode_matmul_cast_bias_gelu_residual_add_relu")                                                \
+  X(relax_amd_decode_matmul_cast_bias_gelu_residual_multiply_relu,                                   \
+    "decode_matmul_cast_bias_gelu_residual_multiply_relu")
+
+WQ_DECODE_MATMUL_LIST(WQ_DECODE_MATMUL)
+
+}  // extern "C"
+
+namespace {
+
+struct Entry {
+  std::string name;    // dotted global-registry name
+  const char* symbol;  // exported C symbol
+  WqTVMBackendPackedCFunc fn;
+};
+
+const std::vector<Entry>& table() {
+  static const std::vector<Entry> t = [] {
+    std::vector<Entry> v;
+    v.push_back({"cutlass.ft_preprocess_weight", "cutlass_ft_preprocess_weight", cutlass_ft_preprocess_weight});
+    v.push_back({"relax_amd.ft_preprocess_weight_dps", "relax_amd_ft_preprocess_weight_dps",
+                 relax_amd_ft_preprocess_weight_dps});
+    v.push_back({"relax_amd.q4f16_1_matmul", "relax_amd_q4f16_1_matmul", relax_amd_q4f16_1_matmul});
+    v.push_back({"relax_amd.q4f16_1_matmul_bias", "relax_amd_q4f16_1_matmul_bias", relax_amd_q4f16_1_matmul_bias});
+    v.push_back({"relax_amd.q4f16_1_matmul_bias_residual", "relax_amd_q4f16_1_matmul_bias_residual",
+                 relax_amd_q4f16_1_matmul_bias_residual});
+    v.push_back({"relax_amd.q4f16_1_decode", "relax_amd_q4f16_1_decode", relax_amd_q4f16_1_decode});
+#define WQ_ENTRY(sym, op) v.push_back({std::string("relax_amd.") + op, #sym, sym});
+    WQ_DECODE_MATMUL_LIST(WQ_ENTRY)
+#undef WQ_ENTRY
+    return v;
+  }();
+  return t;
+}
+
+// Adapter from the registry's TVMPackedCFunc (return through TVMCFuncSetReturn) to the
+// exported-symbol signature (return through out pointers).
+int registry_trampoline(TVMValue* args, int* type_codes, int num_args, TVMRetValueHandle ret,
+                        void* resource_handle) {
+  const Entry* e = static_cast<const Entry*>(resource_handle);
+  TVMValue rv;
+  rv.v_handle = nullptr;
+  int rcode = kTVMNullptr;
+  const int rc = e->fn(args, type_codes, num_args, &rv, &rcode, nullptr);
+  if (rc != 0) return rc;
+  if (rcode != kTVMNullptr) {
+    wq::HostRuntime& h = wq::host();
+    if (!h.set_return) return -1;
+    return h.set_return(ret, &rv, &rcode, 1);
+  }
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int wq_tvm_num_functions(void) { return (int)table().size(); }
+extern "C" const char* wq_tvm_function_name(int i) {
+  return i >= 0 && i < (int)table().size() ? table()[i].name.c_str() : nullptr;
+}
+extern "C" const char* wq_tvm_function_symbol(int i) {
+  return i >= 0 && i < (int)table().size() ? table()[i].symbol : nullptr;
+}
+extern "C" void wq_tvm_set_stream_getter(wq_stream_getter_t getter) { wq::g_stream_getter = getter; }
+
+extern "C" int wq_tvm_register_globals(void) {
+  wq::HostRuntime& h = wq::host();
+  if (!h.present) return 0;
+  int n = 0;
+  for (const Entry& e : table()) {
+    TVMFunctionHandle f = nullptr;
+    if (h.func_create(registry_trampoline, const_cast<Entry*>(&e), nullptr, &f) != 0) return -1;
+    if (h.func_register(e.name.c_str(), f, /*override=*/1) != 0) return -1;
+    ++n;
+  }
+  return n;
+}
+
+// Registers with a TVM runtime that is already in the process when the library is loaded.
+__attribute__((constructor)) static void wq_tvm_autoregister() { (void)wq_tvm_register_globals(); }

@@ -1,0 +1,111 @@
+"""The PackedFunc symbols on device tensors: arguments marshalled as the Relax VM does
+(TVMValue[] + type codes, NDArray handles), results against the CPU oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+
+    assert torch.cuda.is_available()
+    from relax_amd import _lib
+    from tests import gpu_util, tvm_abi_util
+
+    lib = _lib.lib()
+    # kernels go to torch's current stream, supplied through the stream-getter hook
+    getter_t = ctypes.CFUNCTYPE(ctypes.c_void_p)
+    getter = getter_t(lambda: torch.cuda.current_stream().cuda_stream)
+    lib.wq_tvm_set_stream_getter(getter)
+    yield lib, gpu_util, tvm_abi_util, torch
+    lib.wq_tvm_set_stream_getter(None)
+
+
+def test_q4f16_1_matmul_family(env, oracle):
+    lib, u, T, torch = env
+    M, N, K = 3, 200, 512
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=3)
+    rng = np.random.default_rng(1)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    dW, dS, dx, db, dr = u.dev(W), u.dev(S), u.dev(x.reshape(M, 1, K)), u.dev(bias), u.dev(res.reshape(M, 1, N))
+    y = torch.empty((M, 1, N), dtype=torch.float16, device="cuda")
+    tW, _ = T.from_torch(dW, "uint32")
+    tS, _ = T.from_torch(dS)
+    tx, _ = T.from_torch(dx)
+    tb, _ = T.from_torch(db)
+    tr, _ = T.from_torch(dr)
+    ty, _ = T.from_torch(y)
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_matmul, tW, tS, tx, ty)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y).reshape(M, N), oracle.q4g32_linear(W, S, x), "packed q4 matmul")
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_matmul_bias_residual, tW, tS, tx, tb, tr, ty)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y).reshape(M, N), oracle.q4g32_linear(W, S, x, bias=bias, residual=res), "packed q4 epilogue")
+    # prefill-sized M goes to the MFMA kernel through the same symbol
+    M2 = 96
+    x2 = rng.standard_normal((M2, K)).astype(np.float16)
+    dx2 = u.dev(x2)
+    y2 = torch.empty((M2, N), dtype=torch.float16, device="cuda")
+    tx2, _ = T.from_torch(dx2)
+    ty2, _ = T.from_torch(y2)
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_matmul_bias, tW, tS, tx2, tb, ty2)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y2), oracle.q4g32_linear(W, S, x2, bias=bias, nthreads=4), "packed q4 prefill")
+    # decode alone, bit-exact
+    dq = torch.empty((N, K), dtype=torch.float16, device="cuda")
+    tq, _ = T.from_torch(dq)
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_decode, tW, tS, tq)
+    assert rc == 0
+    assert np.array_equal(u.host(dq).view(np.uint16), oracle.q4g32_dequant(W, S).view(np.uint16))
+    # shape errors come back as -1 with a message
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_matmul, tW, tS, tx2, ty)
+    assert rc == -1 and b"inconsistent" in lib.wq_last_error()
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_decode_matmul_composites(env, oracle, nbit):
+    lib, u, T, torch = env
+    M, N, K = 48, 128, 256
+    x, A, s = oracle.make_intb_inputs(M, N, K, nbit, seed=nbit)
+    rng = np.random.default_rng(2)
+    bias = rng.standard_normal((1, N)).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    dA = u.dev(A)
+    # weight reordering through the DPS PackedFunc on device tensors
+    P = torch.empty_like(dA)
+    tA, _ = T.from_torch(dA)
+    tP, _ = T.from_torch(P)
+    rc, _, _ = T.call(lib.relax_amd_ft_preprocess_weight_dps, tA, 80, int(nbit == 4), tP)
+    assert rc == 0, lib.wq_last_error()
+    assert np.array_equal(u.host(P), oracle.ft_preprocess(A, nbit == 4, 80))
+    dx, ds, db, dr = u.dev(x), u.dev(s.reshape(1, N)), u.dev(bias), u.dev(res)
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    tx, _ = T.from_torch(dx)
+    ts, _ = T.from_torch(ds)
+    tb, _ = T.from_torch(db)
+    tr, _ = T.from_torch(dr)
+    to, _ = T.from_torch(out)
+    cases = [
+        ("relax_amd_decode_matmul", (tx, tP, ts, to), {}),
+        ("relax_amd_decode_matmul_cast_bias", (tx, tP, ts, tb, to), dict(bias=bias)),
+        ("relax_amd_decode_matmul_bias_gelu", (tx, tP, ts, tb, to), dict(bias=bias, activation="gelu")),
+        ("relax_amd_decode_matmul_bias_residual_add", (tx, tP, ts, tb, tr, to), dict(bias=bias, residual=res, binary_op="plus")),
+        ("relax_amd_decode_matmul_bias_gelu_residual_multiply_relu", (tx, tP, ts, tb, tr, to),
+         dict(bias=bias, activation="gelu", residual=res, binary_op="multiply", unary_op="relu")),
+    ]
+    for sym, args, okw in cases:
+        rc, _, _ = T.call(getattr(lib, sym), *args)
+        assert rc == 0, (sym, lib.wq_last_error())
+        ref = oracle.intb_linear(x, A, s, nbit, nthreads=4, **{k: (v.reshape(-1) if k == "bias" else v) for k, v in okw.items()})
+        u.assert_close(u.host(out), ref, sym)
+    # a bias that varies along M selects bias_stride = N (python/tvm/contrib/cutlass/build.py:728-734)
+    bias2 = rng.standard_normal((M, N)).astype(np.float16)
+    tb2, _ = T.from_torch(u.dev(bias2))
+    rc, _, _ = T.call(lib.relax_amd_decode_matmul_bias, tx, tP, ts, tb2, to)
+    assert rc == 0
+    u.assert_close(u.host(out), oracle.intb_linear(x, A, s, nbit, bias=bias2, bias_stride=N, nthreads=4), "full bias")
