@@ -173,3 +173,22 @@ def test_registers_with_a_tvm_runtime_when_present(tmp_path):
     out = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
     assert "registry ok" in out.stdout
+
+
+def test_source_compatible_headers_compile_and_run(tmp_path, lib):
+    """Host code written against cutlass_kernels/*.h of the reference's external library
+    compiles against include/ and links the shared library (host-only call, no GPU)."""
+    exe = tmp_path / "ft_api_host"
+    libdir = os.path.join(ROOT, "relax_amd")
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-I", INC, os.path.join(ROOT, "tests", "cpp", "ft_api_host.cc"),
+                           "-o", str(exe), "-L", libdir, "-lrelax_amd_wq", f"-Wl,-rpath,{libdir}",
+                           "-Wl,-rpath,/opt/rocm/lib"])
+    g = np.load(GOLD)
+    for case, is_int4 in (("int8_256x64", 0), ("int4_256x128", 1)):
+        a, want = g[case + "_in"], g[case + "_out"]
+        fin, fout = tmp_path / "in.bin", tmp_path / "out.bin"
+        a.tofile(fin)
+        rows, cols = a.shape[0], a.shape[1] * (2 if is_int4 else 1)
+        r = subprocess.run([str(exe), str(fin), str(fout), str(rows), str(cols), str(is_int4)], capture_output=True, text=True)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert np.array_equal(np.fromfile(fout, np.int8).reshape(a.shape), want)
