@@ -120,7 +120,7 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
                         bias_stride, activation, binary_op, unary_op};
   if (m <= 4 && wq_gemm_cfg_override() == 0)
     return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
-  const int cfg = wq_gemm_cfg_override() ? wq_gemm_cfg_override() : choose_gemm_cfg(m, n);
+  const int cfg = wq_gemm_cfg_override() ? wq_gemm_cfg_override() : choose_gemm_cfg(m, n, false);
   const IntbGemmEpilogue gep{ep, (int)n};
   if (nbit == 8) {
     const IntbLoader<8>::Args bargs{(const uint4_t*)B, (const half_t*)scales, group};

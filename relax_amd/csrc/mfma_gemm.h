@@ -223,9 +223,12 @@ static int launch_mfma_gemm_cfg(int cfg, const char* who, const typename Loader:
   }
 }
 
-inline int choose_gemm_cfg(int64_t M, int64_t N) {
+// Default tile shape: 64x128 for small M, else 128x256 — for format A the fully
+// LDS-staged kernel (12), which falls back to the register-staged one (2) when the
+// shape is not eligible; the other shapes are kept for measurement.
+inline int choose_gemm_cfg(int64_t M, int64_t N, bool lds_staged) {
   (void)N;
-  return M <= 64 ? 3 : 2;
+  return M <= 64 ? 3 : lds_staged ? 12 : 2;
 }
 
 }  // namespace wq

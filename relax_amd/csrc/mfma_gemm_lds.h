@@ -1,0 +1,268 @@
+// Format A prefill GEMM, fully LDS-staged variant for the gfx950 matrix cores:
+//   y[m,n] = epilogue( sum_k x[m,k] * ((code[n,k] - 7) * S[n,k/32]) )
+//
+// Every operand of a K-step (64 k) travels global -> LDS with the direct
+// global_load_lds_dwordx4 path: no staging registers, no VALU work, and the loads
+// of step ks+2 are in flight while step ks is multiplied (3-slot ring).  Per slot:
+//   A   BM rows x 128 B of activations, 16-byte chunk c of row r at slot position
+//       c ^ ((r >> 1) & 7) (the swizzle is applied to the GLOBAL address each lane fetches,
+//       because the LDS side of a direct load is fixed: lane l writes 16 bytes at
+//       base + 16*l);
+//   B   BN rows x 32 B of packed codes (8 words), chunk (n, h) at (2n + h) * 16;
+//   S   BN rows x 4 B: the two scales of the step.
+// A wavefront then reads, per K-step, TM*4 activation fragments, and per weight
+// sub-tile ONE 16-byte piece of codes plus one scale: MFMA lane (j, h) needs 8
+// K-values of column j, which is one packed word, so the weights are dequantized
+// in registers (q4_word_dequant_natural: bit-exact, natural K order, hence no
+// rearrangement of the activations) and never exist in LDS as fp16.
+//
+// Synchronisation per K-step: issue the loads of step ks+2; multiply step ks;
+// s_waitcnt vmcnt(loads of one step) — vector memory operations retire in order,
+// so this wavefront's loads of step ks+1 have landed; s_barrier — so have everyone
+// else's, and everyone is done reading slot ks%3, which the next iteration refills.
+// (A raw s_barrier is used: the fence in __syncthreads would force vmcnt(0).)
+#ifndef RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
+#define RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
+
+#include "wq_device.h"
+#include "wq_host.h"
+
+namespace wq {
+
+template <int TM, int TN, int WM, int WN>
+struct LdsGemmCfg {
+  static_assert(WM * WN == 4, "four wavefronts per workgroup");
+  static constexpr int kThreads = 256;
+  static constexpr int BM = 32 * TM * WM;
+  static constexpr int BN = 32 * TN * WN;
+  static constexpr int kStages = 3;
+  static constexpr int kAOff = 0;
+  static constexpr int kBOff = BM * 128;
+  static constexpr int kSOff = kBOff + BN * 32;
+  static constexpr int kStageBytes = kSOff + BN * 4;
+  static constexpr int kLdsBytes = kStages * kStageBytes;
+  static constexpr int kALoads = BM / 32;   // direct loads per wavefront per step (64 chunks each)
+  static constexpr int kBLoads = BN / 128;
+  static_assert(BN % 128 == 0 && BN <= 256, "B tile: 128 or 256 columns");
+  static constexpr int kLoadsPerStage = kALoads + kBLoads + 1;
+};
+
+// XOR pattern of the activation tile: consecutive rows alternate between the two
+// 128-byte halves of the bank space, so pairs of rows share one pattern value.
+#define WQ_SWZ(r) (((r) >> 1) & 7)
+#define WQ_WAITCNT_VM(n) __builtin_amdgcn_s_waitcnt(((n)&0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+typedef const void __attribute__((address_space(1))) * wq_gptr_t;
+typedef void __attribute__((address_space(3))) * wq_lptr_t;
+
+template <class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU, bool INTERLEAVE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restrict__ S,
+                           const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epilogue,
+                           int M, int N, int K, int tiles_m, int tiles_n) {
+  using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int lj = lane & 31, lh = lane >> 5;
+
+  // XCD-aware tile order: each XCD (own L2) gets a contiguous range, walked M-fastest.
+  const int nblk = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  {
+    const int per = nblk / 8, rem = nblk % 8;
+    const int xcd = pid & 7, idx = pid >> 3;
+    pid = xcd * per + min(xcd, rem) + idx;
+  }
+  const int tile_m = pid % tiles_m, tile_n = pid / tiles_m;
+  const int m0 = tile_m * Cfg::BM, n0 = tile_n * Cfg::BN;
+  const int G = K >> 5;
+  const int ksteps = K >> 6;
+
+  // ---- global sources of this lane's direct loads (rows past M / N are clamped:
+  //      they only feed accumulators that are never stored) ----
+  const char* a_src[Cfg::kALoads];
+#pragma unroll
+  for (int i = 0; i < Cfg::kALoads; ++i) {
+    const int s = (wave * Cfg::kALoads + i) * 64 + lane;  // LDS chunk slot
+    const int r = s >> 3, c = (s & 7) ^ WQ_SWZ(r);
+    a_src[i] = reinterpret_cast<const char*>(X + (int64_t)min(m0 + r, M - 1) * K) + c * 16;
+  }
+  const char* b_src[Cfg::kBLoads];
+#pragma unroll
+  for (int i = 0; i < Cfg::kBLoads; ++i) {
+    const int q = (wave * Cfg::kBLoads + i) * 64 + lane;
+    const int n = q >> 1, h = q & 1;
+    b_src[i] = reinterpret_cast<const char*>(W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
+  }
+  // (with BN = 128 wavefronts 2 and 3 repeat the loads of wavefronts 0 and 1)
+  const int s_row = (wave * 64) % Cfg::BN + lane;
+  const char* s_src = reinterpret_cast<const char*>(S + (int64_t)min(n0 + s_row, N - 1) * G);
+
+  auto issue_loads = [&](int ks) {
+    unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
+#pragma unroll
+    for (int i = 0; i < Cfg::kALoads; ++i)
+      __builtin_amdgcn_global_load_lds((wq_gptr_t)(a_src[i] + (int64_t)ks * 128),
+                                       (wq_lptr_t)(slot + Cfg::kAOff + (wave * Cfg::kALoads + i) * 1024),
+                                       16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < Cfg::kBLoads; ++i)
+      __builtin_amdgcn_global_load_lds((wq_gptr_t)(b_src[i] + (int64_t)ks * 32),
+                                       (wq_lptr_t)(slot + Cfg::kBOff + (wave * Cfg::kBLoads + i) * 1024),
+                                       16, 0, 0);
+    __builtin_amdgcn_global_load_lds((wq_gptr_t)(s_src + (int64_t)ks * 4),
+                                     (wq_lptr_t)(slot + Cfg::kSOff + (wave * 64 % Cfg::BN) * 4), 4, 0, 0);
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.0f;
+
+  auto compute = [&](int ks) {
+    const unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
+    // this lane's packed weights and scale for the whole step
+    uint4_t bw[TN];
+    half_t bs[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+      const int n = (wn * TN + t) * 32 + lj;
+      bw[t] = *reinterpret_cast<const uint4_t*>(slot + Cfg::kBOff + (n * 2 + lh) * 16);
+      bs[t] = *reinterpret_cast<const half_t*>(slot + Cfg::kSOff + n * 4 + lh * 2);
+    }
+    auto read_a = [&](int kk, half8_t (&aop)[TM]) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row = (wm * TM + i) * 32 + lj;
+        aop[i] = *reinterpret_cast<const half8_t*>(slot + Cfg::kAOff + row * 128 +
+                                                   (((4 * lh + kk) ^ WQ_SWZ(row)) << 4));
+      }
+    };
+    auto dequant_b = [&](int kk, half8_t (&bop)[TN]) {
+#pragma unroll
+      for (int t = 0; t < TN; ++t) {
+        const uint32_t word = kk == 0 ? bw[t].x : kk == 1 ? bw[t].y : kk == 2 ? bw[t].z : bw[t].w;
+        const half2_t s2 = {bs[t], bs[t]};
+        half2_t d[4];
+        q4_word_dequant_natural(word, s2, d);
+        bop[t] = half8_t{d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
+      }
+    };
+    half8_t aop[2][TM], bop[2][TN];
+    read_a(0, aop[0]);
+    dequant_b(0, bop[0]);
+    if (!INTERLEAVE) {
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        // operands of column kk+1 are fetched / dequantized before the MFMAs of column kk
+        if (kk < 3) {
+          read_a(kk + 1, aop[(kk + 1) & 1]);
+          dequant_b(kk + 1, bop[(kk + 1) & 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int t = 0; t < TN; ++t)
+            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[kk & 1][i], bop[kk & 1][t],
+                                                               acc[i][t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      // One wavefront per SIMD: nothing else hides VALU time, so the dequantization of
+      // column kk+1 is cut into pairs (5 VALU instructions each) and one pair is issued
+      // after each MFMA of column kk; up to ~5 VALU instructions fit under one MFMA.
+      static_assert(!INTERLEAVE || TM * TN >= TN * 4, "need at least one MFMA per weight pair");
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const int cur = kk & 1, nxt = cur ^ 1;
+        if (kk < 3) read_a(kk + 1, aop[nxt]);
+        half2_t dq[TN][4];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int t = 0; t < TN; ++t) {
+            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[cur][i], bop[cur][t], acc[i][t], 0, 0, 0);
+            const int slice = i * TN + t;  // 0 .. TM*TN-1
+            if (kk < 3 && slice < TN * 4) {
+              const int tt = slice >> 2, j = slice & 3;
+              const uint32_t word = kk + 1 == 1 ? bw[tt].y : kk + 1 == 2 ? bw[tt].z : bw[tt].w;
+              const half2_t s2 = {bs[tt], bs[tt]};
+              dq[tt][j] = q4_pair_dequant_natural(word, j, s2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        if (kk < 3) {
+#pragma unroll
+          for (int t = 0; t < TN; ++t)
+            bop[nxt][t] = half8_t{dq[t][0].x, dq[t][0].y, dq[t][1].x, dq[t][1].y,
+                                  dq[t][2].x, dq[t][2].y, dq[t][3].x, dq[t][3].y};
+        }
+      }
+    }
+  };
+
+  issue_loads(0);
+  if (ksteps > 1) {
+    issue_loads(1);
+    WQ_WAITCNT_VM(Cfg::kLoadsPerStage);
+  } else {
+    WQ_WAITCNT_VM(0);
+  }
+  __builtin_amdgcn_s_barrier();
+
+  for (int ks = 0; ks < ksteps; ++ks) {
+    const bool ahead2 = ks + 2 < ksteps;
+    if (ahead2) issue_loads(ks + 2);
+    compute(ks);
+    if (ahead2) {
+      WQ_WAITCNT_VM(Cfg::kLoadsPerStage);
+    } else {
+      WQ_WAITCNT_VM(0);
+    }
+    __builtin_amdgcn_s_barrier();
+  }
+
+  // ---- epilogue ----
+  // accumulator register r of lane (j, h) is element (row 8*(r/4) + 4*h + r%4, col j)
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    const int n = n0 + (wn * TN + t) * 32 + lj;
+    if (n >= N) continue;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+        if (m < M) Y[(int64_t)m * N + n] = epilogue(acc[i][t][r], m, n);
+      }
+    }
+  }
+}
+
+template <class Epilogue, int TM, int TN, int WM, int WN, int WPE, bool INTERLEAVE = false>
+static int launch_q4g32_gemm_lds(const uint32_t* W, const uint16_t* S, const uint16_t* x, uint16_t* y,
+                                 const Epilogue& ep, int64_t M, int64_t N, int64_t K,
+                                 hipStream_t stream) {
+  using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
+  const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM);
+  const int tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
+  auto kern = q4g32_gemm_lds_kernel<Epilogue, TM, TN, WM, WN, WPE, INTERLEAVE>;
+  WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
+  WQ_LAUNCH("wq_q4g32_gemm", kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), Cfg::kLdsBytes,
+            stream, W, (const half_t*)S, (const half_t*)x, (half_t*)y, ep, (int)M, (int)N, (int)K,
+            tiles_m, tiles_n);
+  return WQ_OK;
+}
+
+}  // namespace wq
+#endif  // RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_

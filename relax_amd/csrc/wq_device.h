@@ -58,6 +58,27 @@ __device__ __forceinline__ void q4_word_dequant(uint32_t w, half2_t s2, half2_t 
   for (int i = 0; i < 4; ++i) out[i] = d[i] * s2;
 }
 
+// Same value as q4_word_dequant but in NATURAL order: out[j] = (w_{2j}, w_{2j+1}).
+// One instruction more per pair (shift, shift-or to move the odd code into the high
+// half-word, and-or); used where rearranging the other operand would cost more.
+__device__ __forceinline__ void q4_word_dequant_natural(uint32_t w, half2_t s2, half2_t out[4]) {
+  const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t t = (w >> (8 * j)) & 0xFFu;  // codes 2j, 2j+1 in bits 0..7 (v_bfe_u32)
+    const uint32_t u = (t << 12) | t;           // code 2j+1 also in bits 16..19
+    out[j] = (as_half2(and_or(u, 0x000F000Fu, 0x64006400u)) - off) * s2;
+  }
+}
+
+// One pair of the above: (w_{2j}, w_{2j+1}).
+__device__ __forceinline__ half2_t q4_pair_dequant_natural(uint32_t w, int j, half2_t s2) {
+  const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+  const uint32_t t = (w >> (8 * j)) & 0xFFu;
+  const uint32_t u = (t << 12) | t;
+  return (as_half2(and_or(u, 0x000F000Fu, 0x64006400u)) - off) * s2;
+}
+
 // fp32 += a.x*b.x + a.y*b.y with exact fp16 products (v_dot2_f32_f16).
 __device__ __forceinline__ float dot2(half2_t a, half2_t b, float c) {
   return __builtin_amdgcn_fdot2(a, b, c, false);
