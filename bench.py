@@ -92,6 +92,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM measurement")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of through a HIP graph")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 1 GiB device copy a few times (reference point for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of rocprofv3) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -103,6 +106,14 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)  # reads 2^30 bytes and writes 2^30 bytes per launch
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": 1 << 30, "launches": 4}))
+        return
     copies = [make_device_set(torch, 1000 + i) for i in range(args.copies)]
     xs = [torch.randn((1, K), device="cuda", dtype=torch.float16) for _, K in DECODE_SHAPES]
     ys = [torch.empty((1, N), device="cuda", dtype=torch.float16) for N, _ in DECODE_SHAPES]
@@ -209,7 +220,7 @@ def main():
             del W, S, x, y
         tf = tot_flops / tot_ms / 1e9
         out["gemm"] = {
-            "kernel": "q4g32_gemm_kernel",
+            "kernel": "q4g32_gemm_lds_kernel",
             "value": round(tf, 1),
             "unit": "TFLOP/s",
             "shapes": gem,

@@ -15,6 +15,18 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+int cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
 }  // namespace wq
 
 extern "C" const char* wq_last_error(void) { return wq::g_last_error; }

@@ -223,12 +223,15 @@ static int launch_mfma_gemm_cfg(int cfg, const char* who, const typename Loader:
   }
 }
 
-// Default tile shape: 64x128 for small M, else 128x256 — for format A the fully
-// LDS-staged kernel (12), which falls back to the register-staged one (2) when the
-// shape is not eligible; the other shapes are kept for measurement.
+// Default tile shape.  Register-staged kernel (format B, and format A when K is not
+// a multiple of 64): 64x128 for small M, else 128x256.  Fully LDS-staged kernel
+// (format A): 256x256 with one wavefront per SIMD and the dequantization
+// interleaved between the MFMAs (15) from M = 256 up, 128x256 (12) below.
 inline int choose_gemm_cfg(int64_t M, int64_t N, bool lds_staged) {
   (void)N;
-  return M <= 64 ? 3 : lds_staged ? 12 : 2;
+  if (M <= 64) return 3;
+  if (!lds_staged) return 2;
+  return M >= 256 ? 15 : 12;
 }
 
 }  // namespace wq

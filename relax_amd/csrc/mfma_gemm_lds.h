@@ -24,10 +24,15 @@
 #ifndef RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 #define RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 
+#include <algorithm>
+
 #include "wq_device.h"
 #include "wq_host.h"
 
 namespace wq {
+
+// Splitting of the last round's tiles (on by default; switch for measurement).
+inline int g_gemm_tail_split = 1;
 
 template <int TM, int TN, int WM, int WN>
 struct LdsGemmCfg {
@@ -55,39 +60,34 @@ struct LdsGemmCfg {
 typedef const void __attribute__((address_space(1))) * wq_gptr_t;
 typedef void __attribute__((address_space(3))) * wq_lptr_t;
 
-template <class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU, bool INTERLEAVE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
-void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restrict__ S,
-                           const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epilogue,
-                           int M, int N, int K, int tiles_m, int tiles_n) {
+// One output tile of TME*32*WM rows x BN columns starting at (m0, n0).  TME is the
+// number of 32-row sub-tiles per wavefront that are actually computed: TM for a full
+// tile, TM/2 or TM/4 for the split tiles of the last, partially filled round.
+template <class Epilogue, int TM, int TN, int WM, int WN, bool INTERLEAVE, int TME>
+__device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__ W,
+                                                    const half_t* __restrict__ S,
+                                                    const half_t* __restrict__ X,
+                                                    half_t* __restrict__ Y, const Epilogue& epilogue,
+                                                    int M, int N, int K, int m0, int n0,
+                                                    unsigned char* lds) {
   using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-
+  constexpr int kALoadsE = Cfg::kALoads * TME / TM;  // direct A loads per wavefront per step
+  constexpr int kLoadsPerStageE = kALoadsE + Cfg::kBLoads + 1;
+  static_assert(kALoadsE >= 1, "tile too small to split further");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int lj = lane & 31, lh = lane >> 5;
-
-  // XCD-aware tile order: each XCD (own L2) gets a contiguous range, walked M-fastest.
-  const int nblk = tiles_m * tiles_n;
-  int pid = blockIdx.x;
-  {
-    const int per = nblk / 8, rem = nblk % 8;
-    const int xcd = pid & 7, idx = pid >> 3;
-    pid = xcd * per + min(xcd, rem) + idx;
-  }
-  const int tile_m = pid % tiles_m, tile_n = pid / tiles_m;
-  const int m0 = tile_m * Cfg::BM, n0 = tile_n * Cfg::BN;
   const int G = K >> 5;
   const int ksteps = K >> 6;
 
   // ---- global sources of this lane's direct loads (rows past M / N are clamped:
   //      they only feed accumulators that are never stored) ----
-  const char* a_src[Cfg::kALoads];
+  const char* a_src[kALoadsE];
 #pragma unroll
-  for (int i = 0; i < Cfg::kALoads; ++i) {
-    const int s = (wave * Cfg::kALoads + i) * 64 + lane;  // LDS chunk slot
+  for (int i = 0; i < kALoadsE; ++i) {
+    const int s = (wave * kALoadsE + i) * 64 + lane;  // LDS chunk slot
     const int r = s >> 3, c = (s & 7) ^ WQ_SWZ(r);
     a_src[i] = reinterpret_cast<const char*>(X + (int64_t)min(m0 + r, M - 1) * K) + c * 16;
   }
@@ -105,9 +105,9 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
   auto issue_loads = [&](int ks) {
     unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
 #pragma unroll
-    for (int i = 0; i < Cfg::kALoads; ++i)
+    for (int i = 0; i < kALoadsE; ++i)
       __builtin_amdgcn_global_load_lds((wq_gptr_t)(a_src[i] + (int64_t)ks * 128),
-                                       (wq_lptr_t)(slot + Cfg::kAOff + (wave * Cfg::kALoads + i) * 1024),
+                                       (wq_lptr_t)(slot + Cfg::kAOff + (wave * kALoadsE + i) * 1024),
                                        16, 0, 0);
 #pragma unroll
     for (int i = 0; i < Cfg::kBLoads; ++i)
@@ -118,9 +118,9 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
                                      (wq_lptr_t)(slot + Cfg::kSOff + (wave * 64 % Cfg::BN) * 4), 4, 0, 0);
   };
 
-  float16_t acc[TM][TN];
+  float16_t acc[TME][TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TME; ++i)
 #pragma unroll
     for (int t = 0; t < TN; ++t)
 #pragma unroll
@@ -137,10 +137,10 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
       bw[t] = *reinterpret_cast<const uint4_t*>(slot + Cfg::kBOff + (n * 2 + lh) * 16);
       bs[t] = *reinterpret_cast<const half_t*>(slot + Cfg::kSOff + n * 4 + lh * 2);
     }
-    auto read_a = [&](int kk, half8_t (&aop)[TM]) {
+    auto read_a = [&](int kk, half8_t (&aop)[TME]) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = (wm * TM + i) * 32 + lj;
+      for (int i = 0; i < TME; ++i) {
+        const int row = (wm * TME + i) * 32 + lj;
         aop[i] = *reinterpret_cast<const half8_t*>(slot + Cfg::kAOff + row * 128 +
                                                    (((4 * lh + kk) ^ WQ_SWZ(row)) << 4));
       }
@@ -155,7 +155,7 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
         bop[t] = half8_t{d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
       }
     };
-    half8_t aop[2][TM], bop[2][TN];
+    half8_t aop[2][TME], bop[2][TN];
     read_a(0, aop[0]);
     dequant_b(0, bop[0]);
     if (!INTERLEAVE) {
@@ -168,7 +168,7 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TME; ++i)
 #pragma unroll
           for (int t = 0; t < TN; ++t)
             acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[kk & 1][i], bop[kk & 1][t],
@@ -179,7 +179,7 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
       // One wavefront per SIMD: nothing else hides VALU time, so the dequantization of
       // column kk+1 is cut into pairs (5 VALU instructions each) and one pair is issued
       // after each MFMA of column kk; up to ~5 VALU instructions fit under one MFMA.
-      static_assert(!INTERLEAVE || TM * TN >= TN * 4, "need at least one MFMA per weight pair");
+      static_assert(!INTERLEAVE || TME * TN >= TN * 4 || TME < TM, "need at least one MFMA per weight pair");
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const int cur = kk & 1, nxt = cur ^ 1;
@@ -187,7 +187,7 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
         half2_t dq[TN][4];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TME; ++i)
 #pragma unroll
           for (int t = 0; t < TN; ++t) {
             acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[cur][i], bop[cur][t], acc[i][t], 0, 0, 0);
@@ -213,7 +213,7 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
   issue_loads(0);
   if (ksteps > 1) {
     issue_loads(1);
-    WQ_WAITCNT_VM(Cfg::kLoadsPerStage);
+    WQ_WAITCNT_VM(kLoadsPerStageE);
   } else {
     WQ_WAITCNT_VM(0);
   }
@@ -224,7 +224,7 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
     if (ahead2) issue_loads(ks + 2);
     compute(ks);
     if (ahead2) {
-      WQ_WAITCNT_VM(Cfg::kLoadsPerStage);
+      WQ_WAITCNT_VM(kLoadsPerStageE);
     } else {
       WQ_WAITCNT_VM(0);
     }
@@ -238,13 +238,50 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
     const int n = n0 + (wn * TN + t) * 32 + lj;
     if (n >= N) continue;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TME; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + (wm * TM + i) * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+        const int m = m0 + (wm * TME + i) * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
         if (m < M) Y[(int64_t)m * N + n] = epilogue(acc[i][t][r], m, n);
       }
     }
+  }
+}
+
+// Workgroup -> work item.  The first n_full workgroups compute whole tiles (as many
+// as fill complete rounds of the machine); the tiles of the last, partially filled
+// round are cut into `split` row slices of TM/split sub-tiles so that the round is
+// shorter instead of leaving most CUs idle while a few finish whole tiles.
+template <class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU, bool INTERLEAVE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
+void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restrict__ S,
+                           const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epilogue,
+                           int M, int N, int K, int tiles_m, int tiles_n, int n_full, int split) {
+  using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int pid = blockIdx.x;
+  if (pid < n_full) {
+    // XCD-aware order: each XCD (own L2) gets a contiguous range of tiles, M-fastest.
+    const int per = n_full / 8, rem = n_full % 8;
+    const int xcd = pid & 7, idx = pid >> 3;
+    pid = xcd * per + min(xcd, rem) + idx;
+    const int tile_m = pid % tiles_m, tile_n = pid / tiles_m;
+    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, INTERLEAVE, TM>(
+        W, S, X, Y, epilogue, M, N, K, tile_m * Cfg::BM, tile_n * Cfg::BN, lds);
+    return;
+  }
+  const int t = n_full + (pid - n_full) / split, part = (pid - n_full) % split;
+  const int tile_m = t % tiles_m, tile_n = t / tiles_m;
+  const int m0 = tile_m * Cfg::BM + part * (Cfg::BM / split), n0 = tile_n * Cfg::BN;
+  if (m0 >= M) return;  // a slice that lies entirely past the last row
+  if (split == 2) {
+    if constexpr (TM % 2 == 0)
+      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, false, TM / 2>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+  } else if (split == 4) {
+    if constexpr (TM % 4 == 0)
+      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, false, TM / 4>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+  } else {
+    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, INTERLEAVE, TM>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
   }
 }
 
@@ -258,9 +295,25 @@ static int launch_q4g32_gemm_lds(const uint32_t* W, const uint16_t* S, const uin
   auto kern = q4g32_gemm_lds_kernel<Epilogue, TM, TN, WM, WN, WPE, INTERLEAVE>;
   WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                              hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
-  WQ_LAUNCH("wq_q4g32_gemm", kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), Cfg::kLdsBytes,
+  // Whole rounds of the machine run whole tiles; the tiles of the last, partial
+  // round are cut into 2 or 4 row slices when that lets them all run at once.
+  const int per_cu = std::max(1, std::min(WPE, (160 * 1024) / Cfg::kLdsBytes));
+  const int slots = cu_count() * per_cu;
+  const int total = tiles_m * tiles_n;
+  const int n_full = (total / slots) * slots;
+  const int rest = total - n_full;
+  int split = 1;
+  if (g_gemm_tail_split) {
+    for (int sp : {4, 2}) {
+      if (TM % sp == 0 && Cfg::kALoads % sp == 0 && rest * sp <= slots) {
+        split = sp;
+        break;
+      }
+    }
+  }
+  WQ_LAUNCH("wq_q4g32_gemm", kern, dim3((unsigned)(n_full + rest * split)), dim3(256), Cfg::kLdsBytes,
             stream, W, (const half_t*)S, (const half_t*)x, (half_t*)y, ep, (int)M, (int)N, (int)K,
-            tiles_m, tiles_n);
+            tiles_m, tiles_n, n_full, split);
   return WQ_OK;
 }
 

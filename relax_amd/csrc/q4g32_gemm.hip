@@ -71,6 +71,9 @@ extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemm_config(
   g_gemm_cfg_override = cfg;
 }
 int wq_gemm_cfg_override() { return g_gemm_cfg_override; }
+extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemm_tail_split(int on) {
+  wq::g_gemm_tail_split = on;
+}
 
 extern "C" int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                              const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M,
@@ -100,7 +103,7 @@ extern "C" int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_
       default: return fail(WQ_EINVAL, "wq_q4g32_gemm: unknown tile configuration %d", cfg);
     }
   }
-  if (cfg >= 11) cfg = cfg == 11 ? 1 : 2;  // not eligible: register-staged kernel of the same tile
+  if (cfg >= 11) cfg = (cfg == 11 || cfg >= 14) ? 1 : 2;  // not eligible: register-staged kernel, same tile
   return launch_mfma_gemm_cfg<Q4G32Loader, Q4G32Epilogue>(cfg, "wq_q4g32_gemm", bargs, x, y, ep, M,
                                                           N, K, stream);
 }

@@ -260,18 +260,6 @@ static int g_gemv_rows = 0;  // 0 = choose from the shape
 static int g_gemv_gpl = 0;
 static int g_gemv_blocks_per_cu = 0;
 
-static int cu_count() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-      cus = prop.multiProcessorCount;
-    if (cus <= 0) cus = 256;
-  }
-  return cus;
-}
-
 template <int ROWS, int MB, int GPL>
 static int launch_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                        const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t N,

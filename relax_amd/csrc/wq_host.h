@@ -15,6 +15,9 @@ namespace wq {
 // Stores a printf-style message for wq_last_error() on this thread and returns `code`.
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
+// Number of compute units of the current device (cached).
+int cu_count();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace wq
