@@ -33,6 +33,12 @@ PREFILL_SHAPES = [(11008, 4096), (4096, 11008)]
 PREFILL_M = 2048
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch, averaged over the four decode shapes resp. the two prefill
+# shapes: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one run each) of this script,
+# scaled by what the same counters read for a plain 1 GiB device copy
+# (`--calibrate-copy`): x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28726775
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 273100000
 
 
 def gemv_bytes(M, N, K):
@@ -186,7 +192,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
             "avg_launch_us": round(avg_launch_us, 3),
             "bytes_per_launch": bytes_per_launch,
         },
@@ -225,7 +231,8 @@ def main():
             "unit": "TFLOP/s",
             "shapes": gem,
             "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                         "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                         "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH},
         }
 
     if not args.no_cpu:
