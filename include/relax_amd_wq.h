@@ -70,14 +70,22 @@ int wq_q4g32_dequantize(const uint32_t* W, const uint16_t* S, uint16_t* out, int
                         wq_stream_t stream);
 
 /* y = x @ dequant(W,S)^T (+ bias[n] in fp32, then fp16, then + residual[m,n] in fp16).
- * x fp16 [M,K], y fp16 [M,N]; bias / residual may be NULL.  Chooses the decode
- * GEMV (M <= WQ_GEMV_MAX_M) or the MFMA GEMM from M. */
+ * x fp16 [M,K], y fp16 [M,N]; bias / residual may be NULL.  Chooses from the shape
+ * between the decode GEMV (M <= 2), the small-batch kernel (M <= 64, or two passes
+ * of it up to M = 128 on a small matrix) and the MFMA GEMM. */
 int wq_q4g32_linear(const uint32_t* W, const uint16_t* S, const uint16_t* x, const uint16_t* bias,
                     const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
                     wq_stream_t stream);
 
-/* The two kernels behind wq_q4g32_linear, selectable for tests and measurement. */
+/* The kernels behind wq_q4g32_linear, selectable for tests and measurement.
+ * wq_q4g32_small_batch (M <= WQ_SMALL_BATCH_MAX_M, K % 64 == 0) streams the weights
+ * once for all rows and multiplies on the matrix cores: the counterpart of
+ * python/tvm/dlight/gpu/low_batch_gemv.py. */
 #define WQ_GEMV_MAX_M 8
+#define WQ_SMALL_BATCH_MAX_M 64
+int wq_q4g32_small_batch(const uint32_t* W, const uint16_t* S, const uint16_t* x, const uint16_t* bias,
+                         const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
+                         wq_stream_t stream);
 int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x, const uint16_t* bias,
                   const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
                   wq_stream_t stream);

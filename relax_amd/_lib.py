@@ -23,6 +23,7 @@ SIGNATURES = {
     "wq_q4g32_linear": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_gemv": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "wq_q4g32_small_batch": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_ft_preprocess_weight_host": [_vp, _vp, _i64, _i64, _i64, _int, _int],
     "wq_ft_preprocess_weight": [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp],
     "wq_intb_dequantize": [_vp, _vp, _vp, _i64, _i64, _int, _i64, _vp],

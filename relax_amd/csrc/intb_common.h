@@ -22,5 +22,29 @@ int intb_gemv_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scale
                        int64_t m, int64_t n, int64_t k, int64_t group, int nbit,
                        const IntbEpilogue& ep, hipStream_t stream);
 
+// Matrix-core streaming kernel for 2 <= m <= 64 (intb_skinny.hip).
+int intb_small_batch_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scales, uint16_t* C,
+                              int64_t m, int64_t n, int64_t k, int64_t group, int nbit,
+                              const IntbEpilogue& ep, hipStream_t stream);
+
+#ifdef __HIPCC__
+// act(acc + bias) [binary residual] [unary], all in fp32, one rounding at the store
+struct IntbGemmEpilogue {
+  IntbEpilogue e;
+  int N;
+  __device__ half_t operator()(float v, int m, int n) const {
+    if (e.bias) v += (float)e.bias[e.bias_stride ? (int64_t)m * e.bias_stride + n : n];
+    v = apply_activation(v, e.activation);
+    if (e.residual) {
+      const float r = (float)e.residual[(int64_t)m * N + n];
+      if (e.binary_op == 1) v += r;
+      if (e.binary_op == 2) v *= r;
+    }
+    if (e.unary_op == 1) v = v > 0.0f ? v : 0.0f;
+    return (half_t)v;
+  }
+};
+#endif
+
 }  // namespace wq
 #endif  // RELAX_AMD_CSRC_INTB_COMMON_H_

@@ -1,8 +1,9 @@
 // Format B GEMM entry points: fp16 activations x preprocessed int8 / int4 weights,
 // the MI355X-native counterpart of fastertransformer::gemm_fp16_int_bias_act and
 // gemm_fp16_int_bias_act_residual (call sites python/tvm/contrib/cutlass/gemm_operation.py:441-458).
-// m <= 4 goes to the streaming GEMV (intb_gemv.hip); larger m to the shared MFMA
-// GEMM (mfma_gemm.h) with the weight loaders below.
+// m <= 2 goes to the streaming GEMV (intb_gemv.hip), m <= 64 to the small-batch
+// kernel (intb_skinny.hip), larger m to the shared MFMA GEMM (mfma_gemm.h) with the
+// weight loaders below.
 #include "intb_common.h"
 #include "mfma_gemm.h"
 
@@ -75,22 +76,6 @@ struct IntbLoader {
   }
 };
 
-// act(acc + bias) [binary residual] [unary], all in fp32, one rounding at the store
-struct IntbGemmEpilogue {
-  IntbEpilogue e;
-  int N;
-  __device__ half_t operator()(float v, int m, int n) const {
-    if (e.bias) v += (float)e.bias[e.bias_stride ? (int64_t)m * e.bias_stride + n : n];
-    v = apply_activation(v, e.activation);
-    if (e.residual) {
-      const float r = (float)e.residual[(int64_t)m * N + n];
-      if (e.binary_op == 1) v += r;
-      if (e.binary_op == 2) v *= r;
-    }
-    if (e.unary_op == 1) v = v > 0.0f ? v : 0.0f;
-    return (half_t)v;
-  }
-};
 
 static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
                             const uint16_t* scales, const uint16_t* bias, const uint16_t* residual,
@@ -118,8 +103,13 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
   const int group = (group_size > 0 && group_size != k) ? 64 : 0;
   const IntbEpilogue ep{(const half_t*)bias, binary_op ? (const half_t*)residual : nullptr,
                         bias_stride, activation, binary_op, unary_op};
-  if (m <= 4 && wq_gemm_cfg_override() == 0)
-    return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
+  if (wq_gemm_cfg_override() == 0) {
+    // one or two rows: the VALU streaming kernel; up to 64 rows: still one pass over the
+    // weights, products on the matrix cores; beyond that the tiled GEMM
+    if (m <= 2) return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
+    if (m <= WQ_SMALL_BATCH_MAX_M)
+      return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
+  }
   const int cfg = wq_gemm_cfg_override() ? wq_gemm_cfg_override() : choose_gemm_cfg(m, n, false);
   const IntbGemmEpilogue gep{ep, (int)n};
   if (nbit == 8) {

@@ -223,14 +223,18 @@ static int launch_mfma_gemm_cfg(int cfg, const char* who, const typename Loader:
   }
 }
 
-// Default tile shape.  Register-staged kernel (format B, and format A when K is not
-// a multiple of 64): 64x128 for small M, else 128x256.  Fully LDS-staged kernel
-// (format A): 256x256 with one wavefront per SIMD and the dequantization
-// interleaved between the MFMAs (15) from M = 256 up, 128x256 (12) below.
+// Tile shape from the problem shape, from timings at M = 96 .. 512 and 2048 of the
+// Llama-7B shapes (format A) and of K = 8192, N = 28672 (format B): what matters at
+// mid M is the number of tiles against 256 CUs.  Register-staged kernel (format B,
+// and format A when K is not a multiple of 64): 64x128 up to M = 128, 128x128 up to
+// 256, else 128x256.  Fully LDS-staged kernel (format A): 64x128 register-staged
+// tiles up to M = 128 when N is large, 128x256 (12) below M = 256, and from there
+// 256x256 with one wavefront per SIMD and the dequantization interleaved between the
+// MFMAs (15).
 inline int choose_gemm_cfg(int64_t M, int64_t N, bool lds_staged) {
-  (void)N;
   if (M <= 64) return 3;
-  if (!lds_staged) return 2;
+  if (!lds_staged) return M <= 128 ? 3 : M <= 256 ? 4 : 2;
+  if (M <= 128 && N >= 8192) return 3;
   return M >= 256 ? 15 : 12;
 }
 

@@ -3,6 +3,7 @@
 // loader for the q4f16_1 layout and the epilogue of the reference's prefill
 // PrimFunc (tests/python/dlight/test_gpu_matmul.py:378-401).
 #include "mfma_gemm.h"
+#include "q4g32_common.h"
 #include "mfma_gemm_lds.h"
 
 namespace wq {
@@ -50,18 +51,6 @@ struct Q4G32Loader {
   }
 };
 
-// (matmul_f32 + f32(bias)) -> fp16 -> + residual in fp16
-struct Q4G32Epilogue {
-  const half_t* bias;
-  const half_t* residual;
-  int N;
-  __device__ half_t operator()(float acc, int m, int n) const {
-    if (bias) acc += (float)bias[n];
-    half_t h = (half_t)acc;
-    if (residual) h = h + residual[(int64_t)m * N + n];
-    return h;
-  }
-};
 
 }  // namespace wq
 

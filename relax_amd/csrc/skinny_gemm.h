@@ -1,0 +1,303 @@
+// Small-batch weight-streaming GEMM (2 <= M <= 64) shared by both weight formats.
+//
+// At small M a quantized linear layer is still a weight stream (HBM-bound), but the
+// products are done by the matrix cores so that all M rows share ONE pass over the
+// weights (the GEMV kernels re-read the weights every few rows and pay VALU work per
+// row).  This is the counterpart of the reference's dlight LowBatchGEMV rule
+// (python/tvm/dlight/gpu/low_batch_gemv.py).
+//
+// Work split.  A workgroup (WAVES wavefronts, arranged NW x KW) owns 16*NW output
+// columns and all M rows.  Wavefront (nw, kw) owns columns n0 + 16*nw .. +15 and the
+// K-steps kw, kw + KW, kw + 2*KW, ... of 128 k each.  One step of one wavefront is
+// 4*TM MFMA 16x16x32: lane (j, kq) holds, for both operands, the 32 consecutive k
+// 128*step + 32*kq .. +31 of column j (row j of the activations), of which MFMA t takes
+// k 8t .. 8t+7.  The weight format (a Policy) says where those 32 codes live, how
+// many 16-byte pieces they are and how they unpack into the four B operands, in
+// natural k order, so the activations need no rearrangement.
+//
+// Everything travels global -> LDS with direct loads into a ring of `stages` slots,
+// `stages - 1` steps ahead: per step the rows x 128 activation slab of each kw
+// (shared by the NW wavefronts of that kw, each loading a part), and per wavefront
+// its codes and scales.  A wavefront waits for its own loads with s_waitcnt vmcnt(n);
+// when NW > 1 one s_barrier per step makes the shared slab visible.  The KW partial
+// sums of a column block meet in LDS at the end.
+//
+// What bounds it: per 16 columns every workgroup re-reads all of the activations
+// (from L2), and unpacking costs about two VALU operations per weight, so eight
+// wavefronts per workgroup (two per SIMD) are used to overlap one wavefront's
+// unpacking with another's loads, and NW grows with M and N to cut the re-reads.
+#ifndef RELAX_AMD_CSRC_SKINNY_GEMM_H_
+#define RELAX_AMD_CSRC_SKINNY_GEMM_H_
+
+#include "wq_device.h"
+#include "wq_host.h"
+
+namespace wq {
+
+#define WQ_SK_WAITCNT_VM(n) __builtin_amdgcn_s_waitcnt(((n)&0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+typedef const void __attribute__((address_space(1))) * wq_sk_gptr_t;
+typedef void __attribute__((address_space(3))) * wq_sk_lptr_t;
+
+// A Policy provides
+//   kPieces            16-byte pieces of codes per lane and step (32 k)
+//   kScaleDma          true: a scale per lane and step, fetched as the 4-byte pair that holds it
+//   Args, Lane         kernel argument block / per-lane state
+//   init(lane, args, n, K, N)
+//   w_addr(lane, k0, p)        address of piece p of the 32 codes starting at k0 (k0 % 32 == 0)
+//   s_addr(lane, k0)           4-byte aligned address of the pair holding the scale for k0   (kScaleDma)
+//   pick_scale(lane, pair, kq) the lane's half of that pair                                  (kScaleDma)
+//   const_scale(lane)          the lane's scale                                              (!kScaleDma)
+//   dequant(pieces, s, out[4]) -> B operands of MFMA 0..3 (k 8t .. 8t+7 each), scaled
+template <typename Policy, int TH, int NW, int WAVES>
+struct SkinnyCfg {
+  static constexpr int KW = WAVES / NW;
+  static_assert(NW * KW == WAVES && (WAVES == 4 || WAVES == 8), "wavefront arrangement");
+  static constexpr int kRows = 8 * TH;                   // activation rows held (M <= kRows)
+  static constexpr int TM = (TH + 1) / 2;                // 16-row MFMA tiles
+  static_assert((2 * TH) % NW == 0, "the slab loads divide among the wavefronts of one kw");
+  static constexpr int kSlabBytes = kRows * 256;         // rows x 128 k
+  static constexpr int kXBytes = KW * kSlabBytes;
+  static constexpr int kWBytes = WAVES * Policy::kPieces * 1024;
+  static constexpr int kStageBytes = kXBytes + kWBytes + (Policy::kScaleDma ? WAVES * 256 : 0);
+  static constexpr int kXLoads = 2 * TH / NW;            // slab loads (4 rows each) per wavefront and step
+  static constexpr int kLoadsPerStep = kXLoads + Policy::kPieces + (Policy::kScaleDma ? 1 : 0);
+  static constexpr int kMaxAhead = 63 / kLoadsPerStep;   // vmcnt holds 6 bits
+  static constexpr int kRedBytes = WAVES * TM * 4 * 64 * 4;
+};
+
+// s_waitcnt vmcnt(groups * L) for a wavefront-uniform run-time `groups` (<= 8)
+template <int L>
+__device__ __forceinline__ void wait_newer_groups(int groups) {
+  switch (groups) {
+    case 0: WQ_SK_WAITCNT_VM(0); break;
+    case 1: WQ_SK_WAITCNT_VM(1 * L <= 63 ? 1 * L : 63); break;
+    case 2: WQ_SK_WAITCNT_VM(2 * L <= 63 ? 2 * L : 63); break;
+    case 3: WQ_SK_WAITCNT_VM(3 * L <= 63 ? 3 * L : 63); break;
+    case 4: WQ_SK_WAITCNT_VM(4 * L <= 63 ? 4 * L : 63); break;
+    case 5: WQ_SK_WAITCNT_VM(5 * L <= 63 ? 5 * L : 63); break;
+    case 6: WQ_SK_WAITCNT_VM(6 * L <= 63 ? 6 * L : 63); break;
+    case 7: WQ_SK_WAITCNT_VM(7 * L <= 63 ? 7 * L : 63); break;
+    default: WQ_SK_WAITCNT_VM(8 * L <= 63 ? 8 * L : 63); break;
+  }
+}
+
+template <typename Policy, typename Epilogue, int TH, int NW, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
+    typename Policy::Args pargs, const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epi,
+    int M, int N, int K, int stages) {
+  using Cfg = SkinnyCfg<Policy, TH, NW, WAVES>;
+  constexpr int KW = Cfg::KW, TM = Cfg::TM, P = Policy::kPieces;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nw = wave / KW, kw = wave % KW;
+  const int lj = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.x * (16 * NW);
+  const int total_steps = (K + 127) >> 7;               // 128-k steps over K
+  const int nsteps = (total_steps + KW - 1) / KW;       // per wavefront (the last may be partly empty)
+  const int ahead = stages - 1;
+
+  // ---- per-lane sources ----
+  // slab load i of this wavefront: rows 4*li .. 4*li+3 of the slab, li = nw*kXLoads + i;
+  // LDS position p of a row holds the 16-byte chunk p ^ (row & 15) (bank-conflict-free reads)
+  const char* x_row[Cfg::kXLoads];
+  int x_chunk[Cfg::kXLoads];
+#pragma unroll
+  for (int i = 0; i < Cfg::kXLoads; ++i) {
+    const int li = nw * Cfg::kXLoads + i;
+    const int row = 4 * li + (lane >> 4);
+    x_chunk[i] = (lane & 15) ^ (row & 15);
+    x_row[i] = reinterpret_cast<const char*>(X + (int64_t)min(row, M - 1) * K);
+  }
+  typename Policy::Lane pl;
+  Policy::init(pl, pargs, min(n0 + 16 * nw + lj, N - 1), K, N);  // clamped columns are never stored
+  half_t s_fixed = (half_t)0.0f;
+  if (!Policy::kScaleDma) s_fixed = Policy::const_scale(pl);
+
+  unsigned char* const w_area = lds + Cfg::kXBytes + wave * (P * 1024);
+  unsigned char* const s_area = lds + Cfg::kXBytes + Cfg::kWBytes + wave * 256;
+
+  auto issue = [&](int it, int slot) {
+    const int stage_off = slot * Cfg::kStageBytes;
+    const int ks = it * KW + kw;
+    const int k0 = 128 * ks + 32 * kq;             // this lane's 32 weights
+    const int k0c = k0 < K ? k0 : 0;               // past the end: any valid address (scale is zeroed)
+#pragma unroll
+    for (int i = 0; i < Cfg::kXLoads; ++i) {
+      const int kchunk = ks * 16 + x_chunk[i];     // 16-byte chunk index along the row
+      const int64_t off = (kchunk * 8 < K) ? (int64_t)kchunk * 16 : 0;
+      __builtin_amdgcn_global_load_lds(
+          (wq_sk_gptr_t)(x_row[i] + off),
+          (wq_sk_lptr_t)(lds + stage_off + kw * Cfg::kSlabBytes + (nw * Cfg::kXLoads + i) * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int p = 0; p < P; ++p)
+      __builtin_amdgcn_global_load_lds((wq_sk_gptr_t)Policy::w_addr(pl, k0c, p),
+                                       (wq_sk_lptr_t)(w_area + stage_off + p * 1024), 16, 0, 0);
+    if (Policy::kScaleDma)
+      __builtin_amdgcn_global_load_lds((wq_sk_gptr_t)Policy::s_addr(pl, k0c),
+                                       (wq_sk_lptr_t)(s_area + stage_off), 4, 0, 0);
+  };
+
+  float4_t acc[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) acc[i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  auto compute = [&](int it, int slot) {
+    const int stage_off = slot * Cfg::kStageBytes;
+    const int k0 = 128 * (it * KW + kw) + 32 * kq;
+    uint4_t pieces[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p)
+      pieces[p] = *reinterpret_cast<const uint4_t*>(w_area + stage_off + p * 1024 + lane * 16);
+    half_t s = s_fixed;
+    if (Policy::kScaleDma)
+      s = Policy::pick_scale(pl, *reinterpret_cast<const half2_t*>(s_area + stage_off + lane * 4), kq);
+    if (k0 >= K) s = (half_t)0.0f;  // code * 0 = exact zero for the weights past K
+    half8_t bop[4];
+    Policy::dequant(pieces, s, bop);
+    const unsigned char* slab = lds + stage_off + kw * Cfg::kSlabBytes;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        // rows past the slab (M <= 8 uses half a tile) re-read a held row: never stored
+        const int row = (16 * i + lj < Cfg::kRows) ? 16 * i + lj : 16 * i + (lj & 7);
+        const half8_t aop =
+            *reinterpret_cast<const half8_t*>(slab + row * 256 + (((4 * kq + t) ^ (row & 15)) << 4));
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, bop[t], acc[i], 0, 0, 0);
+      }
+    }
+  };
+
+  // ---- prologue: fill the ring ----
+  for (int p = 0; p < ahead && p < nsteps; ++p) issue(p, p);
+  int cslot = 0;                       // slot of the step being computed
+  int islot = ahead % stages;          // slot the next issue goes to
+  for (int it = 0; it < nsteps; ++it) {
+    const int newer = min(ahead - 1, nsteps - 1 - it);  // steps issued after step `it`
+    wait_newer_groups<Cfg::kLoadsPerStep>(newer);
+    if (NW > 1) __builtin_amdgcn_s_barrier();
+    // the slot refilled now was computed in the previous iteration (by everyone: barrier above)
+    if (it + ahead < nsteps) {
+      issue(it + ahead, islot);
+      islot = islot + 1 == stages ? 0 : islot + 1;
+    }
+    compute(it, cslot);
+    cslot = cslot + 1 == stages ? 0 : cslot + 1;
+  }
+
+  // ---- reduce the KW partial sums of each column block through LDS, then store ----
+  if (KW > 1) {
+    __syncthreads();  // all ring slots idle
+    float* red = reinterpret_cast<float*>(lds);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[((wave * TM + i) * 4 + r) * 64 + lane] = acc[i][r];
+    __syncthreads();
+    if (kw == 0) {
+#pragma unroll
+      for (int o = 1; o < KW; ++o)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[i][r] += red[(((wave + o) * TM + i) * 4 + r) * 64 + lane];
+    }
+  }
+  if (kw == 0) {
+    const int col = n0 + 16 * nw + lj;
+    if (col < N) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = 16 * i + 4 * kq + r;
+          if (m < M) Y[(int64_t)m * N + col] = epi(acc[i][r], m, col);
+        }
+    }
+  }
+}
+
+constexpr int kSkinnyLdsBudget = 156 * 1024;  // of the 160 KB of a CU
+
+// overrides for tests and measurement (0 = automatic)
+struct SkinnyTuning {
+  int nw, stages, waves;
+};
+SkinnyTuning& skinny_tuning();
+
+template <typename Policy, typename Epilogue, int TH, int NW, int WAVES>
+static int launch_skinny(const char* who, const typename Policy::Args& pargs, const uint16_t* x, uint16_t* y,
+                         const Epilogue& epi, int64_t M, int64_t N, int64_t K, int want_stages,
+                         hipStream_t stream) {
+  using Cfg = SkinnyCfg<Policy, TH, NW, WAVES>;
+  auto kern = skinny_gemm_kernel<Policy, Epilogue, TH, NW, WAVES>;
+  const int64_t blocks = (N + 16 * NW - 1) / (16 * NW);
+  int stages = want_stages;
+  if (stages > Cfg::kMaxAhead + 1) stages = Cfg::kMaxAhead + 1;
+  if (stages > 9) stages = 9;
+  if (stages * Cfg::kStageBytes > kSkinnyLdsBudget) stages = kSkinnyLdsBudget / Cfg::kStageBytes;
+  WQ_REQUIRE(stages >= 2, "%s: internal: no room for a 2-slot ring", who);
+  int lds_bytes = stages * Cfg::kStageBytes;
+  if (lds_bytes < Cfg::kRedBytes) lds_bytes = Cfg::kRedBytes;
+  static bool configured = false;  // per instantiation
+  if (!configured) {
+    WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    configured = true;
+  }
+  WQ_LAUNCH(who, kern, dim3((unsigned)blocks), dim3(64 * WAVES), lds_bytes, stream, pargs,
+            (const half_t*)x, (half_t*)y, epi, (int)M, (int)N, (int)K, stages);
+  return WQ_OK;
+}
+
+// Picks the arrangement from the shape (timings of the Llama-7B layer shapes): few
+// columns per workgroup while the matrix is small, so that every CU gets work; more
+// columns per workgroup for tall matrices and larger M, where the re-reads of the
+// activations (once per workgroup) would otherwise outweigh the weight stream.
+template <typename Policy, typename Epilogue>
+static int launch_skinny_auto(const char* who, const typename Policy::Args& pargs, const uint16_t* x,
+                              uint16_t* y, const Epilogue& epi, int64_t M, int64_t N, int64_t K,
+                              hipStream_t stream) {
+  const SkinnyTuning& t = skinny_tuning();
+  const int64_t per_cu = (N / 16) / cu_count();
+  int nw = 1;
+  if (per_cu >= 2) nw = M <= 8 ? (per_cu >= 4 ? 2 : 1) : M <= 16 ? 2 : 4;
+  if (t.nw) nw = t.nw;
+  if (M <= 8 && nw == 4) nw = 2;  // 8 rows are two slab loads: at most two wavefronts share them
+  const int stages = t.stages ? t.stages : (nw == 4 ? 3 : 2);
+  // eight wavefronts where two ring slots of that arrangement fit LDS, else four
+#define WQ_SK_GO(TH, NW, WAVES)                                                                        \
+  do {                                                                                                 \
+    if constexpr (2 * SkinnyCfg<Policy, TH, NW, WAVES>::kStageBytes <= kSkinnyLdsBudget)               \
+      return launch_skinny<Policy, Epilogue, TH, NW, WAVES>(who, pargs, x, y, epi, M, N, K, stages,    \
+                                                            stream);                                   \
+    else                                                                                               \
+      return launch_skinny<Policy, Epilogue, TH, NW, 4>(who, pargs, x, y, epi, M, N, K, stages,        \
+                                                        stream);                                       \
+  } while (0)
+  if (M <= 8) {
+    if (nw == 2) WQ_SK_GO(1, 2, 8);
+    WQ_SK_GO(1, 1, 8);
+  }
+  if (M <= 16) {
+    if (nw == 4) WQ_SK_GO(2, 4, 8);
+    if (nw == 2) WQ_SK_GO(2, 2, 8);
+    WQ_SK_GO(2, 1, 8);
+  }
+  if (M <= 32) {
+    if (nw == 4) WQ_SK_GO(4, 4, 8);
+    if (nw == 2) WQ_SK_GO(4, 2, 8);
+    WQ_SK_GO(4, 1, 8);
+  }
+  if (nw == 4) WQ_SK_GO(8, 4, 8);
+  if (nw == 2) WQ_SK_GO(8, 2, 8);
+  WQ_SK_GO(8, 1, 8);
+#undef WQ_SK_GO
+}
+
+}  // namespace wq
+#endif  // RELAX_AMD_CSRC_SKINNY_GEMM_H_

@@ -107,7 +107,7 @@ def q4g32_linear(W: torch.Tensor, S: torch.Tensor, x: torch.Tensor, bias: Option
         if out.numel() != M * N:
             raise ValueError("out must have M*N elements")
     fn = {"auto": _lib.lib().wq_q4g32_linear, "gemv": _lib.lib().wq_q4g32_gemv,
-          "gemm": _lib.lib().wq_q4g32_gemm}[kernel]
+          "gemm": _lib.lib().wq_q4g32_gemm, "small_batch": _lib.lib().wq_q4g32_small_batch}[kernel]
     check(fn(_ptr(W), _ptr(S), _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), M, N, K, _stream()),
           f"wq_q4g32_{kernel}")
     return out
