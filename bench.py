@@ -11,7 +11,10 @@ reads a different copy of the weights (a ring of copies larger than the
 Prints ONE JSON line.  `value` is algorithmic bytes per second over the whole
 step; `roofline` describes the decode GEMV kernel, `gemm` the M=2048 prefill
 GEMM of the same quantization scheme, `cpu_baseline` the CPU restatement of the
-reference's path timed on this machine's host cores.
+reference's path timed on this machine's host cores.  Further objects on the same
+line: `stack` (32 decoder layers' linears run as one captured instruction list at
+M = 1, 8, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
+128, 512) and `calibration` (measured pure-read and MFMA-only ceilings).
 """
 from __future__ import annotations
 
@@ -89,6 +92,118 @@ def cpu_baseline(budget_s=8.0):
     }
 
 
+def _time_on_stream(torch, stream, fn, reps):
+    """Average milliseconds of `fn()` over `reps` calls, with events recorded on `stream`."""
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record(stream)
+    for _ in range(reps):
+        fn()
+    b.record(stream)
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def bench_stack(torch, layers=32, batches=(1, 8, 32), reps=20):
+    """The four quantized linears of `layers` Llama-2-7B decoder layers (3.6 GB of codes and scales,
+    so every step is cache-cold) as one instruction list of PackedFunc calls, planned and replayed
+    as one HIP graph by the library's executor."""
+    from relax_amd import vm
+
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    weights = []
+    for _ in range(layers):
+        layer = {}
+        for name, N, K in vm.LLAMA7B_LINEARS:
+            W = torch.randint(-2**31, 2**31 - 1, (N, K // 8), dtype=torch.int32, device="cuda", generator=g)
+            S = (torch.rand((N, K // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+            layer[name] = (W, S)
+        weights.append(layer)
+    stream = torch.cuda.Stream()
+    res = {"layers": layers, "instructions_per_step": 4 * layers, "launch": "hip_graph of PackedFunc calls", "batches": []}
+    for M in batches:
+        hidden = torch.randn((M, 4096), device="cuda", dtype=torch.float16)
+        attn = torch.randn((M, 4096), device="cuda", dtype=torch.float16)
+        act = torch.randn((M, 11008), device="cuda", dtype=torch.float16)
+        outp = torch.empty((M, 4096), device="cuda", dtype=torch.float16)
+        prog = vm.llama_linear_stack(weights, M, hidden, attn, act, outp)
+        ws = prog.plan()
+        prog.capture(stream)
+        prog.replay(stream)
+        stream.synchronize()
+        ms = _time_on_stream(torch, stream, lambda: prog.replay(stream), reps)
+        nbytes = layers * sum(gemv_bytes(M, N, K) for _, N, K in vm.LLAMA7B_LINEARS)
+        res["batches"].append({"M": M, "ms_per_step": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1),
+                               "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                               "bytes_per_step": nbytes, "workspace_bytes": ws,
+                               "workspace_without_reuse": prog.unplanned_bytes})
+        del prog
+    return res
+
+
+def bench_intb(torch, ops, K=8192, N=28672, batches=(1, 16, 128, 512), copies=3):
+    """fp16 x int8 per-channel weights in the preprocessed layout; `copies` weight copies
+    (more than the last-level cache) are cycled so that small M reads HBM."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    Ws = []
+    for _ in range(copies):
+        q = torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda", generator=g)
+        Ws.append(ops.ft_preprocess_weight(q, 80, False))
+        del q
+    s = (torch.rand((N,), device="cuda", generator=g) * 0.009 + 0.001).to(torch.float16)
+    stream = torch.cuda.current_stream()
+    res = {"K": K, "N": N, "weight": "int8 per-channel", "batches": []}
+    for M in batches:
+        x = torch.randn((M, K), device="cuda", dtype=torch.float16)
+        y = torch.empty((M, N), device="cuda", dtype=torch.float16)
+        it = [0]
+
+        def fn():
+            ops.fpA_intB_gemm(x, Ws[it[0] % copies], s, weight_nbit=8, out=y)
+            it[0] += 1
+
+        for _ in range(copies):
+            fn()
+        ms = _time_on_stream(torch, stream, fn, 4 * copies)
+        nbytes = K * N + N * 2 + M * K * 2 + M * N * 2
+        tf = 2.0 * M * N * K / ms / 1e9
+        res["batches"].append({"M": M, "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
+                               "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                               "TFLOP/s": round(tf, 1), "frac_of_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)})
+    return res
+
+
+def bench_calibration(torch):
+    """What this GPU reaches with no algorithm in the way: a streaming read of 1 GiB and MFMA issue only."""
+    import ctypes
+
+    from relax_amd import _lib
+
+    L = _lib.lib()
+    stream = torch.cuda.current_stream()
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+    scratch = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+
+    def rd():
+        _lib.check(L.wq_calibrate_read(src.data_ptr(), src.numel(), scratch.data_ptr(), stream.cuda_stream), "read")
+
+    rd()
+    ms_read = _time_on_stream(torch, stream, rd, 5)
+    flops = ctypes.c_double(0.0)
+
+    def mf():
+        _lib.check(L.wq_calibrate_mfma_f16(scratch.data_ptr(), scratch.numel(), 4000, ctypes.byref(flops),
+                                           stream.cuda_stream), "mfma")
+
+    mf()
+    ms_mfma = _time_on_stream(torch, stream, mf, 3)
+    return {"read_1GiB_GB/s": round(src.numel() / ms_read / 1e6, 1), "hbm_vendor_peak_GB/s": HBM_PEAK_GBS,
+            "mfma_f16_only_TFLOP/s": round(flops.value / ms_mfma / 1e9, 1),
+            "mfma_f16_vendor_peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,6 +213,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM measurement")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of through a HIP graph")
+    ap.add_argument("--no-stack", action="store_true", help="skip the 32-layer stack measurement")
+    ap.add_argument("--no-intb", action="store_true", help="skip the fpA_intB measurement")
+    ap.add_argument("--no-calibration", action="store_true", help="skip the pure-read / MFMA-only ceilings")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy a few times (reference point for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of rocprofv3) and exit")
@@ -234,6 +352,15 @@ def main():
                          "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH},
         }
+
+    del copies
+    torch.cuda.empty_cache()
+    if not args.no_stack:
+        out["stack"] = bench_stack(torch)
+    if not args.no_intb:
+        out["fpA_intB"] = bench_intb(torch, ops)
+    if not args.no_calibration:
+        out["calibration"] = bench_calibration(torch)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()

@@ -146,6 +146,20 @@ int wq_activation_from_string(const char* name);
 int wq_binary_op_from_string(const char* name);
 int wq_unary_op_from_string(const char* name);
 
+/* ------------------------------------------------------------------------- *
+ * Calibration kernels: the measured ceilings reported next to the vendor peaks
+ * (no counterpart in the reference; its methodology precedent is the cache-flush
+ * protocol of src/runtime/profiling.cc:879-895).
+ * ------------------------------------------------------------------------- */
+/* Issues `iters` x 8 independent v_mfma_f32_32x32x16_f16 per wavefront, four wavefronts
+ * per CU, no memory traffic.  scratch: device memory of >= 4 bytes x 256 x number of CUs.
+ * *flops receives the floating-point operations of one launch. */
+int wq_calibrate_mfma_f16(void* scratch, int64_t scratch_bytes, int iters, double* flops,
+                          wq_stream_t stream);
+/* Streams `bytes` of device memory through the CUs with 16-byte loads and no store
+ * (scratch: 4 bytes of device memory, practically never written). */
+int wq_calibrate_read(const void* src, int64_t bytes, void* scratch, wq_stream_t stream);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

@@ -1,4 +1,4 @@
-"""Loads ``librelax_amd_wq.so`` and declares the C ABI of ``include/relax_amd_wq.h``.
+"""Loads ``librelax_amd_wq.so`` and declares the C ABI of ``include/relax_amd_wq.h`` and ``include/relax_amd_vm.h``.
 
 There is no fallback: if the library is missing or a symbol is absent the import
 fails with an error that says how to build it.
@@ -29,11 +29,27 @@ SIGNATURES = {
     "wq_intb_dequantize": [_vp, _vp, _vp, _i64, _i64, _int, _i64, _vp],
     "wq_fpA_intB_gemm": [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
     "wq_fpA_intB_gemm_residual": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
+    "wq_calibrate_mfma_f16": [_vp, _i64, _int, ctypes.POINTER(ctypes.c_double), _vp],
+    "wq_calibrate_read": [_vp, _i64, _vp, _vp],
+    "wq_program_create": [],
+    "wq_program_destroy": [_vp],
+    "wq_program_add_external": [_vp, _int, _int, _int, ctypes.POINTER(_i64), _vp, _int],
+    "wq_program_add_planned": [_vp, _int, _int, _int, ctypes.POINTER(_i64)],
+    "wq_program_rebind": [_vp, _int, _vp],
+    "wq_program_add_call": [_vp, ctypes.c_char_p, _int, ctypes.POINTER(_i64), ctypes.POINTER(_int)],
+    "wq_program_plan": [_vp],
+    "wq_program_unplanned_bytes": [_vp],
+    "wq_program_set_workspace": [_vp, _vp, _i64],
+    "wq_program_run": [_vp, _vp],
+    "wq_program_capture": [_vp, _vp],
+    "wq_program_replay": [_vp, _vp],
+    "wq_program_num_instructions": [_vp],
     "wq_activation_from_string": [ctypes.c_char_p],
     "wq_binary_op_from_string": [ctypes.c_char_p],
     "wq_unary_op_from_string": [ctypes.c_char_p],
 }
-_RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p}
+_RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p, "wq_program_create": _vp,
+             "wq_program_destroy": None, "wq_program_plan": _i64, "wq_program_unplanned_bytes": _i64}
 
 _lib = None
 

@@ -44,9 +44,12 @@ HostRuntime& host() {
 }
 
 wq_stream_getter_t g_stream_getter = nullptr;
+thread_local bool t_stream_override_on = false;
+thread_local void* t_stream_override = nullptr;
 
 // The stream a PackedFunc call enqueues on.
 void* current_stream() {
+  if (t_stream_override_on) return t_stream_override;  // set by the instruction-list executor
   if (g_stream_getter) return g_stream_getter();
   HostRuntime& h = host();
   if (h.func_get_global && h.func_call) {
@@ -482,6 +485,20 @@ int registry_trampoline(TVMValue* args, int* type_codes, int num_args, TVMRetVal
 }
 
 }  // namespace
+
+namespace wq {
+// Used by the instruction-list executor (dps_program.cc).
+void set_stream_override(bool on, void* stream) {
+  t_stream_override_on = on;
+  t_stream_override = stream;
+}
+// Looks a PackedFunc of this library up by its dotted global name or its C symbol.
+WqTVMBackendPackedCFunc find_packed_function(const char* name) {
+  for (const Entry& e : table())
+    if (e.name == name || std::strcmp(e.symbol, name) == 0) return e.fn;
+  return nullptr;
+}
+}  // namespace wq
 
 extern "C" int wq_tvm_num_functions(void) { return (int)table().size(); }
 extern "C" const char* wq_tvm_function_name(int i) {

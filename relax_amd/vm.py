@@ -1,0 +1,144 @@
+"""Instruction-list executor for the library's PackedFuncs (``include/relax_amd_vm.h``) with torch tensors.
+
+Mirrors what a built Relax module does around the quantized linears: every op is a
+``call_dps_packed`` (src/runtime/relax_vm/vm.cc:691-775), intermediates live in one planned
+workspace (StaticPlanBlockMemory) and the whole list is replayed as one HIP graph
+(RewriteCUDAGraph, python/tvm/relax/pipeline.py:90-91).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, List, Sequence, Tuple, Union
+
+import torch
+
+from . import _lib
+from ._lib import check
+
+_DTYPES = {torch.float16: (2, 16), torch.float32: (2, 32), torch.int8: (0, 8), torch.uint8: (1, 8),
+           torch.int32: (0, 32), torch.int64: (0, 64)}
+kDLCPU, kDLROCM = 1, 10
+
+
+class Reg(int):
+    """A tensor register of a :class:`DpsProgram`."""
+
+
+class DpsProgram:
+    def __init__(self):
+        self._l = _lib.lib()
+        self._p = self._l.wq_program_create()
+        self._keep: List[torch.Tensor] = []
+        self._shapes: Dict[int, Tuple[Tuple[int, ...], torch.dtype]] = {}
+        self._workspace = None
+
+    def __del__(self):
+        if getattr(self, "_p", None):
+            self._l.wq_program_destroy(self._p)
+            self._p = None
+
+    # ---- registers ----
+    def external(self, t: torch.Tensor, as_uint32: bool = False) -> Reg:
+        """A tensor that owns its storage (weights, inputs, kept outputs).  ``as_uint32`` declares an
+        int32 tensor as uint32 (torch has no uint32 arithmetic; the bytes are the same)."""
+        if not t.is_contiguous():
+            raise ValueError("tensors must be contiguous")
+        code, bits = _DTYPES[t.dtype]
+        if as_uint32:
+            if t.dtype != torch.int32:
+                raise ValueError("as_uint32 needs an int32 tensor")
+            code = 1
+        shape = (ctypes.c_int64 * max(1, t.dim()))(*t.shape)
+        r = self._l.wq_program_add_external(self._p, code, bits, t.dim(), shape, t.data_ptr(),
+                                            kDLROCM if t.is_cuda else kDLCPU)
+        check(min(r, 0), "wq_program_add_external")
+        self._keep.append(t)
+        self._shapes[r] = (tuple(t.shape), t.dtype)
+        return Reg(r)
+
+    def planned(self, shape: Sequence[int], dtype: torch.dtype = torch.float16) -> Reg:
+        """An intermediate whose storage the memory plan assigns."""
+        code, bits = _DTYPES[dtype]
+        shp = (ctypes.c_int64 * max(1, len(shape)))(*shape)
+        r = self._l.wq_program_add_planned(self._p, code, bits, len(shape), shp)
+        check(min(r, 0), "wq_program_add_planned")
+        self._shapes[r] = (tuple(shape), dtype)
+        return Reg(r)
+
+    def rebind(self, reg: Reg, t: torch.Tensor) -> None:
+        shape, dtype = self._shapes[int(reg)]
+        if tuple(t.shape) != shape or t.dtype != dtype or not t.is_contiguous():
+            raise ValueError("rebind needs a contiguous tensor of the declared shape and dtype")
+        check(self._l.wq_program_rebind(self._p, int(reg), t.data_ptr()), "wq_program_rebind")
+        self._keep.append(t)
+
+    # ---- instructions ----
+    def call(self, func: str, *args: Union[Reg, int]) -> None:
+        """``call_dps_packed(func, inputs..., outputs...)``; ``Reg`` arguments are tensors, plain ints immediates."""
+        n = len(args)
+        vals = (ctypes.c_int64 * max(1, n))(*[int(a) for a in args])
+        kinds = (ctypes.c_int * max(1, n))(*[1 if isinstance(a, Reg) else 0 for a in args])
+        check(self._l.wq_program_add_call(self._p, func.encode(), n, vals, kinds), f"wq_program_add_call({func})")
+
+    # ---- memory plan ----
+    def plan(self, device: str = "cuda") -> int:
+        """Plans the workspace, allocates it (once, here — never while running) and returns its size in bytes."""
+        need = self._l.wq_program_plan(self._p)
+        check(min(need, 0), "wq_program_plan")
+        self._workspace = torch.zeros(max(need, 256), dtype=torch.uint8, device=device)
+        check(self._l.wq_program_set_workspace(self._p, self._workspace.data_ptr(), self._workspace.numel()),
+              "wq_program_set_workspace")
+        return int(need)
+
+    @property
+    def unplanned_bytes(self) -> int:
+        return int(self._l.wq_program_unplanned_bytes(self._p))
+
+    @property
+    def num_instructions(self) -> int:
+        return int(self._l.wq_program_num_instructions(self._p))
+
+    # ---- execution ----
+    def run(self, stream: torch.cuda.Stream = None) -> None:
+        s = (stream or torch.cuda.current_stream()).cuda_stream
+        check(self._l.wq_program_run(self._p, s), "wq_program_run")
+
+    def capture(self, stream: torch.cuda.Stream) -> None:
+        check(self._l.wq_program_capture(self._p, stream.cuda_stream), "wq_program_capture")
+
+    def replay(self, stream: torch.cuda.Stream) -> None:
+        check(self._l.wq_program_replay(self._p, stream.cuda_stream), "wq_program_replay")
+
+
+# The four quantized linears of one Llama-2-7B decoder layer, as (name, N, K).
+LLAMA7B_LINEARS = (("qkv_proj", 12288, 4096), ("o_proj", 4096, 4096), ("gate_up_proj", 22016, 4096),
+                   ("down_proj", 4096, 11008))
+
+
+def llama_linear_stack(weights, M: int, hidden: torch.Tensor, attn_out: torch.Tensor, mlp_act: torch.Tensor,
+                       out: torch.Tensor, linears=LLAMA7B_LINEARS) -> DpsProgram:
+    """Program of ``len(weights)`` decoder layers' quantized linears (q4f16_1), batch ``M``.
+
+    ``weights[l][name] = (W int32 [N, K/8], S fp16 [N, K/32])``.  Only the linears are present, so two
+    inputs stand in for what the missing ops would produce: ``attn_out`` [M, 4096] feeds every o_proj
+    and ``mlp_act`` [M, 11008] every down_proj.  ``hidden`` [M, 4096] enters layer 0; each layer's
+    down_proj output is the next layer's hidden state; the last one lands in ``out``.
+    """
+    p = DpsProgram()
+    h = p.external(hidden)
+    a = p.external(attn_out)
+    g = p.external(mlp_act)
+    dims = {name: (n, k) for name, n, k in linears}
+    L = len(weights)
+    for l, layer in enumerate(weights):
+        regs = {name: (p.external(w, as_uint32=True), p.external(s)) for name, (w, s) in layer.items()}
+        qkv = p.planned((M, dims["qkv_proj"][0]))
+        p.call("relax_amd.q4f16_1_matmul", *regs["qkv_proj"], h, qkv)
+        o = p.planned((M, dims["o_proj"][0]))
+        p.call("relax_amd.q4f16_1_matmul", *regs["o_proj"], a, o)
+        gu = p.planned((M, dims["gate_up_proj"][0]))
+        p.call("relax_amd.q4f16_1_matmul", *regs["gate_up_proj"], o, gu)
+        nxt = p.external(out) if l == L - 1 else p.planned((M, dims["down_proj"][0]))
+        p.call("relax_amd.q4f16_1_matmul", *regs["down_proj"], g, nxt)
+        h = nxt
+    return p

@@ -1,0 +1,173 @@
+"""The instruction-list executor (include/relax_amd_vm.h): planning and error paths on the CPU,
+execution, memory reuse and HIP-graph replay against the oracle on the GPU."""
+import ctypes
+
+import numpy as np
+import pytest
+
+
+def _lib():
+    from relax_amd import _lib
+
+    return _lib.lib()
+
+
+def _shape(*dims):
+    return (ctypes.c_int64 * max(1, len(dims)))(*dims)
+
+
+def _call(l, p, name, regs):
+    n = len(regs)
+    vals = (ctypes.c_int64 * n)(*regs)
+    kinds = (ctypes.c_int * n)(*([1] * n))
+    return l.wq_program_add_call(p, name.encode(), n, vals, kinds)
+
+
+def test_plan_reuses_storage_of_dead_tensors():
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        w = l.wq_program_add_external(p, 1, 32, 2, _shape(64, 8), 0x1000, 10)
+        s = l.wq_program_add_external(p, 2, 16, 2, _shape(64, 2), 0x2000, 10)
+        x = l.wq_program_add_external(p, 2, 16, 2, _shape(4, 64), 0x3000, 10)
+        # chain x -> t0 -> t1 -> t2 -> t3: t_i is dead once t_{i+1} is written
+        t = [l.wq_program_add_planned(p, 2, 16, 2, _shape(4, 64)) for _ in range(4)]
+        big = l.wq_program_add_planned(p, 2, 16, 2, _shape(4, 6400))  # never used: costs nothing
+        assert min(t) >= 0 and big >= 0
+        prev = x
+        for r in t:
+            assert _call(l, p, "relax_amd.q4f16_1_matmul", [w, s, prev, r]) == 0
+            prev = r
+        assert l.wq_program_num_instructions(p) == 4
+        need = l.wq_program_plan(p)
+        # an instruction's input and output are live together, so two blocks of 512 bytes, not four
+        assert need == 2 * 512
+        assert l.wq_program_unplanned_bytes(p) == 4 * 512
+        # running without storage is refused
+        assert l.wq_program_run(p, None) != 0
+        assert b"no storage" in l.wq_last_error()
+        assert l.wq_program_set_workspace(p, 0x10000, 100) != 0 and b"needed" in l.wq_last_error()
+        assert l.wq_program_set_workspace(p, 0x10010, 4096) != 0 and b"aligned" in l.wq_last_error()
+    finally:
+        l.wq_program_destroy(p)
+
+
+def test_plan_keeps_overlapping_tensors_apart_and_fits_sizes():
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        w = l.wq_program_add_external(p, 1, 32, 2, _shape(64, 8), 0x1000, 10)
+        s = l.wq_program_add_external(p, 2, 16, 2, _shape(64, 2), 0x2000, 10)
+        x = l.wq_program_add_external(p, 2, 16, 2, _shape(4, 64), 0x3000, 10)
+        a = l.wq_program_add_planned(p, 2, 16, 2, _shape(4, 64))      # 512 B, live 0..3
+        b = l.wq_program_add_planned(p, 2, 16, 2, _shape(40, 64))     # 5120 B, live 1..1
+        c = l.wq_program_add_planned(p, 2, 16, 2, _shape(8, 64))      # 1024 B, live 2..3: fits b's block
+        d = l.wq_program_add_planned(p, 2, 16, 2, _shape(400, 64))    # 51200 B, live 3..3: fits nothing
+        for regs in ([w, s, x, a], [w, s, x, b], [w, s, x, c], [w, s, a, d], ):
+            assert _call(l, p, "relax_amd_q4f16_1_matmul", regs) == 0  # C symbol name works too
+        assert _call(l, p, "relax_amd_q4f16_1_matmul", [w, s, c, d]) == 0
+        assert l.wq_program_plan(p) == 512 + 5120 + 51200
+    finally:
+        l.wq_program_destroy(p)
+
+
+def test_program_argument_errors():
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        assert _call(l, p, "no.such.function", []) != 0 and b"no PackedFunc" in l.wq_last_error()
+        assert l.wq_program_add_planned(p, 2, 12, 1, _shape(4)) < 0
+        assert l.wq_program_add_planned(p, 2, 16, 1, _shape(-4)) < 0
+        r = l.wq_program_add_planned(p, 2, 16, 1, _shape(4))
+        assert r == 0
+        assert _call(l, p, "relax_amd.q4f16_1_matmul", [0, 7]) != 0 and b"does not exist" in l.wq_last_error()
+        assert l.wq_program_rebind(p, r, 0x1000) != 0  # planned storage cannot be rebound
+        assert l.wq_program_replay(p, None) != 0 and b"nothing captured" in l.wq_last_error()
+        assert l.wq_program_set_workspace(p, 0x1000, 1 << 20) != 0  # not planned yet
+    finally:
+        l.wq_program_destroy(p)
+
+
+SMALL_LINEARS = (("qkv_proj", 384, 128), ("o_proj", 128, 128), ("gate_up_proj", 512, 128), ("down_proj", 128, 256))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_linear_stack_program_matches_oracle_eager_and_replayed(oracle, M):
+    import torch
+
+    from relax_amd import vm
+    from tests import gpu_util as u
+
+    L = 3
+    rng = np.random.default_rng(M)
+    host_w, dev_w = [], []
+    for l in range(L):
+        hw, dw = {}, {}
+        for name, N, K in SMALL_LINEARS:
+            _, W, S = oracle.make_q4g32_inputs(1, N, K, seed=100 * l + N + K)
+            hw[name] = (W, S)
+            dw[name] = (u.dev(W), u.dev(S))
+        host_w.append(hw)
+        dev_w.append(dw)
+    hidden = rng.standard_normal((M, 128)).astype(np.float16)
+    attn = rng.standard_normal((M, 128)).astype(np.float16)
+    act = (rng.standard_normal((M, 256)) * 0.5).astype(np.float16)
+    out = torch.zeros((M, 128), dtype=torch.float16, device="cuda")
+    d_hidden = u.dev(hidden)
+    prog = vm.llama_linear_stack(dev_w, M, d_hidden, u.dev(attn), u.dev(act), out, linears=SMALL_LINEARS)
+    assert prog.num_instructions == 4 * L
+    need = prog.plan()
+    # per layer qkv, o, gate_up and the hidden state: storage is reused across layers
+    assert 0 < need < prog.unplanned_bytes
+    assert need <= 2 * M * (384 + 128 + 512 + 128) * 2 + 8 * 256
+
+    # the last down_proj only depends on mlp_act; check it and, through a second program, the o -> gate_up chain
+    want = oracle.q4g32_linear(*host_w[-1]["down_proj"], act, nthreads=4)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        prog.run(stream)
+    stream.synchronize()
+    eager = u.host(out).copy()
+    u.assert_close(eager, want, "stack eager")
+
+    prog.capture(stream)
+    for rep in range(3):
+        out.zero_()                       # eager work between replays
+        torch.cuda.synchronize()
+        prog.replay(stream)
+        stream.synchronize()
+        assert np.array_equal(u.host(out).view(np.uint16), eager.view(np.uint16)), rep
+
+    # chain through planned storage: y = gate_up(o_proj(attn)) with both intermediates planned
+    p2 = vm.DpsProgram()
+    wq, sq = dev_w[0]["o_proj"]
+    wg, sg = dev_w[0]["gate_up_proj"]
+    y = torch.zeros((M, 512), dtype=torch.float16, device="cuda")
+    t = p2.planned((M, 128))
+    p2.call("relax_amd.q4f16_1_matmul", p2.external(wq, as_uint32=True), p2.external(sq), p2.external(u.dev(attn)), t)
+    p2.call("relax_amd.q4f16_1_matmul", p2.external(wg, as_uint32=True), p2.external(sg), t, p2.external(y))
+    p2.plan()
+    p2.run()
+    torch.cuda.synchronize()
+    o_ref = oracle.q4g32_linear(*host_w[0]["o_proj"], attn, nthreads=4)
+    y_ref = oracle.q4g32_linear(*host_w[0]["gate_up_proj"], o_ref, nthreads=4)
+    u.assert_close(u.host(y), y_ref, "planned chain")
+
+
+@pytest.mark.gpu
+def test_program_reports_callee_errors():
+    import torch
+
+    from relax_amd import vm
+    from relax_amd._lib import WqError
+
+    p = vm.DpsProgram()
+    w = p.external(torch.zeros((8, 8), dtype=torch.int32, device="cuda"), as_uint32=True)
+    s = p.external(torch.zeros((8, 2), dtype=torch.float16, device="cuda"))
+    x = p.external(torch.zeros((1, 32), dtype=torch.float16, device="cuda"))  # K mismatch: W says 64
+    y = p.planned((1, 8))
+    p.call("relax_amd.q4f16_1_matmul", w, s, x, y)
+    p.plan()
+    with pytest.raises(WqError, match="instruction 0"):
+        p.run()
