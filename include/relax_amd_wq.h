@@ -147,6 +147,25 @@ int wq_binary_op_from_string(const char* name);
 int wq_unary_op_from_string(const char* name);
 
 /* ------------------------------------------------------------------------- *
+ * Quantizers (device): fp16 weights [N, K] -> packed codes + scales.
+ * ------------------------------------------------------------------------- */
+/* Format B, the reference fixtures' `encode`
+ * (tests/python/relax/test_codegen_cutlass.py:1392-1457 int4, 1631-1676 int8, 2044-2109 group 64):
+ *   scale = max(max |A|, 1e-4) * (0.125 | 0.0078125) over the row (group_size <= 0 or == K)
+ *           or over each 64-k group; q = clip(round(A / scale), lo, hi), round half away
+ *           from zero, float32 arithmetic.
+ * w_out int8 [K, N] or packed int4 [K, N/2] (un-preprocessed: feed it to
+ * wq_ft_preprocess_weight); scales fp16 [N] or [K/64, N].  scale_scratch: N floats of
+ * device memory (per-channel mode only; may be NULL for group 64).  N % 64 == K % 64 == 0. */
+int wq_intb_encode(const uint16_t* A, int8_t* w_out, uint16_t* scales, float* scale_scratch, int64_t N,
+                   int64_t K, int64_t group_size, int weight_nbit, wq_stream_t stream);
+/* Format A (q4f16_1): per group of 32 along K, scale = fp16(max(max |A|, 1e-4) / 7),
+ * code = clip(round(A / scale) + 7, 0, 14); W uint32 [N, K/8], S fp16 [N, K/32].
+ * Inverse of the decode in tests/python/dlight/test_gpu_gemv.py:198; the reference tree
+ * has no encoder for this format, so the rounding convention is this library's. */
+int wq_q4g32_encode(const uint16_t* A, uint32_t* W, uint16_t* S, int64_t N, int64_t K, wq_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Calibration kernels: the measured ceilings reported next to the vendor peaks
  * (no counterpart in the reference; its methodology precedent is the cache-flush
  * protocol of src/runtime/profiling.cc:879-895).

@@ -30,7 +30,14 @@
  *                                        (tlc-pack/cutlass_fpA_intB_gemm, an empty
  *                                        submodule, no pinned revision) is absent:
  *                                        the layout is pinned for sm in [75, 90) only.
- *   wqo_intb_encode_*                    closed form; round-trip and hand cases
+ *   wqo_intb_encode[_grouped]            closed form (numpy restatement in float32 with
+ *                                        half-away-from-zero rounding), full-scale and
+ *                                        hand cases
+ *   wqo_q4g32_encode                     PARITY UNPINNED: the q4f16_1 quantizer is not in
+ *                                        the reference tree (only its decode side is);
+ *                                        the definition used is stated at the function
+ *                                        and checked through decode(encode(w)) error
+ *                                        bounds, code range and a numpy restatement
  *
  * Build: see oracle/Makefile (gcc -O3 -mavx2 -mfma -mf16c -fopenmp).
  */
@@ -499,4 +506,73 @@ void wqo_intb_encode(const uint16_t* A, int8_t* w_out, uint16_t* scales_out, int
       }
     }
   free(scale);
+}
+
+/*
+ * Fine-grained (group 64 along K) form of the same quantizer,
+ * tests/python/relax/test_codegen_cutlass.py:2044-2109: the maximum, the scale and
+ * the division are per (k / 64, n); scales_out is fp16 [K/64, N].  K % 64 == 0.
+ */
+void wqo_intb_encode_grouped(const uint16_t* A, int8_t* w_out, uint16_t* scales_out, int64_t N,
+                             int64_t K, int nbit) {
+  const float c = nbit == 4 ? 0.125f : 0.0078125f;
+  const float lo = nbit == 4 ? -8.0f : -128.0f, hi = nbit == 4 ? 7.0f : 127.0f;
+  if (nbit == 4) memset(w_out, 0, (size_t)(K * N / 2));
+  for (int64_t g = 0; g < K / 64; ++g)
+    for (int64_t n = 0; n < N; ++n) {
+      float mx = -65504.0f;
+      for (int64_t k = g * 64; k < g * 64 + 64; ++k) {
+        float v = fabsf(h2f(A[n * K + k]));
+        if (v > mx) mx = v;
+      }
+      const float scale = (mx > 0.0001f ? mx : 0.0001f) * c;
+      scales_out[g * N + n] = f2h(scale);
+      for (int64_t k = g * 64; k < g * 64 + 64; ++k) {
+        float r = roundf(h2f(A[n * K + k]) / scale);
+        if (r < lo) r = lo;
+        if (r > hi) r = hi;
+        int q = (int)r;
+        if (nbit == 8) {
+          w_out[k * N + n] = (int8_t)q;
+        } else {
+          uint8_t* p = (uint8_t*)&w_out[k * (N / 2) + n / 2];
+          *p = (uint8_t)(*p | ((q & 15) << ((n % 2) * 4)));
+        }
+      }
+    }
+}
+
+/*
+ * q4f16_1 quantizer (Format A), the inverse of the decode in
+ * tests/python/dlight/test_gpu_gemv.py:198.  The reference tree holds no encoder for
+ * this format, so this is a definition, not a restatement (parity unpinned):
+ *   per group of 32 along K:  m = max |a|  (fp16),
+ *   scale = fp16( max(f32(m), 1e-4) / 7 ),
+ *   code  = clip( round( f32(a) / f32(scale) ) + 7, 0, 14 )     round = half away from zero
+ * so that decode gives (code - 7) * scale with |error| <= scale / 2 for every element
+ * (the group maximum maps to code 0 or 14).  W uint32 [N, K/8], S fp16 [N, K/32].
+ */
+void wqo_q4g32_encode(const uint16_t* A, uint32_t* W, uint16_t* S, int64_t N, int64_t K) {
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t g = 0; g < K / 32; ++g) {
+      const uint16_t* a = A + n * K + g * 32;
+      float mx = 0.0f;
+      for (int i = 0; i < 32; ++i) {
+        float v = fabsf(h2f(a[i]));
+        if (v > mx) mx = v;
+      }
+      const uint16_t sh = f2h((mx > 0.0001f ? mx : 0.0001f) / 7.0f);
+      const float scale = h2f(sh);
+      S[n * (K / 32) + g] = sh;
+      for (int j = 0; j < 4; ++j) {
+        uint32_t word = 0;
+        for (int i = 0; i < 8; ++i) {
+          float r = roundf(h2f(a[8 * j + i]) / scale) + 7.0f;
+          if (r < 0.0f) r = 0.0f;
+          if (r > 14.0f) r = 14.0f;
+          word |= (uint32_t)(int)r << (4 * i);
+        }
+        W[n * (K / 8) + g * 4 + j] = word;
+      }
+    }
 }

@@ -253,6 +253,28 @@ def intb_encode(Wf: np.ndarray, nbit: int):
     return w, s
 
 
+def intb_encode_grouped(Wf: np.ndarray, nbit: int):
+    """The fixtures' group-64 quantizer: fp16 [N,K] -> (int8 [K,N] | [K,N/2], fp16 [K/64,N])."""
+    Wf = _c(Wf, np.float16)
+    N, K = Wf.shape
+    assert K % 64 == 0
+    w = np.zeros((K, N if nbit == 8 else N // 2), np.int8)
+    s = np.empty((K // 64, N), np.float16)
+    lib().wqo_intb_encode_grouped(_p(Wf), _p(w), _p(s), i64(N), i64(K), cint(nbit))
+    return w, s
+
+
+def q4g32_encode(Wf: np.ndarray):
+    """q4f16_1 quantizer (a definition: the reference tree has none): fp16 [N,K] -> (uint32 [N,K/8], fp16 [N,K/32])."""
+    Wf = _c(Wf, np.float16)
+    N, K = Wf.shape
+    assert K % 32 == 0
+    W = np.empty((N, K // 8), np.uint32)
+    S = np.empty((N, K // 32), np.float16)
+    lib().wqo_q4g32_encode(_p(Wf), _p(W), _p(S), i64(N), i64(K))
+    return W, S
+
+
 # ------------------------------------------------- synthetic inputs (shared)
 
 

@@ -214,3 +214,32 @@ def fpA_intB_gemm(x: torch.Tensor, B: torch.Tensor, scales: torch.Tensor, bias: 
                                           M, N, K, group_size, weight_nbit, 0, 0, _stream()),
               "wq_fpA_intB_gemm_residual")
     return out
+
+
+def intb_encode(Wf: torch.Tensor, weight_nbit: int, group_size: int = -1):
+    """The reference fixtures' quantizer (tests/python/relax/test_codegen_cutlass.py:1392-1457, 1631-1676,
+    2044-2109): fp16 ``[N, K]`` -> ``(int8 [K, N] | packed int4 [K, N/2], fp16 scales [N] | [K/64, N])``.
+    The codes are not yet in the GEMM's layout: pass them through :func:`ft_preprocess_weight`."""
+    Wf = _dev(Wf, torch.float16, "Wf")
+    if Wf.dim() != 2:
+        raise ValueError("Wf must be [N, K]")
+    N, K = Wf.shape
+    grouped = group_size == 64 and group_size != K
+    w = torch.empty((K, N if weight_nbit == 8 else N // 2), dtype=torch.int8, device=Wf.device)
+    s = torch.empty((K // 64, N) if grouped else (N,), dtype=torch.float16, device=Wf.device)
+    scratch = None if grouped else torch.empty((N,), dtype=torch.float32, device=Wf.device)
+    check(_lib.lib().wq_intb_encode(_ptr(Wf), _ptr(w), _ptr(s), _ptr(scratch), N, K, group_size, weight_nbit,
+                                    _stream()), "wq_intb_encode")
+    return w, s
+
+
+def q4g32_encode(Wf: torch.Tensor):
+    """q4f16_1 quantizer: fp16 ``[N, K]`` -> ``(W int32 [N, K/8] (uint32 bits), S fp16 [N, K/32])``."""
+    Wf = _dev(Wf, torch.float16, "Wf")
+    if Wf.dim() != 2 or Wf.shape[1] % 32:
+        raise ValueError("Wf must be [N, K] with K a multiple of 32")
+    N, K = Wf.shape
+    W = torch.empty((N, K // 8), dtype=torch.int32, device=Wf.device)
+    S = torch.empty((N, K // 32), dtype=torch.float16, device=Wf.device)
+    check(_lib.lib().wq_q4g32_encode(_ptr(Wf), _ptr(W), _ptr(S), N, K, _stream()), "wq_q4g32_encode")
+    return W, S

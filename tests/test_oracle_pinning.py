@@ -217,3 +217,67 @@ def test_intb_encode_closed_form(oracle, nbit):
     # the largest element of every row maps to +-full scale (8 clips to 7 for int4)
     top = np.abs(q).max(axis=0)
     assert np.all(top >= (7 if nbit == 4 else 127))
+
+
+def _round_half_away(r):
+    return np.sign(r) * np.floor(np.abs(r) + np.float32(0.5))
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_intb_encode_grouped_closed_form(oracle, nbit):
+    """group-64 quantizer (tests/python/relax/test_codegen_cutlass.py:2044-2109) against a numpy
+    restatement in float32, and against the per-channel one where they must agree (K = 64)."""
+    rng = np.random.default_rng(3)
+    N, K = 64, 256
+    Wf = (rng.normal(0, 0.02, size=(N, K)) * rng.uniform(0.1, 4, size=(N, 1))).astype(np.float16)
+    Wf[5, 64:128] = 0  # an all-zero group takes the 1e-4 floor
+    w, s = oracle.intb_encode_grouped(Wf, nbit)
+    q = oracle.intb_unpack(w, nbit).astype(np.int64)  # [K, N]
+    c = np.float32(0.125 if nbit == 4 else 0.0078125)
+    lo, hi = (-8, 7) if nbit == 4 else (-128, 127)
+    g = Wf.reshape(N, K // 64, 64)
+    scale = np.maximum(np.abs(g).max(axis=2).astype(np.float32), np.float32(1e-4)) * c  # [N, K/64]
+    assert np.array_equal(s.view(np.uint16), scale.T.astype(np.float16).view(np.uint16))
+    want = np.clip(_round_half_away(g.astype(np.float32) / scale[:, :, None]), lo, hi).reshape(N, K)
+    assert np.array_equal(q, want.T.astype(np.int64))
+    assert np.all(q[64:128, 5] == 0)
+    w1, s1 = oracle.intb_encode(Wf[:, :64].copy(), nbit)
+    wg, sg = oracle.intb_encode_grouped(Wf[:, :64].copy(), nbit)
+    assert np.array_equal(w1, wg) and np.array_equal(s1.view(np.uint16), sg[0].view(np.uint16))
+
+
+def test_q4g32_encode_definition_and_round_trip(oracle):
+    """The format-A quantizer has no counterpart in the reference tree (parity unpinned): checked are
+    the stated definition (numpy restatement), the code range, the error bound of decode(encode(w))
+    and that weights which are already on a quantization grid survive unchanged."""
+    rng = np.random.default_rng(4)
+    N, K = 48, 256
+    Wf = (rng.normal(0, 0.05, size=(N, K)) * rng.uniform(0.05, 8, size=(N, 1))).astype(np.float16)
+    Wf[3, 32:64] = 0
+    W, S = oracle.q4g32_encode(Wf)
+    q = oracle.q4_unpack(W).astype(np.int64)
+    assert q.min() >= 0 and q.max() <= 14
+    g = Wf.reshape(N, K // 32, 32)
+    m = np.abs(g).max(axis=2).astype(np.float32)
+    s_want = (np.maximum(m, np.float32(1e-4)) / np.float32(7)).astype(np.float16)
+    assert np.array_equal(S.view(np.uint16), s_want.view(np.uint16))
+    r = g.astype(np.float32) / s_want.astype(np.float32)[:, :, None]
+    want = np.clip(_round_half_away(r) + 7, 0, 14).reshape(N, K)
+    assert np.array_equal(q, want.astype(np.int64))
+    assert np.all(q[3, 32:64] == 7)
+    # error bound: half a step, plus the fp16 roundings of scale and product
+    deq = oracle.q4g32_dequant(W, S).astype(np.float64)
+    step = np.repeat(S.astype(np.float64), 32, axis=1)
+    assert np.all(np.abs(deq - Wf.astype(np.float64)) <= 0.5 * step * 1.01 + 1e-7)
+    # every group reaches full scale on one side
+    qq = q.reshape(N, K // 32, 32)
+    nz = m > 1e-4
+    assert np.all(((qq.min(axis=2) == 0) | (qq.max(axis=2) == 14))[nz])
+    # grid weights: codes with full-scale groups and power-of-two scales are reproduced exactly
+    codes = rng.integers(0, 15, size=(N, K)).astype(np.uint8)
+    codes[:, ::32] = 14
+    W0 = oracle.q4_pack(codes)
+    S0 = np.full((N, K // 32), 2.0 ** -6, np.float16)
+    Wgrid = oracle.q4g32_dequant(W0, S0)
+    W1, S1 = oracle.q4g32_encode(Wgrid)
+    assert np.array_equal(oracle.q4g32_dequant(W1, S1).view(np.uint16), Wgrid.view(np.uint16))
