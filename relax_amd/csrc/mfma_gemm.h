@@ -229,13 +229,12 @@ static int launch_mfma_gemm_cfg(int cfg, const char* who, const typename Loader:
 // and format A when K is not a multiple of 64): 64x128 up to M = 128, 128x128 up to
 // 256, else 128x256.  Fully LDS-staged kernel (format A): 64x128 register-staged
 // tiles up to M = 128 when N is large, 128x256 (12) below M = 256, and from there
-// 256x256 with one wavefront per SIMD and the dequantization interleaved between the
-// MFMAs (15).
+// 256x256 with one wavefront per SIMD (11).
 inline int choose_gemm_cfg(int64_t M, int64_t N, bool lds_staged) {
   if (M <= 64) return 3;
   if (!lds_staged) return M <= 128 ? 3 : M <= 256 ? 4 : 2;
   if (M <= 128 && N >= 8192) return 3;
-  return M >= 256 ? 15 : 12;
+  return M >= 256 ? 11 : 12;
 }
 
 }  // namespace wq

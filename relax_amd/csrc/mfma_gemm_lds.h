@@ -16,15 +16,16 @@
 // in registers (q4_word_dequant_natural: bit-exact, natural K order, hence no
 // rearrangement of the activations) and never exist in LDS as fp16.
 //
-// Synchronisation per K-step: issue the loads of step ks+2; multiply step ks;
-// s_waitcnt vmcnt(loads of one step) — vector memory operations retire in order,
-// so this wavefront's loads of step ks+1 have landed; s_barrier — so have everyone
-// else's, and everyone is done reading slot ks%3, which the next iteration refills.
-// (A raw s_barrier is used: the fence in __syncthreads would force vmcnt(0).)
+// Synchronisation: vector memory operations retire in order, so s_waitcnt vmcnt(loads of
+// one step) means "this wavefront's loads of the step before have landed"; one raw
+// s_barrier per K-step then says the same for the whole workgroup (the fence in
+// __syncthreads would force vmcnt(0)).  The schedule inside a K-step is described at
+// q4g32_gemm_lds_tile.
 #ifndef RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 #define RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 
 #include <algorithm>
+#include <type_traits>
 
 #include "wq_device.h"
 #include "wq_host.h"
@@ -56,6 +57,8 @@ struct LdsGemmCfg {
 // 128-byte halves of the bank space, so pairs of rows share one pattern value.
 #define WQ_SWZ(r) (((r) >> 1) & 7)
 #define WQ_WAITCNT_VM(n) __builtin_amdgcn_s_waitcnt(((n)&0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+// the same with lgkmcnt(0): this wavefront's LDS reads have returned as well
+#define WQ_WAITCNT_VM_LGKM0(n) __builtin_amdgcn_s_waitcnt(((n)&0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0x0 << 8))
 
 typedef const void __attribute__((address_space(1))) * wq_gptr_t;
 typedef void __attribute__((address_space(3))) * wq_lptr_t;
@@ -63,7 +66,23 @@ typedef void __attribute__((address_space(3))) * wq_lptr_t;
 // One output tile of TME*32*WM rows x BN columns starting at (m0, n0).  TME is the
 // number of 32-row sub-tiles per wavefront that are actually computed: TM for a full
 // tile, TM/2 or TM/4 for the split tiles of the last, partially filled round.
-template <class Epilogue, int TM, int TN, int WM, int WN, bool INTERLEAVE, int TME>
+//
+// Schedule of one K-step (four phases kk = 0..3 of TME*TN MFMAs each).  Nothing but
+// MFMAs may sit on the critical path of a wavefront that has its SIMD to itself, so
+// every other instruction is slotted between them:
+//   phases 0-2  after some MFMAs: one direct load of step ks+2 (their issue is what
+//               the texture path accepts, 64 B per cycle and CU — issued in a burst they
+//               block the wavefront for hundreds of cycles), and the unpacking of one
+//               weight pair of phase kk+1; at the phase start the LDS reads of the
+//               activation fragments of phase kk+1;
+//   phase 3     first s_waitcnt vmcnt (this wavefront's loads of step ks+1 have landed)
+//               and s_barrier (everyone's have); then, between its MFMAs, the packed
+//               weights, the first activation fragments and the first weight pairs of
+//               step ks+1, so that step ks+1 starts multiplying at once.
+// One barrier per K-step suffices: slot (ks+2)%3 (= (ks-1)%3) is refilled by loads issued
+// after the barrier of step ks-1, and every wavefront has waited for its last LDS reads of
+// that slot (the phase-3 fragments of step ks-1) before that barrier.
+template <class Epilogue, int TM, int TN, int WM, int WN, int TME>
 __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__ W,
                                                     const half_t* __restrict__ S,
                                                     const half_t* __restrict__ X,
@@ -72,7 +91,9 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
                                                     unsigned char* lds) {
   using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
   constexpr int kALoadsE = Cfg::kALoads * TME / TM;  // direct A loads per wavefront per step
-  constexpr int kLoadsPerStageE = kALoadsE + Cfg::kBLoads + 1;
+  constexpr int L = kALoadsE + Cfg::kBLoads + 1;     // direct loads per wavefront per step
+  constexpr int NSLOT = TME * TN;                    // MFMAs per phase
+  constexpr int NPAIR = TN * 4;                      // weight pairs to unpack per phase
   static_assert(kALoadsE >= 1, "tile too small to split further");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -102,20 +123,20 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   const int s_row = (wave * 64) % Cfg::BN + lane;
   const char* s_src = reinterpret_cast<const char*>(S + (int64_t)min(n0 + s_row, N - 1) * G);
 
-  auto issue_loads = [&](int ks) {
+  // direct load number idx (0 .. L-1) of step ks
+  auto issue_one = [&](int ks, int idx) {
     unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
-#pragma unroll
-    for (int i = 0; i < kALoadsE; ++i)
-      __builtin_amdgcn_global_load_lds((wq_gptr_t)(a_src[i] + (int64_t)ks * 128),
-                                       (wq_lptr_t)(slot + Cfg::kAOff + (wave * kALoadsE + i) * 1024),
-                                       16, 0, 0);
-#pragma unroll
-    for (int i = 0; i < Cfg::kBLoads; ++i)
+    if (idx < kALoadsE) {
+      __builtin_amdgcn_global_load_lds((wq_gptr_t)(a_src[idx] + (int64_t)ks * 128),
+                                       (wq_lptr_t)(slot + Cfg::kAOff + (wave * kALoadsE + idx) * 1024), 16, 0, 0);
+    } else if (idx < kALoadsE + Cfg::kBLoads) {
+      const int i = idx - kALoadsE;
       __builtin_amdgcn_global_load_lds((wq_gptr_t)(b_src[i] + (int64_t)ks * 32),
-                                       (wq_lptr_t)(slot + Cfg::kBOff + (wave * Cfg::kBLoads + i) * 1024),
-                                       16, 0, 0);
-    __builtin_amdgcn_global_load_lds((wq_gptr_t)(s_src + (int64_t)ks * 4),
-                                     (wq_lptr_t)(slot + Cfg::kSOff + (wave * 64 % Cfg::BN) * 4), 4, 0, 0);
+                                       (wq_lptr_t)(slot + Cfg::kBOff + (wave * Cfg::kBLoads + i) * 1024), 16, 0, 0);
+    } else {
+      __builtin_amdgcn_global_load_lds((wq_gptr_t)(s_src + (int64_t)ks * 4),
+                                       (wq_lptr_t)(slot + Cfg::kSOff + (wave * 64 % Cfg::BN) * 4), 4, 0, 0);
+    }
   };
 
   float16_t acc[TME][TN];
@@ -126,109 +147,107 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.0f;
 
-  auto compute = [&](int ks) {
-    const unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
-    // this lane's packed weights and scale for the whole step
-    uint4_t bw[TN];
-    half_t bs[TN];
+  uint4_t bw[TN];   // this lane's packed weights of the step being unpacked
+  half_t bs[TN];
+  half8_t aop[2][TME], bop[2][TN];
+  auto read_b = [&](const unsigned char* slot) {
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
       const int n = (wn * TN + t) * 32 + lj;
       bw[t] = *reinterpret_cast<const uint4_t*>(slot + Cfg::kBOff + (n * 2 + lh) * 16);
       bs[t] = *reinterpret_cast<const half_t*>(slot + Cfg::kSOff + n * 4 + lh * 2);
     }
-    auto read_a = [&](int kk, half8_t (&aop)[TME]) {
+  };
+  auto read_a = [&](const unsigned char* slot, int kk, half8_t (&dst)[TME]) {
 #pragma unroll
-      for (int i = 0; i < TME; ++i) {
-        const int row = (wm * TME + i) * 32 + lj;
-        aop[i] = *reinterpret_cast<const half8_t*>(slot + Cfg::kAOff + row * 128 +
-                                                   (((4 * lh + kk) ^ WQ_SWZ(row)) << 4));
-      }
-    };
-    auto dequant_b = [&](int kk, half8_t (&bop)[TN]) {
-#pragma unroll
-      for (int t = 0; t < TN; ++t) {
-        const uint32_t word = kk == 0 ? bw[t].x : kk == 1 ? bw[t].y : kk == 2 ? bw[t].z : bw[t].w;
-        const half2_t s2 = {bs[t], bs[t]};
-        half2_t d[4];
-        q4_word_dequant_natural(word, s2, d);
-        bop[t] = half8_t{d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
-      }
-    };
-    half8_t aop[2][TME], bop[2][TN];
-    read_a(0, aop[0]);
-    dequant_b(0, bop[0]);
-    if (!INTERLEAVE) {
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        // operands of column kk+1 are fetched / dequantized before the MFMAs of column kk
-        if (kk < 3) {
-          read_a(kk + 1, aop[(kk + 1) & 1]);
-          dequant_b(kk + 1, bop[(kk + 1) & 1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < TME; ++i)
-#pragma unroll
-          for (int t = 0; t < TN; ++t)
-            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[kk & 1][i], bop[kk & 1][t],
-                                                               acc[i][t], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    } else {
-      // One wavefront per SIMD: nothing else hides VALU time, so the dequantization of
-      // column kk+1 is cut into pairs (5 VALU instructions each) and one pair is issued
-      // after each MFMA of column kk; up to ~5 VALU instructions fit under one MFMA.
-      static_assert(!INTERLEAVE || TME * TN >= TN * 4 || TME < TM, "need at least one MFMA per weight pair");
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const int cur = kk & 1, nxt = cur ^ 1;
-        if (kk < 3) read_a(kk + 1, aop[nxt]);
-        half2_t dq[TN][4];
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < TME; ++i)
-#pragma unroll
-          for (int t = 0; t < TN; ++t) {
-            acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[cur][i], bop[cur][t], acc[i][t], 0, 0, 0);
-            const int slice = i * TN + t;  // 0 .. TM*TN-1
-            if (kk < 3 && slice < TN * 4) {
-              const int tt = slice >> 2, j = slice & 3;
-              const uint32_t word = kk + 1 == 1 ? bw[tt].y : kk + 1 == 2 ? bw[tt].z : bw[tt].w;
-              const half2_t s2 = {bs[tt], bs[tt]};
-              dq[tt][j] = q4_pair_dequant_natural(word, j, s2);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        if (kk < 3) {
-#pragma unroll
-          for (int t = 0; t < TN; ++t)
-            bop[nxt][t] = half8_t{dq[t][0].x, dq[t][0].y, dq[t][1].x, dq[t][1].y,
-                                  dq[t][2].x, dq[t][2].y, dq[t][3].x, dq[t][3].y};
-        }
-      }
+    for (int i = 0; i < TME; ++i) {
+      const int row = (wm * TME + i) * 32 + lj;
+      dst[i] = *reinterpret_cast<const half8_t*>(slot + Cfg::kAOff + row * 128 +
+                                                 (((4 * lh + kk) ^ WQ_SWZ(row)) << 4));
     }
   };
+  auto word_of = [&](int t, int kk) -> uint32_t {
+    return kk == 0 ? bw[t].x : kk == 1 ? bw[t].y : kk == 2 ? bw[t].z : bw[t].w;
+  };
 
-  issue_loads(0);
+  // ---- prologue: two steps of loads in flight, first operands of step 0 ready ----
+#pragma unroll
+  for (int idx = 0; idx < L; ++idx) issue_one(0, idx);
   if (ksteps > 1) {
-    issue_loads(1);
-    WQ_WAITCNT_VM(kLoadsPerStageE);
+#pragma unroll
+    for (int idx = 0; idx < L; ++idx) issue_one(1, idx);
+    WQ_WAITCNT_VM(L);
   } else {
     WQ_WAITCNT_VM(0);
   }
   __builtin_amdgcn_s_barrier();
+  read_b(lds);
+  read_a(lds, 0, aop[0]);
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    const half2_t s2 = {bs[t], bs[t]};
+    half2_t d[4];
+    q4_word_dequant_natural(bw[t].x, s2, d);
+    bop[0][t] = half8_t{d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
+  }
 
+  // Phase 3 prepares the next step unconditionally: in the last step it reads a slot that
+  // holds stale data and unpacks it for nobody.  (A run-time branch around those LDS reads
+  // would make the compiler wait for them before the first MFMA of the phase.)
   for (int ks = 0; ks < ksteps; ++ks) {
+    const unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
+    const unsigned char* next_slot = lds + ((ks + 1) % Cfg::kStages) * Cfg::kStageBytes;
     const bool ahead2 = ks + 2 < ksteps;
-    if (ahead2) issue_loads(ks + 2);
-    compute(ks);
-    if (ahead2) {
-      WQ_WAITCNT_VM(kLoadsPerStageE);
-    } else {
-      WQ_WAITCNT_VM(0);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int cur = kk & 1, nxt = cur ^ 1;
+      if (kk == 3) {
+        // loads of step ks+1 landed (those of ks+2 may be in flight), own LDS reads done
+        if (ahead2) {
+          WQ_WAITCNT_VM_LGKM0(L);
+        } else {
+          WQ_WAITCNT_VM_LGKM0(0);
+        }
+        __builtin_amdgcn_s_barrier();
+        read_b(next_slot);
+        read_a(next_slot, 0, aop[nxt]);
+      } else {
+        read_a(slot, kk + 1, aop[nxt]);
+      }
+      half2_t dq[TN][4];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int sl = 0; sl < NSLOT; ++sl) {
+        const int i = sl / TN, t = sl % TN;
+        acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[cur][i], bop[cur][t], acc[i][t], 0, 0, 0);
+        // unpack the weight pairs of the next phase; in phase 3 (operands just requested
+        // from LDS) only in the second half of the slots
+        {
+          const int first = kk < 3 ? 0 : NSLOT / 2, span = NSLOT - first;
+          if (sl >= first) {
+            const int p0 = (sl - first) * NPAIR / span, p1 = (sl - first + 1) * NPAIR / span;
+#pragma unroll
+            for (int p = p0; p < p1; ++p) {
+              const int tt = p >> 2, j = p & 3;
+              const half2_t s2 = {bs[tt], bs[tt]};
+              dq[tt][j] = q4_pair_dequant_natural(word_of(tt, (kk + 1) & 3), j, s2);
+            }
+          }
+        }
+        // direct loads of step ks+2, spread over phases 0-2
+        if (kk < 3 && ahead2) {
+          const int g = kk * NSLOT + sl;
+          const int l0 = g * L / (3 * NSLOT), l1 = (g + 1) * L / (3 * NSLOT);
+#pragma unroll
+          for (int idx = l0; idx < l1; ++idx) issue_one(ks + 2, idx);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int t = 0; t < TN; ++t)
+        bop[nxt][t] = half8_t{dq[t][0].x, dq[t][0].y, dq[t][1].x, dq[t][1].y,
+                              dq[t][2].x, dq[t][2].y, dq[t][3].x, dq[t][3].y};
     }
-    __builtin_amdgcn_s_barrier();
   }
 
   // ---- epilogue ----
@@ -252,7 +271,7 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
 // as fill complete rounds of the machine); the tiles of the last, partially filled
 // round are cut into `split` row slices of TM/split sub-tiles so that the round is
 // shorter instead of leaving most CUs idle while a few finish whole tiles.
-template <class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU, bool INTERLEAVE>
+template <class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
 void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restrict__ S,
                            const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epilogue,
@@ -266,7 +285,7 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
     const int xcd = pid & 7, idx = pid >> 3;
     pid = xcd * per + min(xcd, rem) + idx;
     const int tile_m = pid % tiles_m, tile_n = pid / tiles_m;
-    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, INTERLEAVE, TM>(
+    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM>(
         W, S, X, Y, epilogue, M, N, K, tile_m * Cfg::BM, tile_n * Cfg::BN, lds);
     return;
   }
@@ -276,23 +295,23 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
   if (m0 >= M) return;  // a slice that lies entirely past the last row
   if (split == 2) {
     if constexpr (TM % 2 == 0)
-      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, false, TM / 2>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM / 2>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
   } else if (split == 4) {
     if constexpr (TM % 4 == 0)
-      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, false, TM / 4>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM / 4>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
   } else {
-    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, INTERLEAVE, TM>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
   }
 }
 
-template <class Epilogue, int TM, int TN, int WM, int WN, int WPE, bool INTERLEAVE = false>
+template <class Epilogue, int TM, int TN, int WM, int WN, int WPE>
 static int launch_q4g32_gemm_lds(const uint32_t* W, const uint16_t* S, const uint16_t* x, uint16_t* y,
                                  const Epilogue& ep, int64_t M, int64_t N, int64_t K,
                                  hipStream_t stream) {
   using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
   const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM);
   const int tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
-  auto kern = q4g32_gemm_lds_kernel<Epilogue, TM, TN, WM, WN, WPE, INTERLEAVE>;
+  auto kern = q4g32_gemm_lds_kernel<Epilogue, TM, TN, WM, WN, WPE>;
   WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                              hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
   // Whole rounds of the machine run whole tiles; the tiles of the last, partial

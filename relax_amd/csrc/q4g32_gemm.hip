@@ -80,15 +80,13 @@ extern "C" int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_
   int cfg = g_gemm_cfg_override ? g_gemm_cfg_override : choose_gemm_cfg(M, N, true);
   const Q4G32Loader::Args bargs{W, (const half_t*)S};
   const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
-  // 11..13: the fully LDS-staged kernel (needs K % 64 == 0 and 4-byte aligned scale pairs)
+  // 11..14: the fully LDS-staged kernel (needs K % 64 == 0 and 4-byte aligned scale pairs)
   if (cfg >= 11 && K % 64 == 0 && ((uintptr_t)S & 3u) == 0) {
     switch (cfg) {
       case 11: return launch_q4g32_gemm_lds<Q4G32Epilogue, 8, 2, 1, 4, 1>(W, S, x, y, ep, M, N, K, stream);
       case 12: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 2, 1, 4, 2>(W, S, x, y, ep, M, N, K, stream);
       case 13: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 2, 2, 2, 2>(W, S, x, y, ep, M, N, K, stream);
-      case 14: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 4, 2, 2, 1, true>(W, S, x, y, ep, M, N, K, stream);
-      case 15: return launch_q4g32_gemm_lds<Q4G32Epilogue, 8, 2, 1, 4, 1, true>(W, S, x, y, ep, M, N, K, stream);
-      case 16: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 4, 2, 2, 1, false>(W, S, x, y, ep, M, N, K, stream);
+      case 14: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 4, 2, 2, 1>(W, S, x, y, ep, M, N, K, stream);
       default: return fail(WQ_EINVAL, "wq_q4g32_gemm: unknown tile configuration %d", cfg);
     }
   }
