@@ -3,7 +3,7 @@
 //
 // Every operand of a K-step (64 k) travels global -> LDS with the direct
 // global_load_lds_dwordx4 path: no staging registers, no VALU work, and the loads
-// of step ks+2 are in flight while step ks is multiplied (3-slot ring).  Per slot:
+// of the next two to three steps are in flight while a step is multiplied (3-slot ring).  Per slot:
 //   A   BM rows x 128 B of activations, 16-byte chunk c of row r at slot position
 //       c ^ ((r >> 1) & 7) (the swizzle is applied to the GLOBAL address each lane fetches,
 //       because the LDS side of a direct load is fixed: lane l writes 16 bytes at
@@ -70,18 +70,19 @@ typedef void __attribute__((address_space(3))) * wq_lptr_t;
 // Schedule of one K-step (four phases kk = 0..3 of TME*TN MFMAs each).  Nothing but
 // MFMAs may sit on the critical path of a wavefront that has its SIMD to itself, so
 // every other instruction is slotted between them:
-//   phases 0-2  after some MFMAs: one direct load of step ks+2 (their issue is what
-//               the texture path accepts, 64 B per cycle and CU — issued in a burst they
-//               block the wavefront for hundreds of cycles), and the unpacking of one
-//               weight pair of phase kk+1; at the phase start the LDS reads of the
-//               activation fragments of phase kk+1;
+//   phases 0-2  after each MFMA the unpacking of one weight pair of phase kk+1; at the
+//               phase start the LDS reads of the activation fragments of phase kk+1; in
+//               phase 0 also the second half of the direct loads of step ks+2 (direct loads
+//               are slotted between MFMAs because the texture path accepts 64 B per cycle
+//               and CU: issued in a burst they block the wavefront for hundreds of cycles);
 //   phase 3     first s_waitcnt vmcnt (this wavefront's loads of step ks+1 have landed)
 //               and s_barrier (everyone's have); then, between its MFMAs, the packed
 //               weights, the first activation fragments and the first weight pairs of
-//               step ks+1, so that step ks+1 starts multiplying at once.
-// One barrier per K-step suffices: slot (ks+2)%3 (= (ks-1)%3) is refilled by loads issued
-// after the barrier of step ks-1, and every wavefront has waited for its last LDS reads of
-// that slot (the phase-3 fragments of step ks-1) before that barrier.
+//               step ks+1, so that step ks+1 starts multiplying at once, and the first half
+//               of the direct loads of step ks+3 (into the slot of step ks, free by now).
+// One barrier per K-step suffices: slot ks%3 is refilled by loads issued after the barrier
+// of step ks, and every wavefront has waited for its last LDS reads of that slot (the
+// phase-3 fragments) before that barrier.
 template <class Epilogue, int TM, int TN, int WM, int WN, int TME>
 __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__ W,
                                                     const half_t* __restrict__ S,
@@ -94,6 +95,8 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   constexpr int L = kALoadsE + Cfg::kBLoads + 1;     // direct loads per wavefront per step
   constexpr int NSLOT = TME * TN;                    // MFMAs per phase
   constexpr int NPAIR = TN * 4;                      // weight pairs to unpack per phase
+  constexpr int LA = L / 2;                          // loads of a step issued in phase 3 (three steps ahead) ...
+  constexpr int LB = L - LA;                         // ... and in phase 0 of the following step
   static_assert(kALoadsE >= 1, "tile too small to split further");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -170,12 +173,18 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
     return kk == 0 ? bw[t].x : kk == 1 ? bw[t].y : kk == 2 ? bw[t].z : bw[t].w;
   };
 
-  // ---- prologue: two steps of loads in flight, first operands of step 0 ready ----
+  // ---- prologue: steps 0 and 1 and the first part of step 2 in flight, operands of step 0 ready ----
 #pragma unroll
   for (int idx = 0; idx < L; ++idx) issue_one(0, idx);
   if (ksteps > 1) {
 #pragma unroll
     for (int idx = 0; idx < L; ++idx) issue_one(1, idx);
+  }
+  if (ksteps > 2) {
+#pragma unroll
+    for (int idx = 0; idx < LA; ++idx) issue_one(2, idx);
+    WQ_WAITCNT_VM(L + LA);
+  } else if (ksteps > 1) {
     WQ_WAITCNT_VM(L);
   } else {
     WQ_WAITCNT_VM(0);
@@ -197,7 +206,7 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   for (int ks = 0; ks < ksteps; ++ks) {
     const unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
     const unsigned char* next_slot = lds + ((ks + 1) % Cfg::kStages) * Cfg::kStageBytes;
-    const bool ahead2 = ks + 2 < ksteps;
+    const bool ahead2 = ks + 2 < ksteps, ahead3 = ks + 3 < ksteps;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       const int cur = kk & 1, nxt = cur ^ 1;
@@ -234,12 +243,17 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
             }
           }
         }
-        // direct loads of step ks+2, spread over phases 0-2
-        if (kk < 3 && ahead2) {
-          const int g = kk * NSLOT + sl;
-          const int l0 = g * L / (3 * NSLOT), l1 = (g + 1) * L / (3 * NSLOT);
+        // direct loads: the second part of step ks+2 in phase 0; the first part of step
+        // ks+3 in phase 3, into the slot of this step, which nobody reads any more
+        if (kk == 0 && ahead2) {
+          const int l0 = LA + sl * LB / NSLOT, l1 = LA + (sl + 1) * LB / NSLOT;
 #pragma unroll
           for (int idx = l0; idx < l1; ++idx) issue_one(ks + 2, idx);
+        }
+        if (kk == 3 && ahead3) {
+          const int l0 = sl * LA / NSLOT, l1 = (sl + 1) * LA / NSLOT;
+#pragma unroll
+          for (int idx = l0; idx < l1; ++idx) issue_one(ks + 3, idx);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -251,7 +265,54 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   }
 
   // ---- epilogue ----
-  // accumulator register r of lane (j, h) is element (row 8*(r/4) + 4*h + r%4, col j)
+  // accumulator register r of lane (j, h) is element (row 8*(r/4) + 4*h + r%4, col j) of its
+  // 32x32 sub-tile: a lane holds single columns, so direct stores would be 2-byte accesses in
+  // 64-byte runs.  Instead each wavefront transposes through its own piece of LDS (idle now:
+  // every real read of the ring was waited for before the last barrier) RT row sub-tiles at a
+  // time: (acc + bias) -> fp16 -> LDS, then 16 bytes per lane along the row: + residual, store.
+  const bool wide = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(Y) & 15u) == 0) &&
+                    ((reinterpret_cast<uintptr_t>(epilogue.residual) & 15u) == 0);
+  if (wide) {
+    constexpr int RT = (TN >= 4 ? 2 : 4) < TME ? (TN >= 4 ? 2 : 4) : TME;  // sub-tiles per pass: <= 16 KB per wavefront
+    constexpr int kPitch = TN * 64;                                          // bytes per staged row
+    static_assert(4 * RT * 32 * kPitch <= Cfg::kLdsBytes, "epilogue staging exceeds the ring");
+    unsigned char* stage = lds + wave * (RT * 32 * kPitch);
+    float bv[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+      const int n = n0 + (wn * TN + t) * 32 + lj;
+      bv[t] = (epilogue.bias && n < N) ? (float)epilogue.bias[n] : 0.0f;
+    }
+#pragma unroll
+    for (int i0 = 0; i0 < TME; i0 += RT) {
+#pragma unroll
+      for (int ii = 0; ii < RT; ++ii)
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row = ii * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+            *reinterpret_cast<half_t*>(stage + row * kPitch + (t * 32 + lj) * 2) = (half_t)(acc[i0 + ii][t][r] + bv[t]);
+          }
+      // LDS operations of one wavefront execute in order: no barrier between write and read
+      constexpr int kChunksPerRow = TN * 4;                 // 16-byte chunks
+      constexpr int kIters = RT * 32 * kChunksPerRow / 64;
+#pragma unroll
+      for (int it = 0; it < kIters; ++it) {
+        const int c = it * 64 + lane;
+        const int row = c / kChunksPerRow, cc = c % kChunksPerRow;
+        half8_t h = *reinterpret_cast<const half8_t*>(stage + row * kPitch + cc * 16);
+        const int m = m0 + (wm * TME + i0) * 32 + row;
+        const int n = n0 + wn * TN * 32 + cc * 8;
+        if (m < M && n < N) {
+          const int64_t off = (int64_t)m * N + n;
+          if (epilogue.residual) h = h + *reinterpret_cast<const half8_t*>(epilogue.residual + off);
+          *reinterpret_cast<half8_t*>(Y + off) = h;
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < TN; ++t) {
     const int n = n0 + (wn * TN + t) * 32 + lj;
