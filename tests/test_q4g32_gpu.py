@@ -232,3 +232,27 @@ def test_two_pass_small_batch_for_mid_m(ops, u, oracle):
     u.assert_close(got, oracle.q4g32_linear(W, S, x, bias=bias, residual=res, nthreads=8), "two-pass small batch")
     got = u.host(ops.q4g32_linear(u.dev(W), u.dev(S), u.dev(x)))
     u.assert_close(got, oracle.q4g32_linear(W, S, x, nthreads=8), "two-pass small batch, plain")
+
+
+def test_gemm_row_wise_and_element_wise_epilogues_agree(ops, u, oracle):
+    """The GEMM stores 16 bytes per lane when N % 8 == 0 and y / residual are 16-byte aligned, single
+    elements otherwise: both paths, same numbers."""
+    import torch
+
+    M, N, K = 300, 520, 1024
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=31)
+    rng = np.random.default_rng(10)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    ref = oracle.q4g32_linear(W, S, x, bias=bias, residual=res, nthreads=8)
+    dW, dS, dx, db = u.dev(W), u.dev(S), u.dev(x), u.dev(bias)
+    aligned = ops.q4g32_linear(dW, dS, dx, bias=db, residual=u.dev(res), kernel="gemm")
+    u.assert_close(u.host(aligned), ref, "aligned")
+    # y and residual two bytes off a 16-byte boundary
+    ybuf = torch.zeros(M * N + 8, dtype=torch.float16, device="cuda")
+    rbuf = torch.zeros(M * N + 8, dtype=torch.float16, device="cuda")
+    rbuf[1:1 + M * N] = u.dev(res).reshape(-1)
+    y = ybuf[1:1 + M * N].view(M, N)
+    ops.q4g32_linear(dW, dS, dx, bias=db, residual=rbuf[1:1 + M * N].view(M, N), out=y, kernel="gemm")
+    assert torch.equal(y, aligned)
+    assert float(ybuf[0]) == 0.0 and float(ybuf[M * N + 1]) == 0.0  # nothing written outside
