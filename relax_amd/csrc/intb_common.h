@@ -43,6 +43,40 @@ struct IntbGemmEpilogue {
     if (e.unary_op == 1) v = v > 0.0f ? v : 0.0f;
     return (half_t)v;
   }
+  // Row-wise form for 8 consecutive columns n .. n+7 (n % 8 == 0): same arithmetic, 16-byte accesses.
+  // (identity and relu only: eight inlined erf / exp evaluations next to 256 live accumulators
+  // make the compiler spill; silu and gelu keep the element-wise form)
+  __device__ bool wide_ok(int n_cols, const half_t* y) const {
+    return e.activation <= 1 && n_cols % 8 == 0 && e.bias_stride % 8 == 0 &&
+           ((reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(e.bias) |
+             reinterpret_cast<uintptr_t>(e.residual)) & 15u) == 0;
+  }
+  __device__ half8_t apply8(const float (&v)[8], int m, int n) const {
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = v[i];
+    if (e.bias) {
+      const half8_t b = *reinterpret_cast<const half8_t*>(e.bias + (e.bias_stride ? (int64_t)m * e.bias_stride + n : n));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] += (float)b[i];
+    }
+    if (e.activation == 1) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = f[i] > 0.0f ? f[i] : 0.0f;
+    }
+    if (e.residual) {
+      const half8_t r = *reinterpret_cast<const half8_t*>(e.residual + (int64_t)m * N + n);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (e.binary_op == 1) f[i] += (float)r[i];
+        if (e.binary_op == 2) f[i] *= (float)r[i];
+      }
+    }
+    half8_t h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = (half_t)((e.unary_op == 1 && !(f[i] > 0.0f)) ? 0.0f : f[i]);
+    return h;
+  }
 };
 #endif
 

@@ -6,6 +6,7 @@
 // weight loaders below.
 #include "intb_common.h"
 #include "mfma_gemm.h"
+#include "mfma_gemm_lds.h"
 
 int wq_gemm_cfg_override();
 
@@ -77,6 +78,66 @@ struct IntbLoader {
 };
 
 
+// Weight policy of the fully LDS-staged kernel (mfma_gemm_lds.h) for the preprocessed layouts
+// with per-column scales.  A K-step (one 64-row tile) of I = 2 (int8) or 4 (int4) interleaved
+// columns is 128 contiguous bytes, so the B tile is fetched in whole 128-byte lines; the scale
+// of a column never changes and stays in a register.
+template <int NBIT>
+struct IntbLdsPolicy {
+  static constexpr int I = NBIT == 8 ? 2 : 4;
+  static constexpr int kColBytes = 128 / I;
+  static constexpr int kScaleBytes = 0;
+  static constexpr int kStepStride = 128;
+  struct Args {
+    const uint4_t* B;
+    const half_t* scales;
+  };
+  struct Frag {
+    uint4_t w[NBIT == 8 ? 2 : 1];
+  };
+  __device__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
+    const int group = min(n0 / I + (q >> 3), N / I - 1);  // columns past N re-read the last group
+    return reinterpret_cast<const char*>(a.B) + ((int64_t)group * (K >> 6)) * 128 + (q & 7) * 16;
+  }
+  __device__ static const char* s_src(const Args&, int, int) { return nullptr; }
+  __device__ static half_t const_scale(const Args& a, int n) { return a.scales[n]; }
+  __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
+    if (NBIT == 8) {
+      const unsigned char* p = bslot + ((n_local >> 1) * 8 + (n_local & 1) * 4 + 2 * lh) * 16;
+      f.w[0] = *reinterpret_cast<const uint4_t*>(p);
+      f.w[NBIT == 8 ? 1 : 0] = *reinterpret_cast<const uint4_t*>(p + 16);
+    } else {
+      f.w[0] = *reinterpret_cast<const uint4_t*>(bslot + ((n_local >> 2) * 8 + (n_local & 3) * 2 + lh) * 16);
+    }
+  }
+  // int8: piece kk/2 holds 16 k; word j of it holds k = 2j, 2j+1 (bytes 0, 2) and 2j+8, 2j+9 (bytes 1, 3).
+  // int4: word j holds k = 2j + 8i, 2j + 8i + 1 in nibbles i, i + 4.
+  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) {
+    if (NBIT == 8) {
+      const uint4_t& p = f.w[NBIT == 8 ? (kk >> 1) : 0];
+      const uint32_t word = j == 0 ? p.x : j == 1 ? p.y : j == 2 ? p.z : p.w;
+      return u8x2_to_half2(word, (kk & 1) ? 0x04030401u : 0x04020400u) * s2;
+    }
+    const uint32_t word = j == 0 ? f.w[0].x : j == 1 ? f.w[0].y : j == 2 ? f.w[0].z : f.w[0].w;
+    const half2_t off = {(half_t)1032.0f, (half_t)1032.0f};
+    return (as_half2(and_or(word >> (4 * kk), 0x000F000Fu, 0x64006400u)) - off) * s2;
+  }
+};
+
+template <int NBIT>
+static int intb_gemm_lds(int cfg, const char* who, const int8_t* B, const uint16_t* scales, const uint16_t* A,
+                         uint16_t* C, const IntbGemmEpilogue& gep, int64_t m, int64_t n, int64_t k,
+                         hipStream_t stream) {
+  using P = IntbLdsPolicy<NBIT>;
+  const typename P::Args largs{(const uint4_t*)B, (const half_t*)scales};
+  switch (cfg) {
+    case 11: return launch_gemm_lds<P, IntbGemmEpilogue, 8, 2, 1, 4, 1>(who, largs, A, C, gep, m, n, k, stream);
+    case 12: return launch_gemm_lds<P, IntbGemmEpilogue, 4, 2, 1, 4, 2>(who, largs, A, C, gep, m, n, k, stream);
+    case 17: return launch_gemm_lds<P, IntbGemmEpilogue, 4, 1, 1, 4, 2>(who, largs, A, C, gep, m, n, k, stream);
+    default: return fail(WQ_EINVAL, "%s: unknown tile configuration %d", who, cfg);
+  }
+}
+
 static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
                             const uint16_t* scales, const uint16_t* bias, const uint16_t* residual,
                             uint16_t* C, int activation, int binary_op, int unary_op, int64_t m,
@@ -110,8 +171,19 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
     if (m <= WQ_SMALL_BATCH_MAX_M)
       return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
   }
-  const int cfg = wq_gemm_cfg_override() ? wq_gemm_cfg_override() : choose_gemm_cfg(m, n, false);
   const IntbGemmEpilogue gep{ep, (int)n};
+  // per-column scales: the fully LDS-staged kernel (11, 12, 17) except between M = 320 and 1536,
+  // where the 128x256 register-staged tiles fill the CUs better (timings at K = 8192, N = 28672);
+  // fine-grained scales: the register-staged kernel (1..4)
+  int cfg = wq_gemm_cfg_override();
+  if (!cfg) cfg = group ? choose_gemm_cfg(m, n, false) : (m <= 320 ? 17 : m <= 1536 ? 2 : 11);
+  // silu / gelu run the element-wise epilogue, whose inlined exp / erf code does not fit next to
+  // the 256 accumulator registers of the 256x256 tile: stay with 128-row tiles
+  if (!wq_gemm_cfg_override() && activation >= WQ_ACT_SILU && cfg == 11) cfg = 2;
+  if (cfg >= 11 && !group)
+    return nbit == 8 ? intb_gemm_lds<8>(cfg, who, B, scales, A, C, gep, m, n, k, stream)
+                     : intb_gemm_lds<4>(cfg, who, B, scales, A, C, gep, m, n, k, stream);
+  if (cfg >= 11) cfg = cfg == 17 ? 4 : cfg == 11 ? 1 : 2;
   if (nbit == 8) {
     const IntbLoader<8>::Args bargs{(const uint4_t*)B, (const half_t*)scales, group};
     return launch_mfma_gemm_cfg<IntbLoader<8>, IntbGemmEpilogue>(cfg, who, bargs, A, C, gep, m, n, k, stream);

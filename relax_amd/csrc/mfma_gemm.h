@@ -23,6 +23,7 @@
 #ifndef RELAX_AMD_CSRC_MFMA_GEMM_H_
 #define RELAX_AMD_CSRC_MFMA_GEMM_H_
 
+#include "gemm_epilogue.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
@@ -52,8 +53,7 @@ __device__ __forceinline__ int lds_a_offset(int row, int chunk) {
 //   static void init(Lane&, const Args&, int n, int lh, int K, int N);   n is already clamped
 //   static void load(Frag&, const Lane&, const Args&, int ks, int lh, int K, bool ktail);
 //   static void dequant(const Frag&, half8_t out[4]);                    operands of the 4 MFMAs
-// Epilogue policy interface:
-//   half_t operator()(float acc, int m, int n) const;
+// Epilogue policy interface: see gemm_epilogue.h.
 template <class Loader, class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU, bool KTAIL>
 __global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
 void wq_mfma_gemm_kernel(typename Loader::Args bargs, const half_t* __restrict__ X,
@@ -173,7 +173,16 @@ void wq_mfma_gemm_kernel(typename Loader::Args bargs, const half_t* __restrict__
   }
 
   // ---- epilogue ----
-  // accumulator register r of lane (j, h) is element (row 8*(r/4) + 4*h + r%4, col j)
+  // Row-wise through LDS (gemm_epilogue.h): the activation buffers are idle after the last
+  // barrier of the loop, and each wavefront stages in a piece of its own.
+  if (epilogue.wide_ok(N, Y)) {
+    using ECfg = RowwiseEpilogueCfg<TM, TN>;
+    static_assert(WM * WN * ECfg::kBytesPerWave <= Cfg::kLdsBytes, "epilogue staging exceeds the activation buffers");
+    store_tile_rowwise<Epilogue, TM, TN>(acc, epilogue, Y, M, N, m0 + wm * TM * 32, n0 + wn * TN * 32,
+                                         lds + wave * ECfg::kBytesPerWave, lane);
+    return;
+  }
+  // element-wise: accumulator register r of lane (j, h) is element (row 8*(r/4) + 4*h + r%4, col j)
 #pragma unroll
   for (int t = 0; t < TN; ++t) {
     const int n = n0 + (wn * TN + t) * 32 + lj;
@@ -223,18 +232,16 @@ static int launch_mfma_gemm_cfg(int cfg, const char* who, const typename Loader:
   }
 }
 
-// Tile shape from the problem shape, from timings at M = 96 .. 512 and 2048 of the
-// Llama-7B shapes (format A) and of K = 8192, N = 28672 (format B): what matters at
-// mid M is the number of tiles against 256 CUs.  Register-staged kernel (format B,
-// and format A when K is not a multiple of 64): 64x128 up to M = 128, 128x128 up to
-// 256, else 128x256.  Fully LDS-staged kernel (format A): 64x128 register-staged
-// tiles up to M = 128 when N is large, 128x256 (12) below M = 256, and from there
+// Tile shape from the problem shape, from timings at M = 96 .. 2048 of the Llama-7B shapes
+// (format A) and of K = 8192, N = 28672 (format B): what matters at mid M is the number of
+// tiles against 256 CUs.  Register-staged kernel (fine-grained format B, and format A when K is
+// not a multiple of 64): 64x128 up to M = 128, 128x128 up to 256, else 128x256.  Fully
+// LDS-staged kernel: 128x128 tiles, two workgroups per CU (17) up to M = 384, above that
 // 256x256 with one wavefront per SIMD (11).
 inline int choose_gemm_cfg(int64_t M, int64_t N, bool lds_staged) {
-  if (M <= 64) return 3;
+  (void)N;
   if (!lds_staged) return M <= 128 ? 3 : M <= 256 ? 4 : 2;
-  if (M <= 128 && N >= 8192) return 3;
-  return M >= 256 ? 11 : 12;
+  return M <= 384 ? 17 : 11;
 }
 
 }  // namespace wq

@@ -1,5 +1,5 @@
-// Format A prefill GEMM, fully LDS-staged variant for the gfx950 matrix cores:
-//   y[m,n] = epilogue( sum_k x[m,k] * ((code[n,k] - 7) * S[n,k/32]) )
+// Prefill GEMM, fully LDS-staged variant for the gfx950 matrix cores, both weight formats:
+//   y[m,n] = epilogue( sum_k x[m,k] * dequant(w)[n,k] )
 //
 // Every operand of a K-step (64 k) travels global -> LDS with the direct
 // global_load_lds_dwordx4 path: no staging registers, no VALU work, and the loads
@@ -8,25 +8,38 @@
 //       c ^ ((r >> 1) & 7) (the swizzle is applied to the GLOBAL address each lane fetches,
 //       because the LDS side of a direct load is fixed: lane l writes 16 bytes at
 //       base + 16*l);
-//   B   BN rows x 32 B of packed codes (8 words), chunk (n, h) at (2n + h) * 16;
-//   S   BN rows x 4 B: the two scales of the step.
+//   B   BN columns x 32 or 64 B of packed codes, still packed, in the order the weight
+//       format's policy fetches them;
+//   S   (format A only) BN x 4 B: the two scales of the step.
 // A wavefront then reads, per K-step, TM*4 activation fragments, and per weight
-// sub-tile ONE 16-byte piece of codes plus one scale: MFMA lane (j, h) needs 8
-// K-values of column j, which is one packed word, so the weights are dequantized
-// in registers (q4_word_dequant_natural: bit-exact, natural K order, hence no
-// rearrangement of the activations) and never exist in LDS as fp16.
+// sub-tile its 32 codes (16 or 32 bytes) plus one scale: MFMA lane (j, h) needs 8
+// K-values of column j per MFMA, so the weights are dequantized in registers by the
+// policy's bit-exact pair function (natural K order, hence no rearrangement of the
+// activations) and never exist in LDS as fp16.
 //
 // Synchronisation: vector memory operations retire in order, so s_waitcnt vmcnt(loads of
 // one step) means "this wavefront's loads of the step before have landed"; one raw
 // s_barrier per K-step then says the same for the whole workgroup (the fence in
 // __syncthreads would force vmcnt(0)).  The schedule inside a K-step is described at
-// q4g32_gemm_lds_tile.
+// gemm_lds_tile.
+//
+// A weight policy provides
+//   kColBytes            packed bytes per column and K-step (32 or 64)
+//   kScaleBytes          bytes of scales per column and K-step staged in LDS (4 or 0)
+//   Args, Frag           kernel arguments; a lane's packed codes + scale of one column for one step
+//   b_src(args, n0, q, N, K)   global address (step 0) of 16-byte chunk q of the B tile at column n0
+//   kStepStride          bytes between consecutive K-steps of a chunk
+//   s_src(args, n, K)    global address (step 0) of the 4 scale bytes of column n       (kScaleBytes > 0)
+//   const_scale(args, n) the scale of column n                                          (kScaleBytes == 0)
+//   read(frag, bslot, sslot, n_local, lh)   LDS -> registers
+//   pair(frag, kk, j, s2)      dequantized weights (k = 8kk + 2j, 8kk + 2j + 1) of the lane's column
 #ifndef RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 #define RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 
 #include <algorithm>
 #include <type_traits>
 
+#include "gemm_epilogue.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
@@ -35,7 +48,7 @@ namespace wq {
 // Splitting of the last round's tiles (on by default; switch for measurement).
 inline int g_gemm_tail_split = 1;
 
-template <int TM, int TN, int WM, int WN>
+template <class Policy, int TM, int TN, int WM, int WN>
 struct LdsGemmCfg {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
   static constexpr int kThreads = 256;
@@ -44,13 +57,14 @@ struct LdsGemmCfg {
   static constexpr int kStages = 3;
   static constexpr int kAOff = 0;
   static constexpr int kBOff = BM * 128;
-  static constexpr int kSOff = kBOff + BN * 32;
-  static constexpr int kStageBytes = kSOff + BN * 4;
+  static constexpr int kSOff = kBOff + BN * Policy::kColBytes;
+  static constexpr int kStageBytes = kSOff + BN * Policy::kScaleBytes;
   static constexpr int kLdsBytes = kStages * kStageBytes;
   static constexpr int kALoads = BM / 32;   // direct loads per wavefront per step (64 chunks each)
-  static constexpr int kBLoads = BN / 128;
+  static constexpr int kBLoads = BN * Policy::kColBytes / 4096;
   static_assert(BN % 128 == 0 && BN <= 256, "B tile: 128 or 256 columns");
-  static constexpr int kLoadsPerStage = kALoads + kBLoads + 1;
+  static constexpr int kSLoads = Policy::kScaleBytes ? 1 : 0;
+  static constexpr int kLoadsPerStage = kALoads + kBLoads + kSLoads;
 };
 
 // XOR pattern of the activation tile: consecutive rows alternate between the two
@@ -83,16 +97,14 @@ typedef void __attribute__((address_space(3))) * wq_lptr_t;
 // One barrier per K-step suffices: slot ks%3 is refilled by loads issued after the barrier
 // of step ks, and every wavefront has waited for its last LDS reads of that slot (the
 // phase-3 fragments) before that barrier.
-template <class Epilogue, int TM, int TN, int WM, int WN, int TME>
-__device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__ W,
-                                                    const half_t* __restrict__ S,
-                                                    const half_t* __restrict__ X,
-                                                    half_t* __restrict__ Y, const Epilogue& epilogue,
-                                                    int M, int N, int K, int m0, int n0,
-                                                    unsigned char* lds) {
-  using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
+template <class Policy, class Epilogue, int TM, int TN, int WM, int WN, int TME>
+__device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs,
+                                              const half_t* __restrict__ X, half_t* __restrict__ Y,
+                                              const Epilogue& epilogue, int M, int N, int K, int m0,
+                                              int n0, unsigned char* lds) {
+  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN>;
   constexpr int kALoadsE = Cfg::kALoads * TME / TM;  // direct A loads per wavefront per step
-  constexpr int L = kALoadsE + Cfg::kBLoads + 1;     // direct loads per wavefront per step
+  constexpr int L = kALoadsE + Cfg::kBLoads + Cfg::kSLoads;  // direct loads per wavefront per step
   constexpr int NSLOT = TME * TN;                    // MFMAs per phase
   constexpr int NPAIR = TN * 4;                      // weight pairs to unpack per phase
   constexpr int LA = L / 2;                          // loads of a step issued in phase 3 (three steps ahead) ...
@@ -103,7 +115,6 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int lj = lane & 31, lh = lane >> 5;
-  const int G = K >> 5;
   const int ksteps = K >> 6;
 
   // ---- global sources of this lane's direct loads (rows past M / N are clamped:
@@ -117,14 +128,12 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   }
   const char* b_src[Cfg::kBLoads];
 #pragma unroll
-  for (int i = 0; i < Cfg::kBLoads; ++i) {
-    const int q = (wave * Cfg::kBLoads + i) * 64 + lane;
-    const int n = q >> 1, h = q & 1;
-    b_src[i] = reinterpret_cast<const char*>(W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
-  }
-  // (with BN = 128 wavefronts 2 and 3 repeat the loads of wavefronts 0 and 1)
-  const int s_row = (wave * 64) % Cfg::BN + lane;
-  const char* s_src = reinterpret_cast<const char*>(S + (int64_t)min(n0 + s_row, N - 1) * G);
+  for (int i = 0; i < Cfg::kBLoads; ++i)
+    b_src[i] = Policy::b_src(wargs, n0, (wave * Cfg::kBLoads + i) * 64 + lane, N, K);
+  // scales staged per step (format A): 64 columns per wavefront (with BN = 128 wavefronts 2
+  // and 3 repeat the loads of wavefronts 0 and 1)
+  const char* s_src = nullptr;
+  if (Cfg::kSLoads) s_src = Policy::s_src(wargs, min(n0 + (wave * 64) % Cfg::BN + lane, N - 1), K);
 
   // direct load number idx (0 .. L-1) of step ks
   auto issue_one = [&](int ks, int idx) {
@@ -134,7 +143,7 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
                                        (wq_lptr_t)(slot + Cfg::kAOff + (wave * kALoadsE + idx) * 1024), 16, 0, 0);
     } else if (idx < kALoadsE + Cfg::kBLoads) {
       const int i = idx - kALoadsE;
-      __builtin_amdgcn_global_load_lds((wq_gptr_t)(b_src[i] + (int64_t)ks * 32),
+      __builtin_amdgcn_global_load_lds((wq_gptr_t)(b_src[i] + (int64_t)ks * Policy::kStepStride),
                                        (wq_lptr_t)(slot + Cfg::kBOff + (wave * Cfg::kBLoads + i) * 1024), 16, 0, 0);
     } else {
       __builtin_amdgcn_global_load_lds((wq_gptr_t)(s_src + (int64_t)ks * 4),
@@ -150,15 +159,19 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.0f;
 
-  uint4_t bw[TN];   // this lane's packed weights of the step being unpacked
+  typename Policy::Frag bw[TN];   // this lane's packed weights (and scale) of the step being unpacked
   half_t bs[TN];
+  if (!Cfg::kSLoads) {
+#pragma unroll
+    for (int t = 0; t < TN; ++t) bs[t] = Policy::const_scale(wargs, min(n0 + (wn * TN + t) * 32 + lj, N - 1));
+  }
   half8_t aop[2][TME], bop[2][TN];
   auto read_b = [&](const unsigned char* slot) {
 #pragma unroll
     for (int t = 0; t < TN; ++t) {
       const int n = (wn * TN + t) * 32 + lj;
-      bw[t] = *reinterpret_cast<const uint4_t*>(slot + Cfg::kBOff + (n * 2 + lh) * 16);
-      bs[t] = *reinterpret_cast<const half_t*>(slot + Cfg::kSOff + n * 4 + lh * 2);
+      Policy::read(bw[t], slot + Cfg::kBOff, n, lh);
+      if (Cfg::kSLoads) bs[t] = *reinterpret_cast<const half_t*>(slot + Cfg::kSOff + n * 4 + lh * 2);
     }
   };
   auto read_a = [&](const unsigned char* slot, int kk, half8_t (&dst)[TME]) {
@@ -168,9 +181,6 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
       dst[i] = *reinterpret_cast<const half8_t*>(slot + Cfg::kAOff + row * 128 +
                                                  (((4 * lh + kk) ^ WQ_SWZ(row)) << 4));
     }
-  };
-  auto word_of = [&](int t, int kk) -> uint32_t {
-    return kk == 0 ? bw[t].x : kk == 1 ? bw[t].y : kk == 2 ? bw[t].z : bw[t].w;
   };
 
   // ---- prologue: steps 0 and 1 and the first part of step 2 in flight, operands of step 0 ready ----
@@ -196,7 +206,8 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   for (int t = 0; t < TN; ++t) {
     const half2_t s2 = {bs[t], bs[t]};
     half2_t d[4];
-    q4_word_dequant_natural(bw[t].x, s2, d);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) d[j] = Policy::pair(bw[t], 0, j, s2);
     bop[0][t] = half8_t{d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
   }
 
@@ -239,7 +250,7 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
             for (int p = p0; p < p1; ++p) {
               const int tt = p >> 2, j = p & 3;
               const half2_t s2 = {bs[tt], bs[tt]};
-              dq[tt][j] = q4_pair_dequant_natural(word_of(tt, (kk + 1) & 3), j, s2);
+              dq[tt][j] = Policy::pair(bw[tt], (kk + 1) & 3, j, s2);
             }
           }
         }
@@ -265,54 +276,16 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
   }
 
   // ---- epilogue ----
-  // accumulator register r of lane (j, h) is element (row 8*(r/4) + 4*h + r%4, col j) of its
-  // 32x32 sub-tile: a lane holds single columns, so direct stores would be 2-byte accesses in
-  // 64-byte runs.  Instead each wavefront transposes through its own piece of LDS (idle now:
-  // every real read of the ring was waited for before the last barrier) RT row sub-tiles at a
-  // time: (acc + bias) -> fp16 -> LDS, then 16 bytes per lane along the row: + residual, store.
-  const bool wide = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(Y) & 15u) == 0) &&
-                    ((reinterpret_cast<uintptr_t>(epilogue.residual) & 15u) == 0);
-  if (wide) {
-    constexpr int RT = (TN >= 4 ? 2 : 4) < TME ? (TN >= 4 ? 2 : 4) : TME;  // sub-tiles per pass: <= 16 KB per wavefront
-    constexpr int kPitch = TN * 64;                                          // bytes per staged row
-    static_assert(4 * RT * 32 * kPitch <= Cfg::kLdsBytes, "epilogue staging exceeds the ring");
-    unsigned char* stage = lds + wave * (RT * 32 * kPitch);
-    float bv[TN];
-#pragma unroll
-    for (int t = 0; t < TN; ++t) {
-      const int n = n0 + (wn * TN + t) * 32 + lj;
-      bv[t] = (epilogue.bias && n < N) ? (float)epilogue.bias[n] : 0.0f;
-    }
-#pragma unroll
-    for (int i0 = 0; i0 < TME; i0 += RT) {
-#pragma unroll
-      for (int ii = 0; ii < RT; ++ii)
-#pragma unroll
-        for (int t = 0; t < TN; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int row = ii * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            *reinterpret_cast<half_t*>(stage + row * kPitch + (t * 32 + lj) * 2) = (half_t)(acc[i0 + ii][t][r] + bv[t]);
-          }
-      // LDS operations of one wavefront execute in order: no barrier between write and read
-      constexpr int kChunksPerRow = TN * 4;                 // 16-byte chunks
-      constexpr int kIters = RT * 32 * kChunksPerRow / 64;
-#pragma unroll
-      for (int it = 0; it < kIters; ++it) {
-        const int c = it * 64 + lane;
-        const int row = c / kChunksPerRow, cc = c % kChunksPerRow;
-        half8_t h = *reinterpret_cast<const half8_t*>(stage + row * kPitch + cc * 16);
-        const int m = m0 + (wm * TME + i0) * 32 + row;
-        const int n = n0 + wn * TN * 32 + cc * 8;
-        if (m < M && n < N) {
-          const int64_t off = (int64_t)m * N + n;
-          if (epilogue.residual) h = h + *reinterpret_cast<const half8_t*>(epilogue.residual + off);
-          *reinterpret_cast<half8_t*>(Y + off) = h;
-        }
-      }
-    }
+  // Row-wise through LDS (gemm_epilogue.h); the ring is idle now: every real read of it was
+  // waited for before the last barrier, and each wavefront stages in a piece of its own.
+  if (epilogue.wide_ok(N, Y)) {
+    using ECfg = RowwiseEpilogueCfg<TME, TN>;
+    static_assert(4 * ECfg::kBytesPerWave <= Cfg::kLdsBytes, "epilogue staging exceeds the ring");
+    store_tile_rowwise<Epilogue, TME, TN>(acc, epilogue, Y, M, N, m0 + wm * TME * 32, n0 + wn * TN * 32,
+                                          lds + wave * ECfg::kBytesPerWave, lane);
     return;
   }
+  // element-wise: accumulator register r of lane (j, h) is element (row 8*(r/4) + 4*h + r%4, col j)
 #pragma unroll
   for (int t = 0; t < TN; ++t) {
     const int n = n0 + (wn * TN + t) * 32 + lj;
@@ -332,12 +305,12 @@ __device__ __forceinline__ void q4g32_gemm_lds_tile(const uint32_t* __restrict__
 // as fill complete rounds of the machine); the tiles of the last, partially filled
 // round are cut into `split` row slices of TM/split sub-tiles so that the round is
 // shorter instead of leaving most CUs idle while a few finish whole tiles.
-template <class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU>
+template <class Policy, class Epilogue, int TM, int TN, int WM, int WN, int WAVES_PER_EU>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WAVES_PER_EU, WAVES_PER_EU)))
-void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restrict__ S,
-                           const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epilogue,
-                           int M, int N, int K, int tiles_m, int tiles_n, int n_full, int split) {
-  using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
+void gemm_lds_kernel(typename Policy::Args wargs, const half_t* __restrict__ X, half_t* __restrict__ Y,
+                     Epilogue epilogue, int M, int N, int K, int tiles_m, int tiles_n, int n_full,
+                     int split) {
+  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   int pid = blockIdx.x;
   if (pid < n_full) {
@@ -346,8 +319,8 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
     const int xcd = pid & 7, idx = pid >> 3;
     pid = xcd * per + min(xcd, rem) + idx;
     const int tile_m = pid % tiles_m, tile_n = pid / tiles_m;
-    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM>(
-        W, S, X, Y, epilogue, M, N, K, tile_m * Cfg::BM, tile_n * Cfg::BN, lds);
+    gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM>(wargs, X, Y, epilogue, M, N, K,
+                                                        tile_m * Cfg::BM, tile_n * Cfg::BN, lds);
     return;
   }
   const int t = n_full + (pid - n_full) / split, part = (pid - n_full) % split;
@@ -356,23 +329,23 @@ void q4g32_gemm_lds_kernel(const uint32_t* __restrict__ W, const half_t* __restr
   if (m0 >= M) return;  // a slice that lies entirely past the last row
   if (split == 2) {
     if constexpr (TM % 2 == 0)
-      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM / 2>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+      gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM / 2>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   } else if (split == 4) {
     if constexpr (TM % 4 == 0)
-      q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM / 4>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+      gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM / 4>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   } else {
-    q4g32_gemm_lds_tile<Epilogue, TM, TN, WM, WN, TM>(W, S, X, Y, epilogue, M, N, K, m0, n0, lds);
+    gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   }
 }
 
-template <class Epilogue, int TM, int TN, int WM, int WN, int WPE>
-static int launch_q4g32_gemm_lds(const uint32_t* W, const uint16_t* S, const uint16_t* x, uint16_t* y,
-                                 const Epilogue& ep, int64_t M, int64_t N, int64_t K,
-                                 hipStream_t stream) {
-  using Cfg = LdsGemmCfg<TM, TN, WM, WN>;
+template <class Policy, class Epilogue, int TM, int TN, int WM, int WN, int WPE>
+static int launch_gemm_lds(const char* who, const typename Policy::Args& wargs, const uint16_t* x,
+                           uint16_t* y, const Epilogue& ep, int64_t M, int64_t N, int64_t K,
+                           hipStream_t stream) {
+  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN>;
   const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM);
   const int tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
-  auto kern = q4g32_gemm_lds_kernel<Epilogue, TM, TN, WM, WN, WPE>;
+  auto kern = gemm_lds_kernel<Policy, Epilogue, TM, TN, WM, WN, WPE>;
   WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                              hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
   // Whole rounds of the machine run whole tiles; the tiles of the last, partial
@@ -391,9 +364,8 @@ static int launch_q4g32_gemm_lds(const uint32_t* W, const uint16_t* S, const uin
       }
     }
   }
-  WQ_LAUNCH("wq_q4g32_gemm", kern, dim3((unsigned)(n_full + rest * split)), dim3(256), Cfg::kLdsBytes,
-            stream, W, (const half_t*)S, (const half_t*)x, (half_t*)y, ep, (int)M, (int)N, (int)K,
-            tiles_m, tiles_n, n_full, split);
+  WQ_LAUNCH(who, kern, dim3((unsigned)(n_full + rest * split)), dim3(256), Cfg::kLdsBytes, stream, wargs,
+            (const half_t*)x, (half_t*)y, ep, (int)M, (int)N, (int)K, tiles_m, tiles_n, n_full, split);
   return WQ_OK;
 }
 

@@ -52,6 +52,37 @@ struct Q4G32Loader {
 };
 
 
+// Weight policy of the fully LDS-staged kernel (mfma_gemm_lds.h) for format A: per K-step a
+// column is 32 bytes of codes (chunk (n, h) of the B tile = 16 bytes = one scale group) and two
+// scales (4 bytes, staged in LDS with the codes).
+struct Q4G32LdsPolicy {
+  static constexpr int kColBytes = 32;
+  static constexpr int kScaleBytes = 4;
+  static constexpr int kStepStride = 32;
+  struct Args {
+    const uint32_t* W;
+    const half_t* S;
+  };
+  struct Frag {
+    uint4_t w;
+  };
+  __device__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
+    const int n = q >> 1, h = q & 1;
+    return reinterpret_cast<const char*>(a.W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
+  }
+  __device__ static const char* s_src(const Args& a, int n, int K) {
+    return reinterpret_cast<const char*>(a.S + (int64_t)n * (K >> 5));
+  }
+  __device__ static half_t const_scale(const Args&, int) { return (half_t)0.0f; }
+  __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
+    f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
+  }
+  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) {
+    const uint32_t word = kk == 0 ? f.w.x : kk == 1 ? f.w.y : kk == 2 ? f.w.z : f.w.w;
+    return q4_pair_dequant_natural(word, j, s2);
+  }
+};
+
 }  // namespace wq
 
 // Tile shape override for measurement (0 = choose from the problem shape).
@@ -79,18 +110,20 @@ extern "C" int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_
   WQ_REQUIRE(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), "wq_q4g32_gemm: too large");
   int cfg = g_gemm_cfg_override ? g_gemm_cfg_override : choose_gemm_cfg(M, N, true);
   const Q4G32Loader::Args bargs{W, (const half_t*)S};
+  const Q4G32LdsPolicy::Args largs{W, (const half_t*)S};
   const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
-  // 11..14: the fully LDS-staged kernel (needs K % 64 == 0 and 4-byte aligned scale pairs)
+  // 11..17: the fully LDS-staged kernel (needs K % 64 == 0 and 4-byte aligned scale pairs)
   if (cfg >= 11 && K % 64 == 0 && ((uintptr_t)S & 3u) == 0) {
     switch (cfg) {
-      case 11: return launch_q4g32_gemm_lds<Q4G32Epilogue, 8, 2, 1, 4, 1>(W, S, x, y, ep, M, N, K, stream);
-      case 12: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 2, 1, 4, 2>(W, S, x, y, ep, M, N, K, stream);
-      case 13: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 2, 2, 2, 2>(W, S, x, y, ep, M, N, K, stream);
-      case 14: return launch_q4g32_gemm_lds<Q4G32Epilogue, 4, 4, 2, 2, 1>(W, S, x, y, ep, M, N, K, stream);
+      case 11: return launch_gemm_lds<Q4G32LdsPolicy, Q4G32Epilogue, 8, 2, 1, 4, 1>("wq_q4g32_gemm", largs, x, y, ep, M, N, K, stream);
+      case 12: return launch_gemm_lds<Q4G32LdsPolicy, Q4G32Epilogue, 4, 2, 1, 4, 2>("wq_q4g32_gemm", largs, x, y, ep, M, N, K, stream);
+      case 13: return launch_gemm_lds<Q4G32LdsPolicy, Q4G32Epilogue, 4, 2, 2, 2, 2>("wq_q4g32_gemm", largs, x, y, ep, M, N, K, stream);
+      case 14: return launch_gemm_lds<Q4G32LdsPolicy, Q4G32Epilogue, 4, 4, 2, 2, 1>("wq_q4g32_gemm", largs, x, y, ep, M, N, K, stream);
+      case 17: return launch_gemm_lds<Q4G32LdsPolicy, Q4G32Epilogue, 4, 1, 1, 4, 2>("wq_q4g32_gemm", largs, x, y, ep, M, N, K, stream);
       default: return fail(WQ_EINVAL, "wq_q4g32_gemm: unknown tile configuration %d", cfg);
     }
   }
-  if (cfg >= 11) cfg = (cfg == 11 || cfg >= 14) ? 1 : 2;  // not eligible: register-staged kernel, same tile
+  if (cfg >= 11) cfg = cfg == 17 ? 4 : (cfg == 11 || cfg == 14) ? 1 : 2;  // not eligible: register-staged kernel, same tile
   return launch_mfma_gemm_cfg<Q4G32Loader, Q4G32Epilogue>(cfg, "wq_q4g32_gemm", bargs, x, y, ep, M,
                                                           N, K, stream);
 }

@@ -115,7 +115,7 @@ def test_gemm_finegrained(ops, u, oracle, nbit, M):
 
 
 @pytest.mark.parametrize("nbit", [8, 4])
-@pytest.mark.parametrize("M", [2, 48])
+@pytest.mark.parametrize("M", [2, 48, 130])
 @pytest.mark.parametrize("ep", [
     dict(bias="row"), dict(bias="full"), dict(bias="row", activation="relu"), dict(bias="row", activation="silu"),
     dict(bias="row", activation="gelu"), dict(residual=True), dict(bias="row", residual=True, binary_op="plus"),
@@ -142,6 +142,25 @@ def test_small_batch_work_splits(ops, u, oracle, nbit, group_size, nw, stages):
             _run(ops, u, oracle, M, N, K, nbit, seed=M + nw, group_size=group_size)
     finally:
         _lib.lib().wq_debug_set_skinny_config(0, 0, 0)
+
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 17])
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_gemm_tile_configurations(ops, u, oracle, nbit, cfg):
+    """every tile shape of the register-staged (1-4) and the LDS-staged (11, 12, 17) kernel, ragged M,
+    N smaller than a tile, with and without the row-wise epilogue (bias stride not a multiple of 8)."""
+    from relax_amd import _lib
+
+    _lib.lib().wq_debug_set_gemm_config(cfg)
+    try:
+        for M, N, K in [(70, 64, 64), (130, 320, 448), (257, 192, 1024), (300, 576, 512)]:
+            print(f"intb cfg={cfg} nbit={nbit} M={M} N={N} K={K}", flush=True)
+            _run(ops, u, oracle, M, N, K, nbit, seed=M + cfg)
+        _run(ops, u, oracle, 100, 128, 256, nbit, seed=cfg, bias="row", activation="gelu", residual=True,
+             binary_op="multiply", unary_op="relu")
+        _run(ops, u, oracle, 100, 128, 256, nbit, seed=cfg + 1, bias="full")
+    finally:
+        _lib.lib().wq_debug_set_gemm_config(0)
 
 
 @pytest.mark.parametrize("M", [1, 16, 128, 512])
