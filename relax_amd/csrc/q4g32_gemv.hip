@@ -260,10 +260,36 @@ static int g_gemv_rows = 0;  // 0 = choose from the shape
 static int g_gemv_gpl = 0;
 static int g_gemv_blocks_per_cu = 0;
 
+// Workgroups of <ROWS, MB, GPL> for this shape, and how many of them one CU holds at a time.
+template <int ROWS, int MB, int GPL>
+static bool gemv_geometry(int64_t N, int64_t K, int64_t* nblocks, int* resident_per_cu) {
+  const int G = (int)(K / 32);
+  const int parts = (G + 64 * GPL - 1) / (64 * GPL);
+  const int sets_per_block = parts >= 4 ? 1 : 4 / parts;
+  const int threads = 64 * parts * sets_per_block;
+  if (parts > kGemvMaxWaves || threads > gemv_max_threads<GPL>()) return false;
+  const size_t lds = (size_t)MB * K * 2 + (size_t)MB * G * 4;
+  if (lds > 60 * 1024) return false;
+  const int64_t nsets = (N + ROWS - 1) / ROWS;
+  *nblocks = (nsets + sets_per_block - 1) / sets_per_block;
+  static int cached_threads = 0, cached_per_cu = 0;
+  static size_t cached_lds = 0;
+  if (cached_threads != threads || cached_lds != lds) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, q4g32_gemv_kernel<ROWS, MB, GPL>, threads, lds) != hipSuccess)
+      return false;
+    cached_threads = threads;
+    cached_lds = lds;
+    cached_per_cu = n;
+  }
+  *resident_per_cu = cached_per_cu;
+  return true;
+}
+
 template <int ROWS, int MB, int GPL>
 static int launch_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                        const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t N,
-                       int64_t K, hipStream_t stream) {
+                       int64_t K, int blocks_per_cu, hipStream_t stream) {
   const int G = (int)(K / 32);
   const int parts = (G + 64 * GPL - 1) / (64 * GPL);
   const int sets_per_block = parts >= 4 ? 1 : 4 / parts;
@@ -273,10 +299,9 @@ static int launch_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                 threads);
   const int64_t nsets = (N + ROWS - 1) / ROWS;
   int64_t blocks = (nsets + sets_per_block - 1) / sets_per_block;
-  // Very tall matrices run persistent workgroups that take several turns, with the
-  // loads of the next turn in flight during the current one; for the usual sizes
-  // every workgroup takes a single turn (measured to be slightly faster).
-  const int64_t cap = (int64_t)cu_count() * (g_gemv_blocks_per_cu ? g_gemv_blocks_per_cu : 32);
+  // More workgroups than `blocks_per_cu` per CU: persistent workgroups that take several
+  // turns, with the loads of the next turn in flight during the current one.
+  const int64_t cap = (int64_t)cu_count() * (g_gemv_blocks_per_cu ? g_gemv_blocks_per_cu : blocks_per_cu);
   if (blocks > cap) blocks = cap;
   if (K > 8 * 8 * (int64_t)threads)
     return fail(WQ_EUNSUPPORTED, "wq_q4g32_gemv: K=%lld too large for %d threads", (long long)K,
@@ -293,14 +318,35 @@ static int launch_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x,
   return WQ_OK;
 }
 
+// rows == 0 chooses the rows per wavefront from the shape (timings of the Llama-7B layers):
+// what costs most at these kernel lengths (4 .. 12 us) is a second, partly filled round of
+// workgroups, so take the most rows per wavefront (4, 2, 1) for which all workgroups are
+// resident at once and every CU still has at least two; if nothing fits (tall matrices), one
+// row per wavefront and four persistent workgroups per CU, each taking several turns.
 template <int MB, int GPL>
 static int launch_gemv_rows(int rows, const uint32_t* W, const uint16_t* S, const uint16_t* x,
                             const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t N,
                             int64_t K, hipStream_t stream) {
+  int bpc = 32;
+  if (rows == 0) {
+    const int cus = cu_count();
+    int64_t nb = 0;
+    int per_cu = 0;
+    if (gemv_geometry<4, MB, GPL>(N, K, &nb, &per_cu) && nb >= 2 * cus && nb <= (int64_t)cus * per_cu) {
+      rows = 4;
+    } else if (gemv_geometry<2, MB, GPL>(N, K, &nb, &per_cu) && nb >= 2 * cus && nb <= (int64_t)cus * per_cu) {
+      rows = 2;
+    } else if (gemv_geometry<1, MB, GPL>(N, K, &nb, &per_cu) && nb <= (int64_t)cus * per_cu) {
+      rows = 1;
+    } else {
+      rows = 1;
+      bpc = 4;
+    }
+  }
   switch (rows) {
-    case 1: return launch_gemv<1, MB, GPL>(W, S, x, bias, residual, y, N, K, stream);
-    case 2: return launch_gemv<2, MB, GPL>(W, S, x, bias, residual, y, N, K, stream);
-    default: return launch_gemv<4, MB, GPL>(W, S, x, bias, residual, y, N, K, stream);
+    case 1: return launch_gemv<1, MB, GPL>(W, S, x, bias, residual, y, N, K, bpc, stream);
+    case 2: return launch_gemv<2, MB, GPL>(W, S, x, bias, residual, y, N, K, bpc, stream);
+    default: return launch_gemv<4, MB, GPL>(W, S, x, bias, residual, y, N, K, bpc, stream);
   }
 }
 
@@ -336,7 +382,7 @@ extern "C" int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_
   // (rows longer than 256 groups are split over several wavefronts)
   int gpl = g_gemv_gpl ? g_gemv_gpl
                        : (G <= 64 ? 1 : G <= 128 ? 2 : G <= 192 ? 3 : G <= 256 ? 4 : G <= 384 ? 3 : 2);
-  const int rows = g_gemv_rows ? g_gemv_rows : 2;
+  const int rows = g_gemv_rows;  // 0 = from the shape
   // batches of up to 4 rows of x share one pass over the weights
   for (int64_t m0 = 0; m0 < M;) {
     const int64_t left = M - m0;
@@ -345,7 +391,7 @@ extern "C" int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_
     uint16_t* yp = y + m0 * N;
     int rc;
     if (left >= 4) {
-      rc = launch_gemv_rows<4, 1>(rows > 2 ? 2 : rows, W, S, xp, bias, rp, yp, N, K, stream);
+      rc = launch_gemv_rows<4, 1>(rows == 0 || rows > 2 ? 2 : rows, W, S, xp, bias, rp, yp, N, K, stream);
       m0 += 4;
     } else if (left >= 2) {
       rc = gpl >= 2 ? launch_gemv_rows<2, 2>(rows, W, S, xp, bias, rp, yp, N, K, stream)
