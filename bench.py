@@ -40,8 +40,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # shapes: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one run each) of this script,
 # scaled by what the same counters read for a plain 1 GiB device copy
 # (`--calibrate-copy`): x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28726733
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 272900000
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28746825
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 268700000
 
 
 def gemv_bytes(M, N, K):
@@ -344,7 +344,7 @@ def main():
             del W, S, x, y
         tf = tot_flops / tot_ms / 1e9
         out["gemm"] = {
-            "kernel": "q4g32_gemm_lds_kernel",
+            "kernel": "gemm_lds_kernel<Q4G32LdsPolicy>",
             "value": round(tf, 1),
             "unit": "TFLOP/s",
             "shapes": gem,
