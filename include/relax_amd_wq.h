@@ -165,6 +165,14 @@ int wq_intb_encode(const uint16_t* A, int8_t* w_out, uint16_t* scales, float* sc
  * has no encoder for this format, so the rounding convention is this library's. */
 int wq_q4g32_encode(const uint16_t* A, uint32_t* W, uint16_t* S, int64_t N, int64_t K, wq_stream_t stream);
 
+/* K-major q4f16_1 checkpoints (W uint32 [K/8, N], S fp16 [K/32, N]; the layout of
+ * tests/python/dlight/test_gpu_reduction.py:102-120 and test_gpu_gemv.py:813-830) -> the
+ * [N, K/8] / [N, K/32] layout the kernels above read.  A word holds 8 consecutive k of one
+ * column in both layouts, so this is a transpose of words and scales; run it once at load
+ * time.  Not in place. */
+int wq_q4g32_kn_to_nk(const uint32_t* W_kn, const uint16_t* S_kn, uint32_t* W_nk, uint16_t* S_nk,
+                      int64_t N, int64_t K, wq_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Calibration kernels: the measured ceilings reported next to the vendor peaks
  * (no counterpart in the reference; its methodology precedent is the cache-flush

@@ -275,6 +275,26 @@ def q4g32_encode(Wf: np.ndarray):
     return W, S
 
 
+def q4g32_kn_dequant(W_kn: np.ndarray, S_kn: np.ndarray) -> np.ndarray:
+    """K-major form of the same scheme (tests/python/dlight/test_gpu_reduction.py:112-120):
+    B[k, n] = (fp16((W[k // 8, n] >> 4 * (k % 8)) & 15) - 7) * S[k // 32, n], fp16 [K, N].  numpy restatement."""
+    W_kn = _c(W_kn, np.uint32)
+    S_kn = _c(S_kn, np.float16)
+    k8, N = W_kn.shape
+    K = k8 * 8
+    k = np.arange(K)
+    q = (W_kn[k // 8, :] >> (4 * (k % 8)).astype(np.uint32)[:, None]) & np.uint32(15)
+    return (q.astype(np.float16) - np.float16(7)) * S_kn[k // 32, :]
+
+
+def q4g32_kn_linear(W_kn: np.ndarray, S_kn: np.ndarray, x: np.ndarray) -> np.ndarray:
+    """y[m, n] = sum_k x[m, k] * B[k, n], float32 accumulation over the fp16 weights, fp16 result
+    (test_gpu_reduction.py:121-128 with the accumulate mode the build implements)."""
+    B = q4g32_kn_dequant(W_kn, S_kn).astype(np.float32)
+    x = _c(x, np.float16).astype(np.float32)
+    return (x.reshape(-1, x.shape[-1]) @ B).astype(np.float16)
+
+
 # ------------------------------------------------- synthetic inputs (shared)
 
 

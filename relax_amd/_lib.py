@@ -29,6 +29,7 @@ SIGNATURES = {
     "wq_intb_dequantize": [_vp, _vp, _vp, _i64, _i64, _int, _i64, _vp],
     "wq_fpA_intB_gemm": [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
     "wq_fpA_intB_gemm_residual": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
+    "wq_q4g32_kn_to_nk": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
     "wq_intb_encode": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "wq_q4g32_encode": [_vp, _vp, _vp, _i64, _i64, _vp],
     "wq_calibrate_mfma_f16": [_vp, _i64, _int, ctypes.POINTER(ctypes.c_double), _vp],

@@ -243,3 +243,18 @@ def q4g32_encode(Wf: torch.Tensor):
     S = torch.empty((N, K // 32), dtype=torch.float16, device=Wf.device)
     check(_lib.lib().wq_q4g32_encode(_ptr(Wf), _ptr(W), _ptr(S), N, K, _stream()), "wq_q4g32_encode")
     return W, S
+
+
+def q4g32_kn_to_nk(W_kn: torch.Tensor, S_kn: torch.Tensor):
+    """K-major q4f16_1 weights (``W [K/8, N]``, ``S [K/32, N]``; tests/python/dlight/test_gpu_reduction.py:102-120)
+    -> the ``[N, K/8]`` / ``[N, K/32]`` layout of :func:`q4g32_linear`.  Run once when a checkpoint is loaded."""
+    W_kn = _w32(W_kn)
+    S_kn = _dev(S_kn, torch.float16, "S_kn")
+    k8, N = W_kn.shape
+    K = k8 * 8
+    if K % 32 or tuple(S_kn.shape) != (K // 32, N):
+        raise ValueError(f"S_kn must be [K/32, N] = [{K // 32}, {N}], got {tuple(S_kn.shape)}")
+    W = torch.empty((N, k8), dtype=W_kn.dtype, device=W_kn.device)
+    S = torch.empty((N, K // 32), dtype=torch.float16, device=W_kn.device)
+    check(_lib.lib().wq_q4g32_kn_to_nk(_ptr(W_kn), _ptr(S_kn), _ptr(W), _ptr(S), N, K, _stream()), "wq_q4g32_kn_to_nk")
+    return W, S

@@ -281,3 +281,24 @@ def test_q4g32_encode_definition_and_round_trip(oracle):
     Wgrid = oracle.q4g32_dequant(W0, S0)
     W1, S1 = oracle.q4g32_encode(Wgrid)
     assert np.array_equal(oracle.q4g32_dequant(W1, S1).view(np.uint16), Wgrid.view(np.uint16))
+
+
+def test_kn_layout_oracle_matches_loops_and_nk_form(oracle):
+    """K-major q4f16_1: brute-force loops over the TIR expression on a small case, and equality with the
+    NK oracle on the transposed arrays (a word holds the same 8 k of one column in both layouts)."""
+    rng = np.random.default_rng(6)
+    N, K = 5, 64
+    W_kn = rng.integers(0, 2**32, size=(K // 8, N), dtype=np.uint64).astype(np.uint32)
+    S_kn = rng.uniform(0.005, 0.02, size=(K // 32, N)).astype(np.float16)
+    B = oracle.q4g32_kn_dequant(W_kn, S_kn)
+    for k in range(K):
+        for n in range(N):
+            q = (int(W_kn[k // 8, n]) >> (4 * (k % 8))) & 15
+            want = (np.float16(q) - np.float16(7)) * S_kn[k // 32, n]
+            assert B[k, n].view(np.uint16) == np.float16(want).view(np.uint16)
+    nk = oracle.q4g32_dequant(np.ascontiguousarray(W_kn.T), np.ascontiguousarray(S_kn.T))
+    assert np.array_equal(nk.view(np.uint16), np.ascontiguousarray(B.T).view(np.uint16))
+    x = rng.standard_normal((3, K)).astype(np.float16)
+    y = oracle.q4g32_kn_linear(W_kn, S_kn, x)
+    y_nk = oracle.q4g32_linear(np.ascontiguousarray(W_kn.T), np.ascontiguousarray(S_kn.T), x)
+    assert np.allclose(y.astype(np.float32), y_nk.astype(np.float32), rtol=2e-3, atol=2e-3)

@@ -256,3 +256,19 @@ def test_gemm_row_wise_and_element_wise_epilogues_agree(ops, u, oracle):
     ops.q4g32_linear(dW, dS, dx, bias=db, residual=rbuf[1:1 + M * N].view(M, N), out=y, kernel="gemm")
     assert torch.equal(y, aligned)
     assert float(ybuf[0]) == 0.0 and float(ybuf[M * N + 1]) == 0.0  # nothing written outside
+
+
+@pytest.mark.parametrize("N,K", [(1, 32), (70, 96), (4096, 4096), (1000, 11008)])
+def test_kn_layout_conversion_bit_exact_and_linear(ops, u, oracle, N, K):
+    """K-major checkpoints are transposed once on the device; the result is the NK form bit for bit and the
+    linear layer on it agrees with the K-major oracle."""
+    rng = np.random.default_rng(N + K)
+    W_kn = rng.integers(0, 2**32, size=(K // 8, N), dtype=np.uint64).astype(np.uint32)
+    S_kn = rng.uniform(0.005, 0.02, size=(K // 32, N)).astype(np.float16)
+    W, S = ops.q4g32_kn_to_nk(u.dev(W_kn), u.dev(S_kn))
+    assert np.array_equal(u.host(W).view(np.uint32), np.ascontiguousarray(W_kn.T))
+    assert np.array_equal(u.host(S).view(np.uint16), np.ascontiguousarray(S_kn.T).view(np.uint16))
+    if N * K <= 4096 * 4096:
+        x = rng.standard_normal((3, K)).astype(np.float16)
+        got = u.host(ops.q4g32_linear(W, S, u.dev(x)))
+        u.assert_close(got, oracle.q4g32_kn_linear(W_kn, S_kn, x), f"kn linear {N}x{K}")
