@@ -5,7 +5,7 @@ installed PyTorch wheel (torch/quantization/_quantized_conversions.py), an indep
 restatement of the same published layout.  It only accepts device tensors, so this
 script has to run on a machine with a GPU:
 
-    python tests/golden/make_ft_layout_vectors.py gpurun_out/ft_layout_vectors.npz
+    python tests/golden/make_ft_layout_vectors.py /tmp/ft_layout_vectors.npz
 
 and the resulting file is committed as tests/golden/ft_layout_vectors.npz.
 Inputs are seeded random bytes; for each case the file stores the input
@@ -46,4 +46,4 @@ def main(path):
 
 
 if __name__ == "__main__":
-    main(sys.argv[1] if len(sys.argv) > 1 else "gpurun_out/ft_layout_vectors.npz")
+    main(sys.argv[1] if len(sys.argv) > 1 else "/tmp/ft_layout_vectors.npz")
