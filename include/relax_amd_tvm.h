@@ -51,6 +51,15 @@ WQ_PACKED(relax_amd_q4f16_1_matmul_bias);
 WQ_PACKED(relax_amd_q4f16_1_matmul_bias_residual);
 /* "relax_amd.q4f16_1_decode"(W, S, out f16[N,K]): the decode block alone. */
 WQ_PACKED(relax_amd_q4f16_1_decode);
+/* Weight preparation, destination-passing:
+ *   relax_amd.q4f16_1_encode    (A fp16 [N,K], W_out uint32 [N,K/8], S_out fp16 [N,K/32])
+ *   relax_amd.q4f16_1_kn_to_nk  (W_kn uint32 [K/8,N], S_kn fp16 [K/32,N], W_out [N,K/8], S_out [N,K/32])
+ *   relax_amd.fpA_intB_encode   (A fp16 [N,K], w_out int8 [K,N] | [K,N/2], scales_out fp16 [N] | [K/64,N],
+ *                                scratch fp32 [N]) — the fixtures' encode
+ *                                (tests/python/relax/test_codegen_cutlass.py:1392-1457, 1631-1676, 2044-2109) */
+WQ_PACKED(relax_amd_q4f16_1_encode);
+WQ_PACKED(relax_amd_q4f16_1_kn_to_nk);
+WQ_PACKED(relax_amd_fpA_intB_encode);
 
 /* Format B composites, one per pattern name of
  * python/tvm/relax/backend/contrib/cutlass.py:305-312, 344-372.  Arguments are the

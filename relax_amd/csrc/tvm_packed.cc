@@ -401,6 +401,98 @@ WQ_PACKED(relax_amd_q4f16_1_decode) {
   return rc == WQ_OK ? 0 : packed_fail();
 }
 
+// (A fp16 [N, K]) -> (W uint32 [N, K/8], S fp16 [N, K/32]): the q4f16_1 quantizer.
+WQ_PACKED(relax_amd_q4f16_1_encode) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.q4f16_1_encode";
+  Tensor A, W, S;
+  if (num_args != 3) {
+    fail(WQ_EINVAL, "%s: expected (A, W_out, S_out)", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLFloat, 16, "A", &A) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLUInt, 32, "W_out", &W) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLFloat, 16, "S_out", &S))
+    return packed_fail();
+  if (A.t->ndim != 2 || W.t->ndim != 2 || S.t->ndim != 2 || W.t->shape[0] != A.t->shape[0] ||
+      S.t->shape[0] != A.t->shape[0] || W.t->shape[1] * 8 != A.t->shape[1] || S.t->shape[1] * 32 != A.t->shape[1]) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (A [N,K], W [N,K/8], S [N,K/32])", who);
+    return packed_fail();
+  }
+  const int rc = wq_q4g32_encode((const uint16_t*)A.ptr, (uint32_t*)W.ptr, (uint16_t*)S.ptr, A.t->shape[0],
+                                 A.t->shape[1], current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
+// (W uint32 [K/8, N], S fp16 [K/32, N]) -> (W uint32 [N, K/8], S fp16 [N, K/32]): K-major checkpoints.
+WQ_PACKED(relax_amd_q4f16_1_kn_to_nk) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.q4f16_1_kn_to_nk";
+  Tensor Wi, Si, Wo, So;
+  if (num_args != 4) {
+    fail(WQ_EINVAL, "%s: expected (W_kn, S_kn, W_out, S_out)", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W_kn", &Wi) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "S_kn", &Si) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLUInt, 32, "W_out", &Wo) ||
+      !get_tensor(who, args, type_codes, num_args, 3, kDLFloat, 16, "S_out", &So))
+    return packed_fail();
+  if (Wi.t->ndim != 2 || Si.t->ndim != 2 || Wo.t->ndim != 2 || So.t->ndim != 2 ||
+      Si.t->shape[1] != Wi.t->shape[1] || Si.t->shape[0] * 4 != Wi.t->shape[0] ||
+      Wo.t->shape[0] != Wi.t->shape[1] || Wo.t->shape[1] != Wi.t->shape[0] ||
+      So.t->shape[0] != Si.t->shape[1] || So.t->shape[1] != Si.t->shape[0]) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (W_kn [K/8,N], S_kn [K/32,N], W_out [N,K/8], S_out [N,K/32])", who);
+    return packed_fail();
+  }
+  const int rc = wq_q4g32_kn_to_nk((const uint32_t*)Wi.ptr, (const uint16_t*)Si.ptr, (uint32_t*)Wo.ptr,
+                                   (uint16_t*)So.ptr, Wi.t->shape[1], Wi.t->shape[0] * 8, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
+// (A fp16 [N, K]) -> (w int8 [K, N] | [K, N/2], scales fp16 [N] | [K/64, N], scratch fp32 [N]): the
+// reference fixtures' `encode`; int4 and the group size follow from the output shapes.
+WQ_PACKED(relax_amd_fpA_intB_encode) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.fpA_intB_encode";
+  Tensor A, Wq, Sc, Tmp;
+  if (num_args != 4) {
+    fail(WQ_EINVAL, "%s: expected (A, w_out, scales_out, scratch_f32[N])", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLFloat, 16, "A", &A) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLInt, 8, "w_out", &Wq) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLFloat, 16, "scales_out", &Sc) ||
+      !get_tensor(who, args, type_codes, num_args, 3, kDLFloat, 32, "scratch", &Tmp))
+    return packed_fail();
+  if (A.t->ndim != 2 || Wq.t->ndim != 2 || Wq.t->shape[0] != A.t->shape[1]) {
+    fail(WQ_EINVAL, "%s: A must be [N,K] and w_out [K,N] or [K,N/2]", who);
+    return packed_fail();
+  }
+  const int64_t N = A.t->shape[0], K = A.t->shape[1];
+  int nbit;
+  if (Wq.t->shape[1] == N) nbit = 8;
+  else if (Wq.t->shape[1] * 2 == N) nbit = 4;
+  else {
+    fail(WQ_EINVAL, "%s: w_out has %lld columns for N = %lld", who, (long long)Wq.t->shape[1], (long long)N);
+    return packed_fail();
+  }
+  int64_t group;
+  if (Sc.numel == N) group = -1;
+  else if (Sc.numel == (K / 64) * N) group = 64;
+  else {
+    fail(WQ_EINVAL, "%s: scales_out must have N or (K/64)*N elements", who);
+    return packed_fail();
+  }
+  if (Tmp.numel < N) {
+    fail(WQ_EINVAL, "%s: scratch must hold N floats", who);
+    return packed_fail();
+  }
+  const int rc = wq_intb_encode((const uint16_t*)A.ptr, (int8_t*)Wq.ptr, (uint16_t*)Sc.ptr, (float*)Tmp.ptr, N, K,
+                                group, nbit, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
 #define WQ_DECODE_MATMUL(sym, op)                                       \
   WQ_PACKED(sym) {                                                      \
     (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;    \
@@ -458,6 +550,9 @@ const std::vector<Entry>& table() {
     v.push_back({"relax_amd.q4f16_1_matmul_bias_residual", "relax_amd_q4f16_1_matmul_bias_residual",
                  relax_amd_q4f16_1_matmul_bias_residual});
     v.push_back({"relax_amd.q4f16_1_decode", "relax_amd_q4f16_1_decode", relax_amd_q4f16_1_decode});
+    v.push_back({"relax_amd.q4f16_1_encode", "relax_amd_q4f16_1_encode", relax_amd_q4f16_1_encode});
+    v.push_back({"relax_amd.q4f16_1_kn_to_nk", "relax_amd_q4f16_1_kn_to_nk", relax_amd_q4f16_1_kn_to_nk});
+    v.push_back({"relax_amd.fpA_intB_encode", "relax_amd_fpA_intB_encode", relax_amd_fpA_intB_encode});
 #define WQ_ENTRY(sym, op) v.push_back({std::string("relax_amd.") + op, #sym, sym});
     WQ_DECODE_MATMUL_LIST(WQ_ENTRY)
 #undef WQ_ENTRY

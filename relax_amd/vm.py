@@ -56,9 +56,13 @@ class DpsProgram:
         self._shapes[r] = (tuple(t.shape), t.dtype)
         return Reg(r)
 
-    def planned(self, shape: Sequence[int], dtype: torch.dtype = torch.float16) -> Reg:
-        """An intermediate whose storage the memory plan assigns."""
+    def planned(self, shape: Sequence[int], dtype: torch.dtype = torch.float16, as_uint32: bool = False) -> Reg:
+        """An intermediate whose storage the memory plan assigns (``as_uint32``: declare int32 as uint32)."""
         code, bits = _DTYPES[dtype]
+        if as_uint32:
+            if dtype != torch.int32:
+                raise ValueError("as_uint32 needs dtype int32")
+            code = 1
         shp = (ctypes.c_int64 * max(1, len(shape)))(*shape)
         r = self._l.wq_program_add_planned(self._p, code, bits, len(shape), shp)
         check(min(r, 0), "wq_program_add_planned")

@@ -171,3 +171,54 @@ def test_program_reports_callee_errors():
     p.plan()
     with pytest.raises(WqError, match="instruction 0"):
         p.run()
+
+
+@pytest.mark.gpu
+def test_weight_preparation_program(oracle):
+    """fp16 weights -> quantize -> (reorder) -> linear, every step a PackedFunc of the instruction list:
+    q4f16_1 (encode, and a K-major checkpoint through kn_to_nk) and fpA_intB int8 (encode, ft_preprocess DPS,
+    decode_matmul_bias)."""
+    import torch
+
+    from relax_amd import vm
+    from tests import gpu_util as u
+
+    rng = np.random.default_rng(21)
+    M, N, K = 5, 128, 256
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    p = vm.DpsProgram()
+    A = p.external(u.dev(w))
+    X = p.external(u.dev(x))
+    # format A
+    Wq = p.external(torch.zeros((N, K // 8), dtype=torch.int32, device="cuda"), as_uint32=True)
+    Sq = p.external(torch.zeros((N, K // 32), dtype=torch.float16, device="cuda"))
+    ya = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    p.call("relax_amd.q4f16_1_encode", A, Wq, Sq)
+    p.call("relax_amd.q4f16_1_matmul", Wq, Sq, X, p.external(ya))
+    # the same weights arriving K-major
+    W_ref, S_ref = oracle.q4g32_encode(w)
+    Wkn = p.external(u.dev(np.ascontiguousarray(W_ref.T)), as_uint32=True)
+    Skn = p.external(u.dev(np.ascontiguousarray(S_ref.T)))
+    Wt = p.planned((N, K // 8), torch.int32, as_uint32=True)
+    St = p.planned((N, K // 32))
+    yk = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    p.call("relax_amd.q4f16_1_kn_to_nk", Wkn, Skn, Wt, St)
+    p.call("relax_amd.q4f16_1_matmul", Wt, St, X, p.external(yk))
+    # format B int8
+    q8 = p.planned((K, N), torch.int8)
+    sc = p.external(torch.zeros((N,), dtype=torch.float16, device="cuda"))
+    tmp = p.planned((N,), torch.float32)
+    pre = p.planned((K, N), torch.int8)
+    yb = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    p.call("relax_amd.fpA_intB_encode", A, q8, sc, tmp)
+    p.call("relax_amd.ft_preprocess_weight_dps", q8, 80, 0, pre)
+    p.call("relax_amd.decode_matmul_bias", X, pre, sc, p.external(u.dev(bias)), p.external(yb))
+    p.plan()
+    p.run()
+    torch.cuda.synchronize()
+    u.assert_close(u.host(ya), oracle.q4g32_linear(W_ref, S_ref, x), "encoded q4f16_1")
+    assert torch.equal(ya, yk)
+    q_ref, s_ref = oracle.intb_encode(w, 8)
+    u.assert_close(u.host(yb), oracle.intb_linear(x, q_ref, s_ref, 8, bias=bias), "encoded int8")
