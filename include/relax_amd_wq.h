@@ -174,6 +174,46 @@ int wq_q4g32_kn_to_nk(const uint32_t* W_kn, const uint16_t* S_kn, uint32_t* W_nk
                       int64_t N, int64_t K, wq_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * AutoGPTQ checkpoints (tests/python/dlight/test_gpu_gemv.py:636-665):
+ *   qweight uint32 [K/8, N]   code of (k, n) in bits 4*(k%8).. of qweight[k/8][n]
+ *   qzeros  uint32 [G, N/8]   zero of (g, n) in bits 4*(n%8).. of qzeros[g][n/8]
+ *   scales  fp16   [G, N],  g_idx int32 [K] with values in [0, G)
+ *   w[k,n] = (fp16(code) - (fp16(zero) + 1)) * scales[g_idx[k], n]          all in fp16
+ *   y[m,n] = residual[m,n] + fp16(sum_k x[m,k] * w[k,n])
+ * The reference accumulates this sum in fp16 (:653-660) and leaves the function to the
+ * unscheduled fallback (:667-672); this library accumulates in fp32 like its other linears.
+ * ------------------------------------------------------------------------- */
+/* The fp16 weight, bit for bit, straight from the checkpoint layout: out fp16 [K, N].
+ * g_idx entries outside [0, G) are clamped. */
+int wq_gptq_dequantize(const uint32_t* qweight, const uint32_t* qzeros, const uint16_t* scales,
+                       const int32_t* g_idx, uint16_t* out, int64_t K, int64_t N, int64_t G,
+                       wq_stream_t stream);
+/* Load-time conversion to what wq_gptq_linear reads.  Rows are sorted by group (stable), so
+ * every group becomes K/G consecutive rows:
+ *   perm  int32  [K]         perm[k'] = original row at sorted position k'
+ *   W_nk  uint32 [N, K/8]    codes of the sorted rows, 8 per word along K
+ *   SZ    fp16   [N, G, 2]   (scale, zero + 1) per column and group
+ * status_scratch: 4 bytes of device memory used during the call.  *needs_perm (host, may be
+ * NULL) is set to 1 if the sorted order differs from 0..K-1; otherwise wq_gptq_linear may be
+ * given perm = NULL.  Requires K % G == 0, (K/G) % 32 == 0, N % 8 == 0 and a g_idx that
+ * gives each group exactly K/G rows (what AutoGPTQ writes, with or without desc_act);
+ * anything else returns WQ_EUNSUPPORTED.  Synchronises the stream (it reads the check back). */
+int wq_gptq_prepare(const uint32_t* qweight, const uint32_t* qzeros, const uint16_t* scales,
+                    const int32_t* g_idx, uint32_t* W_nk, uint16_t* SZ, int32_t* perm,
+                    int32_t* status_scratch, int* needs_perm, int64_t K, int64_t N, int64_t G,
+                    wq_stream_t stream);
+/* Bytes of workspace wq_gptq_linear needs: M*K*2 for the gathered activations when a row
+ * order is given and M > WQ_GEMV_MAX_M, else 0. */
+size_t wq_gptq_workspace_bytes(int64_t M, int64_t K, int has_perm);
+/* y fp16 [M, N] = epilogue(x fp16 [M, K] . w) over the prepared operands; bias fp16 [N] and
+ * residual fp16 [M, N] may be NULL (epilogue as wq_q4g32_linear).  perm may be NULL (rows
+ * already in group order).  M <= WQ_GEMV_MAX_M streams the weights once per 4 rows of x; larger
+ * M runs the MFMA GEMM (group size % 64 == 0; other group sizes repeat the streaming kernel). */
+int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
+                   const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
+                   int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Calibration kernels: the measured ceilings reported next to the vendor peaks
  * (no counterpart in the reference; its methodology precedent is the cache-flush
  * protocol of src/runtime/profiling.cc:879-895).

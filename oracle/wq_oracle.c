@@ -38,6 +38,15 @@
  *                                        the definition used is stated at the function
  *                                        and checked through decode(encode(w)) error
  *                                        bounds, code range and a numpy restatement
+ *   wqo_gptq_dequant                     a hand-computed case, exhaustive 16 codes x 16
+ *                                        zero points x every scale bit pattern against
+ *                                        numpy.float16 arithmetic, reduction to the pinned
+ *                                        K-major q4f16_1 decode when every zero point is 6
+ *                                        and g_idx[k] = k / 32, and equivariance under a
+ *                                        permutation of the K rows together with g_idx
+ *   wqo_kn_matmul                        float64 matmul over the dequantized weights
+ *                                        (fp32 mode), a sequential numpy.float16 loop on
+ *                                        small cases (fp16 mode), one-hot selection
  *
  * Build: see oracle/Makefile (gcc -O3 -mavx2 -mfma -mf16c -fopenmp).
  */
@@ -574,5 +583,55 @@ void wqo_q4g32_encode(const uint16_t* A, uint32_t* W, uint16_t* S, int64_t N, in
         }
         W[n * (K / 8) + g * 4 + j] = word;
       }
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* AutoGPTQ layout: K-major int4 with packed zero points and g_idx     */
+/* ------------------------------------------------------------------ */
+
+/* tests/python/dlight/test_gpu_gemv.py:636-652 (the "decode" block):
+ *   qweight uint32 [K/8, N], qzeros uint32 [G, N/8], scales fp16 [G, N], g_idx uint32 [K]
+ *   g = g_idx[k]
+ *   B[k,n] = (fp16((qweight[k/8,n] >> 4*(k%8)) & 15)
+ *             - (fp16((qzeros[g, n/8] >> 4*(n%8)) & 15) + fp16(1))) * scales[g,n]     all in fp16
+ * out fp16 [K, N].  Returns -1 if a g_idx entry is outside [0, G).             */
+int wqo_gptq_dequant(const uint32_t* qweight, const uint32_t* qzeros, const uint16_t* scales,
+                     const int32_t* g_idx, uint16_t* out, int64_t K, int64_t N, int64_t G) {
+  const uint16_t one = 0x3c00u;
+  for (int64_t k = 0; k < K; ++k) {
+    const int64_t g = g_idx[k];
+    if (g < 0 || g >= G) return -1;
+    for (int64_t n = 0; n < N; ++n) {
+      const uint32_t code = (qweight[(k / 8) * N + n] >> ((uint32_t)(k % 8) * 4u)) & 15u;
+      const uint32_t zero = (qzeros[g * (N / 8) + n / 8] >> ((uint32_t)(n % 8) * 4u)) & 15u;
+      const uint16_t zp = h_add(f2h((float)zero), one);
+      out[k * N + n] = h_mul(h_sub(f2h((float)code), zp), scales[g * N + n]);
+    }
+  }
+  return 0;
+}
+
+/* The matmul and the add that follow the decode, test_gpu_gemv.py:653-665:
+ *   acc = fp16(0);  acc = acc + x[k] * B[k,n]   (k ascending; product and sum rounded to fp16)
+ *   y = residual + acc                           (fp16 add)
+ * f32acc != 0 switches to the accumulate mode the GPU build implements for every format
+ * (fp32 products and sums over the same fp16 weights, one rounding to fp16, then the
+ * fp16 residual add), the fp32-accumulate convention of test_gpu_reduction.py:411-424.
+ * Bdeq fp16 [K, N], X fp16 [M, K], residual fp16 [M, N] or NULL, Y fp16 [M, N].  */
+void wqo_kn_matmul(const uint16_t* Bdeq, const uint16_t* X, const uint16_t* residual, uint16_t* Y,
+                   int64_t M, int64_t N, int64_t K, int f32acc) {
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t n = 0; n < N; ++n) {
+      uint16_t h;
+      if (f32acc) {
+        float acc = 0.0f;
+        for (int64_t k = 0; k < K; ++k) acc = acc + h2f(X[m * K + k]) * h2f(Bdeq[k * N + n]);
+        h = f2h(acc);
+      } else {
+        h = 0;
+        for (int64_t k = 0; k < K; ++k) h = h_add(h, h_mul(X[m * K + k], Bdeq[k * N + n]));
+      }
+      Y[m * N + n] = residual ? h_add(residual[m * N + n], h) : h;
     }
 }

@@ -322,3 +322,61 @@ def make_intb_inputs(M: int, N: int, K: int, nbit: int, seed: int, group_size: i
     shape = (N,) if group_size <= 0 else (K // group_size, N)
     s = rng.uniform(0.001, 0.01, size=shape).astype(np.float16)
     return x, A, s
+
+
+# ------------------------------------------------- AutoGPTQ layout (K-major, zero points, g_idx)
+
+
+def gptq_dequant(qweight: np.ndarray, qzeros: np.ndarray, scales: np.ndarray, g_idx: np.ndarray) -> np.ndarray:
+    """B[k, n] = (fp16(code) - (fp16(zero) + 1)) * scales[g_idx[k], n], fp16 [K, N]
+    (tests/python/dlight/test_gpu_gemv.py:636-652).  qweight uint32 [K/8, N], qzeros uint32 [G, N/8],
+    scales fp16 [G, N], g_idx int32 [K]."""
+    qweight = _c(qweight, np.uint32)
+    qzeros = _c(qzeros, np.uint32)
+    scales = _c(scales, np.float16)
+    g_idx = _c(g_idx, np.int32)
+    k8, N = qweight.shape
+    K, G = k8 * 8, scales.shape[0]
+    assert qzeros.shape == (G, N // 8) and scales.shape == (G, N) and g_idx.shape == (K,)
+    out = np.empty((K, N), np.float16)
+    rc = lib().wqo_gptq_dequant(_p(qweight), _p(qzeros), _p(scales.view(np.uint16)), _p(g_idx),
+                                _p(out.view(np.uint16)), i64(K), i64(N), i64(G))
+    if rc != 0:
+        raise ValueError("g_idx entry outside [0, G)")
+    return out
+
+
+def kn_matmul(Bdeq: np.ndarray, x: np.ndarray, residual=None, f32acc: bool = True) -> np.ndarray:
+    """y[m, n] = residual[m, n] + sum_k x[m, k] * B[k, n] (test_gpu_gemv.py:653-665); ``f32acc=False`` is the
+    reference's fp16 accumulation, ``True`` the fp32 accumulation the GPU build implements."""
+    Bdeq = _c(Bdeq, np.float16)
+    x = _c(x, np.float16)
+    K, N = Bdeq.shape
+    x2 = x.reshape(-1, K)
+    M = x2.shape[0]
+    res = None if residual is None else _c(residual, np.float16).reshape(M, N)
+    y = np.empty((M, N), np.float16)
+    lib().wqo_kn_matmul(_p(Bdeq.view(np.uint16)), _p(x2.view(np.uint16)),
+                        _opt(None if res is None else res.view(np.uint16)), _p(y.view(np.uint16)),
+                        i64(M), i64(N), i64(K), cint(1 if f32acc else 0))
+    return y
+
+
+def gptq_linear(qweight, qzeros, scales, g_idx, x, residual=None, f32acc: bool = True) -> np.ndarray:
+    return kn_matmul(gptq_dequant(qweight, qzeros, scales, g_idx), x, residual, f32acc)
+
+
+def make_gptq_inputs(M: int, N: int, K: int, group_size: int, seed: int, act_order: bool = False):
+    """x ~ N(0,1) fp16; codes and zero points uniform 0..15; scales ~ U(0.005, 0.02) fp16;
+    g_idx[k] = k // group_size, or (``act_order``) a random permutation of that assignment, which is
+    what AutoGPTQ's desc_act option produces: every group keeps exactly ``group_size`` members."""
+    rng = np.random.default_rng(seed)
+    G = K // group_size
+    x = rng.standard_normal((M, K), dtype=np.float32).astype(np.float16)
+    qweight = rng.integers(0, 2**32, size=(K // 8, N), dtype=np.uint64).astype(np.uint32)
+    qzeros = rng.integers(0, 2**32, size=(G, N // 8), dtype=np.uint64).astype(np.uint32)
+    scales = rng.uniform(0.005, 0.02, size=(G, N)).astype(np.float16)
+    g_idx = (np.arange(K) // group_size).astype(np.int32)
+    if act_order:
+        g_idx = g_idx[rng.permutation(K)]
+    return x, qweight, qzeros, scales, np.ascontiguousarray(g_idx)

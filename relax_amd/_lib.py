@@ -30,6 +30,10 @@ SIGNATURES = {
     "wq_fpA_intB_gemm": [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
     "wq_fpA_intB_gemm_residual": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
     "wq_q4g32_kn_to_nk": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
+    "wq_gptq_dequantize": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "wq_gptq_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_int), _i64, _i64, _i64, _vp],
+    "wq_gptq_workspace_bytes": [_i64, _i64, _int],
+    "wq_gptq_linear": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp],
     "wq_intb_encode": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "wq_q4g32_encode": [_vp, _vp, _vp, _i64, _i64, _vp],
     "wq_calibrate_mfma_f16": [_vp, _i64, _int, ctypes.POINTER(ctypes.c_double), _vp],
@@ -52,7 +56,8 @@ SIGNATURES = {
     "wq_unary_op_from_string": [ctypes.c_char_p],
 }
 _RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p, "wq_program_create": _vp,
-             "wq_program_destroy": None, "wq_program_plan": _i64, "wq_program_unplanned_bytes": _i64}
+             "wq_program_destroy": None, "wq_program_plan": _i64, "wq_program_unplanned_bytes": _i64,
+             "wq_gptq_workspace_bytes": _sz}
 
 _lib = None
 

@@ -1,0 +1,266 @@
+// AutoGPTQ checkpoints: K-major int4 codes with packed zero points and a group index
+// (tests/python/dlight/test_gpu_gemv.py:636-665):
+//   qweight uint32 [K/8, N], qzeros uint32 [G, N/8], scales fp16 [G, N], g_idx int32 [K]
+//   w[k,n] = (fp16(code) - (fp16(zero) + 1)) * scales[g_idx[k], n],   y = residual + x . w
+//
+// The reference's GEMV rule leaves this function unscheduled because the scale depends on k
+// through g_idx.  Here the dependence is removed once, when the checkpoint is loaded:
+//   * the K rows are sorted by group (stable), so that every group is a run of K/G
+//     consecutive rows; `perm` records the order and the activations are gathered through it
+//     (inside the GEMV's activation pass, by a small kernel before the GEMM);
+//   * the words are transposed to the [N, K/8] layout of the other kernels of this library
+//     (a word holds 8 consecutive k of one column in both layouts);
+//   * scale and zero point + 1 are interleaved as fp16 pairs SZ [N, G, 2], the 4 bytes that
+//     one lane needs for one group.
+// After that the weight stream is the one of format A with one more multiply-add per group,
+// and both the streaming GEMV (q4_gemv.h) and the MFMA GEMM (mfma_gemm_lds.h) take it.
+// A g_idx whose groups do not all have K/G members is rejected by the preparation.
+#include "mfma_gemm_lds.h"
+#include "q4_gemv.h"
+#include "q4g32_common.h"
+
+namespace wq {
+
+// ---- the reference's decode, bit for bit, from the checkpoint layout --------------------
+// Thread (kw, n) unpacks the 8 codes of one word: reads coalesced along n, writes 8 rows.
+__global__ __launch_bounds__(256) void gptq_dequant_kernel(const uint32_t* __restrict__ qweight,
+                                                           const uint32_t* __restrict__ qzeros,
+                                                           const half_t* __restrict__ scales,
+                                                           const int* __restrict__ g_idx, half_t* __restrict__ out,
+                                                           int K, int N, int G) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  const int kw = blockIdx.y;
+  if (n >= N) return;
+  const uint32_t word = qweight[(int64_t)kw * N + n];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int k = kw * 8 + i;
+    const int g = min(max(g_idx[k], 0), G - 1);  // entries outside [0, G) are clamped, never followed
+    const uint32_t zero = (qzeros[(int64_t)g * (N >> 3) + (n >> 3)] >> (4 * (n & 7))) & 15u;
+    const half_t zp = (half_t)(float)zero + (half_t)1.0f;
+    const half_t code = (half_t)(float)((word >> (4 * i)) & 15u);
+    out[(int64_t)k * N + n] = (code - zp) * scales[(int64_t)g * N + n];
+  }
+}
+
+// ---- preparation ---------------------------------------------------------------------------
+// One thread per group scans g_idx in ascending k and lists the group's rows.  status bit 0:
+// some group does not have exactly `gs` members (this also catches entries outside [0, G));
+// bit 1: the order differs from 0, 1, 2, ...
+__global__ __launch_bounds__(64) void gptq_perm_kernel(const int* __restrict__ g_idx, int* __restrict__ perm,
+                                                       int* __restrict__ status, int K, int G, int gs) {
+  const int g = blockIdx.x * 64 + threadIdx.x;
+  if (g >= G) return;
+  int count = 0, flags = 0;
+  for (int k = 0; k < K; ++k) {
+    if (g_idx[k] == g) {
+      if (count < gs) {
+        perm[g * gs + count] = k;
+        if (k != g * gs + count) flags |= 2;
+      }
+      ++count;
+    }
+  }
+  if (count != gs) flags |= 1;
+  if (flags) atomicOr(status, flags);
+}
+
+// W_nk[n][kw'] = the 8 codes of column n at rows perm[8kw' .. 8kw'+7]; 64x64 word tiles through
+// LDS: reads coalesced along n, writes coalesced along kw'.
+__global__ __launch_bounds__(256) void gptq_repack_kernel(const uint32_t* __restrict__ qweight,
+                                                          const int* __restrict__ perm, uint32_t* __restrict__ W_nk,
+                                                          int KW, int N) {
+  __shared__ uint32_t tile[64][65];
+  const int kw0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = 0; i < 16; ++i) {
+    const int kw = kw0 + ty * 16 + i, n = n0 + tx;
+    if (kw < KW && n < N) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int k = perm[kw * 8 + c];
+        word |= ((qweight[(int64_t)(k >> 3) * N + n] >> (4 * (k & 7))) & 15u) << (4 * c);
+      }
+      tile[ty * 16 + i][tx] = word;
+    }
+  }
+  __syncthreads();
+  for (int i = 0; i < 16; ++i) {
+    const int n = n0 + ty * 16 + i, kw = kw0 + tx;
+    if (kw < KW && n < N) W_nk[(int64_t)n * KW + kw] = tile[tx][ty * 16 + i];
+  }
+}
+
+// SZ[n][g] = (scales[g][n], fp16(zero[g][n] + 1))
+__global__ __launch_bounds__(256) void gptq_sz_kernel(const uint32_t* __restrict__ qzeros,
+                                                      const half_t* __restrict__ scales, half2_t* __restrict__ SZ,
+                                                      int N, int G) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  const int g = blockIdx.y;
+  if (n >= N) return;
+  const uint32_t zero = (qzeros[(int64_t)g * (N >> 3) + (n >> 3)] >> (4 * (n & 7))) & 15u;
+  SZ[(int64_t)n * G + g] = half2_t{scales[(int64_t)g * N + n], (half_t)(float)(zero + 1u)};
+}
+
+// xp[m][k'] = x[m][perm[k']]
+__global__ __launch_bounds__(256) void gptq_gather_x_kernel(const half_t* __restrict__ x, const int* __restrict__ perm,
+                                                            half_t* __restrict__ xp, int K) {
+  const int k = blockIdx.x * 256 + threadIdx.x;
+  const int64_t m = blockIdx.y;
+  if (k < K) xp[m * K + k] = x[m * K + perm[k]];
+}
+
+// ---- MFMA GEMM policy: the stream of format A with a (scale, zero point) pair per group ------
+// A K-step (64 rows) lies inside one group (group size % 64 == 0), so both lane halves read the
+// same 4 staged bytes.  1024 + code - (1024 + zp) is exact, the multiply rounds once: the
+// reference's fp16 weight, bit for bit.
+struct GptqLdsPolicy {
+  static constexpr int kColBytes = 32;
+  static constexpr int kScaleBytes = 4;
+  static constexpr int kStepStride = 32;
+  struct Args {
+    const uint32_t* W;
+    const half2_t* SZ;
+    int groups;          // per row
+    int steps_per_group; // group size / 64
+    uint32_t inv;        // ceil(2^32 / steps_per_group), unused when steps_per_group == 1
+  };
+  struct Frag {
+    uint4_t w;
+  };
+  struct Scale {
+    half2_t s2;   // scale, twice
+    half2_t off;  // 1024 + zero point, twice
+  };
+  __device__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
+    const int n = q >> 1, h = q & 1;
+    return reinterpret_cast<const char*>(a.W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
+  }
+  __device__ static const char* s_src(const Args& a, int n, int) {
+    return reinterpret_cast<const char*>(a.SZ + (int64_t)n * a.groups);
+  }
+  // ks / steps_per_group by multiplication: exact for ks * steps_per_group < 2^32
+  __device__ static int64_t s_offset(const Args& a, int ks) {
+    const uint32_t g = a.steps_per_group == 1 ? (uint32_t)ks : __umulhi((uint32_t)ks, a.inv);
+    return (int64_t)g * 4;
+  }
+  __device__ static Scale read_scale(const unsigned char* p, int) {
+    const half2_t sz = *reinterpret_cast<const half2_t*>(p);
+    const half_t o = sz.y + (half_t)1024.0f;
+    return Scale{half2_t{sz.x, sz.x}, half2_t{o, o}};
+  }
+  __device__ static Scale const_scale(const Args&, int) { return Scale{}; }
+  __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
+    f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
+  }
+  __device__ static half2_t pair(const Frag& f, int kk, int j, const Scale& sc) {
+    const uint32_t word = kk == 0 ? f.w.x : kk == 1 ? f.w.y : kk == 2 ? f.w.z : f.w.w;
+    const uint32_t t = (word >> (8 * j)) & 0xFFu;  // codes 2j, 2j+1
+    const uint32_t u = (t << 12) | t;
+    return (as_half2(and_or(u, 0x000F000Fu, 0x64006400u)) - sc.off) * sc.s2;
+  }
+};
+
+}  // namespace wq
+
+extern "C" int wq_gptq_dequantize(const uint32_t* qweight, const uint32_t* qzeros, const uint16_t* scales,
+                                  const int32_t* g_idx, uint16_t* out, int64_t K, int64_t N, int64_t G,
+                                  wq_stream_t stream) {
+  using namespace wq;
+  WQ_REQUIRE(K >= 0 && N >= 0 && G >= 0, "wq_gptq_dequantize: negative dimension");
+  WQ_REQUIRE(K % 8 == 0 && N % 8 == 0, "wq_gptq_dequantize: K=%lld and N=%lld must be multiples of 8",
+             (long long)K, (long long)N);
+  if (K == 0 || N == 0) return WQ_OK;
+  WQ_REQUIRE(G > 0, "wq_gptq_dequantize: no groups");
+  WQ_REQUIRE(qweight && qzeros && scales && g_idx && out, "wq_gptq_dequantize: null pointer");
+  WQ_REQUIRE(N < (1ll << 30) && K / 8 < 65536, "wq_gptq_dequantize: too large");
+  WQ_LAUNCH("wq_gptq_dequantize", gptq_dequant_kernel, dim3((unsigned)((N + 255) / 256), (unsigned)(K / 8)),
+            dim3(256), 0, (hipStream_t)stream, qweight, qzeros, (const half_t*)scales, g_idx, (half_t*)out, (int)K,
+            (int)N, (int)G);
+  return WQ_OK;
+}
+
+extern "C" int wq_gptq_prepare(const uint32_t* qweight, const uint32_t* qzeros, const uint16_t* scales,
+                               const int32_t* g_idx, uint32_t* W_nk, uint16_t* SZ, int32_t* perm,
+                               int32_t* status_scratch, int* needs_perm, int64_t K, int64_t N, int64_t G,
+                               wq_stream_t stream_) {
+  using namespace wq;
+  hipStream_t stream = (hipStream_t)stream_;
+  WQ_REQUIRE(K >= 0 && N >= 0 && G >= 0, "wq_gptq_prepare: negative dimension");
+  if (needs_perm) *needs_perm = 0;
+  if (K == 0 || N == 0) return WQ_OK;
+  WQ_REQUIRE(G > 0 && K % G == 0, "wq_gptq_prepare: K=%lld is not a multiple of the %lld groups", (long long)K,
+             (long long)G);
+  const int64_t gs = K / G;
+  WQ_REQUIRE(gs % 32 == 0, "wq_gptq_prepare: group size %lld must be a multiple of 32", (long long)gs);
+  WQ_REQUIRE(N % 8 == 0, "wq_gptq_prepare: N=%lld must be a multiple of 8", (long long)N);
+  WQ_REQUIRE(qweight && qzeros && scales && g_idx && W_nk && SZ && perm && status_scratch,
+             "wq_gptq_prepare: null pointer");
+  WQ_REQUIRE(N < (1ll << 30) && K < (1ll << 24) && G < 65536, "wq_gptq_prepare: too large");
+  // the status word is cleared by a copy of a zero (a fill kernel would do as well); the
+  // call synchronises anyway, it is a load-time step
+  const int32_t zero = 0;
+  WQ_HIP(hipMemcpyAsync(status_scratch, &zero, 4, hipMemcpyHostToDevice, stream));
+  WQ_LAUNCH("wq_gptq_prepare", gptq_perm_kernel, dim3((unsigned)((G + 63) / 64)), dim3(64), 0, stream, g_idx,
+            perm, status_scratch, (int)K, (int)G, (int)gs);
+  int32_t status = 0;
+  WQ_HIP(hipMemcpyAsync(&status, status_scratch, 4, hipMemcpyDeviceToHost, stream));
+  WQ_HIP(hipStreamSynchronize(stream));
+  if (status & 1)
+    return fail(WQ_EUNSUPPORTED,
+                "wq_gptq_prepare: g_idx must assign exactly K/G = %lld rows to each of the %lld groups",
+                (long long)gs, (long long)G);
+  if (needs_perm) *needs_perm = (status & 2) ? 1 : 0;
+  const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K / 8 + 63) / 64));
+  WQ_LAUNCH("wq_gptq_prepare", gptq_repack_kernel, grid, dim3(256), 0, stream, qweight, perm, W_nk, (int)(K / 8),
+            (int)N);
+  WQ_LAUNCH("wq_gptq_prepare", gptq_sz_kernel, dim3((unsigned)((N + 255) / 256), (unsigned)G), dim3(256), 0, stream,
+            qzeros, (const half_t*)scales, (half2_t*)SZ, (int)N, (int)G);
+  return WQ_OK;
+}
+
+extern "C" size_t wq_gptq_workspace_bytes(int64_t M, int64_t K, int has_perm) {
+  return (has_perm && M > WQ_GEMV_MAX_M && M > 0 && K > 0) ? (size_t)M * (size_t)K * 2 : 0;
+}
+
+extern "C" int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
+                              const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
+                              int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream_) {
+  using namespace wq;
+  hipStream_t stream = (hipStream_t)stream_;
+  WQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G >= 0, "wq_gptq_linear: negative dimension");
+  if (M == 0 || N == 0) return WQ_OK;
+  WQ_REQUIRE(K > 0 && G > 0 && K % G == 0, "wq_gptq_linear: K=%lld is not a positive multiple of the %lld groups",
+             (long long)K, (long long)G);
+  const int64_t gs = K / G;
+  WQ_REQUIRE(gs % 32 == 0, "wq_gptq_linear: group size %lld must be a multiple of 32", (long long)gs);
+  WQ_REQUIRE(W_nk && SZ && x && y, "wq_gptq_linear: null pointer");
+  WQ_REQUIRE(aligned16(W_nk) && aligned16(x) && aligned16(perm) && (reinterpret_cast<uintptr_t>(SZ) & 3u) == 0,
+             "wq_gptq_linear: W_nk, x and perm must be 16-byte aligned, SZ 4-byte aligned");
+  WQ_REQUIRE(N < (1ll << 30) && K <= 32768 && M < (1ll << 30),
+             "wq_gptq_linear: N=%lld K=%lld outside the supported range (K <= 32768)", (long long)N, (long long)K);
+  const GemvZp zp{perm, (int)(gs / 32), (int)G};
+  if (M <= WQ_GEMV_MAX_M || gs % 64 != 0)
+    return gemv_dispatch<true>("wq_gptq_linear", W_nk, SZ, zp, x, bias, residual, y, M, N, K, stream);
+  const uint16_t* xg = x;
+  if (perm) {
+    const size_t need = (size_t)M * (size_t)K * 2;
+    WQ_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
+               "wq_gptq_linear: M=%lld with a row order needs a 16-byte aligned workspace of %zu bytes (got %zu)",
+               (long long)M, need, workspace_bytes);
+    WQ_REQUIRE(M < 65536, "wq_gptq_linear: M=%lld too large for the gather", (long long)M);
+    WQ_LAUNCH("wq_gptq_linear", gptq_gather_x_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)M), dim3(256), 0,
+              stream, (const half_t*)x, perm, (half_t*)workspace, (int)K);
+    xg = (const uint16_t*)workspace;
+  }
+  const int spg = (int)(gs / 64);
+  const GptqLdsPolicy::Args largs{W_nk, (const half2_t*)SZ, (int)G, spg,
+                                  spg > 1 ? (uint32_t)(((1ull << 32) + spg - 1) / spg) : 0u};
+  const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
+  if (M <= 384)
+    return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 4, 1, 1, 4, 2>("wq_gptq_linear", largs, xg, y, ep, M, N, K,
+                                                                        stream);
+  return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 8, 2, 1, 4, 1>("wq_gptq_linear", largs, xg, y, ep, M, N, K,
+                                                                      stream);
+}

@@ -99,8 +99,14 @@ struct IntbLdsPolicy {
     const int group = min(n0 / I + (q >> 3), N / I - 1);  // columns past N re-read the last group
     return reinterpret_cast<const char*>(a.B) + ((int64_t)group * (K >> 6)) * 128 + (q & 7) * 16;
   }
+  using Scale = half2_t;  // the column's scale, twice
   __device__ static const char* s_src(const Args&, int, int) { return nullptr; }
-  __device__ static half_t const_scale(const Args& a, int n) { return a.scales[n]; }
+  __device__ static int64_t s_offset(const Args&, int) { return 0; }
+  __device__ static Scale read_scale(const unsigned char*, int) { return Scale{}; }
+  __device__ static Scale const_scale(const Args& a, int n) {
+    const half_t s = a.scales[n];
+    return Scale{s, s};
+  }
   __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
     if (NBIT == 8) {
       const unsigned char* p = bslot + ((n_local >> 1) * 8 + (n_local & 1) * 4 + 2 * lh) * 16;

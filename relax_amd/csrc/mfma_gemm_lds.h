@@ -26,13 +26,17 @@
 // A weight policy provides
 //   kColBytes            packed bytes per column and K-step (32 or 64)
 //   kScaleBytes          bytes of scales per column and K-step staged in LDS (4 or 0)
-//   Args, Frag           kernel arguments; a lane's packed codes + scale of one column for one step
+//   Args, Frag, Scale    kernel arguments; a lane's packed codes of one column for one step; what
+//                        pair() needs besides the codes (the scale in both halves of a register,
+//                        plus the zero point where the format has one)
 //   b_src(args, n0, q, N, K)   global address (step 0) of 16-byte chunk q of the B tile at column n0
 //   kStepStride          bytes between consecutive K-steps of a chunk
 //   s_src(args, n, K)    global address (step 0) of the 4 scale bytes of column n       (kScaleBytes > 0)
-//   const_scale(args, n) the scale of column n                                          (kScaleBytes == 0)
-//   read(frag, bslot, sslot, n_local, lh)   LDS -> registers
-//   pair(frag, kk, j, s2)      dequantized weights (k = 8kk + 2j, 8kk + 2j + 1) of the lane's column
+//   s_offset(args, ks)   byte offset of step ks from there                              (kScaleBytes > 0)
+//   read_scale(p, lh)    Scale from the 4 staged bytes of a column, for lane half lh    (kScaleBytes > 0)
+//   const_scale(args, n) the Scale of column n                                          (kScaleBytes == 0)
+//   read(frag, bslot, n_local, lh)   LDS -> registers
+//   pair(frag, kk, j, scale)   dequantized weights (k = 8kk + 2j, 8kk + 2j + 1) of the lane's column
 #ifndef RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 #define RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 
@@ -146,7 +150,7 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
       __builtin_amdgcn_global_load_lds((wq_gptr_t)(b_src[i] + (int64_t)ks * Policy::kStepStride),
                                        (wq_lptr_t)(slot + Cfg::kBOff + (wave * Cfg::kBLoads + i) * 1024), 16, 0, 0);
     } else {
-      __builtin_amdgcn_global_load_lds((wq_gptr_t)(s_src + (int64_t)ks * 4),
+      __builtin_amdgcn_global_load_lds((wq_gptr_t)(s_src + Policy::s_offset(wargs, ks)),
                                        (wq_lptr_t)(slot + Cfg::kSOff + (wave * 64 % Cfg::BN) * 4), 4, 0, 0);
     }
   };
@@ -160,7 +164,7 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
       for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.0f;
 
   typename Policy::Frag bw[TN];   // this lane's packed weights (and scale) of the step being unpacked
-  half_t bs[TN];
+  typename Policy::Scale bs[TN];
   if (!Cfg::kSLoads) {
 #pragma unroll
     for (int t = 0; t < TN; ++t) bs[t] = Policy::const_scale(wargs, min(n0 + (wn * TN + t) * 32 + lj, N - 1));
@@ -171,7 +175,7 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
     for (int t = 0; t < TN; ++t) {
       const int n = (wn * TN + t) * 32 + lj;
       Policy::read(bw[t], slot + Cfg::kBOff, n, lh);
-      if (Cfg::kSLoads) bs[t] = *reinterpret_cast<const half_t*>(slot + Cfg::kSOff + n * 4 + lh * 2);
+      if (Cfg::kSLoads) bs[t] = Policy::read_scale(slot + Cfg::kSOff + n * 4, lh);
     }
   };
   auto read_a = [&](const unsigned char* slot, int kk, half8_t (&dst)[TME]) {
@@ -204,10 +208,9 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
   read_a(lds, 0, aop[0]);
 #pragma unroll
   for (int t = 0; t < TN; ++t) {
-    const half2_t s2 = {bs[t], bs[t]};
     half2_t d[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) d[j] = Policy::pair(bw[t], 0, j, s2);
+    for (int j = 0; j < 4; ++j) d[j] = Policy::pair(bw[t], 0, j, bs[t]);
     bop[0][t] = half8_t{d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
   }
 
@@ -249,8 +252,7 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
 #pragma unroll
             for (int p = p0; p < p1; ++p) {
               const int tt = p >> 2, j = p & 3;
-              const half2_t s2 = {bs[tt], bs[tt]};
-              dq[tt][j] = Policy::pair(bw[tt], (kk + 1) & 3, j, s2);
+              dq[tt][j] = Policy::pair(bw[tt], (kk + 1) & 3, j, bs[tt]);
             }
           }
         }

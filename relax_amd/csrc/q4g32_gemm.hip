@@ -66,6 +66,7 @@ struct Q4G32LdsPolicy {
   struct Frag {
     uint4_t w;
   };
+  using Scale = half2_t;  // the group's scale, twice
   __device__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
     const int n = q >> 1, h = q & 1;
     return reinterpret_cast<const char*>(a.W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
@@ -73,7 +74,12 @@ struct Q4G32LdsPolicy {
   __device__ static const char* s_src(const Args& a, int n, int K) {
     return reinterpret_cast<const char*>(a.S + (int64_t)n * (K >> 5));
   }
-  __device__ static half_t const_scale(const Args&, int) { return (half_t)0.0f; }
+  __device__ static int64_t s_offset(const Args&, int ks) { return (int64_t)ks * 4; }
+  __device__ static Scale read_scale(const unsigned char* p, int lh) {
+    const half_t s = *reinterpret_cast<const half_t*>(p + lh * 2);
+    return Scale{s, s};
+  }
+  __device__ static Scale const_scale(const Args&, int) { return Scale{(half_t)0.0f, (half_t)0.0f}; }
   __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
     f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
   }

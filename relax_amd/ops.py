@@ -9,9 +9,12 @@ PrimFuncs / PackedFuncs:
   (tests/python/dlight/test_gpu_gemv.py:189, test_gpu_low_batch_gemv.py:30-34)
 * format B: ``(x, w_preprocessed, scales, [bias], [residual]) -> out``
   (tests/python/relax/test_codegen_cutlass.py:1474-1520)
+* AutoGPTQ: ``(qweight uint32[K/8,N], qzeros uint32[G,N/8], scales fp16[G,N], g_idx int32[K], x, residual) -> y``
+  (tests/python/dlight/test_gpu_gemv.py:636-665)
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
@@ -258,3 +261,86 @@ def q4g32_kn_to_nk(W_kn: torch.Tensor, S_kn: torch.Tensor):
     S = torch.empty((N, K // 32), dtype=torch.float16, device=W_kn.device)
     check(_lib.lib().wq_q4g32_kn_to_nk(_ptr(W_kn), _ptr(S_kn), _ptr(W), _ptr(S), N, K, _stream()), "wq_q4g32_kn_to_nk")
     return W, S
+
+
+# ------------------------------------------------------------------ AutoGPTQ checkpoints
+
+
+def _gptq_dims(qweight, qzeros, scales, g_idx):
+    qweight, qzeros = _w32(qweight), _w32(qzeros)
+    scales = _dev(scales, torch.float16, "scales")
+    g_idx = _dev(g_idx, torch.int32, "g_idx")
+    k8, N = qweight.shape
+    K, G = k8 * 8, scales.shape[0]
+    if N % 8 or tuple(qzeros.shape) != (G, N // 8) or tuple(scales.shape) != (G, N) or tuple(g_idx.shape) != (K,):
+        raise ValueError(f"expected qzeros [G, N/8], scales [G, N], g_idx [K] for qweight [K/8, N] = [{k8}, {N}]; got "
+                         f"{tuple(qzeros.shape)}, {tuple(scales.shape)}, {tuple(g_idx.shape)}")
+    return qweight, qzeros, scales, g_idx, K, N, G
+
+
+def gptq_dequantize(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
+                    g_idx: torch.Tensor) -> torch.Tensor:
+    """fp16 ``[K, N]`` weight of an AutoGPTQ layer, bit for bit
+    (tests/python/dlight/test_gpu_gemv.py:636-652): ``(code - (zero + 1)) * scales[g_idx[k], n]``."""
+    qweight, qzeros, scales, g_idx, K, N, G = _gptq_dims(qweight, qzeros, scales, g_idx)
+    out = torch.empty((K, N), dtype=torch.float16, device=qweight.device)
+    check(_lib.lib().wq_gptq_dequantize(_ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(g_idx), _ptr(out), K, N, G,
+                                        _stream()), "wq_gptq_dequantize")
+    return out
+
+
+class GptqWeight:
+    """An AutoGPTQ layer converted for :func:`gptq_linear` (see :func:`gptq_prepare`)."""
+
+    def __init__(self, W_nk, SZ, perm, K, N, G):
+        self.W_nk, self.SZ, self.perm, self.K, self.N, self.G = W_nk, SZ, perm, K, N, G
+
+
+def gptq_prepare(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, g_idx: torch.Tensor) -> GptqWeight:
+    """Load-time conversion of an AutoGPTQ layer: rows sorted by group, words transposed to ``[N, K/8]``,
+    ``(scale, zero + 1)`` pairs ``[N, G, 2]``.  ``perm`` is kept only when the sorted order is not the identity
+    (checkpoints written with ``desc_act``)."""
+    qweight, qzeros, scales, g_idx, K, N, G = _gptq_dims(qweight, qzeros, scales, g_idx)
+    dev = qweight.device
+    W_nk = torch.empty((N, K // 8), dtype=qweight.dtype, device=dev)
+    SZ = torch.empty((N, G, 2), dtype=torch.float16, device=dev)
+    perm = torch.empty((K,), dtype=torch.int32, device=dev)
+    status = torch.empty((1,), dtype=torch.int32, device=dev)
+    needs = ctypes.c_int(0)
+    check(_lib.lib().wq_gptq_prepare(_ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(g_idx), _ptr(W_nk), _ptr(SZ),
+                                     _ptr(perm), _ptr(status), ctypes.byref(needs), K, N, G, _stream()),
+          "wq_gptq_prepare")
+    return GptqWeight(W_nk, SZ, perm if needs.value else None, K, N, G)
+
+
+def gptq_linear(w: GptqWeight, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y = residual + fp16(x . w + bias)`` for a prepared AutoGPTQ layer; ``x`` fp16 ``[..., K]``.
+    A workspace (uint8, :func:`gptq_workspace_bytes`) is allocated when needed and not given."""
+    x = _dev(x, torch.float16, "x")
+    if x.shape[-1] != w.K:
+        raise ValueError(f"x must end in K={w.K}, got {tuple(x.shape)}")
+    M = x.numel() // w.K
+    if bias is not None:
+        bias = _dev(bias, torch.float16, "bias")
+    if residual is not None:
+        residual = _dev(residual, torch.float16, "residual")
+        if residual.numel() != M * w.N:
+            raise ValueError("residual must have M*N elements")
+    if out is None:
+        out = torch.empty((*x.shape[:-1], w.N), dtype=torch.float16, device=x.device)
+    elif not out.is_contiguous() or out.numel() != M * w.N or out.dtype != torch.float16:
+        raise ValueError("out must be a contiguous fp16 tensor of M*N elements")
+    need = _lib.lib().wq_gptq_workspace_bytes(M, w.K, 1 if w.perm is not None else 0)
+    if need and workspace is None:
+        workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
+    check(_lib.lib().wq_gptq_linear(_ptr(w.W_nk), _ptr(w.SZ), _ptr(w.perm), _ptr(x), _ptr(bias), _ptr(residual),
+                                    _ptr(out), M, w.N, w.K, w.G, _ptr(workspace),
+                                    0 if workspace is None else workspace.numel() * workspace.element_size(),
+                                    _stream()), "wq_gptq_linear")
+    return out
+
+
+def gptq_workspace_bytes(M: int, K: int, has_perm: bool) -> int:
+    return int(_lib.lib().wq_gptq_workspace_bytes(M, K, 1 if has_perm else 0))
