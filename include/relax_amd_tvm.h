@@ -61,6 +61,18 @@ WQ_PACKED(relax_amd_q4f16_1_encode);
 WQ_PACKED(relax_amd_q4f16_1_kn_to_nk);
 WQ_PACKED(relax_amd_fpA_intB_encode);
 
+/* AutoGPTQ layers (tests/python/dlight/test_gpu_gemv.py:636-665: qweight u32[K/8,N], qzeros u32[G,N/8],
+ * scales f16[G,N], g_idx u32|i32[K]).  The reference leaves this PrimFunc unscheduled (:667-672).
+ *   relax_amd.autogptq_decode   (qweight, qzeros, scales, g_idx, out f16[K,N])        the decode block
+ *   relax_amd.autogptq_prepare  (qweight, qzeros, scales, g_idx, W_out u32[N,K/8], SZ_out f16[N,G,2],
+ *                                perm_out i32[K], scratch i32[1]) -> int               load time; 1 = pass
+ *                                perm_out to the matmul, 0 = rows already in group order
+ *   relax_amd.autogptq_matmul   (W_nk, SZ, perm | null, x f16[..,K], residual | null, out f16[..,N]
+ *                                [, workspace u8 >= M*K*2 bytes, needed with perm])    matmul + T_add */
+WQ_PACKED(relax_amd_autogptq_decode);
+WQ_PACKED(relax_amd_autogptq_prepare);
+WQ_PACKED(relax_amd_autogptq_matmul);
+
 /* Format B composites, one per pattern name of
  * python/tvm/relax/backend/contrib/cutlass.py:305-312, 344-372.  Arguments are the
  * composite's parameters in their Relax order followed by the output:

@@ -203,12 +203,14 @@ int wq_gptq_prepare(const uint32_t* qweight, const uint32_t* qzeros, const uint1
                     int32_t* status_scratch, int* needs_perm, int64_t K, int64_t N, int64_t G,
                     wq_stream_t stream);
 /* Bytes of workspace wq_gptq_linear needs: M*K*2 for the gathered activations when a row
- * order is given and M > WQ_GEMV_MAX_M, else 0. */
+ * order is given, else 0. */
 size_t wq_gptq_workspace_bytes(int64_t M, int64_t K, int has_perm);
 /* y fp16 [M, N] = epilogue(x fp16 [M, K] . w) over the prepared operands; bias fp16 [N] and
  * residual fp16 [M, N] may be NULL (epilogue as wq_q4g32_linear).  perm may be NULL (rows
- * already in group order).  M <= WQ_GEMV_MAX_M streams the weights once per 4 rows of x; larger
- * M runs the MFMA GEMM (group size % 64 == 0; other group sizes repeat the streaming kernel). */
+ * already in group order); with a row order the activations are first gathered into the
+ * workspace (16-byte aligned, wq_gptq_workspace_bytes).  M <= 2 streams the weights once,
+ * M <= WQ_SMALL_BATCH_MAX_M runs the small-batch kernel (K % 64 == 0), larger M the MFMA GEMM
+ * (group size % 64 == 0); shapes outside those conditions repeat the streaming kernel. */
 int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
                    const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
                    int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream);

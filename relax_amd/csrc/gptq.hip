@@ -7,17 +7,19 @@
 // through g_idx.  Here the dependence is removed once, when the checkpoint is loaded:
 //   * the K rows are sorted by group (stable), so that every group is a run of K/G
 //     consecutive rows; `perm` records the order and the activations are gathered through it
-//     (inside the GEMV's activation pass, by a small kernel before the GEMM);
+//     by a small kernel in front of the linear (one pass over x instead of one per workgroup);
 //   * the words are transposed to the [N, K/8] layout of the other kernels of this library
 //     (a word holds 8 consecutive k of one column in both layouts);
 //   * scale and zero point + 1 are interleaved as fp16 pairs SZ [N, G, 2], the 4 bytes that
 //     one lane needs for one group.
 // After that the weight stream is the one of format A with one more multiply-add per group,
-// and both the streaming GEMV (q4_gemv.h) and the MFMA GEMM (mfma_gemm_lds.h) take it.
+// and the streaming GEMV (q4_gemv.h), the small-batch kernel (skinny_gemm.h) and the MFMA GEMM
+// (mfma_gemm_lds.h) all take it.
 // A g_idx whose groups do not all have K/G members is rejected by the preparation.
 #include "mfma_gemm_lds.h"
 #include "q4_gemv.h"
 #include "q4g32_common.h"
+#include "skinny_gemm.h"
 
 namespace wq {
 
@@ -103,13 +105,86 @@ __global__ __launch_bounds__(256) void gptq_sz_kernel(const uint32_t* __restrict
   SZ[(int64_t)n * G + g] = half2_t{scales[(int64_t)g * N + n], (half_t)(float)(zero + 1u)};
 }
 
-// xp[m][k'] = x[m][perm[k']]
+// xp[m][k'] = x[m][perm[k']]: one row per workgroup, read coalesced into LDS, gathered from there
+// (K <= 32768: 64 KiB), written coalesced as pairs.
 __global__ __launch_bounds__(256) void gptq_gather_x_kernel(const half_t* __restrict__ x, const int* __restrict__ perm,
                                                             half_t* __restrict__ xp, int K) {
-  const int k = blockIdx.x * 256 + threadIdx.x;
-  const int64_t m = blockIdx.y;
-  if (k < K) xp[m * K + k] = x[m * K + perm[k]];
+  extern __shared__ uint4_t gather_smem[];
+  half_t* row = reinterpret_cast<half_t*>(gather_smem);
+  const int64_t m = blockIdx.x;
+  const uint4_t* src = reinterpret_cast<const uint4_t*>(x + m * K);
+  for (int i = threadIdx.x; i < (K >> 3); i += 256) gather_smem[i] = src[i];
+  __syncthreads();
+  half2_t* dst = reinterpret_cast<half2_t*>(xp + m * K);
+  const int2* p2 = reinterpret_cast<const int2*>(perm);
+  for (int i = threadIdx.x; i < (K >> 1); i += 256) {
+    const int2 p = p2[i];
+    dst[i] = half2_t{row[p.x], row[p.y]};
+  }
 }
+
+// The same for a few rows: thread per output pair, straight from global memory.
+__global__ __launch_bounds__(256) void gptq_gather_x_direct_kernel(const half_t* __restrict__ x,
+                                                                   const int* __restrict__ perm,
+                                                                   half_t* __restrict__ xp, int K) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int64_t m = blockIdx.y;
+  if (i < (K >> 1)) {
+    const int2 p = reinterpret_cast<const int2*>(perm)[i];
+    reinterpret_cast<half2_t*>(xp + m * K)[i] = half2_t{x[m * K + p.x], x[m * K + p.y]};
+  }
+}
+
+// ---- small-batch policy: format A's stream with the (scale, zero point) pair of the lane's group ----
+struct GptqSkinnyPolicy {
+  static constexpr int kPieces = 1;
+  static constexpr bool kScaleDma = true;
+  struct Args {
+    const uint32_t* W;
+    const half2_t* SZ;
+    int groups;    // per row
+    int ratio;     // 32-code groups per scale group
+    uint32_t inv;  // ceil(2^32 / ratio), unused when ratio == 1
+  };
+  struct Lane {
+    const char* w;
+    const char* sz;
+    int ratio;
+    uint32_t inv;
+  };
+  using Scale = half2_t;  // (scale, zero point)
+  __device__ static void init(Lane& l, const Args& a, int n, int K, int) {
+    l.w = reinterpret_cast<const char*>(a.W + (int64_t)n * (K >> 3));
+    l.sz = reinterpret_cast<const char*>(a.SZ + (int64_t)n * a.groups);
+    l.ratio = a.ratio;
+    l.inv = a.inv;
+  }
+  __device__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
+  __device__ static const char* s_addr(const Lane& l, int k0) {
+    const uint32_t g32 = (uint32_t)k0 >> 5;
+    return l.sz + (l.ratio == 1 ? g32 : __umulhi(g32, l.inv)) * 4;
+  }
+  __device__ static Scale pick_scale(const Lane&, half2_t pair, int) { return pair; }
+  __device__ static Scale const_scale(const Lane&) { return Scale{}; }
+  __device__ static Scale null_scale() { return Scale{(half_t)0.0f, (half_t)0.0f}; }
+  __device__ static void dequant(const uint4_t* pieces, Scale sz, half8_t out[4]) {
+    const half2_t s2 = {sz.x, sz.x};
+    const half_t o = sz.y + (half_t)1024.0f;
+    const half2_t off = {o, o};
+    const uint32_t words[4] = {pieces[0].x, pieces[0].y, pieces[0].z, pieces[0].w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      half2_t d[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t b = (words[t] >> (8 * j)) & 0xFFu;  // codes 2j, 2j+1
+        const uint32_t u = (b << 12) | b;
+        d[j] = (as_half2(and_or(u, 0x000F000Fu, 0x64006400u)) - off) * s2;
+      }
+      out[t] = half8_t{d[0].x, d[0].y, d[1].x, d[1].y, d[2].x, d[2].y, d[3].x, d[3].y};
+    }
+  }
+};
 
 // ---- MFMA GEMM policy: the stream of format A with a (scale, zero point) pair per group ------
 // A K-step (64 rows) lies inside one group (group size % 64 == 0), so both lane halves read the
@@ -221,7 +296,7 @@ extern "C" int wq_gptq_prepare(const uint32_t* qweight, const uint32_t* qzeros, 
 }
 
 extern "C" size_t wq_gptq_workspace_bytes(int64_t M, int64_t K, int has_perm) {
-  return (has_perm && M > WQ_GEMV_MAX_M && M > 0 && K > 0) ? (size_t)M * (size_t)K * 2 : 0;
+  return (has_perm && M > 0 && K > 0) ? (size_t)M * (size_t)K * 2 : 0;
 }
 
 extern "C" int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
@@ -240,27 +315,42 @@ extern "C" int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const in
              "wq_gptq_linear: W_nk, x and perm must be 16-byte aligned, SZ 4-byte aligned");
   WQ_REQUIRE(N < (1ll << 30) && K <= 32768 && M < (1ll << 30),
              "wq_gptq_linear: N=%lld K=%lld outside the supported range (K <= 32768)", (long long)N, (long long)K);
-  const GemvZp zp{perm, (int)(gs / 32), (int)G};
-  if (M <= WQ_GEMV_MAX_M || gs % 64 != 0)
-    return gemv_dispatch<true>("wq_gptq_linear", W_nk, SZ, zp, x, bias, residual, y, M, N, K, stream);
-  const uint16_t* xg = x;
+  // a row order: gather the activations once, in front of whichever kernel runs
   if (perm) {
     const size_t need = (size_t)M * (size_t)K * 2;
     WQ_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
-               "wq_gptq_linear: M=%lld with a row order needs a 16-byte aligned workspace of %zu bytes (got %zu)",
-               (long long)M, need, workspace_bytes);
-    WQ_REQUIRE(M < 65536, "wq_gptq_linear: M=%lld too large for the gather", (long long)M);
-    WQ_LAUNCH("wq_gptq_linear", gptq_gather_x_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)M), dim3(256), 0,
-              stream, (const half_t*)x, perm, (half_t*)workspace, (int)K);
-    xg = (const uint16_t*)workspace;
+               "wq_gptq_linear: a row order needs a 16-byte aligned workspace of M*K*2 = %zu bytes (got %zu)", need,
+               workspace_bytes);
+    if (M <= 64) {  // few rows: spread each over many workgroups
+      WQ_LAUNCH("wq_gptq_linear", gptq_gather_x_direct_kernel, dim3((unsigned)((K / 2 + 255) / 256), (unsigned)M),
+                dim3(256), 0, stream, (const half_t*)x, perm, (half_t*)workspace, (int)K);
+    } else {
+      auto kern = gptq_gather_x_kernel;
+      const size_t lds = (size_t)K * 2;
+      if (lds > 48 * 1024)
+        WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)lds));
+      WQ_LAUNCH("wq_gptq_linear", kern, dim3((unsigned)M), dim3(256), lds, stream, (const half_t*)x, perm,
+                (half_t*)workspace, (int)K);
+    }
+    x = (const uint16_t*)workspace;
   }
+  const int ratio = (int)(gs / 32);
+  const uint32_t inv32 = ratio > 1 ? (uint32_t)(((1ull << 32) + ratio - 1) / ratio) : 0u;
+  const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
+  if (M <= 2) return gemv_dispatch<true>("wq_gptq_linear", W_nk, SZ, GemvZp{ratio, (int)G}, x, bias, residual, y, M, N, K, stream);
+  if (M <= WQ_SMALL_BATCH_MAX_M && K % 64 == 0) {
+    const GptqSkinnyPolicy::Args pargs{W_nk, (const half2_t*)SZ, (int)G, ratio, inv32};
+    return launch_skinny_auto<GptqSkinnyPolicy, Q4G32Epilogue>("wq_gptq_linear", pargs, x, y, ep, M, N, K, stream);
+  }
+  if (gs % 64 != 0)  // a K-step of the GEMM would straddle two groups: repeat the streaming kernel
+    return gemv_dispatch<true>("wq_gptq_linear", W_nk, SZ, GemvZp{ratio, (int)G}, x, bias, residual, y, M, N, K, stream);
   const int spg = (int)(gs / 64);
   const GptqLdsPolicy::Args largs{W_nk, (const half2_t*)SZ, (int)G, spg,
                                   spg > 1 ? (uint32_t)(((1ull << 32) + spg - 1) / spg) : 0u};
-  const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
   if (M <= 384)
-    return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 4, 1, 1, 4, 2>("wq_gptq_linear", largs, xg, y, ep, M, N, K,
+    return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 4, 1, 1, 4, 2>("wq_gptq_linear", largs, x, y, ep, M, N, K,
                                                                         stream);
-  return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 8, 2, 1, 4, 1>("wq_gptq_linear", largs, xg, y, ep, M, N, K,
+  return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 8, 2, 1, 4, 1>("wq_gptq_linear", largs, x, y, ep, M, N, K,
                                                                       stream);
 }

@@ -40,7 +40,9 @@ struct IntbSkinnyPolicy {
     return reinterpret_cast<const char*>(l.s + (int64_t)(k0 >> 6) * l.N);
   }
   __device__ static half_t pick_scale(const Lane& l, half2_t pair, int) { return l.odd ? pair.y : pair.x; }
+  using Scale = half_t;
   __device__ static half_t const_scale(const Lane& l) { return l.s[0]; }
+  __device__ static half_t null_scale() { return (half_t)0.0f; }
   __device__ static void dequant(const uint4_t* pieces, half_t s, half8_t out[4]) {
     const half2_t s2 = {s, s};
     if (NBIT == 8) {

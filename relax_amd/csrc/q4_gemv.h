@@ -1,4 +1,5 @@
-// Format A decode GEMV: y[m,n] = sum_k x[m,k] * ((code[n,k] - 7) * S[n,k/32]), M <= 8.
+// Decode GEMV over [N, K/8] int4 weights: y[m,n] = sum_k x[m,k] * ((code[n,k] - 7) * S[n,k/32])
+// (format A), or with a zero point per group, (code - zp) * s (template parameter ZP).
 //
 // The kernel is a weight stream bounded by HBM bandwidth, so the design goal is
 // to keep many 16-byte loads in flight per CU, to put nothing (no LDS staging, no
@@ -52,11 +53,10 @@ constexpr int gemv_max_threads() {
 }
 
 // What the zero-point variant adds to the launch: S holds (scale, zero point) fp16 pairs
-// [N, groups], one per `ratio` consecutive 32-code groups, and x may be gathered through `perm`.
+// [N, groups], one per `ratio` consecutive 32-code groups.
 struct GemvZp {
-  const int* perm;  // x'[k] = x[perm[k]], or nullptr
-  int ratio;        // 32-code groups per scale group
-  int groups;       // scale groups per row
+  int ratio;   // 32-code groups per scale group
+  int groups;  // scale groups per row
 };
 
 template <int ROWS, int GPL>
@@ -127,17 +127,7 @@ __global__ __launch_bounds__(gemv_max_threads<GPL>()) void q4g32_gemv_kernel(
 #pragma unroll
     for (int i = 0; i < kMaxXW; ++i) {
       const int wi = tid + i * nthreads;
-      if (wi < nwords) {
-        if (ZP && zp.perm) {  // gather: the weights were reordered along K when they were prepared
-          const int4 p0 = reinterpret_cast<const int4*>(zp.perm)[2 * wi];
-          const int4 p1 = reinterpret_cast<const int4*>(zp.perm)[2 * wi + 1];
-          const half_t* xr = x + (int64_t)m * K;
-          xraw[m][i] = uint4_t{as_u32(half2_t{xr[p0.x], xr[p0.y]}), as_u32(half2_t{xr[p0.z], xr[p0.w]}),
-                               as_u32(half2_t{xr[p1.x], xr[p1.y]}), as_u32(half2_t{xr[p1.z], xr[p1.w]})};
-        } else {
-          xraw[m][i] = reinterpret_cast<const uint4_t*>(x + (int64_t)m * K)[wi];
-        }
-      }
+      if (wi < nwords) xraw[m][i] = reinterpret_cast<const uint4_t*>(x + (int64_t)m * K)[wi];
     }
 
   // ---- 2. weights and scales of the first row set: issued now, consumed last ----
@@ -397,7 +387,7 @@ static int launch_gemv_rows(const char* who, int rows, const uint32_t* W, const 
   }
 }
 
-// Batches of up to 4 rows of x share one pass over the weights.
+// Two rows of x share one pass over the weights (four in registers spill and run slower than two passes).
 template <bool ZP>
 static int gemv_dispatch(const char* who, const uint32_t* W, const uint16_t* S, const GemvZp& zp, const uint16_t* x,
                          const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
@@ -408,17 +398,14 @@ static int gemv_dispatch(const char* who, const uint32_t* W, const uint16_t* S, 
   int gpl = g_gemv_gpl ? g_gemv_gpl
                        : (G <= 64 ? 1 : G <= 128 ? 2 : G <= 192 ? 3 : G <= 256 ? 4 : G <= 384 ? 3 : 2);
   const int rows = g_gemv_rows;  // 0 = from the shape
-  // batches of up to 4 rows of x share one pass over the weights
+  // pairs of rows of x share one pass over the weights
   for (int64_t m0 = 0; m0 < M;) {
     const int64_t left = M - m0;
     const uint16_t* xp = x + m0 * K;
     const uint16_t* rp = residual ? residual + m0 * N : nullptr;
     uint16_t* yp = y + m0 * N;
     int rc;
-    if (left >= 4) {
-      rc = launch_gemv_rows<4, 1, ZP>(who, rows == 0 || rows > 2 ? 2 : rows, W, S, zp, xp, bias, rp, yp, N, K, stream);
-      m0 += 4;
-    } else if (left >= 2) {
+    if (left >= 2) {
       rc = gpl >= 2 ? launch_gemv_rows<2, 2, ZP>(who, rows, W, S, zp, xp, bias, rp, yp, N, K, stream)
                     : launch_gemv_rows<2, 1, ZP>(who, rows, W, S, zp, xp, bias, rp, yp, N, K, stream);
       m0 += 2;

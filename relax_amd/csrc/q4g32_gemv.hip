@@ -26,5 +26,5 @@ extern "C" int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_
   WQ_REQUIRE(N < (1ll << 30) && K <= 32768,
              "wq_q4g32_gemv: N=%lld K=%lld outside the supported range (K <= 32768)",
              (long long)N, (long long)K);
-  return gemv_dispatch<false>("wq_q4g32_gemv", W, S, GemvZp{nullptr, 1, 0}, x, bias, residual, y, M, N, K, stream);
+  return gemv_dispatch<false>("wq_q4g32_gemv", W, S, GemvZp{1, 0}, x, bias, residual, y, M, N, K, stream);
 }

@@ -25,7 +25,9 @@ struct Q4G32SkinnyPolicy {
   __device__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
   __device__ static const char* s_addr(const Lane& l, int k0) { return l.s + ((k0 >> 5) & ~1) * 2; }
   __device__ static half_t pick_scale(const Lane&, half2_t pair, int kq) { return (kq & 1) ? pair.y : pair.x; }
+  using Scale = half_t;
   __device__ static half_t const_scale(const Lane&) { return (half_t)0.0f; }
+  __device__ static half_t null_scale() { return (half_t)0.0f; }
   __device__ static void dequant(const uint4_t* pieces, half_t s, half8_t out[4]) {
     const half2_t s2 = {s, s};
     const uint32_t words[4] = {pieces[0].x, pieces[0].y, pieces[0].z, pieces[0].w};

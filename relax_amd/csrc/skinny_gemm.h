@@ -46,8 +46,10 @@ typedef void __attribute__((address_space(3))) * wq_sk_lptr_t;
 //   init(lane, args, n, K, N)
 //   w_addr(lane, k0, p)        address of piece p of the 32 codes starting at k0 (k0 % 32 == 0)
 //   s_addr(lane, k0)           4-byte aligned address of the pair holding the scale for k0   (kScaleDma)
-//   pick_scale(lane, pair, kq) the lane's half of that pair                                  (kScaleDma)
-//   const_scale(lane)          the lane's scale                                              (!kScaleDma)
+//   Scale                      what dequant needs besides the codes (half_t, or scale and zero point)
+//   pick_scale(lane, pair, kq) the lane's Scale from that pair                               (kScaleDma)
+//   const_scale(lane)          the lane's Scale                                              (!kScaleDma)
+//   null_scale()               a Scale that turns every code into an exact zero (weights past K)
 //   dequant(pieces, s, out[4]) -> B operands of MFMA 0..3 (k 8t .. 8t+7 each), scaled
 template <typename Policy, int TH, int NW, int WAVES>
 struct SkinnyCfg {
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
   }
   typename Policy::Lane pl;
   Policy::init(pl, pargs, min(n0 + 16 * nw + lj, N - 1), K, N);  // clamped columns are never stored
-  half_t s_fixed = (half_t)0.0f;
+  typename Policy::Scale s_fixed = Policy::null_scale();
   if (!Policy::kScaleDma) s_fixed = Policy::const_scale(pl);
 
   unsigned char* const w_area = lds + Cfg::kXBytes + wave * (P * 1024);
@@ -152,10 +154,10 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
 #pragma unroll
     for (int p = 0; p < P; ++p)
       pieces[p] = *reinterpret_cast<const uint4_t*>(w_area + stage_off + p * 1024 + lane * 16);
-    half_t s = s_fixed;
+    typename Policy::Scale s = s_fixed;
     if (Policy::kScaleDma)
       s = Policy::pick_scale(pl, *reinterpret_cast<const half2_t*>(s_area + stage_off + lane * 4), kq);
-    if (k0 >= K) s = (half_t)0.0f;  // code * 0 = exact zero for the weights past K
+    if (k0 >= K) s = Policy::null_scale();  // code * 0 = exact zero for the weights past K
     half8_t bop[4];
     Policy::dequant(pieces, s, bop);
     const unsigned char* slab = lds + stage_off + kw * Cfg::kSlabBytes;

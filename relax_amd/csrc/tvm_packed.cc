@@ -450,6 +450,129 @@ WQ_PACKED(relax_amd_q4f16_1_kn_to_nk) {
   return rc == WQ_OK ? 0 : packed_fail();
 }
 
+// ---- AutoGPTQ layers (tests/python/dlight/test_gpu_gemv.py:636-665) ----
+// g_idx is uint32 in the reference's PrimFunc and int32 in AutoGPTQ checkpoints: same bytes.
+static bool get_index_tensor(const char* who, TVMValue* args, int* tcodes, int n, int i, const char* what, Tensor* t) {
+  const DLTensor* d = i < n && (tcodes[i] == kTVMDLTensorHandle || tcodes[i] == kTVMNDArrayHandle)
+                          ? static_cast<const DLTensor*>(args[i].v_handle)
+                          : nullptr;
+  const int code = (d && d->dtype.code == kDLUInt) ? kDLUInt : kDLInt;
+  return get_tensor(who, args, tcodes, n, i, code, 32, what, t);
+}
+
+static bool gptq_checkpoint_args(const char* who, TVMValue* args, int* tcodes, int n, Tensor* qw, Tensor* qz,
+                                 Tensor* sc, Tensor* gi, int64_t* K, int64_t* N, int64_t* G) {
+  if (!get_tensor(who, args, tcodes, n, 0, kDLUInt, 32, "qweight", qw) ||
+      !get_tensor(who, args, tcodes, n, 1, kDLUInt, 32, "qzeros", qz) ||
+      !get_tensor(who, args, tcodes, n, 2, kDLFloat, 16, "scales", sc) ||
+      !get_index_tensor(who, args, tcodes, n, 3, "g_idx", gi))
+    return false;
+  if (qw->t->ndim != 2 || qz->t->ndim != 2 || sc->t->ndim != 2 || gi->t->ndim != 1) {
+    fail(WQ_EINVAL, "%s: expected qweight [K/8,N], qzeros [G,N/8], scales [G,N], g_idx [K]", who);
+    return false;
+  }
+  *K = qw->t->shape[0] * 8;
+  *N = qw->t->shape[1];
+  *G = sc->t->shape[0];
+  if (sc->t->shape[1] != *N || qz->t->shape[0] != *G || qz->t->shape[1] * 8 != *N || gi->t->shape[0] != *K) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (K=%lld N=%lld G=%lld)", who, (long long)*K, (long long)*N,
+         (long long)*G);
+    return false;
+  }
+  return true;
+}
+
+// (qweight, qzeros, scales, g_idx, out fp16 [K, N]): the decode block alone.
+WQ_PACKED(relax_amd_autogptq_decode) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.autogptq_decode";
+  Tensor qw, qz, sc, gi, out;
+  int64_t K, N, G;
+  if (num_args != 5) {
+    fail(WQ_EINVAL, "%s: expected (qweight, qzeros, scales, g_idx, out)", who);
+    return packed_fail();
+  }
+  if (!gptq_checkpoint_args(who, args, type_codes, num_args, &qw, &qz, &sc, &gi, &K, &N, &G) ||
+      !get_tensor(who, args, type_codes, num_args, 4, kDLFloat, 16, "out", &out))
+    return packed_fail();
+  if (out.numel != K * N) {
+    fail(WQ_EINVAL, "%s: out must have K*N elements", who);
+    return packed_fail();
+  }
+  const int rc = wq_gptq_dequantize((const uint32_t*)qw.ptr, (const uint32_t*)qz.ptr, (const uint16_t*)sc.ptr,
+                                    (const int32_t*)gi.ptr, (uint16_t*)out.ptr, K, N, G, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
+// (qweight, qzeros, scales, g_idx, W_out uint32 [N,K/8], SZ_out fp16 [N,G,2], perm_out int32 [K],
+//  scratch int32 [1]) -> int: 1 if the matmul must be given perm_out, 0 if the rows were already in group order.
+WQ_PACKED(relax_amd_autogptq_prepare) {
+  (void)resource_handle;
+  const char* who = "relax_amd.autogptq_prepare";
+  Tensor qw, qz, sc, gi, Wo, SZ, perm, scratch;
+  int64_t K, N, G;
+  if (num_args != 8) {
+    fail(WQ_EINVAL, "%s: expected (qweight, qzeros, scales, g_idx, W_out, SZ_out, perm_out, scratch)", who);
+    return packed_fail();
+  }
+  if (!gptq_checkpoint_args(who, args, type_codes, num_args, &qw, &qz, &sc, &gi, &K, &N, &G) ||
+      !get_tensor(who, args, type_codes, num_args, 4, kDLUInt, 32, "W_out", &Wo) ||
+      !get_tensor(who, args, type_codes, num_args, 5, kDLFloat, 16, "SZ_out", &SZ) ||
+      !get_tensor(who, args, type_codes, num_args, 6, kDLInt, 32, "perm_out", &perm) ||
+      !get_tensor(who, args, type_codes, num_args, 7, kDLInt, 32, "scratch", &scratch))
+    return packed_fail();
+  if (Wo.numel != N * (K / 8) || SZ.numel != N * G * 2 || perm.numel != K || scratch.numel < 1) {
+    fail(WQ_EINVAL, "%s: outputs must be W_out [N,K/8], SZ_out [N,G,2], perm_out [K], scratch [1]", who);
+    return packed_fail();
+  }
+  int needs = 0;
+  const int rc = wq_gptq_prepare((const uint32_t*)qw.ptr, (const uint32_t*)qz.ptr, (const uint16_t*)sc.ptr,
+                                 (const int32_t*)gi.ptr, (uint32_t*)Wo.ptr, (uint16_t*)SZ.ptr, (int32_t*)perm.ptr,
+                                 (int32_t*)scratch.ptr, &needs, K, N, G, current_stream());
+  if (rc != WQ_OK) return packed_fail();
+  if (out_ret_value && out_ret_tcode) {
+    out_ret_value->v_int64 = needs;
+    *out_ret_tcode = kTVMArgInt;
+  }
+  return 0;
+}
+
+// (W_nk, SZ, perm | null, x, residual | null, out [, workspace uint8]): the matmul and the add of the
+// reference's PrimFunc over the prepared operands, argument order as there (weights, x, residual, out).
+WQ_PACKED(relax_amd_autogptq_matmul) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.autogptq_matmul";
+  Tensor W, SZ, perm, x, res, out, ws;
+  if (num_args != 6 && num_args != 7) {
+    fail(WQ_EINVAL, "%s: expected (W_nk, SZ, perm|null, x, residual|null, out[, workspace])", who);
+    return packed_fail();
+  }
+  const bool has_perm = type_codes[2] != kTVMNullptr, has_res = type_codes[4] != kTVMNullptr;
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W_nk", &W) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "SZ", &SZ) ||
+      (has_perm && !get_tensor(who, args, type_codes, num_args, 2, kDLInt, 32, "perm", &perm)) ||
+      !get_tensor(who, args, type_codes, num_args, 3, kDLFloat, 16, "x", &x) ||
+      (has_res && !get_tensor(who, args, type_codes, num_args, 4, kDLFloat, 16, "residual", &res)) ||
+      !get_tensor(who, args, type_codes, num_args, 5, kDLFloat, 16, "out", &out) ||
+      (num_args == 7 && !get_tensor(who, args, type_codes, num_args, 6, kDLUInt, 8, "workspace", &ws)))
+    return packed_fail();
+  if (W.t->ndim != 2 || SZ.t->ndim != 3 || SZ.t->shape[2] != 2 || SZ.t->shape[0] != W.t->shape[0] || x.t->ndim < 1) {
+    fail(WQ_EINVAL, "%s: expected W_nk [N,K/8] and SZ [N,G,2]", who);
+    return packed_fail();
+  }
+  const int64_t N = W.t->shape[0], K = W.t->shape[1] * 8, G = SZ.t->shape[1];
+  const int64_t m = leading(x.t);
+  if (x.t->shape[x.t->ndim - 1] != K || out.numel != m * N || (has_perm && perm.numel != K) ||
+      (has_res && res.numel != m * N)) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (m=%lld n=%lld k=%lld)", who, (long long)m, (long long)N, (long long)K);
+    return packed_fail();
+  }
+  const int rc = wq_gptq_linear((const uint32_t*)W.ptr, (const uint16_t*)SZ.ptr, (const int32_t*)perm.ptr,
+                                (const uint16_t*)x.ptr, nullptr, (const uint16_t*)res.ptr, (uint16_t*)out.ptr, m, N, K,
+                                G, ws.ptr, num_args == 7 ? (size_t)ws.numel : 0, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
 // (A fp16 [N, K]) -> (w int8 [K, N] | [K, N/2], scales fp16 [N] | [K/64, N], scratch fp32 [N]): the
 // reference fixtures' `encode`; int4 and the group size follow from the output shapes.
 WQ_PACKED(relax_amd_fpA_intB_encode) {
@@ -553,6 +676,9 @@ const std::vector<Entry>& table() {
     v.push_back({"relax_amd.q4f16_1_encode", "relax_amd_q4f16_1_encode", relax_amd_q4f16_1_encode});
     v.push_back({"relax_amd.q4f16_1_kn_to_nk", "relax_amd_q4f16_1_kn_to_nk", relax_amd_q4f16_1_kn_to_nk});
     v.push_back({"relax_amd.fpA_intB_encode", "relax_amd_fpA_intB_encode", relax_amd_fpA_intB_encode});
+    v.push_back({"relax_amd.autogptq_decode", "relax_amd_autogptq_decode", relax_amd_autogptq_decode});
+    v.push_back({"relax_amd.autogptq_prepare", "relax_amd_autogptq_prepare", relax_amd_autogptq_prepare});
+    v.push_back({"relax_amd.autogptq_matmul", "relax_amd_autogptq_matmul", relax_amd_autogptq_matmul});
 #define WQ_ENTRY(sym, op) v.push_back({std::string("relax_amd.") + op, #sym, sym});
     WQ_DECODE_MATMUL_LIST(WQ_ENTRY)
 #undef WQ_ENTRY

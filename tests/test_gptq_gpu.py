@@ -105,8 +105,12 @@ LINEAR_CASES = [  # (M, N, K, group size, act_order)
     (4, 1000, 2048, 1024, False),
     (5, 264, 4096, 4096, True),    # one group
     (8, 2048, 4096, 128, True),
-    (7, 72, 96, 96, True),         # group size not a multiple of 64
-    (16, 512, 1024, 128, True),    # MFMA GEMM from here
+    (7, 72, 96, 96, True),         # K not a multiple of 64: streaming kernel repeated
+    (16, 512, 1024, 128, True),    # small-batch kernel
+    (33, 1032, 4096, 128, True),
+    (64, 4096, 4096, 128, False),
+    (64, 264, 384, 96, True),      # three 32-code groups per scale group
+    (65, 512, 1024, 128, True),    # MFMA GEMM from here
     (16, 512, 1024, 128, False),
     (40, 264, 1152, 192, True),
     (130, 1096, 2048, 64, True),
@@ -138,10 +142,10 @@ def test_linear_bias_and_plain(ops, u, oracle, M):
                    _ref_linear(oracle, qw, qz, s, g_idx, x, bias), "bias")
 
 
-@pytest.mark.parametrize("M", [1, 64])
+@pytest.mark.parametrize("M", [1, 8, 64, 100])
 def test_one_hot_rows_reproduce_the_dequantized_weight(ops, u, oracle, M):
-    """x = e_k selects row k of the weight: exact in the GEMM (it multiplies the reference's fp16
-    weights), one fp16 ulp in the streaming kernel (it applies the scale after the sum)."""
+    """x = e_k selects row k of the weight: exact in the small-batch kernel and the GEMM (they multiply
+    the reference's fp16 weights), one fp16 ulp in the streaming kernel (it applies the scale after the sum)."""
     N, K, gs = 256, 512, 128
     _, qw, qz, s, g_idx = oracle.make_gptq_inputs(1, N, K, gs, seed=11, act_order=True)
     B = oracle.gptq_dequant(qw, qz, s, g_idx)
@@ -150,7 +154,7 @@ def test_one_hot_rows_reproduce_the_dequantized_weight(ops, u, oracle, M):
     x[np.arange(M), ks] = 1
     w = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
     got = u.host(ops.gptq_linear(w, u.dev(x)))
-    if M > 8:
+    if M > 2:
         assert np.array_equal(_bits(got), _bits(B[ks]))
     else:
         assert np.max(np.abs(got.astype(np.float64) - B[ks].astype(np.float64))) <= 2.0**-10 * np.max(np.abs(B))
@@ -164,7 +168,7 @@ def test_linear_argument_errors(ops, u, oracle):
     x, qw, qz, s, g_idx = oracle.make_gptq_inputs(16, 64, 256, 64, seed=1, act_order=True)
     w = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
     assert ops.gptq_workspace_bytes(16, 256, True) == 16 * 256 * 2
-    assert ops.gptq_workspace_bytes(16, 256, False) == 0 and ops.gptq_workspace_bytes(8, 256, True) == 0
+    assert ops.gptq_workspace_bytes(16, 256, False) == 0 and ops.gptq_workspace_bytes(1, 256, True) == 512
     with pytest.raises(WqError, match="workspace"):
         ops.gptq_linear(w, u.dev(x), workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
     with pytest.raises(ValueError):

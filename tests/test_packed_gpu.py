@@ -109,3 +109,79 @@ def test_decode_matmul_composites(env, oracle, nbit):
     rc, _, _ = T.call(lib.relax_amd_decode_matmul_bias, tx, tP, ts, tb2, to)
     assert rc == 0
     u.assert_close(u.host(out), oracle.intb_linear(x, A, s, nbit, bias=bias2, bias_stride=N, nthreads=4), "full bias")
+
+
+def test_autogptq_family(env, oracle):
+    """decode, prepare (returns whether a row order is needed) and matmul + add over an act-order layer,
+    with g_idx typed uint32 as in the reference's PrimFunc (tests/python/dlight/test_gpu_gemv.py:639)."""
+    lib, u, T, torch = env
+    M, N, K, gs = 2, 136, 512, 128
+    G = K // gs
+    x, qw, qz, s, g_idx = oracle.make_gptq_inputs(M, N, K, gs, seed=21, act_order=True)
+    res = np.random.default_rng(4).standard_normal((M, N)).astype(np.float16)
+    d = {k: u.dev(v) for k, v in dict(qw=qw, qz=qz, s=s, g=g_idx, x=x.reshape(M, 1, K), r=res.reshape(M, 1, N)).items()}
+    tqw, _ = T.from_torch(d["qw"], "uint32")
+    tqz, _ = T.from_torch(d["qz"], "uint32")
+    ts, _ = T.from_torch(d["s"])
+    tg, _ = T.from_torch(d["g"], "uint32")
+    tx, _ = T.from_torch(d["x"])
+    tr, _ = T.from_torch(d["r"])
+    B = torch.empty((K, N), dtype=torch.float16, device="cuda")
+    tB, _ = T.from_torch(B)
+    rc, _, _ = T.call(lib.relax_amd_autogptq_decode, tqw, tqz, ts, tg, tB)
+    assert rc == 0, lib.wq_last_error()
+    Bref = oracle.gptq_dequant(qw, qz, s, g_idx)
+    assert np.array_equal(u.host(B).view(np.uint16), Bref.view(np.uint16))
+
+    W = torch.empty((N, K // 8), dtype=torch.int32, device="cuda")
+    SZ = torch.empty((N, G, 2), dtype=torch.float16, device="cuda")
+    perm = torch.empty((K,), dtype=torch.int32, device="cuda")
+    scratch = torch.empty((1,), dtype=torch.int32, device="cuda")
+    tW, _ = T.from_torch(W, "uint32")
+    tSZ, _ = T.from_torch(SZ)
+    tp, _ = T.from_torch(perm)
+    tsc, _ = T.from_torch(scratch)
+    rc, rv, rcode = T.call(lib.relax_amd_autogptq_prepare, tqw, tqz, ts, tg, tW, tSZ, tp, tsc)
+    assert rc == 0, lib.wq_last_error()
+    assert rcode == T.kTVMArgInt and rv.v_int64 == 1
+    assert np.array_equal(u.host(perm), np.argsort(g_idx, kind="stable").astype(np.int32))
+
+    y = torch.empty((M, 1, N), dtype=torch.float16, device="cuda")
+    ty, _ = T.from_torch(y)
+    ws = torch.empty((40 * K * 2,), dtype=torch.uint8, device="cuda")  # gathered activations, up to M = 40
+    tws, _ = T.from_torch(ws)
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul, tW, tSZ, tp, tx, tr, ty, tws)
+    assert rc == 0, lib.wq_last_error()
+    want = oracle.nt_matmul_f32acc(np.ascontiguousarray(Bref.T), x, None, res)
+    u.assert_close(u.host(y).reshape(M, N), want, "packed autogptq matmul + add")
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul, tW, tSZ, tp, tx, None, ty, tws)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y).reshape(M, N), oracle.nt_matmul_f32acc(np.ascontiguousarray(Bref.T), x), "no residual")
+
+    # a row order needs the workspace for the gathered activations
+    M2 = 40
+    x2 = np.random.default_rng(5).standard_normal((M2, K)).astype(np.float16)
+    dx2 = u.dev(x2)
+    y2 = torch.empty((M2, N), dtype=torch.float16, device="cuda")
+    tx2, _ = T.from_torch(dx2)
+    ty2, _ = T.from_torch(y2)
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul, tW, tSZ, tp, tx2, None, ty2)
+    assert rc == -1 and b"workspace" in lib.wq_last_error()
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul, tW, tSZ, tp, tx2, None, ty2, tws)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y2), oracle.nt_matmul_f32acc(np.ascontiguousarray(Bref.T), x2, nthreads=4), "prefill")
+
+    # without act-order the preparation reports that no row order is needed
+    _, qw3, qz3, s3, g3 = oracle.make_gptq_inputs(1, N, K, gs, seed=22)
+    e = [u.dev(v) for v in (qw3, qz3, s3, g3)]
+    t3 = [T.from_torch(e[0], "uint32")[0], T.from_torch(e[1], "uint32")[0], T.from_torch(e[2])[0], T.from_torch(e[3])[0]]
+    rc, rv, rcode = T.call(lib.relax_amd_autogptq_prepare, *t3, tW, tSZ, tp, tsc)
+    assert rc == 0 and rv.v_int64 == 0
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul, tW, tSZ, None, tx, None, ty)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y).reshape(M, N), oracle.gptq_linear(qw3, qz3, s3, g3, x), "identity order")
+    # wrong arity / shapes
+    rc, _, _ = T.call(lib.relax_amd_autogptq_decode, tqw, tqz, ts, tB)
+    assert rc == -1
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul, tW, tSZ, tp, tx2, tr, ty2, tws)
+    assert rc == -1 and b"inconsistent" in lib.wq_last_error()

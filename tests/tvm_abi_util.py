@@ -63,7 +63,7 @@ def from_torch(t, dtype=None):
 
 
 def pack(*items):
-    """items: DLTensor (passed as NDArray handle, what the VM does) or int.  Returns (values, tcodes, n, keep)."""
+    """items: DLTensor (passed as NDArray handle, what the VM does), int or None (a null handle).  Returns (values, tcodes, n, keep)."""
     n = len(items)
     vals = (TVMValue * n)()
     codes = (ctypes.c_int * n)()
@@ -71,6 +71,9 @@ def pack(*items):
         if isinstance(it, DLTensor):
             vals[i].v_handle = ctypes.addressof(it)
             codes[i] = kTVMNDArrayHandle
+        elif it is None:
+            vals[i].v_handle = None
+            codes[i] = kTVMNullptr
         else:
             vals[i].v_int64 = int(it)
             codes[i] = kTVMArgInt
