@@ -175,6 +175,48 @@ def bench_intb(torch, ops, K=8192, N=28672, batches=(1, 16, 128, 512), copies=3)
     return res
 
 
+def bench_autogptq(torch, ops, K=4096, N=4096, group=128, batches=(1, 8), copies=40):
+    """An AutoGPTQ layer of the shape the reference's test uses (int4, zero points, group 128), with and
+    without a row order (desc_act); `copies` prepared layers (more than the last-level cache) are cycled
+    inside one captured graph.  Bytes = codes + (scale, zero point) pairs + x + y (+ the gather's traffic)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(12)
+    G = K // group
+    res = {"K": K, "N": N, "group_size": group, "weight": "int4 + zero points", "cases": []}
+    for act in (False, True):
+        layers = []
+        for _ in range(copies):
+            qw = torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device="cuda", generator=g)
+            qz = torch.randint(-2**31, 2**31 - 1, (G, N // 8), dtype=torch.int32, device="cuda", generator=g)
+            sc = (torch.rand((G, N), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+            gi = (torch.arange(K, device="cuda") // group).to(torch.int32)
+            if act:
+                gi = gi[torch.randperm(K, device="cuda", generator=g)].contiguous()
+            layers.append(ops.gptq_prepare(qw, qz, sc, gi))
+        for M in batches:
+            x = torch.randn((M, K), device="cuda", dtype=torch.float16)
+            y = torch.empty((M, N), device="cuda", dtype=torch.float16)
+            ws = torch.empty((max(1, ops.gptq_workspace_bytes(M, K, act)),), dtype=torch.uint8, device="cuda")
+
+            def step():
+                for w in layers:
+                    ops.gptq_linear(w, x, out=y, workspace=ws)
+
+            step()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            graph.replay()
+            ms = _time_on_stream(torch, torch.cuda.current_stream(), graph.replay, 5) / copies
+            nbytes = N * K // 2 + N * G * 4 + M * K * 2 + M * N * 2 + (M * K * 4 + K * 4 if act else 0)
+            res["cases"].append({"M": M, "row_order": act, "us": round(ms * 1e3, 2),
+                                 "GB/s": round(nbytes / ms / 1e6, 1),
+                                 "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)})
+        del layers
+    return res
+
+
 def bench_calibration(torch):
     """What this GPU reaches with no algorithm in the way: a streaming read of 1 GiB and MFMA issue only."""
     import ctypes
@@ -215,6 +257,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of through a HIP graph")
     ap.add_argument("--no-stack", action="store_true", help="skip the 32-layer stack measurement")
     ap.add_argument("--no-intb", action="store_true", help="skip the fpA_intB measurement")
+    ap.add_argument("--no-autogptq", action="store_true", help="skip the AutoGPTQ layer measurement")
     ap.add_argument("--no-calibration", action="store_true", help="skip the pure-read / MFMA-only ceilings")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy a few times (reference point for scaling "
@@ -359,6 +402,8 @@ def main():
         out["stack"] = bench_stack(torch)
     if not args.no_intb:
         out["fpA_intB"] = bench_intb(torch, ops)
+    if not args.no_autogptq:
+        out["autogptq"] = bench_autogptq(torch, ops)
     if not args.no_calibration:
         out["calibration"] = bench_calibration(torch)
 

@@ -23,6 +23,9 @@ def test_all_entry_points_in_one_graph(oracle):
     q8 = u.dev(rng.integers(-127, 128, size=(K, N)).astype(np.int8))
     sc = u.dev(rng.uniform(0.001, 0.01, size=(N,)).astype(np.float16))
     bias = u.dev(rng.standard_normal(N).astype(np.float16))
+    _, qw, qz, gsc, g_idx = oracle.make_gptq_inputs(1, N, K, 128, seed=2, act_order=True)
+    gw = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(gsc), u.dev(g_idx))   # load time: synchronises, not captured
+    gws = torch.empty((300 * K * 2,), dtype=torch.uint8, device="cuda")     # gathered activations
     outs = {}
 
     def work():
@@ -33,6 +36,8 @@ def test_all_entry_points_in_one_graph(oracle):
         outs["P"] = P
         for M in (1, 8, 100, 300):                    # format B: GEMV, small batch, GEMMs
             outs[f"b{M}"] = ops.fpA_intB_gemm(xs[M], P, sc, bias, weight_nbit=8, activation="relu", out=outs.get(f"b{M}"))
+        for M in (1, 8, 100, 300):                    # AutoGPTQ: gather + GEMV, small batch, GEMMs
+            outs[f"c{M}"] = ops.gptq_linear(gw, xs[M], bias=bias, out=outs.get(f"c{M}"), workspace=gws)
 
     # first pass allocates every output (outside the capture) and sets one-time kernel attributes
     work()
@@ -48,15 +53,17 @@ def test_all_entry_points_in_one_graph(oracle):
             work()
     for rep in range(3):
         for k in outs:
-            if k[0] in "ab":
+            if k[0] in "abc":
                 outs[k].zero_()                       # eager work between replays
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         for k in outs:
-            if k[0] in "ab":
+            if k[0] in "abc":
                 assert torch.equal(outs[k], eager[k]), (rep, k)
     # and the eager results are right
     u.assert_close(u.host(eager["a300"]), oracle.q4g32_linear(W, S, u.host(xs[300]), bias=u.host(bias), nthreads=4), "a300")
     u.assert_close(u.host(eager["b100"]),
                    oracle.intb_linear(u.host(xs[100]), u.host(q8), u.host(sc), 8, bias=u.host(bias), activation="relu"), "b100")
+    B = oracle.gptq_dequant(qw, qz, gsc, g_idx)
+    u.assert_close(u.host(eager["c8"]), oracle.nt_matmul_f32acc(np.ascontiguousarray(B.T), u.host(xs[8]), u.host(bias)), "c8")
