@@ -40,7 +40,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # shapes: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one run each) of this script,
 # scaled by what the same counters read for a plain 1 GiB device copy
 # (`--calibrate-copy`): x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28746825
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28747852
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 268700000
 
 
