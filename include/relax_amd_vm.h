@@ -54,7 +54,8 @@ int wq_program_rebind(wq_program_t* p, int reg, void* data);
 
 /* Appends `func(args...)`.  kinds[i] = 1: args[i] is a tensor register, passed as an
  * NDArray handle (type code 13) as the VM does; kinds[i] = 0: args[i] is an integer
- * immediate (type code 0).  Argument order is the PackedFunc's: inputs, then outputs. */
+ * immediate (type code 0); kinds[i] = 2: a null handle (type code 4) for an optional tensor
+ * that is absent.  Argument order is the PackedFunc's: inputs, then outputs. */
 int wq_program_add_call(wq_program_t* p, const char* func, int num_args, const int64_t* args,
                         const int* kinds);
 

@@ -136,8 +136,12 @@ extern "C" int wq_program_add_call(wq_program_t* p, const char* func, int num_ar
       v.v_handle = &p->regs[(size_t)args[i]].dl;
       in.codes.push_back(kTVMNDArrayHandle);
       in.regs.push_back((int)args[i]);
+    } else if (kinds[i] == 2) {  // an absent optional tensor
+      v.v_handle = nullptr;
+      in.codes.push_back(kTVMNullptr);
+      in.regs.push_back(-1);
     } else {
-      WQ_REQUIRE(kinds[i] == 0, "wq_program_add_call(%s): kinds[%d] must be 0 or 1", func, i);
+      WQ_REQUIRE(kinds[i] == 0, "wq_program_add_call(%s): kinds[%d] must be 0, 1 or 2", func, i);
       v.v_int64 = args[i];
       in.codes.push_back(kTVMArgInt);
       in.regs.push_back(-1);

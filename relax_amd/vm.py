@@ -77,11 +77,12 @@ class DpsProgram:
         self._keep.append(t)
 
     # ---- instructions ----
-    def call(self, func: str, *args: Union[Reg, int]) -> None:
-        """``call_dps_packed(func, inputs..., outputs...)``; ``Reg`` arguments are tensors, plain ints immediates."""
+    def call(self, func: str, *args: Union[Reg, int, None]) -> None:
+        """``call_dps_packed(func, inputs..., outputs...)``; ``Reg`` arguments are tensors, plain ints immediates,
+        ``None`` a null handle (an optional tensor that is absent)."""
         n = len(args)
-        vals = (ctypes.c_int64 * max(1, n))(*[int(a) for a in args])
-        kinds = (ctypes.c_int * max(1, n))(*[1 if isinstance(a, Reg) else 0 for a in args])
+        vals = (ctypes.c_int64 * max(1, n))(*[0 if a is None else int(a) for a in args])
+        kinds = (ctypes.c_int * max(1, n))(*[2 if a is None else 1 if isinstance(a, Reg) else 0 for a in args])
         check(self._l.wq_program_add_call(self._p, func.encode(), n, vals, kinds), f"wq_program_add_call({func})")
 
     # ---- memory plan ----

@@ -222,3 +222,45 @@ def test_weight_preparation_program(oracle):
     assert torch.equal(ya, yk)
     q_ref, s_ref = oracle.intb_encode(w, 8)
     u.assert_close(u.host(yb), oracle.intb_linear(x, q_ref, s_ref, 8, bias=bias), "encoded int8")
+
+
+@pytest.mark.gpu
+def test_autogptq_layer_in_a_program(oracle):
+    """An act-order AutoGPTQ layer run by the instruction list: the load-time preparation eagerly (it
+    synchronises), then matmul + add with the gather workspace as a planned tensor, eager and replayed."""
+    import torch
+
+    from relax_amd import ops, vm
+    from tests import gpu_util as u
+
+    M, N, K, gs = 4, 264, 512, 128
+    x, qw, qz, s, g_idx = oracle.make_gptq_inputs(M, N, K, gs, seed=31, act_order=True)
+    res = np.random.default_rng(2).standard_normal((M, N)).astype(np.float16)
+    w = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
+    p = vm.DpsProgram()
+    W, SZ, perm = p.external(w.W_nk, as_uint32=True), p.external(w.SZ), p.external(w.perm)
+    X, R = p.external(u.dev(x)), p.external(u.dev(res))
+    y1 = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    y2 = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    ws = p.planned((ops.gptq_workspace_bytes(M, K, True),), torch.uint8)
+    h = p.planned((M, N))
+    p.call("relax_amd.autogptq_matmul", W, SZ, perm, X, None, h, ws)          # no residual: a null handle
+    p.call("relax_amd.autogptq_matmul", W, SZ, perm, X, R, p.external(y1), ws)
+    ws2 = p.planned((ops.gptq_workspace_bytes(M, K, True),), torch.uint8)
+    p.call("relax_amd.autogptq_matmul", W, SZ, perm, X, h, p.external(y2), ws2)  # residual = the first result
+    assert p.plan() >= M * K * 2 + M * N * 2
+    p.run()
+    torch.cuda.synchronize()
+    B = np.ascontiguousarray(oracle.gptq_dequant(qw, qz, s, g_idx).T)
+    plain = oracle.nt_matmul_f32acc(B, x)
+    u.assert_close(u.host(y1), oracle.nt_matmul_f32acc(B, x, None, res), "autogptq + residual")
+    u.assert_close(u.host(y2), oracle.nt_matmul_f32acc(B, x, None, plain), "autogptq chained")
+    keep = y2.clone()
+    stream = torch.cuda.Stream()
+    p.capture(stream)
+    for _ in range(2):
+        y2.zero_()
+        torch.cuda.synchronize()
+        p.replay(stream)
+        torch.cuda.synchronize()
+        assert torch.equal(y2, keep)
