@@ -241,7 +241,32 @@ def bench_calibration(torch):
 
     mf()
     ms_mfma = _time_on_stream(torch, stream, mf, 3)
-    return {"read_1GiB_GB/s": round(src.numel() / ms_read / 1e6, 1), "hbm_vendor_peak_GB/s": HBM_PEAK_GBS,
+    # the decode GEMV on a matrix large enough that launch, ramp-up and drain no longer matter
+    # (131072 x 4096, 302 MB per copy, three copies cycled): the kernel's steady-state rate
+    del src
+    from relax_amd import ops
+
+    Nl, Kl = 131072, 4096
+    g = torch.Generator(device="cuda")
+    g.manual_seed(13)
+    Wl = [torch.randint(-2**31, 2**31 - 1, (Nl, Kl // 8), dtype=torch.int32, device="cuda", generator=g) for _ in range(3)]
+    Sl = [(torch.rand((Nl, Kl // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16) for _ in range(3)]
+    xl = torch.randn((1, Kl), device="cuda", dtype=torch.float16)
+    yl = torch.empty((1, Nl), device="cuda", dtype=torch.float16)
+    it = [0]
+
+    def big():
+        ops.q4g32_linear(Wl[it[0] % 3], Sl[it[0] % 3], xl, out=yl)
+        it[0] += 1
+
+    for _ in range(3):
+        big()
+    ms_big = _time_on_stream(torch, stream, big, 12)
+    big_bytes = gemv_bytes(1, Nl, Kl)
+    return {"read_1GiB_GB/s": round((1 << 30) / ms_read / 1e6, 1), "hbm_vendor_peak_GB/s": HBM_PEAK_GBS,
+            "gemv_steady_state": {"N": Nl, "K": Kl, "us": round(ms_big * 1e3, 1),
+                                  "GB/s": round(big_bytes / ms_big / 1e6, 1),
+                                  "frac_of_hbm_peak": round(big_bytes / ms_big / 1e6 / HBM_PEAK_GBS, 4)},
             "mfma_f16_only_TFLOP/s": round(flops.value / ms_mfma / 1e9, 1),
             "mfma_f16_vendor_peak_TFLOP/s": MFMA_F16_PEAK_TFLOPS}
 
