@@ -229,11 +229,13 @@ struct GptqLdsPolicy {
   __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
     f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
   }
-  __device__ static half2_t pair(const Frag& f, int kk, int j, const Scale& sc) {
+  __device__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
     const uint32_t word = kk == 0 ? f.w.x : kk == 1 ? f.w.y : kk == 2 ? f.w.z : f.w.w;
-    const uint32_t t = (word >> (8 * j)) & 0xFFu;  // codes 2j, 2j+1
-    const uint32_t u = (t << 12) | t;
-    return (as_half2(and_or(u, 0x000F000Fu, 0x64006400u)) - sc.off) * sc.s2;
+    return q4_pair_bits_natural(word, j);
+  }
+  __device__ static half2_t pair_finish(uint32_t bits, const Scale& sc) { return (as_half2(bits) - sc.off) * sc.s2; }
+  __device__ static half2_t pair(const Frag& f, int kk, int j, const Scale& sc) {
+    return pair_finish(pair_bits(f, kk, j), sc);
   }
 };
 

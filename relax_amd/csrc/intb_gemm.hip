@@ -118,16 +118,20 @@ struct IntbLdsPolicy {
   }
   // int8: piece kk/2 holds 16 k; word j of it holds k = 2j, 2j+1 (bytes 0, 2) and 2j+8, 2j+9 (bytes 1, 3).
   // int4: word j holds k = 2j + 8i, 2j + 8i + 1 in nibbles i, i + 4.
-  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) {
+  __device__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
     if (NBIT == 8) {
       const uint4_t& p = f.w[NBIT == 8 ? (kk >> 1) : 0];
       const uint32_t word = j == 0 ? p.x : j == 1 ? p.y : j == 2 ? p.z : p.w;
-      return u8x2_to_half2(word, (kk & 1) ? 0x04030401u : 0x04020400u) * s2;
+      return __builtin_amdgcn_perm(0x64646464u, word, (kk & 1) ? 0x04030401u : 0x04020400u);  // 1024 + u8
     }
     const uint32_t word = j == 0 ? f.w[0].x : j == 1 ? f.w[0].y : j == 2 ? f.w[0].z : f.w[0].w;
-    const half2_t off = {(half_t)1032.0f, (half_t)1032.0f};
-    return (as_half2(and_or(word >> (4 * kk), 0x000F000Fu, 0x64006400u)) - off) * s2;
+    return and_or(word >> (4 * kk), 0x000F000Fu, 0x64006400u);                                // 1024 + u4
   }
+  __device__ static half2_t pair_finish(uint32_t bits, half2_t s2) {
+    const half_t o = (half_t)(NBIT == 8 ? 1152.0f : 1032.0f);  // 1024 + the bias of the stored codes
+    return (as_half2(bits) - half2_t{o, o}) * s2;
+  }
+  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) { return pair_finish(pair_bits(f, kk, j), s2); }
 };
 
 template <int NBIT>

@@ -36,7 +36,11 @@
 //   read_scale(p, lh)    Scale from the 4 staged bytes of a column, for lane half lh    (kScaleBytes > 0)
 //   const_scale(args, n) the Scale of column n                                          (kScaleBytes == 0)
 //   read(frag, bslot, n_local, lh)   LDS -> registers
-//   pair(frag, kk, j, scale)   dequantized weights (k = 8kk + 2j, 8kk + 2j + 1) of the lane's column
+//   pair(frag, kk, j, scale)   dequantized weights (k = 8kk + 2j, 8kk + 2j + 1) of the lane's column,
+//                              = pair_finish(pair_bits(frag, kk, j), scale): the two exact fp16 integers
+//                              as a bit pattern, then (integer - offset) * scale.  The K loop runs the two
+//                              halves in different MFMA slots: a chain of four dependent VALU operations
+//                              does not fit behind one MFMA, two do.
 #ifndef RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 #define RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 
@@ -224,6 +228,8 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       const int cur = kk & 1, nxt = cur ^ 1;
+      const unsigned char* const a_from = kk == 3 ? next_slot : slot;  // activation fragments of the next phase
+      const int a_kk = kk == 3 ? 0 : kk + 1;
       if (kk == 3) {
         // loads of step ks+1 landed (those of ks+2 may be in flight), own LDS reads done
         if (ahead2) {
@@ -233,28 +239,29 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
         }
         __builtin_amdgcn_s_barrier();
         read_b(next_slot);
-        read_a(next_slot, 0, aop[nxt]);
-      } else {
-        read_a(slot, kk + 1, aop[nxt]);
       }
       half2_t dq[TN][4];
+      uint32_t pb[NPAIR];
+      // Slots of the unpacking: the bit patterns in the first half of the usable slots, the
+      // arithmetic in the second half; in phase 3 the packed weights were requested from LDS
+      // just above, so the first slots stay free.
+      const int first = kk < 3 ? 0 : NSLOT * 3 / 8, usable = NSLOT - first, half = usable / 2;
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int sl = 0; sl < NSLOT; ++sl) {
         const int i = sl / TN, t = sl % TN;
         acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[cur][i], bop[cur][t], acc[i][t], 0, 0, 0);
-        // unpack the weight pairs of the next phase; in phase 3 (operands just requested
-        // from LDS) only in the second half of the slots
-        {
-          const int first = kk < 3 ? 0 : NSLOT / 2, span = NSLOT - first;
-          if (sl >= first) {
-            const int p0 = (sl - first) * NPAIR / span, p1 = (sl - first + 1) * NPAIR / span;
+        // one activation fragment of the next phase per slot
+        if (sl < TME) {
+          const int row = (wm * TME + sl) * 32 + lj;
+          aop[nxt][sl] = *reinterpret_cast<const half8_t*>(a_from + Cfg::kAOff + row * 128 +
+                                                           (((4 * lh + a_kk) ^ WQ_SWZ(row)) << 4));
+        }
 #pragma unroll
-            for (int p = p0; p < p1; ++p) {
-              const int tt = p >> 2, j = p & 3;
-              dq[tt][j] = Policy::pair(bw[tt], (kk + 1) & 3, j, bs[tt]);
-            }
-          }
+        for (int p = 0; p < NPAIR; ++p) {
+          const int tt = p >> 2, j = p & 3;
+          if (sl == first + p * half / NPAIR) pb[p] = Policy::pair_bits(bw[tt], (kk + 1) & 3, j);
+          if (sl == first + half + p * (usable - half) / NPAIR) dq[tt][j] = Policy::pair_finish(pb[p], bs[tt]);
         }
         // direct loads: the second part of step ks+2 in phase 0; the first part of step
         // ks+3 in phase 3, into the slot of this step, which nobody reads any more

@@ -83,10 +83,15 @@ struct Q4G32LdsPolicy {
   __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
     f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
   }
-  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) {
+  __device__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
     const uint32_t word = kk == 0 ? f.w.x : kk == 1 ? f.w.y : kk == 2 ? f.w.z : f.w.w;
-    return q4_pair_dequant_natural(word, j, s2);
+    return q4_pair_bits_natural(word, j);
   }
+  __device__ static half2_t pair_finish(uint32_t bits, half2_t s2) {
+    const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+    return (as_half2(bits) - off) * s2;
+  }
+  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) { return pair_finish(pair_bits(f, kk, j), s2); }
 };
 
 }  // namespace wq

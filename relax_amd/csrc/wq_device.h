@@ -71,12 +71,16 @@ __device__ __forceinline__ void q4_word_dequant_natural(uint32_t w, half2_t s2, 
   }
 }
 
-// One pair of the above: (w_{2j}, w_{2j+1}).
-__device__ __forceinline__ half2_t q4_pair_dequant_natural(uint32_t w, int j, half2_t s2) {
-  const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+// One pair of the above, in two steps: the fp16 bit pattern (1024 + code_{2j}, 1024 + code_{2j+1}) ...
+__device__ __forceinline__ uint32_t q4_pair_bits_natural(uint32_t w, int j) {
   const uint32_t t = (w >> (8 * j)) & 0xFFu;
   const uint32_t u = (t << 12) | t;
-  return (as_half2(and_or(u, 0x000F000Fu, 0x64006400u)) - off) * s2;
+  return and_or(u, 0x000F000Fu, 0x64006400u);
+}
+// ... and (w_{2j}, w_{2j+1}) from it.
+__device__ __forceinline__ half2_t q4_pair_dequant_natural(uint32_t w, int j, half2_t s2) {
+  const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+  return (as_half2(q4_pair_bits_natural(w, j)) - off) * s2;
 }
 
 // fp32 += a.x*b.x + a.y*b.y with exact fp16 products (v_dot2_f32_f16).
