@@ -48,3 +48,23 @@ def test_host_preprocess_errors(ops):
         ops.ft_preprocess_weight(a.to(torch.int32), 80, False)
     # empty tensors pass through
     assert ops.ft_preprocess_weight(torch.zeros((0, 64), dtype=torch.int8), 80, False).shape == (0, 64)
+
+
+def test_gptq_host_side_checks(ops):
+    """What the AutoGPTQ entry points decide on the host, before any kernel: workspace sizes, shape and
+    pointer checks (null device pointers are never dereferenced: every call below fails its checks first)."""
+    from relax_amd import _lib
+
+    l = _lib.lib()
+    assert ops.gptq_workspace_bytes(1, 4096, True) == 8192
+    assert ops.gptq_workspace_bytes(300, 4096, True) == 300 * 4096 * 2
+    assert ops.gptq_workspace_bytes(300, 4096, False) == 0 and ops.gptq_workspace_bytes(0, 4096, True) == 0
+    # empty problems succeed without touching memory
+    assert l.wq_gptq_linear(0, 0, 0, 0, 0, 0, 0, 0, 64, 256, 2, 0, 0, 0) == 0
+    assert l.wq_gptq_dequantize(0, 0, 0, 0, 0, 0, 64, 2, 0) == 0
+    # K not a multiple of the group count / group size not a multiple of 32 / null pointers
+    assert l.wq_gptq_linear(0, 0, 0, 0, 0, 0, 0, 1, 64, 256, 3, 0, 0, 0) != 0 and b"groups" in l.wq_last_error()
+    assert l.wq_gptq_linear(0, 0, 0, 0, 0, 0, 0, 1, 64, 192, 4, 0, 0, 0) != 0 and b"multiple of 32" in l.wq_last_error()
+    assert l.wq_gptq_linear(0, 0, 0, 0, 0, 0, 0, 1, 64, 256, 2, 0, 0, 0) != 0 and b"null pointer" in l.wq_last_error()
+    assert l.wq_gptq_dequantize(0, 0, 0, 0, 0, 12, 64, 1, 0) != 0 and b"multiples of 8" in l.wq_last_error()
+    assert l.wq_gptq_prepare(0, 0, 0, 0, 0, 0, 0, 0, None, 256, 60, 2, 0) != 0 and b"multiple of 8" in l.wq_last_error()
