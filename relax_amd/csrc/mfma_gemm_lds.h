@@ -92,19 +92,18 @@ typedef void __attribute__((address_space(3))) * wq_lptr_t;
 // Schedule of one K-step (four phases kk = 0..3 of TME*TN MFMAs each).  Nothing but
 // MFMAs may sit on the critical path of a wavefront that has its SIMD to itself, so
 // every other instruction is slotted between them:
-//   phases 0-2  after each MFMA the unpacking of one weight pair of phase kk+1; at the
-//               phase start the LDS reads of the activation fragments of phase kk+1; in
-//               phase 0 also the second half of the direct loads of step ks+2 (direct loads
-//               are slotted between MFMAs because the texture path accepts 64 B per cycle
+//   phases 0-2  per MFMA slot one LDS read of an activation fragment of phase kk+1 (the first
+//               TME slots) and one half of the unpacking of a weight pair of phase kk+1 (bit
+//               pattern in an early slot, arithmetic in a later one); in phase 0 also all direct
+//               loads of step ks+2, one every few slots (the texture path accepts 64 B per cycle
 //               and CU: issued in a burst they block the wavefront for hundreds of cycles);
 //   phase 3     first s_waitcnt vmcnt (this wavefront's loads of step ks+1 have landed)
 //               and s_barrier (everyone's have); then, between its MFMAs, the packed
 //               weights, the first activation fragments and the first weight pairs of
-//               step ks+1, so that step ks+1 starts multiplying at once, and the first half
-//               of the direct loads of step ks+3 (into the slot of step ks, free by now).
-// One barrier per K-step suffices: slot ks%3 is refilled by loads issued after the barrier
-// of step ks, and every wavefront has waited for its last LDS reads of that slot (the
-// phase-3 fragments) before that barrier.
+//               step ks+1, so that step ks+1 starts multiplying at once.
+// One barrier per K-step suffices: slot (ks+2)%3 = (ks-1)%3 is refilled by loads issued after
+// the barrier of step ks-1, and every wavefront has waited for its last LDS reads of that slot
+// (the phase-3 fragments of step ks-1) before that barrier.
 template <class Policy, class Epilogue, int TM, int TN, int WM, int WN, int TME>
 __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs,
                                               const half_t* __restrict__ X, half_t* __restrict__ Y,
@@ -115,8 +114,6 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
   constexpr int L = kALoadsE + Cfg::kBLoads + Cfg::kSLoads;  // direct loads per wavefront per step
   constexpr int NSLOT = TME * TN;                    // MFMAs per phase
   constexpr int NPAIR = TN * 4;                      // weight pairs to unpack per phase
-  constexpr int LA = L / 2;                          // loads of a step issued in phase 3 (three steps ahead) ...
-  constexpr int LB = L - LA;                         // ... and in phase 0 of the following step
   static_assert(kALoadsE >= 1, "tile too small to split further");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -191,18 +188,14 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
     }
   };
 
-  // ---- prologue: steps 0 and 1 and the first part of step 2 in flight, operands of step 0 ready ----
+  // ---- prologue: steps 0 and 1 in flight, operands of step 0 ready ----
 #pragma unroll
   for (int idx = 0; idx < L; ++idx) issue_one(0, idx);
   if (ksteps > 1) {
 #pragma unroll
     for (int idx = 0; idx < L; ++idx) issue_one(1, idx);
   }
-  if (ksteps > 2) {
-#pragma unroll
-    for (int idx = 0; idx < LA; ++idx) issue_one(2, idx);
-    WQ_WAITCNT_VM(L + LA);
-  } else if (ksteps > 1) {
+  if (ksteps > 1) {
     WQ_WAITCNT_VM(L);
   } else {
     WQ_WAITCNT_VM(0);
@@ -224,7 +217,7 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
   for (int ks = 0; ks < ksteps; ++ks) {
     const unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
     const unsigned char* next_slot = lds + ((ks + 1) % Cfg::kStages) * Cfg::kStageBytes;
-    const bool ahead2 = ks + 2 < ksteps, ahead3 = ks + 3 < ksteps;
+    const bool ahead2 = ks + 2 < ksteps;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       const int cur = kk & 1, nxt = cur ^ 1;
@@ -263,17 +256,13 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
           if (sl == first + p * half / NPAIR) pb[p] = Policy::pair_bits(bw[tt], (kk + 1) & 3, j);
           if (sl == first + half + p * (usable - half) / NPAIR) dq[tt][j] = Policy::pair_finish(pb[p], bs[tt]);
         }
-        // direct loads: the second part of step ks+2 in phase 0; the first part of step
-        // ks+3 in phase 3, into the slot of this step, which nobody reads any more
+        // direct loads of step ks+2, all in phase 0 (into the slot of step ks-1, free since the
+        // barrier of its phase 3): timed on the GPU, one phase with loads and three without beat
+        // the same loads spread over two phases (by 1-2 %) or over all four (by 15 %)
         if (kk == 0 && ahead2) {
-          const int l0 = LA + sl * LB / NSLOT, l1 = LA + (sl + 1) * LB / NSLOT;
+          const int l0 = sl * L / NSLOT, l1 = (sl + 1) * L / NSLOT;
 #pragma unroll
           for (int idx = l0; idx < l1; ++idx) issue_one(ks + 2, idx);
-        }
-        if (kk == 3 && ahead3) {
-          const int l0 = sl * LA / NSLOT, l1 = (sl + 1) * LA / NSLOT;
-#pragma unroll
-          for (int idx = l0; idx < l1; ++idx) issue_one(ks + 3, idx);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
