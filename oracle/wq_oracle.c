@@ -234,7 +234,9 @@ void wqo_q4g32_linear(const uint32_t* W, const uint16_t* S, const uint16_t* X,
                       const uint16_t* bias, const uint16_t* residual, uint16_t* Y, int64_t M,
                       int64_t N, int64_t K, int nthreads) {
   uint16_t* B = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)(N * K));
-  wqo_q4g32_dequant(W, S, B, N, K);
+  /* the decode pass row by row (rows are independent: same values with any thread count) */
+#pragma omp parallel for num_threads(nthreads > 0 ? nthreads : 1) schedule(static)
+  for (int64_t n = 0; n < N; ++n) wqo_q4g32_dequant(W + n * (K / 8), S + n * (K / 32), B + n * K, 1, K);
   wqo_nt_matmul_f32acc(B, X, bias, residual, Y, M, N, K, nthreads);
   free(B);
 }
