@@ -268,9 +268,13 @@ static int launch_skinny_auto(const char* who, const typename Policy::Args& parg
   const int64_t per_cu = (N / 16) / cu_count();
   int nw = 1;
   if (per_cu >= 2) nw = M <= 8 ? (per_cu >= 4 ? 2 : 1) : M <= 16 ? 2 : 4;
+  // wide matrices and more than 16 rows: all eight wavefronts side by side (128 columns per
+  // workgroup, each wavefront the whole K), which halves the re-reads of x again, as long as
+  // most CUs still get a workgroup (int8, K = 8192, N = 28672, M = 64: 80 -> 62 us)
+  if (M > 16 && N / 128 >= (cu_count() * 5) / 8) nw = 8;
   if (t.nw) nw = t.nw;
-  if (M <= 8 && nw == 4) nw = 2;  // 8 rows are two slab loads: at most two wavefronts share them
-  const int stages = t.stages ? t.stages : (nw == 4 ? 3 : 2);
+  if (M <= 8 && nw >= 4) nw = 2;  // 8 rows are two slab loads: at most two wavefronts share them
+  const int stages = t.stages ? t.stages : (nw >= 4 ? 3 : 2);
   // eight wavefronts where two ring slots of that arrangement fit LDS, else four
 #define WQ_SK_GO(TH, NW, WAVES)                                                                        \
   do {                                                                                                 \
@@ -285,16 +289,18 @@ static int launch_skinny_auto(const char* who, const typename Policy::Args& parg
     if (nw == 2) WQ_SK_GO(1, 2, 8);
     WQ_SK_GO(1, 1, 8);
   }
-  if (M <= 16) {
+  if (M <= 16 && nw != 8) {
     if (nw == 4) WQ_SK_GO(2, 4, 8);
     if (nw == 2) WQ_SK_GO(2, 2, 8);
     WQ_SK_GO(2, 1, 8);
   }
   if (M <= 32) {
+    if (nw == 8) WQ_SK_GO(4, 8, 8);
     if (nw == 4) WQ_SK_GO(4, 4, 8);
     if (nw == 2) WQ_SK_GO(4, 2, 8);
     WQ_SK_GO(4, 1, 8);
   }
+  if (nw == 8) WQ_SK_GO(8, 8, 8);
   if (nw == 4) WQ_SK_GO(8, 4, 8);
   if (nw == 2) WQ_SK_GO(8, 2, 8);
   WQ_SK_GO(8, 1, 8);

@@ -126,7 +126,7 @@ def test_gemm_epilogues(ops, u, oracle, nbit, M, ep):
     _run(ops, u, oracle, M, 128, 256, nbit, seed=M + 3, **ep)
 
 
-@pytest.mark.parametrize("nw,stages", [(1, 2), (2, 3), (4, 4), (0, 0)])
+@pytest.mark.parametrize("nw,stages", [(1, 2), (2, 3), (4, 4), (8, 3), (0, 0)])
 @pytest.mark.parametrize("nbit", [8, 4])
 @pytest.mark.parametrize("group_size", [-1, 64])
 def test_small_batch_work_splits(ops, u, oracle, nbit, group_size, nw, stages):

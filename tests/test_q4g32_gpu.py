@@ -182,7 +182,7 @@ SMALL_BATCH = [  # (M, N, K): ragged M and N, K/64 not a multiple of the wavefro
 ]
 
 
-@pytest.mark.parametrize("nw,waves,stages", [(1, 0, 2), (2, 0, 3), (4, 0, 5), (1, 0, 3), (2, 0, 2), (4, 0, 4), (0, 0, 0)])
+@pytest.mark.parametrize("nw,waves,stages", [(1, 0, 2), (2, 0, 3), (4, 0, 5), (1, 0, 3), (2, 0, 2), (4, 0, 4), (8, 0, 3), (8, 0, 2), (0, 0, 0)])
 @pytest.mark.parametrize("M,N,K", SMALL_BATCH)
 def test_small_batch_vs_oracle(ops, u, oracle, nw, waves, stages, M, N, K):
     """the matrix-core kernel for 2 <= M <= 64, in each of its work splits (0 = automatic)."""
