@@ -270,15 +270,18 @@ def bench_calibration(torch):
     Sl = [(torch.rand((Nl, Kl // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16) for _ in range(3)]
     xl = torch.randn((1, Kl), device="cuda", dtype=torch.float16)
     yl = torch.empty((1, Nl), device="cuda", dtype=torch.float16)
-    it = [0]
 
     def big():
-        ops.q4g32_linear(Wl[it[0] % 3], Sl[it[0] % 3], xl, out=yl)
-        it[0] += 1
+        for i in range(3):
+            ops.q4g32_linear(Wl[i], Sl[i], xl, out=yl)
 
-    for _ in range(3):
+    big()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
         big()
-    ms_big = _time_on_stream(torch, stream, big, 12)
+    graph.replay()
+    ms_big = _time_on_stream(torch, torch.cuda.current_stream(), graph.replay, 6) / 3
     big_bytes = gemv_bytes(1, Nl, Kl)
     return {"read_1GiB_GB/s": round((1 << 30) / ms_read / 1e6, 1), "hbm_vendor_peak_GB/s": HBM_PEAK_GBS,
             "gemv_steady_state": {"N": Nl, "K": Kl, "us": round(ms_big * 1e3, 1),
