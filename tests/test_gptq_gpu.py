@@ -117,6 +117,9 @@ LINEAR_CASES = [  # (M, N, K, group size, act_order)
     (512, 2048, 4096, 128, True),
     (700, 1024, 1024, 256, False),
     (20, 136, 288, 96, True),      # large M, group size not a multiple of 64: streaming kernel repeated
+    (1, 72, 32768, 128, True),     # the longest supported row: 64 KB of activations staged / gathered through LDS
+    (3, 72, 32768, 256, True),
+    (70, 136, 32768, 2048, True),
 ]
 
 
