@@ -159,32 +159,33 @@ def bench_stack(torch, layers=32, batches=(1, 8, 32), reps=20):
     return res
 
 
-def bench_intb(torch, ops, K=8192, N=28672, batches=(1, 16, 128, 512), copies=3):
-    """fp16 x int8 per-channel weights in the preprocessed layout; `copies` weight copies
-    (more than the last-level cache) are cycled so that small M reads HBM."""
+def bench_intb(torch, ops, K=8192, N=28672, batches=(1, 16, 128, 512), copies=3, nbit=8, group=-1):
+    """fp16 x int8 per-channel weights in the preprocessed layout (or, for the neighbouring schemes,
+    int4 and / or group-64 scales); `copies` weight copies (more than the last-level cache) are cycled so
+    that small M reads HBM."""
     g = torch.Generator(device="cuda")
     g.manual_seed(11)
     Ws = []
     for _ in range(copies):
-        q = torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda", generator=g)
-        Ws.append(ops.ft_preprocess_weight(q, 80, False))
+        q = torch.randint(-127, 128, (K, N if nbit == 8 else N // 2), dtype=torch.int8, device="cuda", generator=g)
+        Ws.append(ops.ft_preprocess_weight(q, 80, nbit == 4))
         del q
-    s = (torch.rand((N,), device="cuda", generator=g) * 0.009 + 0.001).to(torch.float16)
+    s = (torch.rand((N,) if group <= 0 else (K // group, N), device="cuda", generator=g) * 0.009 + 0.001).to(torch.float16)
     stream = torch.cuda.current_stream()
-    res = {"K": K, "N": N, "weight": "int8 per-channel", "batches": []}
+    res = {"K": K, "N": N, "weight": f"int{nbit} " + ("per-channel" if group <= 0 else f"group-{group}"), "batches": []}
     for M in batches:
         x = torch.randn((M, K), device="cuda", dtype=torch.float16)
         y = torch.empty((M, N), device="cuda", dtype=torch.float16)
         it = [0]
 
         def fn():
-            ops.fpA_intB_gemm(x, Ws[it[0] % copies], s, weight_nbit=8, out=y)
+            ops.fpA_intB_gemm(x, Ws[it[0] % copies], s, weight_nbit=nbit, group_size=group, out=y)
             it[0] += 1
 
         for _ in range(copies):
             fn()
         ms = _time_on_stream(torch, stream, fn, 4 * copies)
-        nbytes = K * N + N * 2 + M * K * 2 + M * N * 2
+        nbytes = K * N * nbit // 8 + s.numel() * 2 + M * K * 2 + M * N * 2
         tf = 2.0 * M * N * K / ms / 1e9
         res["batches"].append({"M": M, "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
                                "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
@@ -447,6 +448,11 @@ def main():
         out["stack"] = bench_stack(torch)
     if not args.no_intb:
         out["fpA_intB"] = bench_intb(torch, ops)
+        torch.cuda.empty_cache()
+        # the neighbouring schemes of the same entry point, two batch sizes each
+        out["fpA_intB_variants"] = [bench_intb(torch, ops, batches=(1, 128), copies=4, nbit=4),
+                                    bench_intb(torch, ops, batches=(1, 128), copies=3, nbit=8, group=64)]
+        torch.cuda.empty_cache()
     if not args.no_autogptq:
         out["autogptq"] = bench_autogptq(torch, ops)
     if not args.no_calibration:
