@@ -82,15 +82,18 @@ struct IntbLoader {
 // with per-column scales.  A K-step (one 64-row tile) of I = 2 (int8) or 4 (int4) interleaved
 // columns is 128 contiguous bytes, so the B tile is fetched in whole 128-byte lines; the scale
 // of a column never changes and stays in a register.
-template <int NBIT>
+// GROUPED (scales fp16 [K/64, N], one per column and K-step): a lane stages the 4 bytes that hold
+// the scales of its column and the neighbouring one, and the reader takes its half.
+template <int NBIT, bool GROUPED = false>
 struct IntbLdsPolicy {
   static constexpr int I = NBIT == 8 ? 2 : 4;
   static constexpr int kColBytes = 128 / I;
-  static constexpr int kScaleBytes = 0;
+  static constexpr int kScaleBytes = GROUPED ? 4 : 0;
   static constexpr int kStepStride = 128;
   struct Args {
     const uint4_t* B;
     const half_t* scales;
+    int N;
   };
   struct Frag {
     uint4_t w[NBIT == 8 ? 2 : 1];
@@ -100,9 +103,17 @@ struct IntbLdsPolicy {
     return reinterpret_cast<const char*>(a.B) + ((int64_t)group * (K >> 6)) * 128 + (q & 7) * 16;
   }
   using Scale = half2_t;  // the column's scale, twice
-  __device__ static const char* s_src(const Args&, int, int) { return nullptr; }
-  __device__ static int64_t s_offset(const Args&, int) { return 0; }
-  __device__ static Scale read_scale(const unsigned char*, int) { return Scale{}; }
+  __device__ static const char* s_src(const Args& a, int n, int) {
+    return reinterpret_cast<const char*>(a.scales + (n & ~1));  // the aligned pair of columns (N is even)
+  }
+  __device__ static int64_t s_offset(const Args& a, int ks) { return (int64_t)ks * a.N * 2; }
+  // p = the 4 staged bytes of the lane's column; columns are staged 4 bytes apart from an 8-byte
+  // aligned base, so bit 2 of the address is the parity of the column
+  __device__ static Scale read_scale(const unsigned char* p, int) {
+    const half2_t pair = *reinterpret_cast<const half2_t*>(p);
+    const half_t s = (reinterpret_cast<uintptr_t>(p) & 4) ? pair.y : pair.x;
+    return Scale{s, s};
+  }
   __device__ static Scale const_scale(const Args& a, int n) {
     const half_t s = a.scales[n];
     return Scale{s, s};
@@ -134,12 +145,12 @@ struct IntbLdsPolicy {
   __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) { return pair_finish(pair_bits(f, kk, j), s2); }
 };
 
-template <int NBIT>
+template <int NBIT, bool GROUPED>
 static int intb_gemm_lds(int cfg, const char* who, const int8_t* B, const uint16_t* scales, const uint16_t* A,
                          uint16_t* C, const IntbGemmEpilogue& gep, int64_t m, int64_t n, int64_t k,
                          hipStream_t stream) {
-  using P = IntbLdsPolicy<NBIT>;
-  const typename P::Args largs{(const uint4_t*)B, (const half_t*)scales};
+  using P = IntbLdsPolicy<NBIT, GROUPED>;
+  const typename P::Args largs{(const uint4_t*)B, (const half_t*)scales, (int)n};
   switch (cfg) {
     case 11: return launch_gemm_lds<P, IntbGemmEpilogue, 8, 2, 1, 4, 1>(who, largs, A, C, gep, m, n, k, stream);
     case 12: return launch_gemm_lds<P, IntbGemmEpilogue, 4, 2, 1, 4, 2>(who, largs, A, C, gep, m, n, k, stream);
@@ -182,17 +193,22 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
       return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
   }
   const IntbGemmEpilogue gep{ep, (int)n};
-  // per-column scales: the fully LDS-staged kernel (11, 12, 17) except between M = 320 and 1536,
-  // where the 128x256 register-staged tiles fill the CUs better (timings at K = 8192, N = 28672);
-  // fine-grained scales: the register-staged kernel (1..4)
+  // the fully LDS-staged kernel (11, 12, 17) except between M = 320 and 1536, where the 128x256
+  // register-staged tiles fill the CUs better (timings at K = 8192, N = 28672); fine-grained
+  // scales whose pairs are not 4-byte aligned: the register-staged kernel (1..4)
+  const bool lds_ok = !group || (reinterpret_cast<uintptr_t>(scales) & 3u) == 0;
   int cfg = wq_gemm_cfg_override();
-  if (!cfg) cfg = group ? choose_gemm_cfg(m, n, false) : (m <= 320 ? 17 : m <= 1536 ? 2 : 11);
+  if (!cfg) cfg = !lds_ok ? choose_gemm_cfg(m, n, false) : (m <= 320 ? 17 : m <= 1536 ? 2 : 11);
   // silu / gelu run the element-wise epilogue, whose inlined exp / erf code does not fit next to
   // the 256 accumulator registers of the 256x256 tile: stay with 128-row tiles
   if (!wq_gemm_cfg_override() && activation >= WQ_ACT_SILU && cfg == 11) cfg = 2;
-  if (cfg >= 11 && !group)
-    return nbit == 8 ? intb_gemm_lds<8>(cfg, who, B, scales, A, C, gep, m, n, k, stream)
-                     : intb_gemm_lds<4>(cfg, who, B, scales, A, C, gep, m, n, k, stream);
+  if (cfg >= 11 && lds_ok) {
+    if (group)
+      return nbit == 8 ? intb_gemm_lds<8, true>(cfg, who, B, scales, A, C, gep, m, n, k, stream)
+                       : intb_gemm_lds<4, true>(cfg, who, B, scales, A, C, gep, m, n, k, stream);
+    return nbit == 8 ? intb_gemm_lds<8, false>(cfg, who, B, scales, A, C, gep, m, n, k, stream)
+                     : intb_gemm_lds<4, false>(cfg, who, B, scales, A, C, gep, m, n, k, stream);
+  }
   if (cfg >= 11) cfg = cfg == 17 ? 4 : cfg == 11 ? 1 : 2;
   if (nbit == 8) {
     const IntbLoader<8>::Args bargs{(const uint4_t*)B, (const half_t*)scales, group};

@@ -159,6 +159,11 @@ def test_gemm_tile_configurations(ops, u, oracle, nbit, cfg):
         _run(ops, u, oracle, 100, 128, 256, nbit, seed=cfg, bias="row", activation="gelu", residual=True,
              binary_op="multiply", unary_op="relu")
         _run(ops, u, oracle, 100, 128, 256, nbit, seed=cfg + 1, bias="full")
+        # fine-grained (group-64) scales through the same tiles
+        for M, N, K in [(70, 64, 64), (130, 320, 448), (300, 576, 512)]:
+            print(f"intb cfg={cfg} nbit={nbit} g=64 M={M} N={N} K={K}", flush=True)
+            _run(ops, u, oracle, M, N, K, nbit, seed=M + cfg + 1, group_size=64)
+        _run(ops, u, oracle, 100, 128, 256, nbit, seed=cfg + 2, group_size=64, bias="row", activation="relu")
     finally:
         _lib.lib().wq_debug_set_gemm_config(0)
 
