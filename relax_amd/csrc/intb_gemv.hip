@@ -147,6 +147,10 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
     for (int m = 0; m < MB; ++m) acc[r][m] = 0.0f;
 
   const uint32_t magic = 0x64006400u;
+  // fine-grained scales [K/64, N]: the R*I columns of this wavefront are adjacent, so one 8-byte
+  // (int8) or 16-byte (int4) load per tile fetches the scales of all of them (gset is a multiple of
+  // R and N / I of 16: the load stays inside the row); needs 16-byte aligned scales
+  const bool vec_scales = group > 0 && (reinterpret_cast<uintptr_t>(scales) & 15u) == 0;
   for (int p0 = 0; p0 < pieces; p0 += 64 * U) {
     uint4_t wv[R][U];
 #pragma unroll
@@ -156,6 +160,21 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
       for (int u = 0; u < U; ++u) {
         const int p = min(p0 + 64 * u + lane, pieces - 1);
         wv[r][u] = __builtin_nontemporal_load(&src[p]);
+      }
+    }
+    uint4_t sv[U];
+    if (vec_scales) {
+      static_assert(R * I * 2 == 8 || R * I * 2 == 16, "scale vector of 8 or 16 bytes");
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int tile_u = min(p0 + 64 * u + lane, pieces - 1) >> 3;
+        const half_t* sp = scales + (int64_t)tile_u * N + gset * I;
+        if (R * I * 2 == 16) {
+          sv[u] = *reinterpret_cast<const uint4_t*>(sp);
+        } else {
+          const uint2_t t = *reinterpret_cast<const uint2_t*>(sp);
+          sv[u] = uint4_t{t.x, t.y, 0u, 0u};
+        }
       }
     }
 #pragma unroll
@@ -231,7 +250,13 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         float sf = ok ? 1.0f : 0.0f;
-        if (group > 0) {
+        if (vec_scales) {
+          // half (r * I + col_in_group) of the vector
+          const int h = r * I + col_in_group;
+          const uint32_t word = (h >> 1) == 0 ? sv[u].x : (h >> 1) == 1 ? sv[u].y : (h >> 1) == 2 ? sv[u].z : sv[u].w;
+          const half2_t pair = as_half2(word);
+          sf = ok ? (float)((h & 1) ? pair.y : pair.x) : 0.0f;
+        } else if (group > 0) {
           const int n = min(gset + r, ngroups - 1) * I + col_in_group;
           sf = ok ? (float)scales[(int64_t)tile * N + n] : 0.0f;
         }

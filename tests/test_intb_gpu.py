@@ -226,3 +226,24 @@ def test_argument_errors(ops, u, oracle):
         ops.fpA_intB_gemm(u.dev(x[:, :32].copy()), P, u.dev(s), weight_nbit=8)
     with pytest.raises(ValueError):
         ops.fpA_intB_gemm(u.dev(x), P, u.dev(s[:10].copy()), weight_nbit=8)
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_grouped_gemv_with_scales_at_any_alignment(ops, u, oracle, nbit):
+    """group-64 scales: the streaming kernel fetches them as 8- or 16-byte vectors when the buffer is
+    16-byte aligned and one by one otherwise; both must give the same result."""
+    import torch
+
+    M, N, K = 2, 192, 512
+    x, A, s = oracle.make_intb_inputs(M, N, K, nbit, seed=5, group_size=64)
+    P = ops.ft_preprocess_weight(u.dev(A), 80, nbit == 4)
+    ref = oracle.intb_linear(x, A, s, nbit, group_size=64)
+    aligned = u.dev(s)
+    backing = torch.empty(s.size + 2, dtype=torch.float16, device="cuda")
+    shifted = backing[2:].view(s.shape)  # 4 bytes past a 16-byte boundary
+    shifted.copy_(aligned)
+    assert aligned.data_ptr() % 16 == 0 and shifted.data_ptr() % 16 == 4
+    got_a = ops.fpA_intB_gemm(u.dev(x), P, aligned, weight_nbit=nbit, group_size=64)
+    got_s = ops.fpA_intB_gemm(u.dev(x), P, shifted, weight_nbit=nbit, group_size=64)
+    assert torch.equal(got_a, got_s)
+    u.assert_close(u.host(got_a), ref, f"grouped gemv int{nbit}")
