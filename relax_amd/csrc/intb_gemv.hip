@@ -150,7 +150,8 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
   // fine-grained scales [K/64, N]: the R*I columns of this wavefront are adjacent, so one 8-byte
   // (int8) or 16-byte (int4) load per tile fetches the scales of all of them (gset is a multiple of
   // R and N / I of 16: the load stays inside the row); needs 16-byte aligned scales
-  const bool vec_scales = group > 0 && (reinterpret_cast<uintptr_t>(scales) & 15u) == 0;
+  constexpr bool kVecFits = R * I * 2 == 8 || R * I * 2 == 16;
+  const bool vec_scales = kVecFits && group > 0 && (reinterpret_cast<uintptr_t>(scales) & 15u) == 0;
   for (int p0 = 0; p0 < pieces; p0 += 64 * U) {
     uint4_t wv[R][U];
 #pragma unroll
@@ -164,7 +165,6 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
     }
     uint4_t sv[U];
     if (vec_scales) {
-      static_assert(R * I * 2 == 8 || R * I * 2 == 16, "scale vector of 8 or 16 bytes");
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int tile_u = min(p0 + 64 * u + lane, pieces - 1) >> 3;
