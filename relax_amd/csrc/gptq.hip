@@ -164,6 +164,8 @@ struct GptqSkinnyPolicy {
     const uint32_t g32 = (uint32_t)k0 >> 5;
     return l.sz + (l.ratio == 1 ? g32 : __umulhi(g32, l.inv)) * 4;
   }
+  __device__ static const char* s_pair_addr(const Lane& l, int k0) { return s_addr(l, k0); }
+  static bool pair_aligned(const Args&) { return true; }
   __device__ static Scale pick_scale(const Lane&, half2_t pair, int) { return pair; }
   __device__ static Scale const_scale(const Lane&) { return Scale{}; }
   __device__ static Scale null_scale() { return Scale{(half_t)0.0f, (half_t)0.0f}; }

@@ -39,6 +39,11 @@ struct IntbSkinnyPolicy {
   __device__ static const char* s_addr(const Lane& l, int k0) {
     return reinterpret_cast<const char*>(l.s + (int64_t)(k0 >> 6) * l.N);
   }
+  __device__ static const char* s_pair_addr(const Lane& l, int k0) {
+    if (GROUPED) return s_addr(l, k0);
+    return reinterpret_cast<const char*>(reinterpret_cast<uintptr_t>(l.s) & ~(uintptr_t)3);  // &scales[n & ~1]
+  }
+  static bool pair_aligned(const Args& a) { return (reinterpret_cast<uintptr_t>(a.scales) & 3u) == 0; }
   __device__ static half_t pick_scale(const Lane& l, half2_t pair, int) { return l.odd ? pair.y : pair.x; }
   using Scale = half_t;
   __device__ static half_t const_scale(const Lane& l) { return l.s[0]; }

@@ -24,6 +24,8 @@ struct Q4G32SkinnyPolicy {
   }
   __device__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
   __device__ static const char* s_addr(const Lane& l, int k0) { return l.s + ((k0 >> 5) & ~1) * 2; }
+  __device__ static const char* s_pair_addr(const Lane& l, int k0) { return s_addr(l, k0); }
+  static bool pair_aligned(const Args& a) { return (reinterpret_cast<uintptr_t>(a.S) & 3u) == 0; }
   __device__ static half_t pick_scale(const Lane&, half2_t pair, int kq) { return (kq & 1) ? pair.y : pair.x; }
   using Scale = half_t;
   __device__ static half_t const_scale(const Lane&) { return (half_t)0.0f; }

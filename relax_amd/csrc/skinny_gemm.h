@@ -51,6 +51,8 @@ typedef void __attribute__((address_space(3))) * wq_sk_lptr_t;
 //   const_scale(lane)          the lane's Scale                                              (!kScaleDma)
 //   null_scale()               a Scale that turns every code into an exact zero (weights past K)
 //   dequant(pieces, s, out[4]) -> B operands of MFMA 0..3 (k 8t .. 8t+7 each), scaled
+//   s_pair_addr(lane, k0)      like s_addr, for every policy (a fixed scale: the pair that holds it)
+//   pair_aligned(args)         host: whether those pairs are 4-byte aligned
 template <typename Policy, int TH, int NW, int WAVES>
 struct SkinnyCfg {
   static constexpr int KW = WAVES / NW;
@@ -223,9 +225,194 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
   }
 }
 
+
 constexpr int kSkinnyLdsBudget = 156 * 1024;  // of the 160 KB of a CU
 
+// ---------------------------------------------------------------------------------
+// M <= 16: the activations stay in registers.
+//
+// The ring kernel above re-reads the activations once per workgroup and keeps two thirds
+// of its loads in flight on those slabs; loads retire in order, so its weight stream is
+// only as deep as the slab ring.  For one 16-row tile the activations fit the register
+// file instead: a workgroup's WAVES wavefronts split K into contiguous runs of NSTEP
+// steps of 128 k, and wavefront w keeps the MFMA A operands of its run (16 rows x
+// 128*NSTEP k: 16*NSTEP registers) for the whole kernel.  The workgroups are persistent
+// (one per CU) and walk over 16-column tiles; the only loads inside the walk are the
+// codes and scales, through a wavefront-private ring in LDS that runs kDepth steps ahead
+// (across tiles).  Per tile the WAVES partial sums meet in LDS and one wavefront (taking
+// turns) adds them and stores.  Measured: with loads only it streams 2 TB/s from eight
+// wavefronts per CU however deep the ring, so it wins where the ring kernel pays most
+// for the slabs (K = 8192) and loses at K = 4096.
+//
+// Every policy hands its scale over as a 4-byte pair per lane and step here
+// (Policy::s_pair_addr), so that the walk has no load the compiler must wait for.
+template <typename Policy, int NSTEP, int WAVES>
+struct XregCfg {
+  static constexpr int kStepBytes = Policy::kPieces * 1024 + 256;
+  static constexpr int kLoadsPerStep = Policy::kPieces + 1;
+  static constexpr int kRedBytes = 2 * WAVES * 1024;
+  static constexpr int kFit = (kSkinnyLdsBudget - kRedBytes) / (WAVES * kStepBytes);
+  static constexpr int kCount = 63 / kLoadsPerStep + 1;  // vmcnt holds 6 bits
+  static constexpr int kWant = 3 * NSTEP;
+  static constexpr int kDepth = kFit < kCount ? (kFit < kWant ? kFit : kWant) : (kCount < kWant ? kCount : kWant);
+  static_assert(kDepth >= 2, "ring too small");
+  static constexpr int kLdsBytes = WAVES * kDepth * kStepBytes + kRedBytes;
+};
+
+template <typename Policy, typename Epilogue, int NSTEP, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void skinny_xreg_kernel(
+    typename Policy::Args pargs, const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epi,
+    int M, int N, int K) {
+  using Cfg = XregCfg<Policy, NSTEP, WAVES>;
+  constexpr int P = Policy::kPieces, L = Cfg::kLoadsPerStep, D = Cfg::kDepth;
+  constexpr int QA = D / NSTEP;  // the step D ahead of step s is step (s + D) % NSTEP, QA or QA + 1 tiles ahead
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lj = lane & 15, kq = lane >> 4;
+  const int tiles = (N + 15) >> 4;
+  const int grid = gridDim.x;
+  unsigned char* const ring = lds + wave * (D * Cfg::kStepBytes);
+  float4_t* const red = reinterpret_cast<float4_t*>(lds + WAVES * D * Cfg::kStepBytes);
+
+  // ---- the A operands of this wavefront's run of K (zero past M and past K) ----
+  half8_t a[NSTEP][4];
+  int k0c[NSTEP];  // this lane's 32 weights of step s (any valid k when past K: they meet zeros)
+#pragma unroll
+  for (int s = 0; s < NSTEP; ++s) {
+    const int k0 = (wave * NSTEP + s) * 128 + 32 * kq;
+    const bool held = lj < M && k0 < K;
+    k0c[s] = k0 < K ? k0 : 0;
+    const half_t* src = held ? X + (int64_t)lj * K + k0 : X;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const half8_t v = *reinterpret_cast<const half8_t*>(src + 8 * t);
+      a[s][t] = held ? v : half8_t{};
+    }
+  }
+
+  // lane state of the tiles QA and QA + 1 tiles ahead (whose loads are being issued)
+  typename Policy::Lane pl[2];
+  bool valid[2] = {false, false};
+  auto set_tile = [&](int which, int tile) {
+    valid[which] = tile < tiles;  // past the end: every lane re-reads one address
+    Policy::init(pl[which], pargs, min(min(tile, tiles - 1) * 16 + lj, N - 1), K, N);
+  };
+  auto issue = [&](int which, int s, int slot) {
+    unsigned char* dst = ring + slot * Cfg::kStepBytes;
+#pragma unroll
+    for (int p = 0; p < P; ++p)
+      __builtin_amdgcn_global_load_lds(
+          (wq_sk_gptr_t)(valid[which] ? Policy::w_addr(pl[which], k0c[s], p) : reinterpret_cast<const char*>(X)),
+          (wq_sk_lptr_t)(dst + p * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(
+        (wq_sk_gptr_t)(valid[which] ? Policy::s_pair_addr(pl[which], k0c[s]) : reinterpret_cast<const char*>(X)),
+        (wq_sk_lptr_t)(dst + P * 1024), 4, 0, 0);
+  };
+
+  // ---- prologue: the first D steps (slot = flat step % D) ----
+#pragma unroll
+  for (int f = 0; f < D; ++f) {
+    if (f % NSTEP == 0) set_tile(0, blockIdx.x + (f / NSTEP) * grid);
+    issue(0, f % NSTEP, f);
+  }
+  // the activations are in registers before the walk starts
+#pragma unroll
+  for (int s = 0; s < NSTEP; ++s)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) asm volatile("" : "+v"(a[s][t]));
+  typename Policy::Lane pl0;  // for pick_scale, which depends on the lane only
+  Policy::init(pl0, pargs, min(blockIdx.x * 16 + lj, N - 1), K, N);
+  set_tile(0, blockIdx.x + QA * grid);
+
+  int slot = 0;  // of step 0 of the current tile
+  int turn = 0;
+  for (int tile = blockIdx.x; tile < tiles; tile += grid) {
+    set_tile(1, tile + (QA + 1) * grid);
+    float4_t acc = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int s = 0; s < NSTEP; ++s) {
+      WQ_SK_WAITCNT_VM((D - 1) * L);  // issued after this step's loads: the D - 1 steps that follow it
+      int sl = slot + s;
+      if (sl >= D) sl -= D;
+      const unsigned char* src = ring + sl * Cfg::kStepBytes;
+      uint4_t pieces[P];
+#pragma unroll
+      for (int p = 0; p < P; ++p) pieces[p] = *reinterpret_cast<const uint4_t*>(src + p * 1024 + lane * 16);
+      const half2_t pair = *reinterpret_cast<const half2_t*>(src + P * 1024 + lane * 4);
+      half8_t bop[4];
+      Policy::dequant(pieces, Policy::pick_scale(pl0, pair, kq), bop);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s][t], bop[t], acc, 0, 0, 0);
+      // the slot is free once its contents are in registers; it takes the step D ahead
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      issue((s + D) / NSTEP - QA, (s + D) % NSTEP, sl);
+    }
+    slot = (slot + NSTEP) % D;
+    pl[0] = pl[1];
+    valid[0] = valid[1];
+
+    // ---- the WAVES partial sums of the tile meet in LDS (two buffers, by turns) ----
+    float4_t* const buf = red + (turn & 1) * (WAVES * 64);
+    buf[wave * 64 + lane] = acc;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (wave == turn % WAVES) {
+      float4_t sum = buf[lane];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) {
+        const float4_t v = buf[w * 64 + lane];
+        sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+      }
+      const int col = tile * 16 + lj;
+      if (col < N) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = 4 * kq + r;
+          if (m < M) Y[(int64_t)m * N + col] = epi(sum[r], m, col);
+        }
+      }
+    }
+    ++turn;
+  }
+  WQ_SK_WAITCNT_VM(0);  // the loads past the last tile land before the LDS is given back
+}
+
+template <typename Policy, typename Epilogue, int NSTEP, int WAVES>
+static int launch_xreg(const char* who, const typename Policy::Args& pargs, const uint16_t* x, uint16_t* y,
+                       const Epilogue& epi, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
+  using Cfg = XregCfg<Policy, NSTEP, WAVES>;
+  auto kern = skinny_xreg_kernel<Policy, Epilogue, NSTEP, WAVES>;
+  const int64_t tiles = (N + 15) / 16;
+  const int64_t blocks = tiles < cu_count() ? tiles : cu_count();
+  static bool configured = false;  // per instantiation
+  if (!configured) {
+    WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    configured = true;
+  }
+  WQ_LAUNCH(who, kern, dim3((unsigned)blocks), dim3(64 * WAVES), Cfg::kLdsBytes, stream, pargs,
+            (const half_t*)x, (half_t*)y, epi, (int)M, (int)N, (int)K);
+  return WQ_OK;
+}
+
+// K up to 64 steps of 128 (8192) is held by 8 wavefronts x 4 or 8 steps (64 or 128 registers;
+// 11 steps for K = 11008 spill)
+inline bool xreg_fits(int64_t M, int64_t K) { return M <= 16 && K <= 64 * 128; }
+
+template <typename Policy, typename Epilogue>
+static int launch_xreg_auto(const char* who, const typename Policy::Args& pargs, const uint16_t* x,
+                            uint16_t* y, const Epilogue& epi, int64_t M, int64_t N, int64_t K,
+                            hipStream_t stream) {
+  const int64_t steps = (K + 127) / 128;
+  if (steps <= 32) return launch_xreg<Policy, Epilogue, 4, 8>(who, pargs, x, y, epi, M, N, K, stream);
+  return launch_xreg<Policy, Epilogue, 8, 8>(who, pargs, x, y, epi, M, N, K, stream);
+}
+
 // overrides for tests and measurement (0 = automatic)
+// waves: 1 = the ring kernel, 2 = the kernel that holds the activations in registers (where it fits)
 struct SkinnyTuning {
   int nw, stages, waves;
 };
@@ -265,6 +452,12 @@ static int launch_skinny_auto(const char* who, const typename Policy::Args& parg
                               uint16_t* y, const Epilogue& epi, int64_t M, int64_t N, int64_t K,
                               hipStream_t stream) {
   const SkinnyTuning& t = skinny_tuning();
+  // activations in registers where that kernel is the faster one: 4096 < K <= 8192 and at least
+  // four column tiles per CU (N = 28672, K = 8192: q4f16_1 at M = 16 58 -> 47 us, int8 at M = 4
+  // 60 -> 48 us; with two tiles per CU, or at K = 4096, its eight wavefronts per CU stream the
+  // weights more slowly than the ring kernel's twenty-four)
+  if (xreg_fits(M, K) && Policy::pair_aligned(pargs) && (t.waves == 2 || (t.waves == 0 && K > 4096 && N / 16 >= 4 * (int64_t)cu_count())))
+    return launch_xreg_auto<Policy, Epilogue>(who, pargs, x, y, epi, M, N, K, stream);
   const int64_t per_cu = (N / 16) / cu_count();
   int nw = 1;
   if (per_cu >= 2) nw = M <= 8 ? (per_cu >= 4 ? 2 : 1) : M <= 16 ? 2 : 4;

@@ -126,19 +126,19 @@ def test_gemm_epilogues(ops, u, oracle, nbit, M, ep):
     _run(ops, u, oracle, M, 128, 256, nbit, seed=M + 3, **ep)
 
 
-@pytest.mark.parametrize("nw,stages", [(1, 2), (2, 3), (4, 4), (8, 3), (0, 0)])
+@pytest.mark.parametrize("nw,stages,waves", [(1, 2, 0), (2, 3, 0), (4, 4, 0), (8, 3, 0), (0, 0, 0), (0, 0, 1), (0, 0, 2)])
 @pytest.mark.parametrize("nbit", [8, 4])
 @pytest.mark.parametrize("group_size", [-1, 64])
-def test_small_batch_work_splits(ops, u, oracle, nbit, group_size, nw, stages):
+def test_small_batch_work_splits(ops, u, oracle, nbit, group_size, nw, stages, waves):
     """3 <= M <= 64 runs the matrix-core streaming kernel; every work split of it, ragged M,
     K not a multiple of its 128-k step."""
     from relax_amd import _lib
 
-    _lib.lib().wq_debug_set_skinny_config(nw, stages, 0)
+    _lib.lib().wq_debug_set_skinny_config(nw, stages, waves)
     try:
         for M, N, K in [(3, 64, 64), (8, 320, 448), (9, 128, 4096), (16, 320, 448), (24, 64, 1024),
-                        (32, 2048, 512), (40, 320, 448), (64, 192, 2112)]:
-            print(f"intb small batch nbit={nbit} g={group_size} nw={nw} M={M} N={N} K={K}", flush=True)
+                        (32, 2048, 512), (40, 320, 448), (64, 192, 2112), (16, 4288, 8192), (5, 8192, 5184)]:
+            print(f"intb small batch nbit={nbit} g={group_size} nw={nw} waves={waves} M={M} N={N} K={K}", flush=True)
             _run(ops, u, oracle, M, N, K, nbit, seed=M + nw, group_size=group_size)
     finally:
         _lib.lib().wq_debug_set_skinny_config(0, 0, 0)

@@ -179,13 +179,16 @@ def test_gemm_epilogue(ops, u, oracle):
 SMALL_BATCH = [  # (M, N, K): ragged M and N, K/64 not a multiple of the wavefronts that split K
     (2, 64, 64), (5, 100, 192), (8, 4096, 4096), (16, 1001, 320), (17, 12288, 4096),
     (32, 4096, 11008), (33, 520, 1024), (64, 22016, 4096), (9, 31, 128),
+    (3, 12288, 4096), (16, 4112, 8192), (12, 5000, 5184), (7, 16, 8192),
 ]
 
 
-@pytest.mark.parametrize("nw,waves,stages", [(1, 0, 2), (2, 0, 3), (4, 0, 5), (1, 0, 3), (2, 0, 2), (4, 0, 4), (8, 0, 3), (8, 0, 2), (0, 0, 0)])
+@pytest.mark.parametrize("nw,waves,stages", [(1, 0, 2), (2, 0, 3), (4, 0, 5), (1, 0, 3), (2, 0, 2), (4, 0, 4), (8, 0, 3), (8, 0, 2), (0, 0, 0),
+                                             (0, 1, 0), (0, 2, 0)])
 @pytest.mark.parametrize("M,N,K", SMALL_BATCH)
 def test_small_batch_vs_oracle(ops, u, oracle, nw, waves, stages, M, N, K):
-    """the matrix-core kernel for 2 <= M <= 64, in each of its work splits (0 = automatic)."""
+    """the matrix-core kernels for 2 <= M <= 64, in each of their work splits (0 = automatic; waves 1: the
+    ring kernel, 2: activations in registers where M <= 16 and K <= 8192)."""
     from relax_amd import _lib
 
     x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=nw + M + N + K)
