@@ -240,9 +240,10 @@ constexpr int kSkinnyLdsBudget = 156 * 1024;  // of the 160 KB of a CU
 // (one per CU) and walk over 16-column tiles; the only loads inside the walk are the
 // codes and scales, through a wavefront-private ring in LDS that runs kDepth steps ahead
 // (across tiles).  Per tile the WAVES partial sums meet in LDS and one wavefront (taking
-// turns) adds them and stores.  Measured: with loads only it streams 2 TB/s from eight
-// wavefronts per CU however deep the ring, so it wins where the ring kernel pays most
-// for the slabs (K = 8192) and loses at K = 4096.
+// turns) adds them and stores.  Measured: with loads only it streams 2 TB/s however
+// deep the ring (and no more from sixteen wavefronts than from eight), so it wins where
+// the ring kernel pays most for the slabs (K = 8192, many tiles per CU) and loses at
+// K = 4096.
 //
 // Every policy hands its scale over as a 4-byte pair per lane and step here
 // (Policy::s_pair_addr), so that the walk has no load the compiler must wait for.
@@ -454,8 +455,7 @@ static int launch_skinny_auto(const char* who, const typename Policy::Args& parg
   const SkinnyTuning& t = skinny_tuning();
   // activations in registers where that kernel is the faster one: 4096 < K <= 8192 and at least
   // four column tiles per CU (N = 28672, K = 8192: q4f16_1 at M = 16 58 -> 47 us, int8 at M = 4
-  // 60 -> 48 us; with two tiles per CU, or at K = 4096, its eight wavefronts per CU stream the
-  // weights more slowly than the ring kernel's twenty-four)
+  // 60 -> 48 us; with two tiles per CU, or at K = 4096, the ring kernel is the faster one)
   if (xreg_fits(M, K) && Policy::pair_aligned(pargs) && (t.waves == 2 || (t.waves == 0 && K > 4096 && N / 16 >= 4 * (int64_t)cu_count())))
     return launch_xreg_auto<Policy, Epilogue>(who, pargs, x, y, epi, M, N, K, stream);
   const int64_t per_cu = (N / 16) / cu_count();
