@@ -139,6 +139,7 @@ __global__ __launch_bounds__(256) void gptq_gather_x_direct_kernel(const half_t*
 struct GptqSkinnyPolicy {
   static constexpr int kPieces = 1;
   static constexpr bool kScaleDma = true;
+  static constexpr bool kCanScaleBlock = false;
   struct Args {
     const uint32_t* W;
     const half2_t* SZ;

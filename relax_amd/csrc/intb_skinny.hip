@@ -15,6 +15,7 @@ template <int NBIT, bool GROUPED>
 struct IntbSkinnyPolicy {
   static constexpr int kPieces = NBIT == 8 ? 2 : 1;
   static constexpr bool kScaleDma = GROUPED;
+  static constexpr bool kCanScaleBlock = false;
   struct Args {
     const uint4_t* B;
     const half_t* scales;

@@ -10,6 +10,7 @@ namespace wq {
 struct Q4G32SkinnyPolicy {
   static constexpr int kPieces = 1;
   static constexpr bool kScaleDma = true;
+  static constexpr bool kCanScaleBlock = true;
   struct Args {
     const uint32_t* W;
     const half_t* S;
@@ -25,6 +26,11 @@ struct Q4G32SkinnyPolicy {
   __device__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
   __device__ static const char* s_addr(const Lane& l, int k0) { return l.s + ((k0 >> 5) & ~1) * 2; }
   __device__ static const char* s_pair_addr(const Lane& l, int k0) { return s_addr(l, k0); }
+  __device__ static const char* sblock_addr(const Lane& l, int g) { return l.s + g * 2; }
+  // rows of K/16 bytes: every 8 scales are 16 aligned bytes when K % 256 == 0 and S is aligned
+  static bool scale_block_ok(const Args& a, int64_t K) {
+    return K % 256 == 0 && (reinterpret_cast<uintptr_t>(a.S) & 15u) == 0;
+  }
   static bool pair_aligned(const Args& a) { return (reinterpret_cast<uintptr_t>(a.S) & 3u) == 0; }
   __device__ static half_t pick_scale(const Lane&, half2_t pair, int kq) { return (kq & 1) ? pair.y : pair.x; }
   using Scale = half_t;

@@ -52,8 +52,16 @@ typedef void __attribute__((address_space(3))) * wq_sk_lptr_t;
 //   null_scale()               a Scale that turns every code into an exact zero (weights past K)
 //   dequant(pieces, s, out[4]) -> B operands of MFMA 0..3 (k 8t .. 8t+7 each), scaled
 //   s_pair_addr(lane, k0)      like s_addr, for every policy (a fixed scale: the pair that holds it)
+//   kCanScaleBlock             true (needs kScaleDma): the scales of a column are 2-byte values, contiguous
+//                              along K, one per 32 k; where scale_block_ok(args, K) the ring kernel may
+//                              fetch all scales of a column block once, 16 bytes per lane, instead of a
+//                              pair per lane and step
+//   sblock_addr(lane, g)       address of scale g of the lane's column (g % 8 == 0)       (kCanScaleBlock)
+//   scale_block_ok(args, K)    host: every 8 scales of a column are 16 aligned bytes      (kCanScaleBlock)
 //   pair_aligned(args)         host: whether those pairs are 4-byte aligned
-template <typename Policy, int TH, int NW, int WAVES>
+constexpr int kScaleBlockMaxK = 4096;  // a column block's scales for all of K stay in LDS: 4 KB
+
+template <typename Policy, int TH, int NW, int WAVES, bool SB = false>
 struct SkinnyCfg {
   static constexpr int KW = WAVES / NW;
   static_assert(NW * KW == WAVES && (WAVES == 4 || WAVES == 8), "wavefront arrangement");
@@ -63,9 +71,11 @@ struct SkinnyCfg {
   static constexpr int kSlabBytes = kRows * 256;         // rows x 128 k
   static constexpr int kXBytes = KW * kSlabBytes;
   static constexpr int kWBytes = WAVES * Policy::kPieces * 1024;
-  static constexpr int kStageBytes = kXBytes + kWBytes + (Policy::kScaleDma ? WAVES * 256 : 0);
+  static constexpr bool kStepScale = Policy::kScaleDma && !SB;  // a scale load per lane and step
+  static constexpr int kStageBytes = kXBytes + kWBytes + (kStepScale ? WAVES * 256 : 0);
+  static constexpr int kSBlockBytes = SB ? NW * kScaleBlockMaxK : 0;  // after the ring
   static constexpr int kXLoads = 2 * TH / NW;            // slab loads (4 rows each) per wavefront and step
-  static constexpr int kLoadsPerStep = kXLoads + Policy::kPieces + (Policy::kScaleDma ? 1 : 0);
+  static constexpr int kLoadsPerStep = kXLoads + Policy::kPieces + (kStepScale ? 1 : 0);
   static constexpr int kMaxAhead = 63 / kLoadsPerStep;   // vmcnt holds 6 bits
   static constexpr int kRedBytes = WAVES * TM * 4 * 64 * 4;
 };
@@ -86,11 +96,11 @@ __device__ __forceinline__ void wait_newer_groups(int groups) {
   }
 }
 
-template <typename Policy, typename Epilogue, int TH, int NW, int WAVES>
+template <typename Policy, typename Epilogue, int TH, int NW, int WAVES, bool SB>
 __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
     typename Policy::Args pargs, const half_t* __restrict__ X, half_t* __restrict__ Y, Epilogue epi,
     int M, int N, int K, int stages) {
-  using Cfg = SkinnyCfg<Policy, TH, NW, WAVES>;
+  using Cfg = SkinnyCfg<Policy, TH, NW, WAVES, SB>;
   constexpr int KW = Cfg::KW, TM = Cfg::TM, P = Policy::kPieces;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -122,6 +132,9 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
 
   unsigned char* const w_area = lds + Cfg::kXBytes + wave * (P * 1024);
   unsigned char* const s_area = lds + Cfg::kXBytes + Cfg::kWBytes + wave * 256;
+  // SB: all scales of the column block (K / 32 per column), as chunks of 32 per column: chunk c is
+  // one load of one wavefront, lane (j, q) bringing scales 32c + 8q .. + 7 of column j
+  unsigned char* const s_block = lds + stages * Cfg::kStageBytes + nw * kScaleBlockMaxK;
 
   auto issue = [&](int it, int slot) {
     const int stage_off = slot * Cfg::kStageBytes;
@@ -140,7 +153,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
     for (int p = 0; p < P; ++p)
       __builtin_amdgcn_global_load_lds((wq_sk_gptr_t)Policy::w_addr(pl, k0c, p),
                                        (wq_sk_lptr_t)(w_area + stage_off + p * 1024), 16, 0, 0);
-    if (Policy::kScaleDma)
+    if constexpr (Cfg::kStepScale)
       __builtin_amdgcn_global_load_lds((wq_sk_gptr_t)Policy::s_addr(pl, k0c),
                                        (wq_sk_lptr_t)(s_area + stage_off), 4, 0, 0);
   };
@@ -157,8 +170,13 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
     for (int p = 0; p < P; ++p)
       pieces[p] = *reinterpret_cast<const uint4_t*>(w_area + stage_off + p * 1024 + lane * 16);
     typename Policy::Scale s = s_fixed;
-    if (Policy::kScaleDma)
+    if constexpr (Cfg::kStepScale)
       s = Policy::pick_scale(pl, *reinterpret_cast<const half2_t*>(s_area + stage_off + lane * 4), kq);
+    if constexpr (SB) {
+      const int g = (k0 < K ? k0 : 0) >> 5;  // chunk g / 32, fetched by lane (j, (g / 8) % 4)
+      s = *reinterpret_cast<const half_t*>(s_block + (g >> 5) * 1024 + (((g >> 3) & 3) * 16 + lj) * 16 +
+                                           (g & 7) * 2);
+    }
     if (k0 >= K) s = Policy::null_scale();  // code * 0 = exact zero for the weights past K
     half8_t bop[4];
     Policy::dequant(pieces, s, bop);
@@ -176,14 +194,23 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
     }
   };
 
-  // ---- prologue: fill the ring ----
+  // ---- prologue: the scale block (its loads are older than every step's, so each wavefront's
+  // part has landed when its first wait returns; the barrier of step 0 covers the others'), then
+  // fill the ring ----
+  if constexpr (SB) {
+    for (int c = kw; c * 1024 < K; c += KW) {
+      const int g = 32 * c + 8 * kq;
+      __builtin_amdgcn_global_load_lds((wq_sk_gptr_t)Policy::sblock_addr(pl, g * 32 < K ? g : 0),
+                                       (wq_sk_lptr_t)(s_block + c * 1024), 16, 0, 0);
+    }
+  }
   for (int p = 0; p < ahead && p < nsteps; ++p) issue(p, p);
   int cslot = 0;                       // slot of the step being computed
   int islot = ahead % stages;          // slot the next issue goes to
   for (int it = 0; it < nsteps; ++it) {
     const int newer = min(ahead - 1, nsteps - 1 - it);  // steps issued after step `it`
     wait_newer_groups<Cfg::kLoadsPerStep>(newer);
-    if (NW > 1) __builtin_amdgcn_s_barrier();
+    if (NW > 1 || (SB && KW > 1 && it == 0)) __builtin_amdgcn_s_barrier();
     // the slot refilled now was computed in the previous iteration (by everyone: barrier above)
     if (it + ahead < nsteps) {
       issue(it + ahead, islot);
@@ -419,19 +446,27 @@ struct SkinnyTuning {
 };
 SkinnyTuning& skinny_tuning();
 
-template <typename Policy, typename Epilogue, int TH, int NW, int WAVES>
+template <typename Policy, typename Epilogue, int TH, int NW, int WAVES, bool SB = false>
 static int launch_skinny(const char* who, const typename Policy::Args& pargs, const uint16_t* x, uint16_t* y,
                          const Epilogue& epi, int64_t M, int64_t N, int64_t K, int want_stages,
                          hipStream_t stream) {
-  using Cfg = SkinnyCfg<Policy, TH, NW, WAVES>;
-  auto kern = skinny_gemm_kernel<Policy, Epilogue, TH, NW, WAVES>;
+  // one fetch of all scales where the policy allows it and the block is small (two column
+  // blocks at most: more would cost a workgroup per CU)
+  if constexpr (!SB && Policy::kCanScaleBlock && NW <= 2) {
+    if (K <= kScaleBlockMaxK && Policy::scale_block_ok(pargs, K))
+      return launch_skinny<Policy, Epilogue, TH, NW, WAVES, true>(who, pargs, x, y, epi, M, N, K, want_stages,
+                                                                  stream);
+  }
+  using Cfg = SkinnyCfg<Policy, TH, NW, WAVES, SB>;
+  auto kern = skinny_gemm_kernel<Policy, Epilogue, TH, NW, WAVES, SB>;
   const int64_t blocks = (N + 16 * NW - 1) / (16 * NW);
   int stages = want_stages;
   if (stages > Cfg::kMaxAhead + 1) stages = Cfg::kMaxAhead + 1;
   if (stages > 9) stages = 9;
-  if (stages * Cfg::kStageBytes > kSkinnyLdsBudget) stages = kSkinnyLdsBudget / Cfg::kStageBytes;
+  if (stages * Cfg::kStageBytes + Cfg::kSBlockBytes > kSkinnyLdsBudget)
+    stages = (kSkinnyLdsBudget - Cfg::kSBlockBytes) / Cfg::kStageBytes;
   WQ_REQUIRE(stages >= 2, "%s: internal: no room for a 2-slot ring", who);
-  int lds_bytes = stages * Cfg::kStageBytes;
+  int lds_bytes = stages * Cfg::kStageBytes + Cfg::kSBlockBytes;
   if (lds_bytes < Cfg::kRedBytes) lds_bytes = Cfg::kRedBytes;
   static bool configured = false;  // per instantiation
   if (!configured) {
