@@ -18,7 +18,8 @@
 // Everything travels global -> LDS with direct loads into a ring of `stages` slots,
 // `stages - 1` steps ahead: per step the rows x 128 activation slab of each kw
 // (shared by the NW wavefronts of that kw, each loading a part), and per wavefront
-// its codes and scales.  A wavefront waits for its own loads with s_waitcnt vmcnt(n);
+// its codes and scales (or, where the policy and K allow, all scales of the column block
+// once, ahead of the ring).  A wavefront waits for its own loads with s_waitcnt vmcnt(n);
 // when NW > 1 one s_barrier per step makes the shared slab visible.  The KW partial
 // sums of a column block meet in LDS at the end.
 //
