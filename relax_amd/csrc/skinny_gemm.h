@@ -60,7 +60,8 @@ typedef void __attribute__((address_space(3))) * wq_sk_lptr_t;
 //   sblock_addr(lane, g)       address of scale g of the lane's column (g % 8 == 0)       (kCanScaleBlock)
 //   scale_block_ok(args, K)    host: every 8 scales of a column are 16 aligned bytes      (kCanScaleBlock)
 //   pair_aligned(args)         host: whether those pairs are 4-byte aligned
-constexpr int kScaleBlockMaxK = 4096;  // a column block's scales for all of K stay in LDS: 4 KB
+constexpr int kScaleBlockMaxK = 11264;  // a column block's scales for all of K stay in LDS: K bytes
+inline int scale_block_stride(int K) { return ((K + 1023) >> 10) << 10; }
 
 template <typename Policy, int TH, int NW, int WAVES, bool SB = false>
 struct SkinnyCfg {
@@ -74,7 +75,6 @@ struct SkinnyCfg {
   static constexpr int kWBytes = WAVES * Policy::kPieces * 1024;
   static constexpr bool kStepScale = Policy::kScaleDma && !SB;  // a scale load per lane and step
   static constexpr int kStageBytes = kXBytes + kWBytes + (kStepScale ? WAVES * 256 : 0);
-  static constexpr int kSBlockBytes = SB ? NW * kScaleBlockMaxK : 0;  // after the ring
   static constexpr int kXLoads = 2 * TH / NW;            // slab loads (4 rows each) per wavefront and step
   static constexpr int kLoadsPerStep = kXLoads + Policy::kPieces + (kStepScale ? 1 : 0);
   static constexpr int kMaxAhead = 63 / kLoadsPerStep;   // vmcnt holds 6 bits
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_gemm_kernel(
   unsigned char* const s_area = lds + Cfg::kXBytes + Cfg::kWBytes + wave * 256;
   // SB: all scales of the column block (K / 32 per column), as chunks of 32 per column: chunk c is
   // one load of one wavefront, lane (j, q) bringing scales 32c + 8q .. + 7 of column j
-  unsigned char* const s_block = lds + stages * Cfg::kStageBytes + nw * kScaleBlockMaxK;
+  unsigned char* const s_block = lds + stages * Cfg::kStageBytes + nw * ((((K + 1023) >> 10)) << 10);
 
   auto issue = [&](int it, int slot) {
     const int stage_off = slot * Cfg::kStageBytes;
@@ -454,7 +454,9 @@ static int launch_skinny(const char* who, const typename Policy::Args& pargs, co
   // one fetch of all scales where the policy allows it and the block is small (two column
   // blocks at most: more would cost a workgroup per CU)
   if constexpr (!SB && Policy::kCanScaleBlock && NW <= 2) {
-    if (K <= kScaleBlockMaxK && Policy::scale_block_ok(pargs, K))
+    if (K <= kScaleBlockMaxK && Policy::scale_block_ok(pargs, K) &&
+        2 * SkinnyCfg<Policy, TH, NW, WAVES, true>::kStageBytes + NW * scale_block_stride((int)K) <=
+            kSkinnyLdsBudget)
       return launch_skinny<Policy, Epilogue, TH, NW, WAVES, true>(who, pargs, x, y, epi, M, N, K, want_stages,
                                                                   stream);
   }
@@ -464,10 +466,11 @@ static int launch_skinny(const char* who, const typename Policy::Args& pargs, co
   int stages = want_stages;
   if (stages > Cfg::kMaxAhead + 1) stages = Cfg::kMaxAhead + 1;
   if (stages > 9) stages = 9;
-  if (stages * Cfg::kStageBytes + Cfg::kSBlockBytes > kSkinnyLdsBudget)
-    stages = (kSkinnyLdsBudget - Cfg::kSBlockBytes) / Cfg::kStageBytes;
+  const int sblock_bytes = SB ? NW * scale_block_stride((int)K) : 0;  // after the ring
+  if (stages * Cfg::kStageBytes + sblock_bytes > kSkinnyLdsBudget)
+    stages = (kSkinnyLdsBudget - sblock_bytes) / Cfg::kStageBytes;
   WQ_REQUIRE(stages >= 2, "%s: internal: no room for a 2-slot ring", who);
-  int lds_bytes = stages * Cfg::kStageBytes + Cfg::kSBlockBytes;
+  int lds_bytes = stages * Cfg::kStageBytes + sblock_bytes;
   if (lds_bytes < Cfg::kRedBytes) lds_bytes = Cfg::kRedBytes;
   static bool configured = false;  // per instantiation
   if (!configured) {
