@@ -106,7 +106,10 @@ WQ_PACKED(relax_amd_decode_matmul_cast_bias_gelu_residual_multiply_relu);
 /* Registers every function above in the TVM global registry of the current
  * process (TVMFuncCreateFromCFunc + TVMFuncRegisterGlobal, looked up with
  * dlsym).  Returns the number of names registered, 0 when no TVM runtime is
- * loaded, -1 on error.  Called automatically when the library is loaded. */
+ * loaded, -1 on error.  Called automatically when the library is loaded.  The
+ * "relax_amd.*" names replace an earlier registration of the same name; the host's own
+ * name "cutlass.ft_preprocess_weight" is registered only when the host does not have it
+ * (a TVM built with its CUTLASS back end keeps its function). */
 int wq_tvm_register_globals(void);
 
 /* Number of PackedFunc names and the i-th dotted name / C symbol (for tools and tests). */

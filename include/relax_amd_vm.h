@@ -49,7 +49,8 @@ int wq_program_add_external(wq_program_t* p, int dtype_code, int dtype_bits, int
 int wq_program_add_planned(wq_program_t* p, int dtype_code, int dtype_bits, int ndim,
                            const int64_t* shape);
 /* Points an external register at other storage of the same shape (next batch of inputs).
- * A captured graph keeps the addresses it was captured with: capture again afterwards. */
+ * A captured graph keeps the addresses it was captured with, so the graph is dropped here:
+ * wq_program_replay fails ("nothing captured") until wq_program_capture is called again. */
 int wq_program_rebind(wq_program_t* p, int reg, void* data);
 
 /* Appends `func(args...)`.  kinds[i] = 1: args[i] is a tensor register, passed as an

@@ -43,18 +43,44 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(verbose: bool = True) -> str:
-    """Compile every source and link the shared library; returns its path."""
+def _deps(src: str, seen=None):
+    """`src` and every file it includes with quotes, transitively."""
+    seen = seen if seen is not None else set()
+    if src in seen or not os.path.exists(src):
+        return seen
+    seen.add(src)
+    with open(src) as f:
+        for line in f:
+            line = line.strip()
+            if line.startswith('#include "'):
+                _deps(os.path.normpath(os.path.join(os.path.dirname(src), line.split('"')[1])), seen)
+    return seen
+
+
+def _stale(src: str) -> bool:
+    obj = os.path.join(OBJDIR, os.path.basename(src) + ".o")
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    return any(os.path.getmtime(d) > t for d in _deps(src)) or os.path.getmtime(__file__) > t
+
+
+def build(verbose: bool = True, incremental: bool = False) -> str:
+    """Compile every source (with `incremental`, only those newer than their object file, headers
+    included) and link the shared library; returns its path."""
     os.makedirs(OBJDIR, exist_ok=True)
     srcs = sources()
-    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
+    todo = [s for s in srcs if _stale(s)] if incremental else srcs
+    if todo:
+        with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(todo))) as ex:
+            list(ex.map(_compile, todo))
+    objs = [os.path.join(OBJDIR, os.path.basename(s) + ".o") for s in srcs]
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     subprocess.check_call(cmd)
     if verbose:
-        print(f"built {LIB} from {len(srcs)} sources", flush=True)
+        print(f"built {LIB}: compiled {len(todo)} of {len(srcs)} sources", flush=True)
     return LIB
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv)

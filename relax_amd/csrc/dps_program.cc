@@ -115,6 +115,7 @@ extern "C" int wq_program_rebind(wq_program_t* p, int reg, void* data) {
   WQ_REQUIRE(p && reg >= 0 && reg < (int)p->regs.size(), "wq_program_rebind: no such register %d", reg);
   WQ_REQUIRE(!p->regs[reg].planned, "wq_program_rebind: register %d is planned storage", reg);
   p->regs[reg].dl.data = data;
+  drop_graph(p);  // a captured graph holds the old address: replay must fail until captured again
   return WQ_OK;
 }
 

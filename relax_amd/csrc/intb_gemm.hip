@@ -189,7 +189,8 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
     // one or two rows: the VALU streaming kernel; up to 64 rows: still one pass over the
     // weights, products on the matrix cores; beyond that the tiled GEMM
     if (m <= 2) return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
-    if (m <= WQ_SMALL_BATCH_MAX_M)
+    // fine-grained scales whose pairs are not 4-byte aligned go to the register-staged GEMM below
+    if (m <= WQ_SMALL_BATCH_MAX_M && (!group || (reinterpret_cast<uintptr_t>(scales) & 3u) == 0))
       return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
   }
   const IntbGemmEpilogue gep{ep, (int)n};

@@ -23,6 +23,7 @@ struct HostRuntime {
   int (*func_call)(TVMFunctionHandle, TVMValue*, int*, int, TVMValue*, int*) = nullptr;
   int (*set_return)(TVMRetValueHandle, TVMValue*, int*, int) = nullptr;
   int (*array_alloc)(const tvm_index_t*, int, int, int, int, int, int, TVMArrayHandle*) = nullptr;
+  int (*array_free)(TVMArrayHandle) = nullptr;
   bool present = false;
 };
 
@@ -37,6 +38,7 @@ HostRuntime& host() {
     r.func_call = reinterpret_cast<decltype(r.func_call)>(sym("TVMFuncCall"));
     r.set_return = reinterpret_cast<decltype(r.set_return)>(sym("TVMCFuncSetReturn"));
     r.array_alloc = reinterpret_cast<decltype(r.array_alloc)>(sym("TVMArrayAlloc"));
+    r.array_free = reinterpret_cast<decltype(r.array_free)>(sym("TVMArrayFree"));
     r.present = r.func_create && r.func_register;
     return r;
   }();
@@ -338,8 +340,10 @@ WQ_PACKED(cutlass_ft_preprocess_weight) {
     fail(WQ_EDEVICE, "%s: TVMArrayAlloc failed", who);
     return packed_fail();
   }
-  if (preprocess_into(who, in, sm, is_int4, static_cast<char*>(out->data) + out->byte_offset) != 0)
+  if (preprocess_into(who, in, sm, is_int4, static_cast<char*>(out->data) + out->byte_offset) != 0) {
+    if (h.array_free) (void)h.array_free(out);  // the result never reaches the caller: give it back
     return packed_fail();
+  }
   // ownership of the new array moves to the caller (packed_func.h:975-982)
   out_ret_value->v_handle = out;
   *out_ret_tcode = kTVMNDArrayHandle;
@@ -736,8 +740,16 @@ extern "C" int wq_tvm_register_globals(void) {
   int n = 0;
   for (const Entry& e : table()) {
     TVMFunctionHandle f = nullptr;
+    // Names of this library ("relax_amd.*") are replaced on a second call; a name that belongs
+    // to the host ("cutlass.ft_preprocess_weight" of a TVM built with CUTLASS) is left alone
+    // when the host already has it.
+    const bool ours = e.name.rfind("relax_amd.", 0) == 0;
+    if (!ours && h.func_get_global) {
+      TVMFunctionHandle have = nullptr;
+      if (h.func_get_global(e.name.c_str(), &have) == 0 && have) continue;
+    }
     if (h.func_create(registry_trampoline, const_cast<Entry*>(&e), nullptr, &f) != 0) return -1;
-    if (h.func_register(e.name.c_str(), f, /*override=*/1) != 0) return -1;
+    if (h.func_register(e.name.c_str(), f, /*override=*/ours ? 1 : 0) != 0) return -1;
     ++n;
   }
   return n;

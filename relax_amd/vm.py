@@ -28,7 +28,7 @@ class DpsProgram:
     def __init__(self):
         self._l = _lib.lib()
         self._p = self._l.wq_program_create()
-        self._keep: List[torch.Tensor] = []
+        self._keep: Dict[int, torch.Tensor] = {}  # register -> the tensor that owns its storage
         self._shapes: Dict[int, Tuple[Tuple[int, ...], torch.dtype]] = {}
         self._workspace = None
 
@@ -52,7 +52,7 @@ class DpsProgram:
         r = self._l.wq_program_add_external(self._p, code, bits, t.dim(), shape, t.data_ptr(),
                                             kDLROCM if t.is_cuda else kDLCPU)
         check(min(r, 0), "wq_program_add_external")
-        self._keep.append(t)
+        self._keep[r] = t
         self._shapes[r] = (tuple(t.shape), t.dtype)
         return Reg(r)
 
@@ -74,7 +74,7 @@ class DpsProgram:
         if tuple(t.shape) != shape or t.dtype != dtype or not t.is_contiguous():
             raise ValueError("rebind needs a contiguous tensor of the declared shape and dtype")
         check(self._l.wq_program_rebind(self._p, int(reg), t.data_ptr()), "wq_program_rebind")
-        self._keep.append(t)
+        self._keep[int(reg)] = t  # the previous tensor of this register is released
 
     # ---- instructions ----
     def call(self, func: str, *args: Union[Reg, int, None]) -> None:
@@ -121,14 +121,22 @@ LLAMA7B_LINEARS = (("qkv_proj", 12288, 4096), ("o_proj", 4096, 4096), ("gate_up_
 
 
 def llama_linear_stack(weights, M: int, hidden: torch.Tensor, attn_out: torch.Tensor, mlp_act: torch.Tensor,
-                       out: torch.Tensor, linears=LLAMA7B_LINEARS) -> DpsProgram:
+                       out: torch.Tensor, linears=LLAMA7B_LINEARS, taps=None) -> DpsProgram:
     """Program of ``len(weights)`` decoder layers' quantized linears (q4f16_1), batch ``M``.
 
     ``weights[l][name] = (W int32 [N, K/8], S fp16 [N, K/32])``.  Only the linears are present, so two
     inputs stand in for what the missing ops would produce: ``attn_out`` [M, 4096] feeds every o_proj
     and ``mlp_act`` [M, 11008] every down_proj.  ``hidden`` [M, 4096] enters layer 0; each layer's
     down_proj output is the next layer's hidden state; the last one lands in ``out``.
+    ``taps`` maps ``(layer, name)`` to a tensor [M, N] that receives that linear's output instead of
+    planned storage (to look at an intermediate of the stack).
     """
+    taps = taps or {}
+
+    def dest(l, name):
+        t = taps.get((l, name))
+        return p.external(t) if t is not None else p.planned((M, dims[name][0]))
+
     p = DpsProgram()
     h = p.external(hidden)
     a = p.external(attn_out)
@@ -137,13 +145,13 @@ def llama_linear_stack(weights, M: int, hidden: torch.Tensor, attn_out: torch.Te
     L = len(weights)
     for l, layer in enumerate(weights):
         regs = {name: (p.external(w, as_uint32=True), p.external(s)) for name, (w, s) in layer.items()}
-        qkv = p.planned((M, dims["qkv_proj"][0]))
+        qkv = dest(l, "qkv_proj")
         p.call("relax_amd.q4f16_1_matmul", *regs["qkv_proj"], h, qkv)
-        o = p.planned((M, dims["o_proj"][0]))
+        o = dest(l, "o_proj")
         p.call("relax_amd.q4f16_1_matmul", *regs["o_proj"], a, o)
-        gu = p.planned((M, dims["gate_up_proj"][0]))
+        gu = dest(l, "gate_up_proj")
         p.call("relax_amd.q4f16_1_matmul", *regs["gate_up_proj"], o, gu)
-        nxt = p.external(out) if l == L - 1 else p.planned((M, dims["down_proj"][0]))
+        nxt = p.external(out) if l == L - 1 else dest(l, "down_proj")
         p.call("relax_amd.q4f16_1_matmul", *regs["down_proj"], g, nxt)
         h = nxt
     return p

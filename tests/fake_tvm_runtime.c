@@ -2,7 +2,7 @@
  * A tiny stand-in for the handful of TVM runtime C-API entry points the PackedFunc
  * layer looks up with dlsym (TVMFuncCreateFromCFunc, TVMFuncRegisterGlobal,
  * TVMFuncGetGlobal, TVMFuncCall, TVMCFuncSetReturn, TVMAPISetLastError,
- * TVMArrayAlloc).  Test double only: it lets the CPU tests check that the library
+ * TVMArrayAlloc, TVMArrayFree).  Test double only: it lets the CPU tests check that the library
  * registers its global names when a runtime is present and that a registry call
  * round-trips arguments and a returned NDArray.  Host (kDLCPU) arrays only.
  */
@@ -12,7 +12,7 @@
 
 #include "../include/relax_amd_tvm_abi.h"
 
-#define MAXF 64
+#define MAXF 256
 typedef struct {
   TVMPackedCFunc fn;
   void* resource;
@@ -22,6 +22,7 @@ static char g_names[MAXF][96];
 static Func* g_named[MAXF];
 static int g_nfuncs = 0, g_nnames = 0;
 static char g_last_error[512];
+static int g_live_arrays = 0;
 
 typedef struct {
   TVMValue value;
@@ -43,7 +44,12 @@ int TVMFuncCreateFromCFunc(TVMPackedCFunc func, void* resource_handle, TVMPacked
   return 0;
 }
 int TVMFuncRegisterGlobal(const char* name, TVMFunctionHandle f, int override) {
-  (void)override;
+  for (int i = 0; i < g_nnames; ++i)
+    if (!strcmp(g_names[i], name)) {
+      if (!override) return -1;  /* "already registered" */
+      g_named[i] = (Func*)f;
+      return 0;
+    }
   if (g_nnames >= MAXF) return -1;
   strncpy(g_names[g_nnames], name, 95);
   g_named[g_nnames++] = (Func*)f;
@@ -89,8 +95,33 @@ int TVMArrayAlloc(const tvm_index_t* shape, int ndim, int dtype_code, int dtype_
   t->device.device_type = (DLDeviceType)device_type;
   t->device.device_id = device_id;
   t->data = malloc((size_t)(n * dtype_bits / 8 + 64));
+  ++g_live_arrays;
   *out = t;
   return 0;
+}
+int TVMArrayFree(TVMArrayHandle h) {
+  DLTensor* t = (DLTensor*)h;
+  free(t->data);
+  free(t->shape);
+  free(t);
+  --g_live_arrays;
+  return 0;
+}
+int fake_live_arrays(void) { return g_live_arrays; }
+/* a function of the host's own, to check that the library does not replace it */
+static int host_own_fn(TVMValue* a, int* c, int n, TVMRetValueHandle r, void* res) {
+  (void)a; (void)c; (void)n; (void)r; (void)res;
+  return 0;
+}
+int fake_register_host_function(const char* name) {
+  TVMFunctionHandle f;
+  if (TVMFuncCreateFromCFunc(host_own_fn, NULL, NULL, &f) != 0) return -1;
+  return TVMFuncRegisterGlobal(name, f, 0);
+}
+int fake_is_host_function(const char* name) {
+  TVMFunctionHandle f = NULL;
+  TVMFuncGetGlobal(name, &f);
+  return f && ((Func*)f)->fn == host_own_fn;
 }
 int fake_num_registered(void) { return g_nnames; }
 const char* fake_registered_name(int i) { return g_names[i]; }

@@ -1,6 +1,25 @@
 """Helpers shared by the GPU parity tests."""
+import os
+import subprocess
+
 import numpy as np
 import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def build_cpp_program(name: str, force: bool = False) -> str:
+    """Compiles tests/cpp/<name>.cc (host code against include/ and the shared library, HIP runtime API
+    only) into tests/cpp/bin/<name> unless an up-to-date binary is there; returns its path."""
+    src = os.path.join(ROOT, "tests", "cpp", name + ".cc")
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", name)
+    libdir = os.path.join(ROOT, "relax_amd")
+    if force or not os.path.exists(exe) or os.path.getmtime(exe) < os.path.getmtime(src):
+        os.makedirs(os.path.dirname(exe), exist_ok=True)
+        subprocess.check_call(["g++", "-std=c++17", "-O1", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"),
+                               "-I", "/opt/rocm/include", src, "-o", exe, "-L", libdir, "-lrelax_amd_wq",
+                               "-L", "/opt/rocm/lib", "-lamdhip64", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"])
+    return exe
 
 
 def dev(a: np.ndarray) -> torch.Tensor:

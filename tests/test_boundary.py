@@ -168,11 +168,41 @@ def test_registers_with_a_tvm_runtime_when_present(tmp_path):
         assert fake.TVMFuncCall(f, vals, codes, n, ctypes.byref(rv), ctypes.byref(rc_code)) == -1
         fake.TVMGetLastError.restype = ctypes.c_char_p
         assert b"sm=95" in fake.TVMGetLastError()
+        # the array allocated for the failed call went back to the runtime: only the first result is live
+        assert fake.fake_live_arrays() == 1, fake.fake_live_arrays()
         print("registry ok", len(names))
     """)
     out = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
     assert "registry ok" in out.stdout
+
+
+def test_host_keeps_its_own_ft_preprocess_weight(tmp_path):
+    """A host whose registry already holds 'cutlass.ft_preprocess_weight' (a TVM built with its CUTLASS
+    back end) keeps it: the library registers its own 'relax_amd.*' names only."""
+    fake = tmp_path / "libfake_tvm_runtime.so"
+    subprocess.check_call(["gcc", "-shared", "-fPIC", "-O1", "-o", str(fake), os.path.join(ROOT, "tests", "fake_tvm_runtime.c")])
+    script = textwrap.dedent(f"""
+        import ctypes, sys
+        sys.path.insert(0, {ROOT!r})
+        fake = ctypes.CDLL({str(fake)!r}, mode=ctypes.RTLD_GLOBAL)
+        assert fake.fake_register_host_function(b"cutlass.ft_preprocess_weight") == 0
+        from relax_amd import _lib
+        lib = _lib.lib()
+        fake.fake_registered_name.restype = ctypes.c_char_p
+        names = [fake.fake_registered_name(i).decode() for i in range(fake.fake_num_registered())]
+        assert fake.fake_is_host_function(b"cutlass.ft_preprocess_weight") == 1
+        assert names.count("cutlass.ft_preprocess_weight") == 1
+        assert "relax_amd.ft_preprocess_weight_dps" in names and "relax_amd.q4f16_1_matmul" in names
+        assert len(names) == lib.wq_tvm_num_functions()
+        # a second registration replaces the library's own names and still leaves the host's alone
+        assert lib.wq_tvm_register_globals() == lib.wq_tvm_num_functions() - 1
+        assert fake.fake_is_host_function(b"cutlass.ft_preprocess_weight") == 1
+        print("policy ok")
+    """)
+    out = subprocess.run([sys.executable, "-c", script], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "policy ok" in out.stdout
 
 
 def test_source_compatible_headers_compile_and_run(tmp_path, lib):

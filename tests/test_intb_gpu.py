@@ -184,8 +184,16 @@ def test_int8_full_size_sampled(ops, u, oracle, M):
     got = u.host(ops.fpA_intB_gemm(u.dev(x), P, u.dev(s), weight_nbit=8))
     cols = np.concatenate([np.arange(0, 64), np.arange(14000, 14064), np.arange(N - 64, N)])
     A_cols = u.host(dA[:, torch.from_numpy(cols).cuda()].contiguous())
-    ref = oracle.intb_linear(x[: min(M, 8)], A_cols, s[cols], 8, nthreads=8)
-    u.assert_close(got[: min(M, 8)][:, cols], ref, f"int8 full M={M}")
+    # rows from every row tile of the kernels that serve these M (tiles of 128 and 256 rows)
+    rows = np.unique(np.clip(np.array([0, 7, 8, 15, 31, 32, 63, 64, 127, 128, 129, 255, 256, 300, 383, 384, 511]), 0, M - 1))
+    ref = oracle.intb_linear(x[rows], A_cols, s[cols], 8, nthreads=8)
+    u.assert_close(got[rows][:, cols], ref, f"int8 full M={M}")
+    if M > 2:
+        # every 61st row against the streaming kernel (an independent kernel), all columns
+        pick = np.arange(0, M, 61)
+        for r in pick:
+            yv = u.host(ops.fpA_intB_gemm(u.dev(x[r:r + 1]), P, u.dev(s), weight_nbit=8))
+            u.assert_close(got[r:r + 1], yv, f"int8 full M={M} row {r} vs gemv")
     if M == 1:
         xh = np.zeros((1, K), np.float16)
         xh[0, 4321] = 1

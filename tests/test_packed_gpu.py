@@ -67,14 +67,80 @@ def test_q4f16_1_matmul_family(env, oracle):
     assert rc == -1 and b"inconsistent" in lib.wq_last_error()
 
 
+def _decode_matmul_names():
+    """The 22 composite names of python/tvm/relax/backend/contrib/cutlass.py:305-312 (6 plain) and
+    :344-372 (16 residual blocks: {bias, bias_gelu} x {cast, no cast} x {add, multiply} x {relu, none})."""
+    names = ["decode_matmul", "decode_matmul_bias", "decode_matmul_cast", "decode_matmul_cast_bias",
+             "decode_matmul_bias_gelu", "decode_matmul_cast_bias_gelu"]
+    for cast in ("", "_cast"):
+        for act in ("", "_gelu"):
+            for op in ("add", "multiply"):
+                for relu in ("", "_relu"):
+                    names.append(f"decode_matmul{cast}_bias{act}_residual_{op}{relu}")
+    return names
+
+
+def test_decode_matmul_name_table_is_complete(env):
+    lib = env[0]
+    lib.wq_tvm_function_name.restype = ctypes.c_char_p
+    have = {lib.wq_tvm_function_name(i).decode() for i in range(lib.wq_tvm_num_functions())}
+    want = {"relax_amd." + n for n in _decode_matmul_names()}
+    assert len(want) == 22
+    assert want == {n for n in have if n.startswith("relax_amd.decode_matmul")}
+
+
 @pytest.mark.parametrize("nbit", [8, 4])
-def test_decode_matmul_composites(env, oracle, nbit):
+@pytest.mark.parametrize("name", _decode_matmul_names())
+def test_decode_matmul_composites(env, oracle, name, nbit):
+    """Every composite PackedFunc, epilogue derived from its name, against the oracle; M = 48 runs the
+    small-batch kernel, M = 200 the MFMA GEMM."""
+    from relax_amd import ops
+
+    lib, u, T, torch = env
+    N, K = 128, 256
+    okw = {}
+    if "_bias" in name:
+        okw["bias"] = True
+    if "_gelu" in name:
+        okw["activation"] = "gelu"
+    if "_residual_add" in name:
+        okw["binary_op"] = "plus"
+    if "_residual_multiply" in name:
+        okw["binary_op"] = "multiply"
+    if name.endswith("_relu"):
+        okw["unary_op"] = "relu"
+    sym = getattr(lib, "relax_amd_" + name)
+    for M in (48, 200):
+        x, A, s = oracle.make_intb_inputs(M, N, K, nbit, seed=nbit + M)
+        rng = np.random.default_rng(2 + M)
+        bias = rng.standard_normal((1, N)).astype(np.float16)
+        res = rng.standard_normal((M, N)).astype(np.float16)
+        P = ops.ft_preprocess_weight(u.dev(A), 80, nbit == 4)
+        out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        tens = [T.from_torch(t)[0] for t in (u.dev(x), P, u.dev(s.reshape(1, N)))]
+        kw = dict(okw)
+        if "bias" in kw:
+            tens.append(T.from_torch(u.dev(bias))[0])
+            kw["bias"] = bias.reshape(-1)
+        if "binary_op" in kw:
+            tens.append(T.from_torch(u.dev(res))[0])
+            kw["residual"] = res
+        tens.append(T.from_torch(out)[0])
+        print(f"{name} int{nbit} M={M}", flush=True)
+        rc, _, _ = T.call(sym, *tens)
+        assert rc == 0, (name, lib.wq_last_error())
+        u.assert_close(u.host(out), oracle.intb_linear(x, A, s, nbit, nthreads=4, **kw), f"{name} int{nbit} M={M}")
+        # one argument short is refused
+        rc, _, _ = T.call(sym, *tens[:-1])
+        assert rc == -1, name
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_decode_matmul_preprocess_and_full_bias(env, oracle, nbit):
     lib, u, T, torch = env
     M, N, K = 48, 128, 256
     x, A, s = oracle.make_intb_inputs(M, N, K, nbit, seed=nbit)
     rng = np.random.default_rng(2)
-    bias = rng.standard_normal((1, N)).astype(np.float16)
-    res = rng.standard_normal((M, N)).astype(np.float16)
     dA = u.dev(A)
     # weight reordering through the DPS PackedFunc on device tensors
     P = torch.empty_like(dA)
@@ -83,26 +149,10 @@ def test_decode_matmul_composites(env, oracle, nbit):
     rc, _, _ = T.call(lib.relax_amd_ft_preprocess_weight_dps, tA, 80, int(nbit == 4), tP)
     assert rc == 0, lib.wq_last_error()
     assert np.array_equal(u.host(P), oracle.ft_preprocess(A, nbit == 4, 80))
-    dx, ds, db, dr = u.dev(x), u.dev(s.reshape(1, N)), u.dev(bias), u.dev(res)
     out = torch.empty((M, N), dtype=torch.float16, device="cuda")
-    tx, _ = T.from_torch(dx)
-    ts, _ = T.from_torch(ds)
-    tb, _ = T.from_torch(db)
-    tr, _ = T.from_torch(dr)
+    tx, _ = T.from_torch(u.dev(x))
+    ts, _ = T.from_torch(u.dev(s.reshape(1, N)))
     to, _ = T.from_torch(out)
-    cases = [
-        ("relax_amd_decode_matmul", (tx, tP, ts, to), {}),
-        ("relax_amd_decode_matmul_cast_bias", (tx, tP, ts, tb, to), dict(bias=bias)),
-        ("relax_amd_decode_matmul_bias_gelu", (tx, tP, ts, tb, to), dict(bias=bias, activation="gelu")),
-        ("relax_amd_decode_matmul_bias_residual_add", (tx, tP, ts, tb, tr, to), dict(bias=bias, residual=res, binary_op="plus")),
-        ("relax_amd_decode_matmul_bias_gelu_residual_multiply_relu", (tx, tP, ts, tb, tr, to),
-         dict(bias=bias, activation="gelu", residual=res, binary_op="multiply", unary_op="relu")),
-    ]
-    for sym, args, okw in cases:
-        rc, _, _ = T.call(getattr(lib, sym), *args)
-        assert rc == 0, (sym, lib.wq_last_error())
-        ref = oracle.intb_linear(x, A, s, nbit, nthreads=4, **{k: (v.reshape(-1) if k == "bias" else v) for k, v in okw.items()})
-        u.assert_close(u.host(out), ref, sym)
     # a bias that varies along M selects bias_stride = N (python/tvm/contrib/cutlass/build.py:728-734)
     bias2 = rng.standard_normal((M, N)).astype(np.float16)
     tb2, _ = T.from_torch(u.dev(bias2))
@@ -185,3 +235,41 @@ def test_autogptq_family(env, oracle):
     assert rc == -1
     rc, _, _ = T.call(lib.relax_amd_autogptq_matmul, tW, tSZ, tp, tx2, tr, ty2, tws)
     assert rc == -1 and b"inconsistent" in lib.wq_last_error()
+
+
+@pytest.mark.parametrize("case,nbit,group,M", [("int8_percol", 8, -1, 40), ("int8_nobias", 8, -1, 1),
+                                               ("int8_percol", 8, -1, 300), ("int4_fine", 4, 64, 24),
+                                               ("int4_fine", 4, 64, 260)])
+def test_emitted_host_code_runs_on_device(env, oracle, tmp_path, case, nbit, group, M):
+    """tests/cpp/ft_api_device.cc calls fastertransformer::gemm_fp16_int_bias_act<uint8_t, PER_COLUMN_SCALE_ONLY>
+    and ..._residual<cutlass::uint4b_t, FINEGRAINED_SCALE_ONLY> on device buffers with the argument lists the
+    reference emits (python/tvm/contrib/cutlass/gemm_operation.py:441-458), as its own process."""
+    import subprocess
+
+    from relax_amd import ops
+
+    lib, u, T, torch = env
+    N, K = 192, 512
+    x, A, s = oracle.make_intb_inputs(M, N, K, nbit, seed=M + nbit, group_size=group)
+    rng = np.random.default_rng(M)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    P = u.host(ops.ft_preprocess_weight(u.dev(A), 80, nbit == 4))
+    x.tofile(tmp_path / "A.bin")
+    P.tofile(tmp_path / "B.bin")
+    s.tofile(tmp_path / "scales.bin")
+    kw = {}
+    if case != "int8_nobias":
+        bias.tofile(tmp_path / "bias.bin")
+        kw["bias"] = bias
+    if case == "int8_percol":
+        kw["activation"] = "gelu"
+    if case == "int4_fine":
+        res.tofile(tmp_path / "residual.bin")
+        kw.update(residual=res, binary_op="plus", unary_op="relu", group_size=64)
+    exe = u.build_cpp_program("ft_api_device")
+    print(f"ft_api_device {case} M={M}", flush=True)
+    r = subprocess.run([exe, case, str(tmp_path), str(M), str(N), str(K)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(tmp_path / "C.bin", np.float16).reshape(M, N)
+    u.assert_close(got, oracle.intb_linear(x, A, s, nbit, nthreads=4, **kw), f"emitted host code {case} M={M}")

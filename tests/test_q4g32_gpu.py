@@ -202,6 +202,19 @@ def test_small_batch_vs_oracle(ops, u, oracle, nw, waves, stages, M, N, K):
     u.assert_close(got, ref, f"small batch nw{nw} waves{waves} {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M", [8, 32])
+@pytest.mark.parametrize("N,K", [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)])
+def test_llama7b_shapes_at_decode_batches(ops, u, oracle, M, N, K):
+    """The four Llama-2-7B linears at the batch sizes of the 32-layer stack, at full size: the
+    small-batch kernel selected explicitly and whatever the automatic dispatch picks."""
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=M + N + K)
+    print(f"llama shape M={M} N={N} K={K}", flush=True)
+    ref = oracle.q4g32_linear(W, S, x, nthreads=8)
+    dW, dS, dx = u.dev(W), u.dev(S), u.dev(x)
+    u.assert_close(u.host(ops.q4g32_linear(dW, dS, dx, kernel="small_batch")), ref, f"small batch {M}x{N}x{K}")
+    u.assert_close(u.host(ops.q4g32_linear(dW, dS, dx)), ref, f"automatic {M}x{N}x{K}")
+
+
 def test_small_batch_epilogue_and_dispatch(ops, u, oracle):
     M, N, K = 24, 200, 512
     x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=19)

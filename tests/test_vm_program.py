@@ -156,6 +156,109 @@ def test_linear_stack_program_matches_oracle_eager_and_replayed(oracle, M):
 
 
 @pytest.mark.gpu
+def test_llama7b_stack_full_size_matches_oracle(oracle):
+    """The real 32-layer program (128 instructions, 3.6 GB of codes and scales) at M = 1, 8, 32, eager and
+    replayed.  Checked against the oracle: `out` (the last down_proj, which depends only on mlp_act), and
+    two taps in the middle of the stack that each sit behind a dependency through planned storage:
+    gate_up_proj of layer 15 (reads that layer's o_proj result) and qkv_proj of layer 16 (reads the hidden
+    state written by layer 15's down_proj)."""
+    import torch
+
+    from relax_amd import vm
+    from tests import gpu_util as u
+
+    L = 32
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    weights = []
+    for _ in range(L):
+        layer = {}
+        for name, N, K in vm.LLAMA7B_LINEARS:
+            W = torch.randint(-2**31, 2**31 - 1, (N, K // 8), dtype=torch.int32, device="cuda", generator=g)
+            S = (torch.rand((N, K // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+            layer[name] = (W, S)
+        weights.append(layer)
+
+    def host_ws(l, name):
+        W, S = weights[l][name]
+        return u.host(W).view(np.uint32), u.host(S)
+
+    stream = torch.cuda.Stream()
+    for M in (1, 8, 32):
+        print(f"llama stack M={M}", flush=True)
+        rng = np.random.default_rng(40 + M)
+        hidden = rng.standard_normal((M, 4096)).astype(np.float16)
+        attn = rng.standard_normal((M, 4096)).astype(np.float16)
+        act = (rng.standard_normal((M, 11008)) * 0.5).astype(np.float16)
+        out = torch.zeros((M, 4096), dtype=torch.float16, device="cuda")
+        tap_gu = torch.zeros((M, 22016), dtype=torch.float16, device="cuda")
+        tap_qkv = torch.zeros((M, 12288), dtype=torch.float16, device="cuda")
+        prog = vm.llama_linear_stack(weights, M, u.dev(hidden), u.dev(attn), u.dev(act), out,
+                                     taps={(15, "gate_up_proj"): tap_gu, (16, "qkv_proj"): tap_qkv})
+        assert prog.num_instructions == 4 * L
+        prog.plan()
+        want_out = oracle.q4g32_linear(*host_ws(L - 1, "down_proj"), act, nthreads=8)
+        o15 = oracle.q4g32_linear(*host_ws(15, "o_proj"), attn, nthreads=8)
+        want_gu = oracle.q4g32_linear(*host_ws(15, "gate_up_proj"), o15, nthreads=8)
+        h16 = oracle.q4g32_linear(*host_ws(15, "down_proj"), act, nthreads=8)
+        want_qkv = oracle.q4g32_linear(*host_ws(16, "qkv_proj"), h16, nthreads=8)
+
+        def check(what):
+            u.assert_close(u.host(out), want_out, f"stack M={M} {what}: out")
+            u.assert_close(u.host(tap_gu), want_gu, f"stack M={M} {what}: gate_up of layer 15")
+            u.assert_close(u.host(tap_qkv), want_qkv, f"stack M={M} {what}: qkv of layer 16")
+
+        prog.run(stream)
+        stream.synchronize()
+        check("eager")
+        eager = [t.clone() for t in (out, tap_gu, tap_qkv)]
+        prog.capture(stream)
+        for rep in range(2):
+            for t in (out, tap_gu, tap_qkv):
+                t.zero_()
+            torch.cuda.synchronize()
+            prog.replay(stream)
+            stream.synchronize()
+            check(f"replay {rep}")
+            for t, e in zip((out, tap_gu, tap_qkv), eager):
+                assert torch.equal(t, e), (M, rep)
+        del prog
+
+
+@pytest.mark.gpu
+def test_rebind_drops_the_captured_graph(oracle):
+    """After a rebind the captured graph would still address the old tensor: replay is refused until the
+    program is captured again, and the new capture reads the new tensor."""
+    import torch
+
+    from relax_amd import vm
+    from relax_amd._lib import WqError
+    from tests import gpu_util as u
+
+    M, N, K = 2, 64, 128
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=4)
+    x2 = (x * 0.5).astype(np.float16)
+    p = vm.DpsProgram()
+    X = p.external(u.dev(x))
+    y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    p.call("relax_amd.q4f16_1_matmul", p.external(u.dev(W), as_uint32=True), p.external(u.dev(S)), X, p.external(y))
+    p.plan()
+    stream = torch.cuda.Stream()
+    p.capture(stream)
+    p.replay(stream)
+    stream.synchronize()
+    u.assert_close(u.host(y), oracle.q4g32_linear(W, S, x), "first binding")
+    p.rebind(X, u.dev(x2))
+    with pytest.raises(WqError, match="nothing captured"):
+        p.replay(stream)
+    p.capture(stream)
+    p.replay(stream)
+    stream.synchronize()
+    u.assert_close(u.host(y), oracle.q4g32_linear(W, S, x2), "second binding")
+    assert len(p._keep) == 4  # one tensor per external register: the first x was released
+
+
+@pytest.mark.gpu
 def test_program_reports_callee_errors():
     import torch
 
