@@ -117,15 +117,17 @@ def test_decode_matmul_composites(env, oracle, name, nbit):
         res = rng.standard_normal((M, N)).astype(np.float16)
         P = ops.ft_preprocess_weight(u.dev(A), 80, nbit == 4)
         out = torch.empty((M, N), dtype=torch.float16, device="cuda")
-        tens = [T.from_torch(t)[0] for t in (u.dev(x), P, u.dev(s.reshape(1, N)))]
+        held = [u.dev(x), P, u.dev(s.reshape(1, N))]  # device tensors stay referenced during the call
         kw = dict(okw)
         if "bias" in kw:
-            tens.append(T.from_torch(u.dev(bias))[0])
+            held.append(u.dev(bias))
             kw["bias"] = bias.reshape(-1)
         if "binary_op" in kw:
-            tens.append(T.from_torch(u.dev(res))[0])
+            held.append(u.dev(res))
             kw["residual"] = res
-        tens.append(T.from_torch(out)[0])
+        held.append(out)
+        packed = [T.from_torch(t) for t in held]
+        tens = [t for t, _ in packed]
         print(f"{name} int{nbit} M={M}", flush=True)
         rc, _, _ = T.call(sym, *tens)
         assert rc == 0, (name, lib.wq_last_error())
@@ -150,12 +152,14 @@ def test_decode_matmul_preprocess_and_full_bias(env, oracle, nbit):
     assert rc == 0, lib.wq_last_error()
     assert np.array_equal(u.host(P), oracle.ft_preprocess(A, nbit == 4, 80))
     out = torch.empty((M, N), dtype=torch.float16, device="cuda")
-    tx, _ = T.from_torch(u.dev(x))
-    ts, _ = T.from_torch(u.dev(s.reshape(1, N)))
+    dx, ds = u.dev(x), u.dev(s.reshape(1, N))
+    tx, _ = T.from_torch(dx)
+    ts, _ = T.from_torch(ds)
     to, _ = T.from_torch(out)
     # a bias that varies along M selects bias_stride = N (python/tvm/contrib/cutlass/build.py:728-734)
     bias2 = rng.standard_normal((M, N)).astype(np.float16)
-    tb2, _ = T.from_torch(u.dev(bias2))
+    db2 = u.dev(bias2)
+    tb2, _ = T.from_torch(db2)
     rc, _, _ = T.call(lib.relax_amd_decode_matmul_bias, tx, tP, ts, tb2, to)
     assert rc == 0
     u.assert_close(u.host(out), oracle.intb_linear(x, A, s, nbit, bias=bias2, bias_stride=N, nthreads=4), "full bias")
