@@ -215,6 +215,19 @@ int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm
                    const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
                    int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream);
 
+/* wq_gptq_linear for callers that cannot allocate device memory and have no workspace to
+ * pass (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same arguments and results as wq_gptq_linear without the
+ * workspace: with a row order the gathered activations go to a buffer built into the library
+ * (WQ_GPTQ_NOALLOC_MAX_BYTES of device memory per GPU, held until the process ends), so
+ * M*K*2 must not exceed that size; larger problems are refused with WQ_EINVAL.  The call
+ * allocates nothing.  Every call on a GPU shares that GPU's buffer: calls that overlap in time
+ * on one GPU (different streams) race; calls on one stream are ordered. */
+#define WQ_GPTQ_NOALLOC_MAX_BYTES (1u << 20)
+int wq_gptq_linear_noalloc(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
+                           const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
+                           int64_t K, int64_t G, wq_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * Calibration kernels: the measured ceilings reported next to the vendor peaks
  * (no counterpart in the reference; its methodology precedent is the cache-flush

@@ -34,6 +34,7 @@ SIGNATURES = {
     "wq_gptq_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_int), _i64, _i64, _i64, _vp],
     "wq_gptq_workspace_bytes": [_i64, _i64, _int],
     "wq_gptq_linear": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp],
+    "wq_gptq_linear_noalloc": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "wq_intb_encode": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "wq_q4g32_encode": [_vp, _vp, _vp, _i64, _i64, _vp],
     "wq_calibrate_mfma_f16": [_vp, _i64, _int, ctypes.POINTER(ctypes.c_double), _vp],

@@ -16,6 +16,8 @@
 // and the streaming GEMV (q4_gemv.h), the small-batch kernel (skinny_gemm.h) and the MFMA GEMM
 // (mfma_gemm_lds.h) all take it.
 // A g_idx whose groups do not all have K/G members is rejected by the preparation.
+#include <mutex>
+
 #include "mfma_gemm_lds.h"
 #include "q4_gemv.h"
 #include "q4g32_common.h"
@@ -304,11 +306,75 @@ extern "C" size_t wq_gptq_workspace_bytes(int64_t M, int64_t K, int has_perm) {
   return (has_perm && M > 0 && K > 0) ? (size_t)M * (size_t)K * 2 : 0;
 }
 
+namespace wq {
+static int gptq_linear_impl(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
+                            const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
+                            int64_t K, int64_t G, void* workspace, size_t workspace_bytes, hipStream_t stream);
+}
+
 extern "C" int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
                               const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
-                              int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream_) {
+                              int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream) {
+  return wq::gptq_linear_impl(W_nk, SZ, perm, x, bias, residual, y, M, N, K, G, workspace, workspace_bytes,
+                              (hipStream_t)stream);
+}
+
+// ---- the same linear for callers that cannot allocate: the gathered activations live in a
+// ---- file-scope device array instead of a caller workspace
+namespace wq {
+
+constexpr size_t kGptqScratchBytes = WQ_GPTQ_NOALLOC_MAX_BYTES;
+// One copy per GPU, held until the process ends.  In host code this name is only a handle
+// for hipGetSymbolAddress; kernels receive the address looked up below.
+static __device__ __align__(256) unsigned char scratch[kGptqScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int gptq_scratch_for_current_device(void** out) {
+  int dev = -1;
+  WQ_HIP(hipGetDevice(&dev));
+  WQ_REQUIRE(dev >= 0 && dev < kMaxDevices, "wq_gptq_linear_noalloc: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    WQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    WQ_REQUIRE(p && aligned16(p), "wq_gptq_linear_noalloc: no device address for the scratch array");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return WQ_OK;
+}
+
+}  // namespace wq
+
+extern "C" int wq_gptq_linear_noalloc(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm,
+                                      const uint16_t* x, const uint16_t* bias, const uint16_t* residual,
+                                      uint16_t* y, int64_t M, int64_t N, int64_t K, int64_t G,
+                                      wq_stream_t stream) {
   using namespace wq;
-  hipStream_t stream = (hipStream_t)stream_;
+  void* ws = nullptr;
+  size_t ws_bytes = 0;
+  if (perm && M > 0 && N > 0 && K > 0) {
+    WQ_REQUIRE(M < (1ll << 30) && K <= 32768, "wq_gptq_linear_noalloc: M=%lld K=%lld outside the supported range",
+               (long long)M, (long long)K);
+    const size_t need = (size_t)M * (size_t)K * 2;
+    WQ_REQUIRE(need <= kGptqScratchBytes,
+               "wq_gptq_linear_noalloc: the gathered activations need M*K*2 = %zu bytes, the built-in scratch "
+               "buffer holds %zu; use wq_gptq_linear with a workspace",
+               need, kGptqScratchBytes);
+    if (int rc = gptq_scratch_for_current_device(&ws)) return rc;
+    ws_bytes = kGptqScratchBytes;
+  }
+  return gptq_linear_impl(W_nk, SZ, perm, x, bias, residual, y, M, N, K, G, ws, ws_bytes, (hipStream_t)stream);
+}
+
+static int wq::gptq_linear_impl(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
+                                const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
+                                int64_t K, int64_t G, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  using namespace wq;
   WQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G >= 0, "wq_gptq_linear: negative dimension");
   if (M == 0 || N == 0) return WQ_OK;
   WQ_REQUIRE(K > 0 && G > 0 && K % G == 0, "wq_gptq_linear: K=%lld is not a positive multiple of the %lld groups",
