@@ -93,6 +93,46 @@ int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x, const
                   const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
                   wq_stream_t stream);
 
+/* A list of decode linears (M = 1 each) as ONE launch: what a decoder layer, or a whole stack
+ * of them, asks of python/tvm/dlight/gpu/gemv.py:216-530 one generated kernel at a time.  A grid
+ * of persistent workgroups walks the list; the weights of the next linear are already streaming
+ * while the current one finishes, and a linear whose x is the y of an earlier linear of the list
+ * (found from the addresses) waits on a device-side counter instead of a kernel boundary.
+ *   create  validates, finds the dependencies, uploads the descriptor table into `workspace`
+ *           (256-byte aligned device memory of wq_q4g32_gemv_list_workspace_bytes(n) bytes, owned
+ *           by the caller and left alone until destroy) and synchronises `stream`: a load-time call.
+ *           Outputs must not overlap any operand of an earlier linear of the list other than as that
+ *           dependency (refused with WQ_EUNSUPPORTED); bias / residual must come from outside the list.
+ *   run     one asynchronous launch on `stream`; no allocation, no synchronisation: capturable.
+ *           Launches of one list must not overlap in time (they share the counters).
+ *   status  synchronises `stream` and reports a wait that ran into the spin limit (WQ_EDEVICE):
+ *           this happens only if the grid could not be resident at once, e.g. while another
+ *           kernel holds CUs; the results of that launch are undefined.
+ * NULL from create / non-zero from the others: see wq_last_error(). */
+typedef struct wq_q4g32_gemv_desc {
+  const uint32_t* W;        /* uint32 [N, K/8] */
+  const uint16_t* S;        /* fp16 [N, K/32] */
+  const uint16_t* x;        /* fp16 [K] */
+  const uint16_t* bias;     /* fp16 [N] or NULL */
+  const uint16_t* residual; /* fp16 [N] or NULL */
+  uint16_t* y;              /* fp16 [N] */
+  int64_t N, K;             /* K % 32 == 0, K <= WQ_GEMV_LIST_MAX_K */
+} wq_q4g32_gemv_desc;
+typedef struct wq_gemv_list wq_gemv_list_t;
+#define WQ_GEMV_LIST_MAX 4096
+#define WQ_GEMV_LIST_MAX_K 16384
+size_t wq_q4g32_gemv_list_workspace_bytes(int n);
+wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* descs, int n, void* workspace,
+                                          size_t workspace_bytes, wq_stream_t stream);
+int wq_q4g32_gemv_list_run(wq_gemv_list_t* list, wq_stream_t stream);
+int wq_q4g32_gemv_list_status(wq_gemv_list_t* list, wq_stream_t stream);
+void wq_q4g32_gemv_list_destroy(wq_gemv_list_t* list);
+/* How many linears of the list wait for an earlier one, and how many of those for the linear
+ * directly in front of them (those cannot overlap with it; order lists to keep this number low). */
+int wq_q4g32_gemv_list_info(const wq_gemv_list_t* list, int* dependencies, int* adjacent);
+/* Upper bound of one wait in ticks of the 100 MHz wall clock (default 2 s). */
+int wq_q4g32_gemv_list_set_spin_limit(wq_gemv_list_t* list, long long ticks);
+
 /* ------------------------------------------------------------------------- *
  * Format B — fp16 activations x int8 / int4 weights (per-channel or group-64 scales).
  *   packed weight  int8 [K, N]   or  int4 as int8 [K, N/2] (two's complement

@@ -24,6 +24,13 @@ SIGNATURES = {
     "wq_q4g32_gemv": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_small_batch": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "wq_q4g32_gemv_list_workspace_bytes": [_int],
+    "wq_q4g32_gemv_list_create": [_vp, _int, _vp, _sz, _vp],
+    "wq_q4g32_gemv_list_run": [_vp, _vp],
+    "wq_q4g32_gemv_list_status": [_vp, _vp],
+    "wq_q4g32_gemv_list_destroy": [_vp],
+    "wq_q4g32_gemv_list_info": [_vp, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)],
+    "wq_q4g32_gemv_list_set_spin_limit": [_vp, ctypes.c_longlong],
     "wq_ft_preprocess_weight_host": [_vp, _vp, _i64, _i64, _i64, _int, _int],
     "wq_ft_preprocess_weight": [_vp, _vp, _i64, _i64, _i64, _int, _int, _vp],
     "wq_intb_dequantize": [_vp, _vp, _vp, _i64, _i64, _int, _i64, _vp],
@@ -58,7 +65,8 @@ SIGNATURES = {
 }
 _RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p, "wq_program_create": _vp,
              "wq_program_destroy": None, "wq_program_plan": _i64, "wq_program_unplanned_bytes": _i64,
-             "wq_gptq_workspace_bytes": _sz}
+             "wq_gptq_workspace_bytes": _sz, "wq_q4g32_gemv_list_workspace_bytes": _sz,
+             "wq_q4g32_gemv_list_create": _vp, "wq_q4g32_gemv_list_destroy": None}
 
 _lib = None
 

@@ -11,6 +11,8 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+if os.path.dirname(HERE) not in sys.path:
+    sys.path.insert(0, os.path.dirname(HERE))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librelax_amd_wq.so")
 OBJDIR = os.path.join(HERE, "build")
@@ -62,7 +64,7 @@ def _stale(src: str) -> bool:
     if not os.path.exists(obj):
         return True
     t = os.path.getmtime(obj)
-    return any(os.path.getmtime(d) > t for d in _deps(src)) or os.path.getmtime(__file__) > t
+    return any(os.path.getmtime(d) > t for d in _deps(src))
 
 
 def build(verbose: bool = True, incremental: bool = False) -> str:
@@ -74,6 +76,11 @@ def build(verbose: bool = True, incremental: bool = False) -> str:
     if todo:
         with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(todo))) as ex:
             list(ex.map(_compile, todo))
+    if any(os.path.basename(s) == "q4g32_gemv_list.hip" for s in todo):
+        # that kernel waits for its inline-assembly loads by hand: verify the generated code
+        from relax_amd import check_ring_asm
+
+        check_ring_asm.main(HIPCC, [f for f in FLAGS if f != "-fPIC"])
     objs = [os.path.join(OBJDIR, os.path.basename(s) + ".o") for s in srcs]
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     subprocess.check_call(cmd)

@@ -1,0 +1,112 @@
+"""Build-time check of the generated code of ``csrc/q4g32_gemv_list.hip``.
+
+The compute wavefronts of that kernel load their weight stream with inline-assembly loads into a
+ring of registers and wait for them by hand, so the compiler does not know that those registers are
+in flight between a load and its wait.  The source makes every read of a ring register an asm
+statement that depends on the wait; what is left to chance is register allocation (a copy or a
+spill of a ring register inserted between load and wait would read it too early).  This script
+compiles the file to assembly and verifies, in the kernel's text, that
+
+* every ring register (destination of a ``global_load_* ... nt`` instruction) is read only by the
+  three unpack instructions the source uses (``v_and_or_b32``, ``v_lshrrev_b32 .., 8, ..``,
+  ``v_cvt_f32_f16``), never by a move, a store or anything else, and
+* each ring slot keeps one register in the prologue and in the loop (no renaming copies).
+
+Registers that the compiler also uses for short-lived temporaries while a slot is empty are
+recognised by being written by another instruction first.
+"""
+from __future__ import annotations
+
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "csrc", "q4g32_gemv_list.hip")
+ALLOWED_READERS = ("v_and_or_b32", "v_lshrrev_b32", "v_cvt_f32_f16")
+
+
+def _regs(tok: str):
+    """'v[4:7]' -> {4,5,6,7}; 'v12' -> {12}; anything else -> empty."""
+    m = re.fullmatch(r"v\[(\d+):(\d+)\]", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.fullmatch(r"v(\d+)", tok)
+    return {int(m.group(1))} if m else set()
+
+
+def _check_function(body: list[str]) -> list[str]:
+    errors = []
+    ring = set()
+    for l in body:
+        if l.startswith("global_load_") and l.endswith(" nt"):
+            ring |= _regs(l.split()[1].rstrip(","))
+    if not ring:
+        return []
+    # walk the text; a ring register is "loaded" after a ring load wrote it and until something else writes it
+    loaded = set()
+    for l in body:
+        parts = l.replace(",", " ").split()
+        op, ops = parts[0], parts[1:]
+        if op.startswith("global_load_") and l.endswith(" nt"):
+            loaded |= _regs(ops[0])
+            continue
+        if not ops:
+            continue
+        stores = ("global_store", "ds_write", "buffer_store", "scratch_store", "global_atomic", "ds_add")
+        writes = _regs(ops[0]) if not op.startswith(("s_",) + stores) else set()
+        reads = set()
+        for t in (ops if not writes else ops[1:]):
+            reads |= _regs(t)
+        if op.startswith(stores):
+            reads |= _regs(ops[0])
+        hit = reads & loaded
+        if hit and not op.startswith(ALLOWED_READERS):
+            errors.append(f"ring register(s) {sorted(hit)} read by `{l}`")
+        if op.startswith("v_lshrrev_b32") and hit and ops[1] != "8":
+            errors.append(f"unexpected shift of a ring register: `{l}`")
+        loaded -= writes  # now a temporary of the compiler
+    return errors
+
+
+def check(asm_text: str) -> list[str]:
+    """Checks every kernel of the file on its own (register names mean nothing across kernels)."""
+    lines = [l.split(";")[0].strip() for l in asm_text.splitlines()]
+    functions, cur = [], None
+    for l in lines:
+        if not l:
+            continue
+        if l.endswith(":") and not l.startswith("."):  # a function label
+            cur = []
+            functions.append(cur)
+        elif l.startswith(".Lfunc_end"):
+            cur = None
+        elif cur is not None and not l.startswith(".") and not l.endswith(":"):
+            cur.append(l)
+    errors, with_ring = [], 0
+    for body in functions:
+        if any(l.startswith("global_load_") and l.endswith(" nt") for l in body):
+            with_ring += 1
+            errors += _check_function(body)
+    if with_ring == 0:
+        return ["no ring loads found (expected global_load_* ... nt in q4g32_gemv_list_kernel)"]
+    return errors
+
+
+def main(hipcc="/opt/rocm/bin/hipcc", flags=()):
+    with tempfile.TemporaryDirectory() as td:
+        out = os.path.join(td, "k.s")
+        subprocess.check_call([hipcc, *flags, "-S", "--cuda-device-only", SRC, "-o", out], stderr=subprocess.DEVNULL)
+        errs = check(open(out).read())
+    if errs:
+        raise RuntimeError("q4g32_gemv_list.hip: the generated code touches in-flight ring registers:\n  " + "\n  ".join(errs[:20]))
+    return True
+
+
+if __name__ == "__main__":
+    from relax_amd import build as _b  # noqa: E402
+
+    main(_b.HIPCC, [f for f in _b.FLAGS if f != "-fPIC"])
+    print("ring registers: ok")

@@ -1,0 +1,706 @@
+// A list of format-A (q4f16_1) decode linears, M = 1 each, in ONE launch.
+//
+// Why.  One decode linear reads 9 .. 50 MB; as a kernel of its own it lasts 4 .. 11 us, of which
+// about 2.7 us are launch gap, ramp-up and drain.  A decoder layer is a list of such linears, so the
+// list is executed by one grid of persistent workgroups that walks it: the weight stream of the
+// next linear is already in flight while the current one finishes, and a linear that reads what an
+// earlier one wrote waits on a device-side counter instead of a kernel boundary.
+//
+// Workgroup = NC compute wavefronts + 2 service wavefronts, one workgroup per CU.
+//   * A compute wavefront owns whole rows: row r of a linear belongs to wavefront r mod (all
+//     compute wavefronts of the grid).  A row is streamed in chunks of 64 scale groups (2048 k,
+//     1 KiB of codes: one 16-byte load and one scale per lane).  The chunks of all its rows, over
+//     all linears, form one stream that runs through a ring of D register slots: the loads of chunk
+//     f + D are issued when chunk f has been consumed, also across the boundary between two
+//     linears.  Compute wavefronts issue no other vector memory operation, so the compiler's
+//     s_waitcnt vmcnt(2(D-1)) in front of each consume is exact.  Arithmetic per chunk as in the
+//     single-linear kernel (q4_gemv.h): 1 shift + 4 v_and_or + 4 v_dot2 per 8 weights, zero point
+//     and scale applied once per group.  Row sums go to LDS, not to memory.
+//   * The service wavefronts do everything irregular, each at its own pace, up to NB (2..4) linears
+//     ahead of or behind the compute wavefronts; LDS words (ListFlags) hand the NB buffer slots over.
+//     The x wavefront waits for a producer linear (bounded spin), loads the activations of a coming
+//     linear, rearranges them to the pairing of the unpack, computes the zero-point constants and
+//     writes both to LDS.  The y wavefront takes the finished row sums of a linear from LDS, applies
+//     bias / cast / residual, stores y, and signals completion.
+//
+// Dependencies.  Linear i may read the y of an earlier linear `dep` of the same list.  Each
+// workgroup adds 1 to one of 8 counters of linear `dep` once its stores of y (device scope, written
+// through) have completed; the x wavefront of a consumer spins until the 8 counters sum to the number
+// of workgroups and then reads x with device-scope loads (no cache is written back or invalidated:
+// a release / acquire fence pair at agent scope costs about 10 us per linear here), for at most `spin_limit` ticks of the 100 MHz wall clock: after that it raises the
+// error word, stops waiting for anything and lets every wavefront run to the end (results are then
+// undefined, the host reads the error word).  The grid is sized so that all workgroups are resident
+// at once; the bounded wait is what keeps a launch that is not (another kernel holding CUs) from
+// hanging.  If dep == i - 1 nothing can overlap: the compute wavefronts idle (their ring stays
+// loaded) until the producer has finished everywhere; callers order lists so that this is rare.
+// The last workgroup to finish clears the counters for the next launch.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <vector>
+
+#include "wq_device.h"
+#include "wq_host.h"
+
+namespace wq {
+
+struct GemvListDesc {  // 64 bytes, device memory
+  const char* W;       // uint32 [N, K/8]
+  const char* S;       // fp16   [N, K/32]
+  const half_t* x;     // fp16   [K]
+  const half_t* bias;  // fp16   [N] or null
+  const half_t* residual;  // fp16 [N] or null
+  half_t* y;           // fp16   [N]
+  int32_t N;
+  int32_t q;           // row groups / workgroups  (a row group is 2^gs consecutive rows)
+  uint32_t g_dep;      // bits 0..15: K / 32; bits 16..30: 1 + the linear of this list that writes x (0: none);
+                       // bit 31: a later linear reads y
+  uint16_t rem;        // row groups % workgroups
+  uint16_t off;        // rotation: workgroup b owns the row groups local * workgroups + ((b - off) mod workgroups)
+};
+static_assert(sizeof(GemvListDesc) == 64, "descriptor layout");
+constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y
+
+typedef const GemvListDesc __attribute__((address_space(4)))* gemv_desc_ptr;  // scalar loads
+
+constexpr int kCounterStride = 16;   // ints between two counters (64 bytes: one cache line each)
+constexpr int kCountersPerLinear = 8;
+constexpr int kChunkBytes = 4096 + 256;
+constexpr int kBufferFlags = 0x00020000;  // buffer resource word 3: 32-bit data format, no swizzle
+constexpr int kDeviceScope = 16;          // cache policy bit sc1: the access is coherent over the whole device  // LDS bytes per chunk of x: 4 x 64 uint4 + 64 floats
+
+// sync layout (ints): [lin][8] counters at stride kCounterStride, then `finished`, then `error`
+__host__ __device__ inline int sync_counter_index(int lin, int k) { return (lin * kCountersPerLinear + k) * kCounterStride; }
+__host__ __device__ inline int sync_finished_index(int nlin) { return sync_counter_index(nlin, 0); }
+__host__ __device__ inline int sync_error_index(int nlin) { return sync_counter_index(nlin, 1); }
+__host__ __device__ inline int sync_ints(int nlin) { return sync_counter_index(nlin, 2); }
+
+__device__ __forceinline__ void lds_done_then_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// ---- where a workgroup's rows are: its rows of all linears, in list order, form one sequence of
+// ---- positions 0, 1, 2, ...; a cursor maps a position to (linear, local row).  Forward only.
+struct RowCursor {
+  int lin;          // current linear (nlin: past the end)
+  int base;         // position of its first row
+  int R;            // positions of it that belong to this workgroup (whole row groups)
+  int rb;           // (b - off) mod workgroups: row group = local group * workgroups + rb
+  int N;            // rows of the linear (positions of a last, partial row group beyond N are empty)
+  int C, glast;     // chunks per row, groups in the last chunk (1..64)
+  int row_w, row_s; // bytes per row of W and S
+  const char* W;
+  const char* S;
+};
+
+__device__ __forceinline__ void row_cursor_load(RowCursor& cu, gemv_desc_ptr descs, int nlin, int b, int nwg, int gs) {
+  if (cu.lin >= nlin) {
+    cu.R = 0x7fffffff;  // every position from here on is "past the end"
+    return;
+  }
+  // the whole descriptor with one scalar load (W, S: words 0..3; N, q, g_dep, rem | off << 16: 12..15)
+  typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
+  const words_ptr p = (words_ptr)(descs + cu.lin);
+  uint32_t w[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) w[i] = p[i];
+  const int G = (int)(w[14] & 0xffffu);
+  const int K = G << 5;
+  int rb = b - (int)(w[15] >> 16);
+  if (rb < 0) rb += nwg;
+  cu.rb = rb;
+  cu.N = (int)w[12];
+  cu.R = ((int)w[13] + (rb < (int)(w[15] & 0xffffu) ? 1 : 0)) << gs;
+  cu.C = (G + 63) >> 6;
+  cu.glast = G - (cu.C - 1) * 64;
+  cu.row_w = K >> 1;
+  cu.row_s = G * 2;
+  cu.W = reinterpret_cast<const char*>(((uint64_t)w[1] << 32) | w[0]);
+  cu.S = reinterpret_cast<const char*>(((uint64_t)w[3] << 32) | w[2]);
+}
+
+// moves the cursor to the linear that holds position `pos`
+__device__ __forceinline__ void row_cursor_seek(RowCursor& cu, int pos, gemv_desc_ptr descs, int nlin, int b, int nwg, int gs) {
+  while (cu.lin < nlin && pos >= cu.base + cu.R) {
+    cu.base += cu.R;
+    ++cu.lin;
+    row_cursor_load(cu, descs, nlin, b, nwg, gs);
+  }
+}
+
+// row of the linear at position `pos` of the workgroup's sequence (may be >= N in a partial last group)
+__device__ __forceinline__ int64_t row_cursor_row(const RowCursor& cu, int pos, int nwg, int gs) {
+  const int lp = pos - cu.base;
+  return ((((int64_t)(lp >> gs)) * nwg + cu.rb) << gs) + (lp & ((1 << gs) - 1));
+}
+
+// LDS words that hand the buffers over inside a workgroup.  Activations live in NB (2 or 4) slots
+// (slot = linear mod NB), row sums in kYSlots slots (linear mod kYSlots):
+//   x_ready[slot]  = j + 1 once the activations of linear j are staged            (written by an x wavefront)
+//   left[slot]     += 1 by every compute wavefront that is done with a linear of that slot (cumulative)
+//   flushed        = j + 1 once the row sums of linears 0..j have been stored to y (written by the y wavefront)
+constexpr int kMaxSlots = 4;
+constexpr int kYSlots = 8;
+struct ListFlags {
+  int x_ready[kMaxSlots];
+  int left[kMaxSlots];
+  int flushed;
+  int next_pos;  // the next position of the workgroup's row sequence that nobody has taken
+  int pad[6];
+};
+
+__device__ __forceinline__ void lds_spin_until(const int* flag, int target) {
+  while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) __builtin_amdgcn_s_sleep(1);
+  asm volatile("" ::: "memory");  // LDS is served in order: what was written before the flag is visible now
+}
+
+#ifdef WQ_LIST_TRACE
+__device__ long long* g_list_trace = nullptr;  // [workgroup 0 | workgroup 100][64] wall-clock stamps
+#define WQ_TR(i)                                                                                   \
+  do {                                                                                             \
+    if (g_list_trace && (blockIdx.x == 0 || blockIdx.x == 100) && (threadIdx.x & 63) == 0 && (i) < 64) \
+      g_list_trace[(blockIdx.x ? 64 : 0) + (i)] = wall_clock64();                                  \
+  } while (0)
+#else
+#define WQ_TR(i) do { } while (0)
+#endif
+
+template <int NC, int XW, int D>
+__global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(const GemvListDesc* __restrict__ descs_,
+                                                                        int nlin, int* __restrict__ sync,
+                                                                        long long spin_limit, int xbuf_bytes,
+                                                                        int ybuf_floats, int nb_log2, int gs, int use_sync) {
+  const int nb = 1 << nb_log2;
+  extern __shared__ uint4_t smem[];
+  const gemv_desc_ptr descs = (gemv_desc_ptr)descs_;
+  char* lds = reinterpret_cast<char*>(smem);
+  // flags, then nb x buffers of xbuf_bytes each, then kYSlots y buffers of ybuf_floats floats
+  ListFlags* flags = reinterpret_cast<ListFlags*>(lds);
+  char* xbuf = lds + sizeof(ListFlags);
+  float* ybuf = reinterpret_cast<float*>(xbuf + nb * xbuf_bytes);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nwg = gridDim.x;
+
+  if (wave < NC) {
+    // =========================== compute wavefront ===========================
+    // Rows are taken one at a time from the workgroup's sequence (an LDS counter), so the NC
+    // wavefronts stay balanced whatever the row lengths; the next position is fetched one row ahead.
+    const int b = blockIdx.x;
+    const uint32_t lane16 = lane * 16;
+    if (tid < (int)(sizeof(ListFlags) / sizeof(int))) reinterpret_cast<int*>(flags)[tid] = 0;
+    lds_done_then_barrier();  // LDS starts undefined: the flags are cleared before anyone looks
+
+    auto take_position = [&]() {
+      int p = 0;
+      if (lane == 0) p = __hip_atomic_fetch_add(&flags->next_pos, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      return p;  // valid in lane 0; read with readfirstlane where it is used
+    };
+
+    // The ring.  Its loads are written in assembly and waited for by hand: loads retire in order and
+    // a compute wavefront issues no other vector memory operation, so with all D slots in flight the
+    // oldest one has landed when at most 2 (D - 1) loads are outstanding.  (Left to the compiler, the
+    // counts come out right only as long as every path through the loop issues the same loads.)
+    // A wavefront issues one instruction every four cycles, so what a chunk costs is its instruction
+    // count: everything a chunk needs when it is consumed (where its activations are, where its row
+    // sum goes) is worked out when it is issued, once per row where possible, and kept per slot.
+    uint4_t rw[D];
+    uint32_t rs[D];
+    int slot_lin[D];    // linear of the chunk in the slot; -1: the slot is empty
+    int slot_x[D];      // LDS byte offset of the chunk's activations
+    int slot_y[D];      // LDS byte offset of the row sum if this is the row's last chunk, else -1
+    int slot_gl[D];     // groups in the chunk (64, or fewer in a partial last chunk)
+    int inflight = 0;   // slots issued and not yet consumed
+    const int xbuf0 = (int)sizeof(ListFlags);
+    const int ybuf0 = xbuf0 + nb * xbuf_bytes;
+
+    // issue side: the row being issued, and the next position (fetched one row ahead)
+    RowCursor ic;
+    ic.lin = 0;
+    ic.base = 0;
+    row_cursor_load(ic, descs, nlin, b, nwg, gs);
+    int inext = take_position();
+    int i_c = 0, i_xbase = 0, i_ypos = 0;
+    const char* i_wb = nullptr;
+    const char* i_sb = nullptr;
+    uint32_t i_part16 = 0;  // lane offset in a partial last chunk: idle lanes shadow the last group
+    int i_part_lin = -1;
+    auto next_row = [&]() {  // the next position that holds a row (a last, partial row group has empty ones)
+      int64_t row;
+      int pos;
+      do {
+        pos = __builtin_amdgcn_readfirstlane(inext);
+        inext = take_position();
+        row_cursor_seek(ic, pos, descs, nlin, b, nwg, gs);
+        row = row_cursor_row(ic, pos, nwg, gs);
+      } while (ic.lin < nlin && row >= ic.N);
+      if (ic.lin >= nlin) return;
+      if (i_part_lin != ic.lin) {
+        i_part_lin = ic.lin;
+        i_part16 = min(lane, ic.glast - 1) * 16;
+      }
+      i_c = 0;
+      i_wb = ic.W + row * ic.row_w;
+      i_sb = ic.S + row * ic.row_s;
+      i_xbase = xbuf0 + (ic.lin & (nb - 1)) * xbuf_bytes;
+      i_ypos = ybuf0 + ((ic.lin & (kYSlots - 1)) * ybuf_floats + (pos - ic.base)) * 4;
+    };
+    next_row();
+
+    auto issue = [&](uint4_t& w, uint32_t& s, int& slin, int& sx, int& sy, int& sgl) {
+      slin = -1;
+      if (ic.lin >= nlin) return;
+      const bool last = i_c == ic.C - 1;
+      const bool partial = last && ic.glast < 64;
+      const uint32_t voff = partial ? i_part16 : lane16;
+      const uint32_t soff = voff >> 3;
+      asm volatile(
+          "global_load_dwordx4 %0, %2, %3 nt\n\t"
+          "global_load_ushort %1, %4, %5 nt"
+          : "=&v"(w), "=&v"(s)
+          : "v"(voff), "s"(i_wb), "v"(soff), "s"(i_sb));
+      slin = ic.lin;
+      sx = i_xbase + i_c * kChunkBytes;
+      sy = last ? i_ypos : -1;
+      sgl = partial ? ic.glast : 64;
+      ++inflight;
+      if (last) {
+        next_row();
+      } else {
+        ++i_c;
+        i_wb += 1024;
+        i_sb += 128;
+      }
+    };
+
+    // Every compute wavefront passes through every linear, also those in which it takes no row:
+    // leaving linear e says "my row sums of e are in LDS and I no longer read its activations".
+    int entered = -1;
+    auto advance_to = [&](int lin) {
+      while (entered < lin) {
+        if (entered >= 0) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          if (lane == 0)
+            __hip_atomic_fetch_add(&flags->left[entered & (nb - 1)], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        ++entered;
+        if (entered < nlin) lds_spin_until(&flags->x_ready[entered & (nb - 1)], entered + 1);
+      }
+    };
+
+    // `magic` (0x6400 in both halves, OR-ed under every code) doubles as the token that orders the
+    // reads of a ring slot behind the wait for it: the wait is an asm statement that "modifies"
+    // magic, and every instruction that reads a ring register is an asm statement that takes magic as
+    // an operand.  The ring registers themselves appear in no other statement, so nothing can read
+    // or copy them between their load and their wait (the build checks this in the generated code).
+    uint32_t magic = 0x64006400u;
+    float acc = 0.0f;
+    auto ring_shr8 = [&](uint32_t word) {
+      uint32_t r;
+      asm("v_lshrrev_b32 %0, 8, %1 ; %2" : "=v"(r) : "v"(word), "v"(magic));
+      return r;
+    };
+    auto ring_scale = [&](uint32_t s16) {
+      float r;
+      asm("v_cvt_f32_f16 %0, %1 ; %2" : "=v"(r) : "v"(s16), "v"(magic));
+      return r;
+    };
+    auto consume = [&](const uint4_t& w4, const uint32_t& s16, int lin, int sx, int sy, int gl) {
+      if (lin != entered) advance_to(lin);
+      uint32_t lo = lane16;
+      if (gl < 64) lo = min(lane, gl - 1) * 16;
+      const char* xb = lds + sx;
+      uint4_t xv[4];
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) xv[ch] = *reinterpret_cast<const uint4_t*>(xb + ch * 1024 + lo);
+      float grp = *reinterpret_cast<const float*>(xb + 4096 + (lo >> 2));
+      // this slot is the oldest in flight
+      if (inflight == D) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"(2 * (D - 1)));
+      else asm volatile("s_waitcnt vmcnt(0)" : "+v"(magic));
+      --inflight;
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) {
+        const uint32_t word = ch == 0 ? w4.x : ch == 1 ? w4.y : ch == 2 ? w4.z : w4.w;
+        const uint32_t w8 = ring_shr8(word);
+        const half2_t t0 = as_half2(and_or(word, 0x000F000Fu, magic));  // 1024 + (q0, q4)
+        const half2_t t1 = as_half2(and_or(word, 0x00F000F0u, magic));  // 1024 + 16*(q1, q5)
+        const half2_t t2 = as_half2(and_or(w8, 0x000F000Fu, magic));    // 1024 + (q2, q6)
+        const half2_t t3 = as_half2(and_or(w8, 0x00F000F0u, magic));    // 1024 + 16*(q3, q7)
+        grp = dot2(t0, as_half2(xv[ch].x), grp);
+        grp = dot2(t1, as_half2(xv[ch].y), grp);
+        grp = dot2(t2, as_half2(xv[ch].z), grp);
+        grp = dot2(t3, as_half2(xv[ch].w), grp);
+      }
+      float sf = ring_scale(s16);
+      if (gl < 64 && lane >= gl) sf = 0.0f;
+      acc = fmaf(sf, grp, acc);
+      if (sy >= 0) {
+        const float tot = wave_sum_to_lane63(acc);
+        if (lane == 63) *reinterpret_cast<float*>(lds + sy) = tot;
+        acc = 0.0f;
+      }
+    };
+
+#pragma unroll
+    for (int s = 0; s < D; ++s) issue(rw[s], rs[s], slot_lin[s], slot_x[s], slot_y[s], slot_gl[s]);
+    while (inflight > 0) {
+#pragma unroll
+      for (int s = 0; s < D; ++s) {
+        if (slot_lin[s] >= 0) consume(rw[s], rs[s], slot_lin[s], slot_x[s], slot_y[s], slot_gl[s]);
+        issue(rw[s], rs[s], slot_lin[s], slot_x[s], slot_y[s], slot_gl[s]);
+      }
+    }
+    advance_to(nlin);
+    return;
+  }
+
+  lds_done_then_barrier();  // the flags are cleared
+  bool aborted = false;
+
+  if (wave < NC + XW) {
+    // ====================== x wavefronts: activations -> LDS ======================
+    // x wavefront k stages the linears k, k + XW, k + 2 XW, ...
+    // until every workgroup has signalled linear `dep`, or the spin limit passes
+    auto wait_for = [&](int dep) {
+      if (aborted) return;
+      const long long t0 = wall_clock64();
+      while (true) {
+        int v = 0;
+        if (lane < kCountersPerLinear)
+          v = __hip_atomic_load(sync + sync_counter_index(dep, lane), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 4, 64);
+        if (__builtin_amdgcn_readfirstlane(v) >= nwg) break;
+        if (wall_clock64() - t0 > spin_limit) {
+          aborted = true;
+          if (lane == 0)
+            __hip_atomic_store(sync + sync_error_index(nlin), dep + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+    };
+
+    const half2_t k1031 = {(half_t)1031.0f, (half_t)1031.0f};
+    const half2_t k71 = {(half_t)71.0f, (half_t)71.0f};
+    const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+    for (int j = wave - NC; j < nlin; j += XW) {
+      const int slot = j & (nb - 1);
+      // the slot is free once every compute wavefront has left the linear that used it before; the
+      // row-sum slot of linear j once the sums of linear j - kYSlots have been stored
+      if (j >= nb) lds_spin_until(&flags->left[slot], NC * (((j - nb) >> nb_log2) + 1));
+      if (j >= kYSlots) lds_spin_until(&flags->flushed, j - kYSlots + 1);
+      const int dep = (int)((descs[j].g_dep >> 16) & 0x7fffu) - 1;
+      if (dep >= 0) wait_for(dep);
+      if (j < 16) WQ_TR(32 + j);
+      const int K = (int)(descs[j].g_dep & 0xffffu) << 5;
+      // an x that other workgroups of this launch have written is read with device-scope loads
+      // (sc1), which see what device-scope stores followed by the counter update have published,
+      // without invalidating any cache; an x from outside the list with ordinary loads
+      const __amdgpu_buffer_rsrc_t xr =
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(descs[j].x), 0, K * 2, kBufferFlags);
+      char* xb = xbuf + slot * xbuf_bytes;
+      const int nwords = K >> 3;  // 16-byte words of 8 activations; a multiple of 4
+      constexpr int U = 16;       // loads in flight per lane: one round trip per 16 KiB of x
+      for (int base = 0; base < nwords; base += 64 * U) {
+        uint4_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int wi = base + u * 64 + lane;
+          if (wi < nwords)
+            v[u] = dep >= 0 ? __builtin_amdgcn_raw_buffer_load_b128(xr, wi * 16, 0, kDeviceScope)
+                            : __builtin_amdgcn_raw_buffer_load_b128(xr, wi * 16, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int wi = base + u * 64 + lane;
+          if (wi < nwords) {  // a quad of lanes (one group) is in or out together
+            const uint32_t in[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+            uint32_t o[4];
+            pair_i_i4(in, o);  // o[i] = (x_i, x_{i+4})
+            float c = dot2(as_half2(o[0]), k1031, 0.0f);
+            c = dot2(as_half2(o[1]), k71, c);
+            c = dot2(as_half2(o[2]), k1031, c);
+            c = dot2(as_half2(o[3]), k71, c);
+            c += dpp_shift<0xb1, 0xf>(c);  // the 4 words of a group sit in 4 adjacent lanes
+            c += dpp_shift<0x4e, 0xf>(c);
+            const int grp = wi >> 2, ch = wi & 3;
+            char* cb = xb + (grp >> 6) * kChunkBytes;
+            *reinterpret_cast<uint4_t*>(cb + ch * 1024 + (grp & 63) * 16) =
+                uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
+            if (ch == 0) *reinterpret_cast<float*>(cb + 4096 + (grp & 63) * 4) = -c;
+          }
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      if (lane == 0) __hip_atomic_store(&flags->x_ready[slot], j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (j < 16) WQ_TR(48 + j);
+    }
+    return;
+  }
+
+  // ================== y wavefront: row sums -> y, completion signals ==================
+  for (int j = 0; j < nlin; ++j) {
+    const int slot = j & (nb - 1);
+    lds_spin_until(&flags->left[slot], NC * ((j >> nb_log2) + 1));
+    if (j < 16) WQ_TR(j);
+    const half_t* bias = descs[j].bias;
+    const half_t* residual = descs[j].residual;
+    const float* yb = ybuf + (j & (kYSlots - 1)) * ybuf_floats;
+    int rb = (int)blockIdx.x - (int)descs[j].off;
+    if (rb < 0) rb += nwg;
+    const int N = descs[j].N;
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[j].y, 0, N * 2, kBufferFlags);
+    const int R = (descs[j].q + (rb < (int)descs[j].rem ? 1 : 0)) << gs;
+    for (int idx = lane; idx < R; idx += 64) {
+      const int64_t n = ((((int64_t)(idx >> gs)) * nwg + rb) << gs) + (idx & ((1 << gs) - 1));
+      if (n < N) {
+        float v = yb[idx];
+        if (bias) v += (float)bias[n];
+        half_t h = (half_t)v;
+        if (residual) h = h + residual[n];
+        // device-scope store: written through, so that a counter update after it publishes it
+        __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (int)n * 2, 0, kDeviceScope);
+      }
+    }
+    // the row sums are in registers or stored: the slot may be written again
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (lane == 0) __hip_atomic_store(&flags->flushed, j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (descs[j].g_dep & kSignal) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores of this workgroup have been written through
+      if (lane == 0)
+        __hip_atomic_fetch_add(sync + sync_counter_index(j, blockIdx.x & (kCountersPerLinear - 1)), 1,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (j < 16) WQ_TR(16 + j);
+  }
+  if (!use_sync) return;
+  // the last workgroup to get here clears the counters for the next launch (every wait of this
+  // workgroup lies behind it: its last row sums could only be stored after all its activations were staged)
+  int last = 0;
+  if (lane == 0)
+    last = __hip_atomic_fetch_add(sync + sync_finished_index(nlin), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+           nwg - 1;
+  if (__builtin_amdgcn_readfirstlane(last)) {
+    for (int i = lane; i < nlin * kCountersPerLinear; i += 64)
+      __hip_atomic_store(sync + i * kCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0)
+      __hip_atomic_store(sync + sync_finished_index(nlin), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+}  // namespace wq
+
+namespace wq {
+// ------------------------------------------------------------------ host side
+struct GemvListConfig {
+  int nc, depth, blocks_per_cu;
+};
+
+static bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a && b && na && nb && a0 < b0 + nb && b0 < a0 + na;
+}
+
+}  // namespace wq
+
+struct wq_gemv_list {
+  std::vector<wq::GemvListDesc> descs;
+  int n = 0;
+  void* table = nullptr;  // device: descriptors
+  int* sync = nullptr;    // device: counters
+  int blocks = 0, threads = 0;
+  size_t lds = 0;
+  int xbuf_bytes = 0, ybuf_floats = 0;
+  int late = 0, deps = 0;
+  int nb = 2;
+  int gs = 2;  // log2 of the rows per row group
+  int depth = 4;
+  long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
+};
+
+namespace wq {
+
+constexpr int kListNC = 13;    // compute wavefronts per workgroup
+constexpr int kListXW = 2;     // wavefronts that stage activations
+constexpr int kListDepth = 4;  // ring slots (KiB of codes in flight) per compute wavefront: 52 KiB per CU
+constexpr size_t kListAlign = 256;
+
+typedef void (*list_kernel_t)(const GemvListDesc*, int, int*, long long, int, int, int, int, int);
+static list_kernel_t list_kernel_for(int depth) {
+  switch (depth) {
+    case 2: return q4g32_gemv_list_kernel<kListNC, kListXW, 2>;
+    case 3: return q4g32_gemv_list_kernel<kListNC, kListXW, 3>;
+    case 4: return q4g32_gemv_list_kernel<kListNC, kListXW, 4>;
+    case 6: return q4g32_gemv_list_kernel<kListNC, kListXW, 6>;
+    default: return nullptr;
+  }
+}
+
+static size_t list_table_bytes(int n) { return ((size_t)n * sizeof(GemvListDesc) + kListAlign - 1) / kListAlign * kListAlign; }
+
+}  // namespace wq
+
+extern "C" size_t wq_q4g32_gemv_list_workspace_bytes(int n) {
+  if (n <= 0) return 0;
+  return wq::list_table_bytes(n) + (size_t)wq::sync_ints(n) * sizeof(int);
+}
+
+extern "C" void wq_q4g32_gemv_list_destroy(wq_gemv_list_t* l) { delete l; }
+
+extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d, int n, void* workspace,
+                                                     size_t workspace_bytes, wq_stream_t stream_) {
+  using namespace wq;
+  hipStream_t stream = (hipStream_t)stream_;
+#define bad(code, ...) ((void)fail(code, __VA_ARGS__), (wq_gemv_list_t*)nullptr)
+  if (!d || n <= 0 || n > WQ_GEMV_LIST_MAX) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: need 1 .. %d linears, got %d", WQ_GEMV_LIST_MAX, n);
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & (kListAlign - 1)) ||
+      workspace_bytes < wq_q4g32_gemv_list_workspace_bytes(n))
+    return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: workspace must be 256-byte aligned device memory of %zu bytes",
+               wq_q4g32_gemv_list_workspace_bytes(n));
+  std::unique_ptr<wq_gemv_list> l(new wq_gemv_list());
+  l->n = n;
+  l->descs.resize(n);
+  int cmax = 1;
+  for (int i = 0; i < n; ++i) {
+    const wq_q4g32_gemv_desc& s = d[i];
+    if (s.N <= 0 || s.K <= 0 || s.K % 32 != 0 || s.K > WQ_GEMV_LIST_MAX_K || s.N >= (1ll << 30))
+      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: N=%lld K=%lld (K must be a positive multiple of 32, at most %d)",
+                 i, (long long)s.N, (long long)s.K, WQ_GEMV_LIST_MAX_K);
+    if (!s.W || !s.S || !s.x || !s.y) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: null pointer", i);
+    if (!aligned16(s.W) || !aligned16(s.x))
+      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: W and x must be 16-byte aligned", i);
+    GemvListDesc& g = l->descs[i];
+    g.W = reinterpret_cast<const char*>(s.W);
+    g.S = reinterpret_cast<const char*>(s.S);
+    g.x = reinterpret_cast<const half_t*>(s.x);
+    g.bias = reinterpret_cast<const half_t*>(s.bias);
+    g.residual = reinterpret_cast<const half_t*>(s.residual);
+    g.y = reinterpret_cast<half_t*>(s.y);
+    g.N = (int32_t)s.N;
+    g.q = 0;  // q, rem, off: once the grid is known
+    g.g_dep = (uint32_t)(s.K / 32);
+    g.rem = 0;
+    g.off = 0;
+    cmax = std::max(cmax, (int)((s.K / 32 + 63) / 64));
+  }
+  // Who reads what an earlier linear of the list wrote.  Writing over something an earlier linear
+  // still reads or wrote is refused: workgroups are not synchronised except through `dep`.
+  for (int i = 0; i < n; ++i) {
+    const wq_q4g32_gemv_desc& a = d[i];
+    for (int j = i - 1; j >= 0; --j) {
+      const wq_q4g32_gemv_desc& b = d[j];
+      const size_t yb = (size_t)b.N * 2, ya = (size_t)a.N * 2;
+      if (((l->descs[i].g_dep >> 16) & 0x7fffu) == 0 && ranges_overlap(a.x, (size_t)a.K * 2, b.y, yb))
+        l->descs[i].g_dep |= (uint32_t)(j + 1) << 16;
+      if (ranges_overlap(a.residual, ya, b.y, yb) || ranges_overlap(a.bias, ya, b.y, yb))
+        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i, j);
+      if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, (size_t)b.K * 2) ||
+          ranges_overlap(a.y, ya, b.residual, yb) || ranges_overlap(a.y, ya, b.bias, yb))
+        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the output of linear %d overlaps an operand of linear %d", i, j);
+    }
+    if (ranges_overlap(a.y, (size_t)a.N * 2, a.x, (size_t)a.K * 2))
+      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: y overlaps x", i);
+    const int dep = (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1;
+    if (dep >= 0) {
+      l->descs[dep].g_dep |= kSignal;
+      ++l->deps;
+      if (dep == i - 1) ++l->late;
+    }
+  }
+  // launch shape: one workgroup of 16 wavefronts per CU.  Workgroup b owns the rows
+  // n = local * workgroups + ((b - off) mod workgroups); `off` continues the round-robin where the
+  // previous linear ended, so that the remainders of all linears spread over the workgroups.
+  l->threads = 64 * (kListNC + kListXW + 1);
+  l->blocks = std::min(cu_count(), 32768);
+  l->gs = getenv("WQ_LIST_GS") ? atoi(getenv("WQ_LIST_GS")) : 2;
+  int64_t turns = 1;
+  int64_t off = 0;
+  for (int i = 0; i < n; ++i) {
+    GemvListDesc& g = l->descs[i];
+    const int64_t groups = (d[i].N + (1 << l->gs) - 1) >> l->gs;
+    g.q = (int32_t)(groups / l->blocks);
+    g.rem = (uint16_t)(groups % l->blocks);
+    g.off = (uint16_t)off;
+    off = (off + groups) % l->blocks;
+    turns = std::max<int64_t>(turns, ((groups + l->blocks - 1) / l->blocks) << l->gs);
+  }
+  l->xbuf_bytes = cmax * kChunkBytes;
+  l->ybuf_floats = (int)((turns + 63) / 64 * 64);
+  // 4 buffer slots (linears the service wavefronts may run ahead of or behind the compute wavefronts) if they fit, else 2
+  const size_t fixed = sizeof(ListFlags) + (size_t)kYSlots * l->ybuf_floats * sizeof(float);
+  const size_t room = fixed < 150 * 1024 ? 150 * 1024 - fixed : 0;
+  l->nb = room / l->xbuf_bytes >= 4 ? 4 : room / l->xbuf_bytes >= 2 ? 2 : 0;
+  if (l->nb < 2) return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations and row sums do not fit the LDS");
+  l->lds = fixed + (size_t)l->nb * l->xbuf_bytes;
+  l->depth = getenv("WQ_LIST_D") ? atoi(getenv("WQ_LIST_D")) : kListDepth;
+  auto kern = list_kernel_for(l->depth);
+  if (!kern) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: no kernel for ring depth %d", l->depth);
+  if (l->lds > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)l->lds) != hipSuccess)
+    return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
+  int resident = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
+    return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: the workgroup does not fit a CU (%zu bytes of LDS)", l->lds);
+  l->table = workspace;
+  l->sync = reinterpret_cast<int*>(static_cast<char*>(workspace) + list_table_bytes(n));
+  if (hipMemcpyAsync(l->table, l->descs.data(), (size_t)n * sizeof(GemvListDesc), hipMemcpyHostToDevice, stream) != hipSuccess ||
+      hipMemsetAsync(l->sync, 0, (size_t)sync_ints(n) * sizeof(int), stream) != hipSuccess ||
+      hipStreamSynchronize(stream) != hipSuccess)
+    return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: could not upload the descriptor table");
+  return l.release();
+#undef bad
+}
+
+extern "C" int wq_q4g32_gemv_list_run(wq_gemv_list_t* l, wq_stream_t stream) {
+  using namespace wq;
+  WQ_REQUIRE(l && l->table, "wq_q4g32_gemv_list_run: null list");
+  WQ_LAUNCH("wq_q4g32_gemv_list_run", list_kernel_for(l->depth), dim3((unsigned)l->blocks),
+            dim3((unsigned)l->threads), l->lds, (hipStream_t)stream, (const GemvListDesc*)l->table, l->n, l->sync,
+            l->spin_limit, l->xbuf_bytes, l->ybuf_floats, l->nb == 4 ? 2 : 1, l->gs, l->deps > 0 ? 1 : 0);
+  return WQ_OK;
+}
+
+extern "C" int wq_q4g32_gemv_list_status(wq_gemv_list_t* l, wq_stream_t stream) {
+  using namespace wq;
+  WQ_REQUIRE(l && l->table, "wq_q4g32_gemv_list_status: null list");
+  int err = 0;
+  int* p = l->sync + sync_error_index(l->n);
+  WQ_HIP(hipMemcpyAsync(&err, p, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  WQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+  if (err == 0) return WQ_OK;
+  // the counters may be mid-count after an abandoned wait: start clean
+  WQ_HIP(hipMemsetAsync(l->sync, 0, (size_t)sync_ints(l->n) * sizeof(int), (hipStream_t)stream));
+  WQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return fail(WQ_EDEVICE,
+              "wq_q4g32_gemv_list: a wait for linear %d timed out (the grid was not resident at once?); "
+              "results of that launch are undefined",
+              err - 1);
+}
+
+extern "C" int wq_q4g32_gemv_list_info(const wq_gemv_list_t* l, int* dependencies, int* adjacent) {
+  using namespace wq;
+  WQ_REQUIRE(l, "wq_q4g32_gemv_list_info: null list");
+  if (dependencies) *dependencies = l->deps;
+  if (adjacent) *adjacent = l->late;
+  return WQ_OK;
+}
+
+extern "C" int wq_q4g32_gemv_list_set_spin_limit(wq_gemv_list_t* l, long long ticks) {
+  using namespace wq;
+  WQ_REQUIRE(l && ticks >= 0, "wq_q4g32_gemv_list_set_spin_limit: bad argument");
+  l->spin_limit = ticks;
+  return WQ_OK;
+}
+
+#ifdef WQ_LIST_TRACE
+extern "C" __attribute__((visibility("default"))) int wq_debug_list_trace(long long* device_buffer) {
+  return hipMemcpyToSymbol(HIP_SYMBOL(wq::g_list_trace), &device_buffer, sizeof(device_buffer)) == hipSuccess ? 0 : -1;
+}
+#endif

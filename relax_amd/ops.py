@@ -116,6 +116,74 @@ def q4g32_linear(W: torch.Tensor, S: torch.Tensor, x: torch.Tensor, bias: Option
     return out
 
 
+class GemvDesc(ctypes.Structure):
+    """``wq_q4g32_gemv_desc`` of include/relax_amd_wq.h."""
+    _fields_ = [("W", ctypes.c_void_p), ("S", ctypes.c_void_p), ("x", ctypes.c_void_p), ("bias", ctypes.c_void_p),
+                ("residual", ctypes.c_void_p), ("y", ctypes.c_void_p), ("N", ctypes.c_int64), ("K", ctypes.c_int64)]
+
+
+class Q4G32GemvList:
+    """A list of decode linears (M = 1 each) run as ONE launch (``wq_q4g32_gemv_list_*``).
+
+    ``linears``: sequence of ``(W, S, x, y)`` or ``(W, S, x, y, bias, residual)`` device tensors; a linear
+    whose ``x`` is the ``y`` of an earlier one waits for it on the device.  The tensors are kept alive by
+    this object; the descriptor table and the counters live in a workspace allocated here, once.
+    """
+
+    def __init__(self, linears):
+        self._l = _lib.lib()
+        n = len(linears)
+        arr = (GemvDesc * max(1, n))()
+        self._keep = []
+        for i, lin in enumerate(linears):
+            W, S, x, y = lin[:4]
+            bias = lin[4] if len(lin) > 4 else None
+            residual = lin[5] if len(lin) > 5 else None
+            W = _w32(W)
+            S = _dev(S, torch.float16, "S")
+            x = _dev(x, torch.float16, "x")
+            y = _dev(y, torch.float16, "y")
+            N, kw = W.shape
+            K = kw * 8
+            if K % 32 or tuple(S.shape) != (N, K // 32):
+                raise ValueError(f"linear {i}: S must be [N, K/32] = [{N}, {K // 32}], got {tuple(S.shape)}")
+            if x.numel() != K or y.numel() != N:
+                raise ValueError(f"linear {i}: x must hold K={K} and y N={N} elements (one row each)")
+            for t, name in ((bias, "bias"), (residual, "residual")):
+                if t is not None and _dev(t, torch.float16, name).numel() != N:
+                    raise ValueError(f"linear {i}: {name} must hold N={N} elements")
+            arr[i] = GemvDesc(_ptr(W), _ptr(S), _ptr(x), _ptr(bias), _ptr(residual), _ptr(y), N, K)
+            self._keep.append((W, S, x, y, bias, residual))
+        need = self._l.wq_q4g32_gemv_list_workspace_bytes(n)
+        self._workspace = torch.zeros(max(int(need), 256), dtype=torch.uint8, device="cuda")
+        self._h = self._l.wq_q4g32_gemv_list_create(arr, n, self._workspace.data_ptr(), self._workspace.numel(),
+                                                    _stream())
+        if not self._h:
+            raise _lib.WqError("wq_q4g32_gemv_list_create failed: " + self._l.wq_last_error().decode())
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._l.wq_q4g32_gemv_list_destroy(self._h)
+            self._h = None
+
+    def run(self) -> None:
+        """One asynchronous launch on torch's current stream."""
+        check(self._l.wq_q4g32_gemv_list_run(self._h, _stream()), "wq_q4g32_gemv_list_run")
+
+    def status(self) -> None:
+        """Synchronises and raises if a device-side wait of an earlier launch timed out."""
+        check(self._l.wq_q4g32_gemv_list_status(self._h, _stream()), "wq_q4g32_gemv_list_status")
+
+    def info(self):
+        """(linears that wait for an earlier one, of which for the one directly in front)."""
+        a, b = ctypes.c_int(0), ctypes.c_int(0)
+        check(self._l.wq_q4g32_gemv_list_info(self._h, ctypes.byref(a), ctypes.byref(b)), "wq_q4g32_gemv_list_info")
+        return a.value, b.value
+
+    def set_spin_limit(self, ticks: int) -> None:
+        check(self._l.wq_q4g32_gemv_list_set_spin_limit(self._h, ticks), "wq_q4g32_gemv_list_set_spin_limit")
+
+
 # ----------------------------------------------------------------- format B
 
 
