@@ -3,10 +3,15 @@
 
 One step = one pass of the four Llama-2-7B-shaped decode linears at batch M=1
 (int4 codes packed 8 per uint32 along K, group 32, fp16 scales, zero point 7):
-4096->12288 (fused QKV), 4096->4096 (o_proj), 4096->22016 (gate/up), 11008->4096 (down).
+4096->12288 (fused QKV), 4096->4096 (o_proj), 4096->22016 (gate/up), 11008->4096 (down),
+issued as ONE launch of the list kernel (wq_q4g32_gemv_list_run).
 Inputs are synthetic and resident in HBM before the timed region.  Each step
 reads a different copy of the weights (a ring of copies larger than the
 256 MB last-level cache), so the reported GB/s is HBM traffic, not cache hits.
+
+Timing protocol (after src/runtime/profiling.cc:862-933 of the reference): untimed warm-up, then
+`--samples` (5) samples, each a whole number of repetitions that lasts at least `--min-sample-ms`
+(100 ms), HIP events on the launch stream; the median is reported, min and max beside it.
 
 Prints ONE JSON line.  `value` is algorithmic bytes per second over the whole
 step; `roofline` describes the decode GEMV kernel, `gemm` the M=2048 prefill
@@ -36,12 +41,19 @@ PREFILL_SHAPES = [(11008, 4096), (4096, 11008)]
 PREFILL_M = 2048
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch, averaged over the four decode shapes resp. the two prefill
-# shapes: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one run each) of this script,
-# scaled by what the same counters read for a plain 1 GiB device copy
-# (`--calibrate-copy`): x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28747852
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 268700000
+# HBM bytes per launch of the two headline kernels come from rocprofv3 counters collected offline
+# (this script cannot read hardware counters): profiles/hbm_traffic.json holds the figures, the
+# summary they were taken from and its date; it is copied into the JSON line, or null if absent.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def offline_traffic(kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)[kernel]
+        return t["bytes_per_launch"], {"file": t["source"], "date": t["date"]}
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def gemv_bytes(M, N, K):
@@ -121,7 +133,25 @@ def _time_on_stream(torch, stream, fn, reps):
     return a.elapsed_time(b) / reps
 
 
-def bench_stack(torch, layers=32, batches=(1, 8, 32), reps=20):
+SAMPLES = 5
+MIN_SAMPLE_MS = 100.0
+
+
+def _measure(torch, stream, fn, min_ms=None, samples=None):
+    """Median / min / max milliseconds per call of `fn()`: `samples` samples, each enough calls to
+    last `min_ms`.  Returns (median, dict with the spread)."""
+    min_ms = MIN_SAMPLE_MS if min_ms is None else min_ms
+    samples = SAMPLES if samples is None else samples
+    fn()
+    one = max(_time_on_stream(torch, stream, fn, 2), 1e-4)
+    reps = max(1, int(np.ceil(min_ms / one)))
+    t = sorted(_time_on_stream(torch, stream, fn, reps) for _ in range(samples))
+    med = t[len(t) // 2] if len(t) % 2 else 0.5 * (t[len(t) // 2 - 1] + t[len(t) // 2])
+    return med, {"samples": samples, "calls_per_sample": reps, "sample_ms": round(med * reps, 1),
+                 "min": round(t[0], 6), "max": round(t[-1], 6)}
+
+
+def bench_stack(torch, layers=32, batches=(1, 8, 32)):
     """The four quantized linears of `layers` Llama-2-7B decoder layers (3.6 GB of codes and scales,
     so every step is cache-cold) as one instruction list of PackedFunc calls, planned and replayed
     as one HIP graph by the library's executor."""
@@ -138,7 +168,8 @@ def bench_stack(torch, layers=32, batches=(1, 8, 32), reps=20):
             layer[name] = (W, S)
         weights.append(layer)
     stream = torch.cuda.Stream()
-    res = {"layers": layers, "instructions_per_step": 4 * layers, "launch": "hip_graph of PackedFunc calls", "batches": []}
+    res = {"layers": layers, "instructions_per_step": 4 * layers,
+           "launch": "hip_graph of PackedFunc calls; runs of decode linears (M = 1) fused into one launch", "batches": []}
     for M in batches:
         hidden = torch.randn((M, 4096), device="cuda", dtype=torch.float16)
         attn = torch.randn((M, 4096), device="cuda", dtype=torch.float16)
@@ -149,10 +180,13 @@ def bench_stack(torch, layers=32, batches=(1, 8, 32), reps=20):
         prog.capture(stream)
         prog.replay(stream)
         stream.synchronize()
-        ms = _time_on_stream(torch, stream, lambda: prog.replay(stream), reps)
+        ms, spread = _measure(torch, stream, lambda: prog.replay(stream))
+        prog.status(stream)
         nbytes = layers * sum(gemv_bytes(M, N, K) for _, N, K in vm.LLAMA7B_LINEARS)
         res["batches"].append({"M": M, "ms_per_step": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1),
                                "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                               "ms_spread": spread, "launches_per_step": 4 * layers - sum(
+                                   len(prog.fused_order(g)) - 1 for g in range(prog.num_fused_groups)),
                                "bytes_per_step": nbytes, "workspace_bytes": ws,
                                "workspace_without_reuse": prog.unplanned_bytes})
         del prog
@@ -184,12 +218,19 @@ def bench_intb(torch, ops, K=8192, N=28672, batches=(1, 16, 128, 512), copies=3,
 
         for _ in range(copies):
             fn()
-        ms = _time_on_stream(torch, stream, fn, 4 * copies)
+        def cycle():
+            for _ in range(copies):
+                fn()
+
+        ms, spread = _measure(torch, stream, cycle, min_ms=MIN_SAMPLE_MS / 2)
+        ms /= copies
         nbytes = K * N * nbit // 8 + s.numel() * 2 + M * K * 2 + M * N * 2
         tf = 2.0 * M * N * K / ms / 1e9
         res["batches"].append({"M": M, "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
                                "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-                               "TFLOP/s": round(tf, 1), "frac_of_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4)})
+                               "TFLOP/s": round(tf, 1), "frac_of_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                               "us_spread": {k: (round(v / copies * 1e3, 2) if k in ("min", "max") else v)
+                                             for k, v in spread.items()}})
     return res
 
 
@@ -226,7 +267,8 @@ def bench_autogptq(torch, ops, K=4096, N=4096, group=128, batches=(1, 8), copies
             with torch.cuda.graph(graph):
                 step()
             graph.replay()
-            ms = _time_on_stream(torch, torch.cuda.current_stream(), graph.replay, 5) / copies
+            ms, _ = _measure(torch, torch.cuda.current_stream(), graph.replay, min_ms=MIN_SAMPLE_MS / 4, samples=3)
+            ms /= copies
             nbytes = N * K // 2 + N * G * 4 + M * K * 2 + M * N * 2 + (M * K * 4 + K * 4 if act else 0)
             res["cases"].append({"M": M, "row_order": act, "us": round(ms * 1e3, 2),
                                  "GB/s": round(nbytes / ms / 1e6, 1),
@@ -250,7 +292,7 @@ def bench_calibration(torch):
         _lib.check(L.wq_calibrate_read(src.data_ptr(), src.numel(), scratch.data_ptr(), stream.cuda_stream), "read")
 
     rd()
-    ms_read = _time_on_stream(torch, stream, rd, 5)
+    ms_read, _ = _measure(torch, stream, rd, min_ms=MIN_SAMPLE_MS / 4, samples=3)
     flops = ctypes.c_double(0.0)
 
     def mf():
@@ -258,7 +300,7 @@ def bench_calibration(torch):
                                            stream.cuda_stream), "mfma")
 
     mf()
-    ms_mfma = _time_on_stream(torch, stream, mf, 3)
+    ms_mfma, _ = _measure(torch, stream, mf, min_ms=MIN_SAMPLE_MS / 4, samples=3)
     # the decode GEMV on a matrix large enough that launch, ramp-up and drain no longer matter
     # (131072 x 4096, 302 MB per copy, three copies cycled): the kernel's steady-state rate
     del src
@@ -282,7 +324,8 @@ def bench_calibration(torch):
     with torch.cuda.graph(graph):
         big()
     graph.replay()
-    ms_big = _time_on_stream(torch, torch.cuda.current_stream(), graph.replay, 6) / 3
+    ms_big, _ = _measure(torch, torch.cuda.current_stream(), graph.replay, min_ms=MIN_SAMPLE_MS / 4, samples=3)
+    ms_big /= 3
     big_bytes = gemv_bytes(1, Nl, Kl)
     return {"read_1GiB_GB/s": round((1 << 30) / ms_read / 1e6, 1), "hbm_vendor_peak_GB/s": HBM_PEAK_GBS,
             "gemv_steady_state": {"N": Nl, "K": Kl, "us": round(ms_big * 1e3, 1),
@@ -298,6 +341,8 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--copies", type=int, default=16, help="distinct weight copies in the ring")
+    ap.add_argument("--samples", type=int, default=5, help="timed samples per measurement (the median is reported)")
+    ap.add_argument("--min-sample-ms", type=float, default=100.0, help="a sample repeats its work until it lasts this long")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-gemm", action="store_true", help="skip the prefill GEMM measurement")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of through a HIP graph")
@@ -327,49 +372,69 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes": 1 << 30, "launches": 4}))
         return
+    global SAMPLES, MIN_SAMPLE_MS
+    SAMPLES, MIN_SAMPLE_MS = args.samples, args.min_sample_ms
     copies = [make_device_set(torch, 1000 + i) for i in range(args.copies)]
     xs = [torch.randn((1, K), device="cuda", dtype=torch.float16) for _, K in DECODE_SHAPES]
     ys = [torch.empty((1, N), device="cuda", dtype=torch.float16) for N, _ in DECODE_SHAPES]
     step_bytes = sum(gemv_bytes(1, N, K) for N, K in DECODE_SHAPES)
-    launches_per_step = len(DECODE_SHAPES)
+    # one list per weight copy: the four linears of a step are ONE launch
+    lists = [ops.Q4G32GemvList([(W, S, x, y) for (W, S), x, y in zip(c, xs, ys)]) for c in copies]
 
     def step(i):
-        for (W, S), x, y in zip(copies[i % args.copies], xs, ys):
-            ops.q4g32_linear(W, S, x, out=y, kernel="gemv")
+        lists[i % args.copies].run()
 
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for i in range(args.warmup):
             step(i)
         stream.synchronize()
-        graph = None
-        if not args.no_graph:
+        if args.no_graph:
+            def run_steps():
+                for i in range(args.steps):
+                    step(i)
+        else:
             # one graph holds all timed steps: the host only issues a single launch
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 for i in range(args.steps):
                     step(i)
-            graph.replay()  # untimed replay (graph upload)
-            stream.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record(stream)
-        if graph is not None:
-            graph.replay()
-        else:
-            for i in range(args.steps):
-                step(i)
-        e1.record(stream)
-        torch.cuda.synchronize()
-        total_ms = e0.elapsed_time(e1)
+            run_steps = graph.replay
+        # EXACTLY `steps` steps per repetition, bracketed by synchronisation; median over samples
+        total_ms, spread = _measure(torch, stream, run_steps)
+        lists[0].status()
 
     ms_per_step = total_ms / args.steps
     gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
-    # the GEMV kernel is the only kernel in the timed region: its average launch
-    # duration (launch gaps included, so a slight under-estimate of the kernel) is
-    avg_launch_us = total_ms * 1e3 / (args.steps * launches_per_step)
-    bytes_per_launch = step_bytes / launches_per_step
-    achieved = bytes_per_launch / (avg_launch_us * 1e-6) / 1e9
+    # the list kernel is the only kernel in the timed region, one launch per step: its average
+    # launch duration (gaps between launches included, so a slight under-estimate of the kernel) is
+    avg_launch_us = ms_per_step * 1e3
+    achieved = step_bytes / (avg_launch_us * 1e-6) / 1e9
+    traffic, traffic_src = offline_traffic("q4g32_gemv_list_kernel")
+
+    # every linear on its own, as a single call of wq_q4g32_linear issues it (the streaming kernel of one
+    # linear per launch), cycling the weight copies inside one graph
+    per_shape = []
+    with torch.cuda.stream(stream):
+        for si, (N, K) in enumerate(DECODE_SHAPES):
+            def one(i, si=si):
+                W, S = copies[i % args.copies][si]
+                ops.q4g32_linear(W, S, xs[si], out=ys[si], kernel="gemv")
+            for i in range(args.copies):
+                one(i)
+            stream.synchronize()
+            g1 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g1, stream=stream):
+                for i in range(4 * args.copies):
+                    one(i)
+            ms1, sp1 = _measure(torch, stream, g1.replay, min_ms=MIN_SAMPLE_MS / 4)
+            us = ms1 * 1e3 / (4 * args.copies)
+            nb = gemv_bytes(1, N, K)
+            per_shape.append({"N": N, "K": K, "us": round(us, 3), "GB/s": round(nb / us / 1e3, 1),
+                              "frac_of_hbm_peak": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": nb,
+                              "us_min": round(sp1["min"] * 1e3 / (4 * args.copies), 3),
+                              "us_max": round(sp1["max"] * 1e3 / (4 * args.copies), 3)})
+            del g1
 
     out = {
         "metric": METRIC,
@@ -389,26 +454,36 @@ def main():
                         "4096->12288, 4096->4096, 4096->22016, 11008->4096",
             "weight_copies_in_ring": args.copies,
             "ring_bytes": step_bytes * args.copies,
-            "launch": "eager" if graph is None else "hip_graph",
+            "launch": ("eager" if args.no_graph else "hip_graph") + ", one launch of the list kernel per step",
             "bytes_per_step": step_bytes,
         },
+        "timing": {"protocol": "median of samples; a sample is a whole number of repetitions of the timed steps "
+                               "lasting at least min_sample_ms; HIP events on the launch stream",
+                   "min_sample_ms": MIN_SAMPLE_MS, **spread,
+                   "ms_per_step_min": round(spread["min"] / args.steps, 6),
+                   "ms_per_step_max": round(spread["max"] / args.steps, 6)},
         "roofline": {
-            "kernel": "q4g32_gemv_kernel",
+            "kernel": "q4g32_gemv_list_kernel",
             "bound": "hbm",
             "achieved": round(achieved, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": traffic,
+            "traffic_source": traffic_src,
             "avg_launch_us": round(avg_launch_us, 3),
-            "bytes_per_launch": bytes_per_launch,
+            "bytes_per_launch": step_bytes,
         },
+        # the same four linears one launch each (what a single wq_q4g32_linear call costs), and the
+        # 4096 x 4096 linear of the single-GEMV configuration on its own
+        "per_linear": per_shape,
+        "single_gemv_4096x4096": next(p for p in per_shape if p["N"] == 4096 and p["K"] == 4096),
     }
 
     if not args.no_gemm:
         gem = []
         tot_flops, tot_ms = 0.0, 0.0
-        reps = 10
+        cur = torch.cuda.current_stream()
         for N, K in PREFILL_SHAPES:
             g = torch.Generator(device="cuda")
             g.manual_seed(N)
@@ -418,20 +493,16 @@ def main():
             y = torch.empty((PREFILL_M, N), device="cuda", dtype=torch.float16)
             for _ in range(3):
                 ops.q4g32_linear(W, S, x, out=y, kernel="gemm")
-            torch.cuda.synchronize()
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for _ in range(reps):
-                ops.q4g32_linear(W, S, x, out=y, kernel="gemm")
-            b.record()
-            torch.cuda.synchronize()
-            ms = a.elapsed_time(b) / reps
+            ms, sp = _measure(torch, cur, lambda: ops.q4g32_linear(W, S, x, out=y, kernel="gemm"))
             fl = 2.0 * PREFILL_M * N * K
-            gem.append({"M": PREFILL_M, "N": N, "K": K, "us": round(ms * 1e3, 2), "tflops": round(fl / ms / 1e9, 1)})
+            gem.append({"M": PREFILL_M, "N": N, "K": K, "us": round(ms * 1e3, 2), "tflops": round(fl / ms / 1e9, 1),
+                        "us_min": round(sp["min"] * 1e3, 2), "us_max": round(sp["max"] * 1e3, 2),
+                        "samples": sp["samples"], "calls_per_sample": sp["calls_per_sample"]})
             tot_flops += fl
             tot_ms += ms
             del W, S, x, y
         tf = tot_flops / tot_ms / 1e9
+        gtraffic, gsrc = offline_traffic("gemm_lds_kernel")
         out["gemm"] = {
             "kernel": "gemm_lds_kernel<Q4G32LdsPolicy>",
             "value": round(tf, 1),
@@ -439,9 +510,10 @@ def main():
             "shapes": gem,
             "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
-                         "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH},
+                         "traffic": gtraffic, "traffic_source": gsrc},
         }
 
+    del lists
     del copies
     torch.cuda.empty_cache()
     if not args.no_stack:

@@ -79,6 +79,26 @@ int wq_program_replay(wq_program_t* p, wq_stream_t stream);
 
 int wq_program_num_instructions(const wq_program_t* p);
 
+/* Fused decode linears.  A run of two or more consecutive relax_amd.q4f16_1_matmul[_bias[_residual]]
+ * instructions with one row of x each (the decode step of a stack of quantized linears) is
+ * executed as ONE launch of the list kernel (wq_q4g32_gemv_list_* of relax_amd_wq.h) instead of
+ * one kernel per instruction, which is what the reference's VM does with the generated kernels
+ * of python/tvm/dlight/gpu/gemv.py.  Inside such a run, independent linears are moved between a
+ * producer and its consumer (results are unchanged: every true, anti and output dependence
+ * between the instructions is kept), and the planned tensors of the run do not share storage.
+ * The descriptor tables live in the workspace (wq_program_plan accounts for them) and are
+ * uploaded by the first wq_program_run / wq_program_capture after the plan or a rebind.
+ * Option "fuse_decode" (default 1) switches this off; set it before wq_program_plan. */
+int wq_program_set_option(wq_program_t* p, const char* name, int value);
+/* Number of runs that are executed fused (after the first run or capture). */
+int wq_program_num_fused_groups(const wq_program_t* p);
+/* The order in which run `group` walks its instructions: writes up to `capacity` instruction
+ * indices to `order` and returns how many the run holds. */
+int wq_program_fused_order(const wq_program_t* p, int group, int* order, int capacity);
+/* Synchronises `stream` and reports a device-side wait of a fused run that hit its spin limit
+ * (see wq_q4g32_gemv_list_status). */
+int wq_program_status(wq_program_t* p, wq_stream_t stream);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

@@ -59,6 +59,10 @@ SIGNATURES = {
     "wq_program_capture": [_vp, _vp],
     "wq_program_replay": [_vp, _vp],
     "wq_program_num_instructions": [_vp],
+    "wq_program_set_option": [_vp, ctypes.c_char_p, _int],
+    "wq_program_num_fused_groups": [_vp],
+    "wq_program_fused_order": [_vp, _int, ctypes.POINTER(_int), _int],
+    "wq_program_status": [_vp, _vp],
     "wq_activation_from_string": [ctypes.c_char_p],
     "wq_binary_op_from_string": [ctypes.c_char_p],
     "wq_unary_op_from_string": [ctypes.c_char_p],

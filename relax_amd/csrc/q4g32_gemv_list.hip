@@ -35,7 +35,6 @@
 // loaded) until the producer has finished everywhere; callers order lists so that this is rare.
 // The last workgroup to finish clears the counters for the next launch.
 #include <algorithm>
-#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <vector>
@@ -149,7 +148,8 @@ struct ListFlags {
   int left[kMaxSlots];
   int flushed;
   int next_pos;  // the next position of the workgroup's row sequence that nobody has taken
-  int pad[6];
+  int next_x;    // the next linear whose activations no x wavefront has taken
+  int pad[5];
 };
 
 __device__ __forceinline__ void lds_spin_until(const int* flag, int target) {
@@ -364,20 +364,32 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
 
   if (wave < NC + XW) {
     // ====================== x wavefronts: activations -> LDS ======================
-    // x wavefront k stages the linears k, k + XW, k + 2 XW, ...
     // until every workgroup has signalled linear `dep`, or the spin limit passes
+    int cur_j = -1;
+    (void)cur_j;
     auto wait_for = [&](int dep) {
       if (aborted) return;
       const long long t0 = wall_clock64();
       while (true) {
+        // read-modify-write (+ 0): performed where the counter lives, never served from a stale cache line
         int v = 0;
         if (lane < kCountersPerLinear)
-          v = __hip_atomic_load(sync + sync_counter_index(dep, lane), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          v = __hip_atomic_fetch_add(sync + sync_counter_index(dep, lane), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         v += __shfl_xor(v, 1, 64);
         v += __shfl_xor(v, 2, 64);
         v += __shfl_xor(v, 4, 64);
         if (__builtin_amdgcn_readfirstlane(v) >= nwg) break;
         if (wall_clock64() - t0 > spin_limit) {
+#ifdef WQ_LIST_TRACE
+          // first time-out of the launch: who waited for what, and the state of its workgroup
+          if (g_list_trace && lane == 0 && atomicCAS((unsigned long long*)&g_list_trace[128], 0ull, 1ull) == 0ull) {
+            long long* t = g_list_trace + 129;
+            t[0] = blockIdx.x; t[1] = cur_j; t[2] = dep; t[3] = nwg;
+            for (int k = 0; k < 8; ++k) t[4 + k] = __hip_atomic_load(sync + sync_counter_index(dep, k), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int k = 0; k < 4; ++k) { t[12 + k] = flags->x_ready[k]; t[16 + k] = flags->left[k]; }
+            t[20] = flags->flushed; t[21] = flags->next_pos; t[22] = flags->next_x;
+          }
+#endif
           aborted = true;
           if (lane == 0)
             __hip_atomic_store(sync + sync_error_index(nlin), dep + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -385,18 +397,28 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         }
         __builtin_amdgcn_s_sleep(4);
       }
+      // whatever this XCD's L2 still holds of an earlier content of x (the addresses are reused
+      // from launch to launch) must not serve the loads that follow
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     };
 
     const half2_t k1031 = {(half_t)1031.0f, (half_t)1031.0f};
     const half2_t k71 = {(half_t)71.0f, (half_t)71.0f};
     const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
-    for (int j = wave - NC; j < nlin; j += XW) {
+    while (true) {
+      // whichever x wavefront is free takes the next linear, so that one slow wait does not hold up
+      // the activations of the linears behind it
+      int j = 0;
+      if (lane == 0) j = __hip_atomic_fetch_add(&flags->next_x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      j = __builtin_amdgcn_readfirstlane(j);
+      if (j >= nlin) break;
       const int slot = j & (nb - 1);
       // the slot is free once every compute wavefront has left the linear that used it before; the
       // row-sum slot of linear j once the sums of linear j - kYSlots have been stored
       if (j >= nb) lds_spin_until(&flags->left[slot], NC * (((j - nb) >> nb_log2) + 1));
       if (j >= kYSlots) lds_spin_until(&flags->flushed, j - kYSlots + 1);
       const int dep = (int)((descs[j].g_dep >> 16) & 0x7fffu) - 1;
+      cur_j = j;
       if (dep >= 0) wait_for(dep);
       if (j < 16) WQ_TR(32 + j);
       const int K = (int)(descs[j].g_dep & 0xffffu) << 5;
@@ -520,8 +542,7 @@ struct wq_gemv_list {
   int xbuf_bytes = 0, ybuf_floats = 0;
   int late = 0, deps = 0;
   int nb = 2;
-  int gs = 2;  // log2 of the rows per row group
-  int depth = 4;
+  int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
   long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
 };
 
@@ -530,18 +551,8 @@ namespace wq {
 constexpr int kListNC = 13;    // compute wavefronts per workgroup
 constexpr int kListXW = 2;     // wavefronts that stage activations
 constexpr int kListDepth = 4;  // ring slots (KiB of codes in flight) per compute wavefront: 52 KiB per CU
+                               // (2, 3, 4 and 6 slots measure the same within 2 %)
 constexpr size_t kListAlign = 256;
-
-typedef void (*list_kernel_t)(const GemvListDesc*, int, int*, long long, int, int, int, int, int);
-static list_kernel_t list_kernel_for(int depth) {
-  switch (depth) {
-    case 2: return q4g32_gemv_list_kernel<kListNC, kListXW, 2>;
-    case 3: return q4g32_gemv_list_kernel<kListNC, kListXW, 3>;
-    case 4: return q4g32_gemv_list_kernel<kListNC, kListXW, 4>;
-    case 6: return q4g32_gemv_list_kernel<kListNC, kListXW, 6>;
-    default: return nullptr;
-  }
-}
 
 static size_t list_table_bytes(int n) { return ((size_t)n * sizeof(GemvListDesc) + kListAlign - 1) / kListAlign * kListAlign; }
 
@@ -619,7 +630,6 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
   // previous linear ended, so that the remainders of all linears spread over the workgroups.
   l->threads = 64 * (kListNC + kListXW + 1);
   l->blocks = std::min(cu_count(), 32768);
-  l->gs = getenv("WQ_LIST_GS") ? atoi(getenv("WQ_LIST_GS")) : 2;
   int64_t turns = 1;
   int64_t off = 0;
   for (int i = 0; i < n; ++i) {
@@ -639,9 +649,7 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
   l->nb = room / l->xbuf_bytes >= 4 ? 4 : room / l->xbuf_bytes >= 2 ? 2 : 0;
   if (l->nb < 2) return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations and row sums do not fit the LDS");
   l->lds = fixed + (size_t)l->nb * l->xbuf_bytes;
-  l->depth = getenv("WQ_LIST_D") ? atoi(getenv("WQ_LIST_D")) : kListDepth;
-  auto kern = list_kernel_for(l->depth);
-  if (!kern) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: no kernel for ring depth %d", l->depth);
+  auto kern = q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>;
   if (l->lds > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)l->lds) != hipSuccess)
     return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
@@ -661,7 +669,7 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
 extern "C" int wq_q4g32_gemv_list_run(wq_gemv_list_t* l, wq_stream_t stream) {
   using namespace wq;
   WQ_REQUIRE(l && l->table, "wq_q4g32_gemv_list_run: null list");
-  WQ_LAUNCH("wq_q4g32_gemv_list_run", list_kernel_for(l->depth), dim3((unsigned)l->blocks),
+  WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>), dim3((unsigned)l->blocks),
             dim3((unsigned)l->threads), l->lds, (hipStream_t)stream, (const GemvListDesc*)l->table, l->n, l->sync,
             l->spin_limit, l->xbuf_bytes, l->ybuf_floats, l->nb == 4 ? 2 : 1, l->gs, l->deps > 0 ? 1 : 0);
   return WQ_OK;

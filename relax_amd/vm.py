@@ -103,6 +103,27 @@ class DpsProgram:
     def num_instructions(self) -> int:
         return int(self._l.wq_program_num_instructions(self._p))
 
+    # ---- fused decode linears ----
+    def set_option(self, name: str, value: int) -> None:
+        """``fuse_decode`` (default 1): run consecutive decode linears as one launch.  Set before :meth:`plan`."""
+        check(self._l.wq_program_set_option(self._p, name.encode(), int(value)), "wq_program_set_option")
+
+    @property
+    def num_fused_groups(self) -> int:
+        return int(self._l.wq_program_num_fused_groups(self._p))
+
+    def fused_order(self, group: int = 0) -> List[int]:
+        n = self._l.wq_program_fused_order(self._p, group, (ctypes.c_int * 1)(), 0)
+        check(min(n, 0), "wq_program_fused_order")
+        buf = (ctypes.c_int * max(1, n))()
+        self._l.wq_program_fused_order(self._p, group, buf, n)
+        return list(buf[:n])
+
+    def status(self, stream: torch.cuda.Stream = None) -> None:
+        """Synchronises and raises if a device-side wait of a fused run timed out."""
+        s = (stream or torch.cuda.current_stream()).cuda_stream
+        check(self._l.wq_program_status(self._p, s), "wq_program_status")
+
     # ---- execution ----
     def run(self, stream: torch.cuda.Stream = None) -> None:
         s = (stream or torch.cuda.current_stream()).cuda_stream

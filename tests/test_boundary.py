@@ -27,7 +27,7 @@ def _declared_symbols():
     for h in ("relax_amd_wq.h", "relax_amd_tvm.h", "relax_amd_vm.h"):
         text = open(os.path.join(INC, h)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names |= set(re.findall(r"^\s*(?:const\s+char\*|int|void|int64_t|size_t|wq_program_t\*)\s+(wq_\w+)\s*\(", text, flags=re.M))
+        names |= set(re.findall(r"^\s*(?:const\s+char\*|int|void|int64_t|size_t|wq_program_t\*|wq_gemv_list_t\*)\s+(wq_\w+)\s*\(", text, flags=re.M))
         names |= set(re.findall(r"^WQ_PACKED\((\w+)\);", text, flags=re.M))
     names.discard("name")
     return sorted(names)

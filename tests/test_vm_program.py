@@ -88,6 +88,61 @@ def test_program_argument_errors():
         l.wq_program_destroy(p)
 
 
+def test_fused_group_order_keeps_dependences_and_separates_producers_from_consumers():
+    """Planning alone (no GPU): a stack of decode linears (one row of x) becomes one fused run whose
+    order is a permutation that keeps every true / anti / output dependence and puts other linears
+    between a producer and its consumer."""
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        L = 6
+        dims = {"q": (384, 128), "o": (128, 128), "g": (512, 128), "d": (128, 256)}
+        addr = [0x100000]
+
+        def ext(code, bits, *shape):
+            addr[0] += 0x100000
+            return l.wq_program_add_external(p, code, bits, len(shape), _shape(*shape), addr[0], 10)
+
+        hidden, attn, act = ext(2, 16, 1, 128), ext(2, 16, 1, 128), ext(2, 16, 1, 256)
+        reads, writes = [], []
+        h = hidden
+        for layer in range(L):
+            w = {k: (ext(1, 32, n, kk // 8), ext(2, 16, n, kk // 32)) for k, (n, kk) in dims.items()}
+            t = {k: l.wq_program_add_planned(p, 2, 16, 2, _shape(1, n)) for k, (n, _) in dims.items()}
+            for k, x in (("q", h), ("o", attn), ("g", t["o"]), ("d", act)):
+                assert _call(l, p, "relax_amd.q4f16_1_matmul", [w[k][0], w[k][1], x, t[k]]) == 0
+                reads.append({w[k][0], w[k][1], x})
+                writes.append(t[k])
+            h = t["d"]
+        n = 4 * L
+        need = l.wq_program_plan(p)
+        # nothing is shared inside the run, and the run's descriptor table is part of the workspace
+        assert need >= l.wq_program_unplanned_bytes(p) + l.wq_q4g32_gemv_list_workspace_bytes(n)
+        buf = (ctypes.c_int * n)()
+        assert l.wq_program_fused_order(p, 0, buf, n) == n
+        order = list(buf)
+        assert sorted(order) == list(range(n))
+        pos = {ins: k for k, ins in enumerate(order)}
+        gaps = []
+        for i in range(n):
+            for j in range(i):
+                raw = writes[j] in reads[i]
+                if raw or writes[i] == writes[j] or writes[i] in reads[j]:
+                    assert pos[j] < pos[i], (j, i)
+                if raw:
+                    gaps.append(pos[i] - pos[j])
+        # at the end of the run nothing independent is left to put between the last producers and
+        # consumers; everywhere else at least three linears lie between
+        assert len(gaps) == 2 * L - 1 and min(gaps[:-2]) >= 4 and min(gaps) >= 2, gaps
+        # switched off: the instructions keep their order and storage is shared again
+        assert l.wq_program_set_option(p, b"fuse_decode", 0) == 0
+        assert l.wq_program_plan(p) < l.wq_program_unplanned_bytes(p)
+        assert l.wq_program_fused_order(p, 0, buf, n) < 0
+        assert l.wq_program_set_option(p, b"no_such_option", 1) != 0
+    finally:
+        l.wq_program_destroy(p)
+
+
 SMALL_LINEARS = (("qkv_proj", 384, 128), ("o_proj", 128, 128), ("gate_up_proj", 512, 128), ("down_proj", 128, 256))
 
 
@@ -117,10 +172,19 @@ def test_linear_stack_program_matches_oracle_eager_and_replayed(oracle, M):
     d_hidden = u.dev(hidden)
     prog = vm.llama_linear_stack(dev_w, M, d_hidden, u.dev(attn), u.dev(act), out, linears=SMALL_LINEARS)
     assert prog.num_instructions == 4 * L
-    need = prog.plan()
-    # per layer qkv, o, gate_up and the hidden state: storage is reused across layers
-    assert 0 < need < prog.unplanned_bytes
-    assert need <= 2 * M * (384 + 128 + 512 + 128) * 2 + 8 * 256
+    if M == 1:
+        # the decode step runs as one fused launch: its tensors do not share storage, and the
+        # workspace also holds the descriptor table and the counters of the run
+        need = prog.plan()
+        assert need >= prog.unplanned_bytes
+        unfused = vm.llama_linear_stack(dev_w, M, d_hidden, u.dev(attn), u.dev(act), out, linears=SMALL_LINEARS)
+        unfused.set_option("fuse_decode", 0)
+        assert 0 < unfused.plan() < unfused.unplanned_bytes
+    else:
+        need = prog.plan()
+        # per layer qkv, o, gate_up and the hidden state: storage is reused across layers
+        assert 0 < need < prog.unplanned_bytes
+        assert need <= 2 * M * (384 + 128 + 512 + 128) * 2 + 8 * 256
 
     # the last down_proj only depends on mlp_act; check it and, through a second program, the o -> gate_up chain
     want = oracle.q4g32_linear(*host_w[-1]["down_proj"], act, nthreads=4)
@@ -130,6 +194,8 @@ def test_linear_stack_program_matches_oracle_eager_and_replayed(oracle, M):
     stream.synchronize()
     eager = u.host(out).copy()
     u.assert_close(eager, want, "stack eager")
+    assert prog.num_fused_groups == (1 if M == 1 else 0)
+    prog.status(stream)
 
     prog.capture(stream)
     for rep in range(3):
@@ -210,6 +276,8 @@ def test_llama7b_stack_full_size_matches_oracle(oracle):
 
         prog.run(stream)
         stream.synchronize()
+        prog.status(stream)
+        assert prog.num_fused_groups == (1 if M == 1 else 0)
         check("eager")
         eager = [t.clone() for t in (out, tap_gu, tap_qkv)]
         prog.capture(stream)
