@@ -283,7 +283,7 @@ def bench_calibration(torch):
 
     from relax_amd import _lib
 
-    L = _lib.lib()
+    L = _lib.calibrate_lib()
     stream = torch.cuda.current_stream()
     src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
     scratch = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")

@@ -93,6 +93,14 @@ int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x, const
                   const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
                   wq_stream_t stream);
 
+/* The decode GEMV with the reference's fp16 accumulation (tests/python/dlight/test_gpu_reduction.py:44-51,
+ * test_gpu_gemv.py:199-206: `NT_matmul += x * decode`, everything fp16): every product and every partial
+ * sum is rounded to fp16.  The order of the sum is free in the reference (its schedules reorder it) and a
+ * tree here, so results agree with a sequential fp16 sum only within fp16 accumulation error.  x fp16 [M, K]
+ * (rows one launch each), y fp16 [M, N]; no epilogue.  wq_q4g32_linear accumulates in fp32 instead. */
+int wq_q4g32_gemv_f16acc(const uint32_t* W, const uint16_t* S, const uint16_t* x, uint16_t* y, int64_t M,
+                         int64_t N, int64_t K, wq_stream_t stream);
+
 /* A list of decode linears (M = 1 each) as ONE launch: what a decoder layer, or a whole stack
  * of them, asks of python/tvm/dlight/gpu/gemv.py:216-530 one generated kernel at a time.  A grid
  * of persistent workgroups walks the list; the weights of the next linear are already streaming
@@ -267,20 +275,6 @@ int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm
 int wq_gptq_linear_noalloc(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
                            const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
                            int64_t K, int64_t G, wq_stream_t stream);
-
-/* ------------------------------------------------------------------------- *
- * Calibration kernels: the measured ceilings reported next to the vendor peaks
- * (no counterpart in the reference; its methodology precedent is the cache-flush
- * protocol of src/runtime/profiling.cc:879-895).
- * ------------------------------------------------------------------------- */
-/* Issues `iters` x 8 independent v_mfma_f32_32x32x16_f16 per wavefront, four wavefronts
- * per CU, no memory traffic.  scratch: device memory of >= 4 bytes x 256 x number of CUs.
- * *flops receives the floating-point operations of one launch. */
-int wq_calibrate_mfma_f16(void* scratch, int64_t scratch_bytes, int iters, double* flops,
-                          wq_stream_t stream);
-/* Streams `bytes` of device memory through the CUs with 16-byte loads and no store
- * (scratch: 4 bytes of device memory, practically never written). */
-int wq_calibrate_read(const void* src, int64_t bytes, void* scratch, wq_stream_t stream);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -24,6 +24,7 @@ SIGNATURES = {
     "wq_q4g32_gemv": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_small_batch": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "wq_q4g32_gemv_f16acc": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_q4g32_gemv_list_workspace_bytes": [_int],
     "wq_q4g32_gemv_list_create": [_vp, _int, _vp, _sz, _vp],
     "wq_q4g32_gemv_list_run": [_vp, _vp],
@@ -44,8 +45,6 @@ SIGNATURES = {
     "wq_gptq_linear_noalloc": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "wq_intb_encode": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp],
     "wq_q4g32_encode": [_vp, _vp, _vp, _i64, _i64, _vp],
-    "wq_calibrate_mfma_f16": [_vp, _i64, _int, ctypes.POINTER(ctypes.c_double), _vp],
-    "wq_calibrate_read": [_vp, _i64, _vp, _vp],
     "wq_program_create": [],
     "wq_program_destroy": [_vp],
     "wq_program_add_external": [_vp, _int, _int, _int, ctypes.POINTER(_i64), _vp, _int],
@@ -72,7 +71,23 @@ _RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p
              "wq_gptq_workspace_bytes": _sz, "wq_q4g32_gemv_list_workspace_bytes": _sz,
              "wq_q4g32_gemv_list_create": _vp, "wq_q4g32_gemv_list_destroy": None}
 
+# include/relax_amd_wq_testing.h: the work-split overrides of the calling thread (all return void)
+TESTING_SIGNATURES = {
+    "wq_debug_set_gemm_config": [_int],
+    "wq_debug_set_gemm_tail_split": [_int],
+    "wq_debug_set_gemv_config": [_int, _int],
+    "wq_debug_set_gemv_blocks_per_cu": [_int],
+    "wq_debug_set_skinny_config": [_int, _int, _int],
+}
+# ... and the calibration kernels of librelax_amd_wq_calibrate.so
+CALIBRATE_LIB_PATH = os.path.join(HERE, "librelax_amd_wq_calibrate.so")
+CALIBRATE_SIGNATURES = {
+    "wq_calibrate_mfma_f16": [_vp, _i64, _int, ctypes.POINTER(ctypes.c_double), _vp],
+    "wq_calibrate_read": [_vp, _i64, _vp, _vp],
+}
+
 _lib = None
+_calibrate_lib = None
 
 
 class WqError(RuntimeError):
@@ -97,8 +112,29 @@ def lib() -> ctypes.CDLL:
             fn = getattr(l, name)  # AttributeError if the symbol is not exported
             fn.argtypes = argtypes
             fn.restype = _RESTYPES.get(name, ctypes.c_int)
+        for name, argtypes in TESTING_SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.argtypes = argtypes
+            fn.restype = None
         _lib = l
     return _lib
+
+
+def calibrate_lib() -> ctypes.CDLL:
+    """The measurement-only library (streaming-read and MFMA-issue ceilings)."""
+    global _calibrate_lib
+    if _calibrate_lib is None:
+        if not os.path.exists(CALIBRATE_LIB_PATH):
+            raise ImportError(f"{CALIBRATE_LIB_PATH} is missing: build it with `python -m relax_amd.build`")
+        import torch  # noqa: F401  (same reason as in lib())
+
+        l = ctypes.CDLL(CALIBRATE_LIB_PATH)
+        for name, argtypes in CALIBRATE_SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        _calibrate_lib = l
+    return _calibrate_lib
 
 
 def check(rc: int, what: str) -> None:

@@ -1,4 +1,5 @@
-"""Compiles the HIP/C++ sources under ``relax_amd/csrc`` into ``librelax_amd_wq.so`` (gfx950).
+"""Compiles the HIP/C++ sources under ``relax_amd/csrc`` into ``librelax_amd_wq.so`` (gfx950), and
+the calibration kernels (``calibrate.hip``: measurement only) into ``librelax_amd_wq_calibrate.so``.
 
 hipcc cross-compiles without a GPU.  The library is built in-tree so that it
 travels with the source tree to the machine that runs it.
@@ -15,6 +16,8 @@ if os.path.dirname(HERE) not in sys.path:
     sys.path.insert(0, os.path.dirname(HERE))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librelax_amd_wq.so")
+CALIBRATE_LIB = os.path.join(HERE, "librelax_amd_wq_calibrate.so")
+CALIBRATE_SOURCES = ("calibrate.hip",)  # not linked into the product library
 OBJDIR = os.path.join(HERE, "build")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -81,9 +84,10 @@ def build(verbose: bool = True, incremental: bool = False) -> str:
         from relax_amd import check_ring_asm
 
         check_ring_asm.main(HIPCC, [f for f in FLAGS if f != "-fPIC"])
-    objs = [os.path.join(OBJDIR, os.path.basename(s) + ".o") for s in srcs]
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
-    subprocess.check_call(cmd)
+    for lib, want in ((LIB, False), (CALIBRATE_LIB, True)):
+        objs = [os.path.join(OBJDIR, os.path.basename(s) + ".o") for s in srcs
+                if (os.path.basename(s) in CALIBRATE_SOURCES) == want]
+        subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *objs])
     if verbose:
         print(f"built {LIB}: compiled {len(todo)} of {len(srcs)} sources", flush=True)
     return LIB

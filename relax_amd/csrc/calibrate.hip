@@ -1,8 +1,10 @@
 // Two microbenchmark kernels that give the measured ceilings the library's kernels are
 // compared with, next to the vendor peak figures: MFMA issue only (no memory traffic)
 // and a pure streaming read (no arithmetic worth mentioning, no write).
+#include "../../include/relax_amd_wq_testing.h"
+#include <hip/hip_runtime.h>
+
 #include "wq_device.h"
-#include "wq_host.h"
 
 namespace wq {
 
@@ -53,27 +55,32 @@ __global__ __launch_bounds__(256) void calibrate_read_kernel(const uint4_t* __re
 
 }  // namespace wq
 
+// This file is a library of its own (librelax_amd_wq_calibrate.so): it reports errors through its
+// return value only (WQ_EINVAL, WQ_EDEVICE) and shares no state with the product library.
+static int launch_status() { return hipGetLastError() == hipSuccess ? WQ_OK : WQ_EDEVICE; }
+
 extern "C" int wq_calibrate_mfma_f16(void* scratch, int64_t scratch_bytes, int iters, double* flops,
                                      wq_stream_t stream) {
   using namespace wq;
-  const int blocks = cu_count();  // one workgroup of four wavefronts per CU
-  WQ_REQUIRE(scratch && scratch_bytes >= (int64_t)blocks * 256 * 4,
-             "wq_calibrate_mfma_f16: scratch must hold %lld bytes", (long long)blocks * 256 * 4);
-  WQ_REQUIRE(iters > 0, "wq_calibrate_mfma_f16: iters must be positive");
-  WQ_LAUNCH("wq_calibrate_mfma_f16", calibrate_mfma_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
-            (float*)scratch, iters, 1.0f);
+  int dev = 0, blocks = 0;  // one workgroup of four wavefronts per CU
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&blocks, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    return WQ_EDEVICE;
+  if (!scratch || scratch_bytes < (int64_t)blocks * 256 * 4 || iters <= 0) return WQ_EINVAL;
+  hipLaunchKernelGGL(calibrate_mfma_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (float*)scratch, iters,
+                     1.0f);
   if (flops) *flops = (double)blocks * 4 * iters * 8 * (2.0 * 32 * 32 * 16);
-  return WQ_OK;
+  return launch_status();
 }
 
 extern "C" int wq_calibrate_read(const void* src, int64_t bytes, void* scratch, wq_stream_t stream) {
   using namespace wq;
-  WQ_REQUIRE(src && scratch && bytes >= 0 && bytes % 16 == 0 && aligned16(src),
-             "wq_calibrate_read: src must be 16-byte aligned, bytes a multiple of 16, scratch 4 bytes");
+  if (!src || !scratch || bytes < 0 || bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(src) & 15u))
+    return WQ_EINVAL;
   if (bytes == 0) return WQ_OK;
   const int64_t blocks = (bytes / 16 + 2047) / 2048;
-  WQ_REQUIRE(blocks < (1ll << 31), "wq_calibrate_read: too large");
-  WQ_LAUNCH("wq_calibrate_read", calibrate_read_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-            (const uint4_t*)src, bytes / 16, (uint32_t*)scratch);
-  return WQ_OK;
+  if (blocks >= (1ll << 31)) return WQ_EINVAL;
+  hipLaunchKernelGGL(calibrate_read_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const uint4_t*)src, bytes / 16, (uint32_t*)scratch);
+  return launch_status();
 }

@@ -398,9 +398,10 @@ static int wq::gptq_linear_impl(const uint32_t* W_nk, const uint16_t* SZ, const 
     } else {
       auto kern = gptq_gather_x_kernel;
       const size_t lds = (size_t)K * 2;
-      if (lds > 48 * 1024)
-        WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)lds));
+      if (lds > 48 * 1024) {
+        static DynamicLdsLimit limit;
+        WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), (int)lds));
+      }
       WQ_LAUNCH("wq_gptq_linear", kern, dim3((unsigned)M), dim3(256), lds, stream, (const half_t*)x, perm,
                 (half_t*)workspace, (int)K);
     }

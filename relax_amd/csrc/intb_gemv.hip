@@ -18,6 +18,7 @@
 // (int4: codes with k%16 >= 8 are taken unshifted as 1024 + 16u and meet
 // activations pre-multiplied by 1/16.)  The per-channel scale multiplies the
 // finished sum; fine-grained scales multiply each 64-row tile.
+#include "tuning.h"
 #include "wq_device.h"
 #include "wq_host.h"
 #include "intb_common.h"
@@ -307,8 +308,8 @@ static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* 
   const size_t lds = (size_t)MB * K * 2 + (size_t)MB * (K / (NBIT == 8 ? 16 : 32)) * 4;
   auto kern = intb_gemv_kernel<NBIT, R, MB>;
   if (lds > 60 * 1024) {
-    WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    static DynamicLdsLimit limit;  // per instantiation
+    WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), (int)lds));
   }
   WQ_LAUNCH("wq_fpA_intB_gemm(gemv)", kern, dim3((unsigned)blocks), dim3(kIntbGemvThreads), lds,
             stream, (const uint4_t*)B, (const half_t*)scales, (const half_t*)A, (half_t*)C, (int)N,

@@ -24,6 +24,7 @@
 #define RELAX_AMD_CSRC_MFMA_GEMM_H_
 
 #include "gemm_epilogue.h"
+#include "tuning.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
@@ -208,8 +209,8 @@ static int launch_mfma_gemm(const char* who, const typename Loader::Args& bargs,
   auto kern = (K % kBK == 0) ? wq_mfma_gemm_kernel<Loader, Epilogue, TM, TN, WM, WN, WPE, false>
                              : wq_mfma_gemm_kernel<Loader, Epilogue, TM, TN, WM, WN, WPE, true>;
   if (Cfg::kLdsBytes > 64 * 1024) {
-    WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
+    static DynamicLdsLimit limit_full, limit_tail;  // one per kernel of this launcher
+    WQ_HIP((K % kBK == 0 ? limit_full : limit_tail).ensure(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes));
   }
   WQ_LAUNCH(who, kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(Cfg::kThreads), Cfg::kLdsBytes,
             stream, bargs, (const half_t*)x, (half_t*)y, ep, (int)M, (int)N, (int)K, tiles_m,

@@ -48,13 +48,11 @@
 #include <type_traits>
 
 #include "gemm_epilogue.h"
+#include "tuning.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
 namespace wq {
-
-// Splitting of the last round's tiles (on by default; switch for measurement).
-inline int g_gemm_tail_split = 1;
 
 template <class Policy, int TM, int TN, int WM, int WN>
 struct LdsGemmCfg {
@@ -344,8 +342,8 @@ static int launch_gemm_lds(const char* who, const typename Policy::Args& wargs, 
   const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM);
   const int tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
   auto kern = gemm_lds_kernel<Policy, Epilogue, TM, TN, WM, WN, WPE>;
-  WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
+  static DynamicLdsLimit limit;
+  WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes));
   // Whole rounds of the machine run whole tiles; the tiles of the last, partial
   // round are cut into 2 or 4 row slices when that lets them all run at once.
   const int per_cu = std::max(1, std::min(WPE, (160 * 1024) / Cfg::kLdsBytes));
@@ -354,7 +352,7 @@ static int launch_gemm_lds(const char* who, const typename Policy::Args& wargs, 
   const int n_full = (total / slots) * slots;
   const int rest = total - n_full;
   int split = 1;
-  if (g_gemm_tail_split) {
+  if (tuning().gemm_tail_split) {
     for (int sp : {4, 2}) {
       if (TM % sp == 0 && Cfg::kALoads % sp == 0 && rest * sp <= slots) {
         split = sp;

@@ -39,6 +39,7 @@
 // a dequantized column bit for bit.  The bit-exact dequantization itself is
 // q4_word_dequant, used by the dequantize entry point and by the MFMA GEMM.
 #pragma once
+#include "tuning.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
@@ -288,10 +289,6 @@ __global__ __launch_bounds__(gemv_max_threads<GPL>()) void q4g32_gemv_kernel(
   }
 }
 
-inline int g_gemv_rows = 0;  // 0 = choose from the shape
-inline int g_gemv_gpl = 0;
-inline int g_gemv_blocks_per_cu = 0;
-
 template <bool ZP>
 constexpr size_t gemv_lds_bytes(int MB, int64_t K) {
   return (size_t)MB * K * 2 + (size_t)MB * (K / 32) * 4 * (ZP ? 2 : 1);
@@ -309,17 +306,19 @@ static bool gemv_geometry(int64_t N, int64_t K, int64_t* nblocks, int* resident_
   if (lds > 60 * 1024) return false;
   const int64_t nsets = (N + ROWS - 1) / ROWS;
   *nblocks = (nsets + sets_per_block - 1) / sets_per_block;
-  static int cached_threads = 0, cached_per_cu = 0;
-  static size_t cached_lds = 0;
-  if (cached_threads != threads || cached_lds != lds) {
+  // the last answer of the occupancy query, per instantiation: (threads, lds, workgroups per CU)
+  // packed into one atomic word, so that concurrent callers read a consistent triple
+  static std::atomic<uint64_t> cache{0};
+  const uint64_t key = ((uint64_t)threads << 48) | ((uint64_t)lds << 16);
+  uint64_t c = cache.load(std::memory_order_acquire);
+  if ((c & ~0xffffull) != key || c == 0) {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, q4g32_gemv_kernel<ROWS, MB, GPL, ZP>, threads, lds) != hipSuccess)
       return false;
-    cached_threads = threads;
-    cached_lds = lds;
-    cached_per_cu = n;
+    c = key | (uint64_t)(n & 0xffff);
+    cache.store(c, std::memory_order_release);
   }
-  *resident_per_cu = cached_per_cu;
+  *resident_per_cu = (int)(c & 0xffff);
   return true;
 }
 
@@ -338,7 +337,8 @@ static int launch_gemv(const char* who, const uint32_t* W, const uint16_t* S, co
   int64_t blocks = (nsets + sets_per_block - 1) / sets_per_block;
   // More workgroups than `blocks_per_cu` per CU: persistent workgroups that take several
   // turns, with the loads of the next turn in flight during the current one.
-  const int64_t cap = (int64_t)cu_count() * (g_gemv_blocks_per_cu ? g_gemv_blocks_per_cu : blocks_per_cu);
+  const int forced_per_cu = tuning().gemv_blocks_per_cu;
+  const int64_t cap = (int64_t)cu_count() * (forced_per_cu ? forced_per_cu : blocks_per_cu);
   if (blocks > cap) blocks = cap;
   if (K > 8 * 8 * (int64_t)threads)
     return fail(WQ_EUNSUPPORTED, "%s: K=%lld too large for %d threads", who, (long long)K,
@@ -346,8 +346,8 @@ static int launch_gemv(const char* who, const uint32_t* W, const uint16_t* S, co
   const size_t lds = gemv_lds_bytes<ZP>(MB, K);
   auto kern = q4g32_gemv_kernel<ROWS, MB, GPL, ZP>;
   if (lds > 60 * 1024) {
-    WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    static DynamicLdsLimit limit;
+    WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), (int)lds));
   }
   WQ_LAUNCH(who, kern, dim3((unsigned)blocks), dim3(threads), lds, stream, (const uint4_t*)W, (const half_t*)S, (const half_t*)x,
             (const half_t*)bias, (const half_t*)residual, (half_t*)y, (int)N, (int)K, parts,
@@ -395,9 +395,9 @@ static int gemv_dispatch(const char* who, const uint32_t* W, const uint16_t* S, 
   const int G = (int)(K / 32);
   // groups per lane: one wavefront covers a whole row when K <= 64*32*GPL
   // (rows longer than 256 groups are split over several wavefronts)
-  int gpl = g_gemv_gpl ? g_gemv_gpl
+  int gpl = tuning().gemv_gpl ? tuning().gemv_gpl
                        : (G <= 64 ? 1 : G <= 128 ? 2 : G <= 192 ? 3 : G <= 256 ? 4 : G <= 384 ? 3 : 2);
-  const int rows = g_gemv_rows;  // 0 = from the shape
+  const int rows = tuning().gemv_rows;  // 0 = from the shape
   // pairs of rows of x share one pass over the weights
   for (int64_t m0 = 0; m0 < M;) {
     const int64_t left = M - m0;

@@ -97,14 +97,7 @@ struct Q4G32LdsPolicy {
 }  // namespace wq
 
 // Tile shape override for measurement (0 = choose from the problem shape).
-static int g_gemm_cfg_override = 0;
-extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemm_config(int cfg) {
-  g_gemm_cfg_override = cfg;
-}
-int wq_gemm_cfg_override() { return g_gemm_cfg_override; }
-extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemm_tail_split(int on) {
-  wq::g_gemm_tail_split = on;
-}
+int wq_gemm_cfg_override() { return wq::tuning().gemm_cfg; }
 
 extern "C" int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                              const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M,
@@ -119,7 +112,7 @@ extern "C" int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_
   WQ_REQUIRE(W && S && x && y, "wq_q4g32_gemm: null pointer");
   WQ_REQUIRE(aligned16(W) && aligned16(x), "wq_q4g32_gemm: W and x must be 16-byte aligned");
   WQ_REQUIRE(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), "wq_q4g32_gemm: too large");
-  int cfg = g_gemm_cfg_override ? g_gemm_cfg_override : choose_gemm_cfg(M, N, true);
+  int cfg = tuning().gemm_cfg ? tuning().gemm_cfg : choose_gemm_cfg(M, N, true);
   const Q4G32Loader::Args bargs{W, (const half_t*)S};
   const Q4G32LdsPolicy::Args largs{W, (const half_t*)S};
   const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};

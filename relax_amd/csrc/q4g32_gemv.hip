@@ -1,16 +1,6 @@
 // Format A (q4f16_1) decode GEMV entry point: the streaming kernel of q4_gemv.h without zero points.
 #include "q4_gemv.h"
 
-// Launch-shape overrides for measurement: rows per row set, groups per lane and
-// resident workgroups per CU (0 = automatic).
-extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemv_config(int rows, int gpl) {
-  wq::g_gemv_rows = rows;
-  wq::g_gemv_gpl = gpl;
-}
-extern "C" __attribute__((visibility("default"))) void wq_debug_set_gemv_blocks_per_cu(int n) {
-  wq::g_gemv_blocks_per_cu = n;
-}
-
 extern "C" int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x,
                              const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M,
                              int64_t N, int64_t K, wq_stream_t stream_) {

@@ -48,17 +48,7 @@ struct Q4G32SkinnyPolicy {
   }
 };
 
-SkinnyTuning& skinny_tuning() {
-  static SkinnyTuning t{0, 0, 0};
-  return t;
-}
-
 }  // namespace wq
-
-extern "C" __attribute__((visibility("default"))) void wq_debug_set_skinny_config(int nw, int stages,
-                                                                                  int waves) {
-  wq::skinny_tuning() = wq::SkinnyTuning{nw, stages, waves};
-}
 
 // Small-batch entry: 1 <= M <= 64, K % 64 == 0.  Called by wq_q4g32_linear.
 extern "C" int wq_q4g32_small_batch(const uint32_t* W, const uint16_t* S, const uint16_t* x,

@@ -30,6 +30,7 @@
 #ifndef RELAX_AMD_CSRC_SKINNY_GEMM_H_
 #define RELAX_AMD_CSRC_SKINNY_GEMM_H_
 
+#include "tuning.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
@@ -416,12 +417,8 @@ static int launch_xreg(const char* who, const typename Policy::Args& pargs, cons
   auto kern = skinny_xreg_kernel<Policy, Epilogue, NSTEP, WAVES>;
   const int64_t tiles = (N + 15) / 16;
   const int64_t blocks = tiles < cu_count() ? tiles : cu_count();
-  static bool configured = false;  // per instantiation
-  if (!configured) {
-    WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    configured = true;
-  }
+  static DynamicLdsLimit limit;  // per instantiation
+  WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), 160 * 1024));
   WQ_LAUNCH(who, kern, dim3((unsigned)blocks), dim3(64 * WAVES), Cfg::kLdsBytes, stream, pargs,
             (const half_t*)x, (half_t*)y, epi, (int)M, (int)N, (int)K);
   return WQ_OK;
@@ -440,12 +437,15 @@ static int launch_xreg_auto(const char* who, const typename Policy::Args& pargs,
   return launch_xreg<Policy, Epilogue, 8, 8>(who, pargs, x, y, epi, M, N, K, stream);
 }
 
-// overrides for tests and measurement (0 = automatic)
+// overrides for tests and measurement (tuning.h; 0 = automatic)
 // waves: 1 = the ring kernel, 2 = the kernel that holds the activations in registers (where it fits)
 struct SkinnyTuning {
   int nw, stages, waves;
 };
-SkinnyTuning& skinny_tuning();
+inline SkinnyTuning skinny_tuning() {
+  const Tuning& t = tuning();
+  return SkinnyTuning{t.skinny_nw, t.skinny_stages, t.skinny_waves};
+}
 
 template <typename Policy, typename Epilogue, int TH, int NW, int WAVES, bool SB = false>
 static int launch_skinny(const char* who, const typename Policy::Args& pargs, const uint16_t* x, uint16_t* y,
@@ -472,12 +472,8 @@ static int launch_skinny(const char* who, const typename Policy::Args& pargs, co
   WQ_REQUIRE(stages >= 2, "%s: internal: no room for a 2-slot ring", who);
   int lds_bytes = stages * Cfg::kStageBytes + sblock_bytes;
   if (lds_bytes < Cfg::kRedBytes) lds_bytes = Cfg::kRedBytes;
-  static bool configured = false;  // per instantiation
-  if (!configured) {
-    WQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    configured = true;
-  }
+  static DynamicLdsLimit limit;  // per instantiation
+  WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), 160 * 1024));
   WQ_LAUNCH(who, kern, dim3((unsigned)blocks), dim3(64 * WAVES), lds_bytes, stream, pargs,
             (const half_t*)x, (half_t*)y, epi, (int)M, (int)N, (int)K, stages);
   return WQ_OK;
@@ -491,7 +487,7 @@ template <typename Policy, typename Epilogue>
 static int launch_skinny_auto(const char* who, const typename Policy::Args& pargs, const uint16_t* x,
                               uint16_t* y, const Epilogue& epi, int64_t M, int64_t N, int64_t K,
                               hipStream_t stream) {
-  const SkinnyTuning& t = skinny_tuning();
+  const SkinnyTuning t = skinny_tuning();
   // activations in registers where that kernel is the faster one: 4096 < K <= 8192 and at least
   // four column tiles per CU (N = 28672, K = 8192: q4f16_1 at M = 16 58 -> 47 us, int8 at M = 4
   // 60 -> 48 us; with two tiles per CU, or at K = 4096, the ring kernel is the faster one)

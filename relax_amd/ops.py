@@ -116,6 +116,26 @@ def q4g32_linear(W: torch.Tensor, S: torch.Tensor, x: torch.Tensor, bias: Option
     return out
 
 
+def q4g32_gemv_f16acc(W: torch.Tensor, S: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """The decode GEMV with fp16 accumulation (the reference's `NT_matmul += x * decode` with every
+    buffer fp16: tests/python/dlight/test_gpu_reduction.py:44-51): each product and each partial sum
+    is rounded to fp16; the sum is a tree (per lane, then over the wavefront)."""
+    W = _w32(W)
+    S = _dev(S, torch.float16, "S")
+    x = _dev(x, torch.float16, "x")
+    N, kw = W.shape
+    K = kw * 8
+    if x.shape[-1] != K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {K}")
+    if K % 32 or tuple(S.shape) != (N, K // 32):
+        raise ValueError(f"S must be [N, K/32] = [{N}, {K // 32}], got {tuple(S.shape)}")
+    M = x.numel() // K if K else 0
+    out = torch.empty(tuple(x.shape[:-1]) + (N,), dtype=torch.float16, device=x.device)
+    check(_lib.lib().wq_q4g32_gemv_f16acc(_ptr(W), _ptr(S), _ptr(x), _ptr(out), M, N, K, _stream()),
+          "wq_q4g32_gemv_f16acc")
+    return out
+
+
 class GemvDesc(ctypes.Structure):
     """``wq_q4g32_gemv_desc`` of include/relax_amd_wq.h."""
     _fields_ = [("W", ctypes.c_void_p), ("S", ctypes.c_void_p), ("x", ctypes.c_void_p), ("bias", ctypes.c_void_p),

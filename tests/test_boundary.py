@@ -22,9 +22,9 @@ def lib():
     return _lib.lib()
 
 
-def _declared_symbols():
+def _declared_symbols(headers=("relax_amd_wq.h", "relax_amd_tvm.h", "relax_amd_vm.h")):
     names = set()
-    for h in ("relax_amd_wq.h", "relax_amd_tvm.h", "relax_amd_vm.h"):
+    for h in headers:
         text = open(os.path.join(INC, h)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names |= set(re.findall(r"^\s*(?:const\s+char\*|int|void|int64_t|size_t|wq_program_t\*|wq_gemv_list_t\*)\s+(wq_\w+)\s*\(", text, flags=re.M))
@@ -42,6 +42,55 @@ def test_every_declared_symbol_is_exported(lib):
     from relax_amd import _lib
 
     assert set(_lib.SIGNATURES) <= set(names)
+    # the product headers hold no test hook and no calibration kernel
+    assert not [n for n in names if n.startswith(("wq_debug_", "wq_calibrate_"))]
+
+
+def test_testing_header_symbols(lib):
+    """include/relax_amd_wq_testing.h: the thread-local overrides live in the product library, the
+    calibration kernels in a library of their own."""
+    from relax_amd import _lib
+
+    names = _declared_symbols(("relax_amd_wq_testing.h",))
+    hooks = sorted(n for n in names if n.startswith("wq_debug_"))
+    calib = sorted(n for n in names if n.startswith("wq_calibrate_"))
+    assert hooks == sorted(_lib.TESTING_SIGNATURES) and calib == sorted(_lib.CALIBRATE_SIGNATURES)
+    assert sorted(names) == hooks + calib or set(names) == set(hooks) | set(calib)
+    for n in hooks:
+        assert hasattr(lib, n), n
+    c = _lib.calibrate_lib()
+    for n in calib:
+        assert hasattr(c, n) and not hasattr(lib, n), n
+    # an override belongs to the thread that set it: an unknown tile configuration is refused before
+    # anything touches a device, and the message names the configuration of the CALLING thread
+    import threading
+
+    W = np.zeros((64, 8), np.uint32)
+    S = np.zeros((64, 2), np.float16)
+    x = np.zeros((64, 64), np.float16)
+    y = np.zeros((64, 64), np.float16)
+
+    def call():
+        rc = lib.wq_q4g32_gemm(W.ctypes.data, S.ctypes.data, x.ctypes.data, None, None, y.ctypes.data, 64, 64, 64, None)
+        return rc, lib.wq_last_error().decode()
+
+    seen = {}
+
+    def other():
+        lib.wq_debug_set_gemm_config(99)
+        seen["other"] = call()
+        lib.wq_debug_set_gemm_config(0)
+
+    lib.wq_debug_set_gemm_config(98)
+    try:
+        t = threading.Thread(target=other)
+        t.start()
+        t.join()
+        seen["main"] = call()
+    finally:
+        lib.wq_debug_set_gemm_config(0)
+    assert seen["other"][0] == -1 and "configuration 99" in seen["other"][1], seen
+    assert seen["main"][0] == -1 and "configuration 98" in seen["main"][1], seen
 
 
 def test_function_table(lib):
