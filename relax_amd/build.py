@@ -79,11 +79,12 @@ def build(verbose: bool = True, incremental: bool = False) -> str:
     if todo:
         with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(todo))) as ex:
             list(ex.map(_compile, todo))
-    if any(os.path.basename(s) == "q4g32_gemv_list.hip" for s in todo):
-        # that kernel waits for its inline-assembly loads by hand: verify the generated code
-        from relax_amd import check_ring_asm
+    from relax_amd import check_ring_asm
 
-        check_ring_asm.main(HIPCC, [f for f in FLAGS if f != "-fPIC"])
+    ring = [os.path.basename(s) for s in todo if os.path.basename(s) in check_ring_asm.SOURCES]
+    if ring:
+        # those kernels wait for their inline-assembly loads by hand: verify the generated code
+        check_ring_asm.main(HIPCC, [f for f in FLAGS if f != "-fPIC"], ring)
     for lib, want in ((LIB, False), (CALIBRATE_LIB, True)):
         objs = [os.path.join(OBJDIR, os.path.basename(s) + ".o") for s in srcs
                 if (os.path.basename(s) in CALIBRATE_SOURCES) == want]

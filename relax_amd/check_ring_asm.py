@@ -1,6 +1,6 @@
-"""Build-time check of the generated code of ``csrc/q4g32_gemv_list.hip``.
+"""Build-time check of the generated code of ``csrc/q4g32_gemv_list.hip`` and ``csrc/q4g32_batch_list.hip``.
 
-The compute wavefronts of that kernel load their weight stream with inline-assembly loads into a
+The compute wavefronts of those kernels load their weight stream with inline-assembly loads into a
 ring of registers and wait for them by hand, so the compiler does not know that those registers are
 in flight between a load and its wait.  The source makes every read of a ring register an asm
 statement that depends on the wait; what is left to chance is register allocation (a copy or a
@@ -24,7 +24,7 @@ import sys
 import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(HERE, "csrc", "q4g32_gemv_list.hip")
+SOURCES = ("q4g32_gemv_list.hip", "q4g32_batch_list.hip")
 ALLOWED_READERS = ("v_and_or_b32", "v_lshrrev_b32", "v_cvt_f32_f16")
 
 
@@ -91,17 +91,19 @@ def check(asm_text: str) -> list[str]:
             with_ring += 1
             errors += _check_function(body)
     if with_ring == 0:
-        return ["no ring loads found (expected global_load_* ... nt in q4g32_gemv_list_kernel)"]
+        return ["no ring loads found (expected global_load_* ... nt in the kernel)"]
     return errors
 
 
-def main(hipcc="/opt/rocm/bin/hipcc", flags=()):
-    with tempfile.TemporaryDirectory() as td:
-        out = os.path.join(td, "k.s")
-        subprocess.check_call([hipcc, *flags, "-S", "--cuda-device-only", SRC, "-o", out], stderr=subprocess.DEVNULL)
-        errs = check(open(out).read())
-    if errs:
-        raise RuntimeError("q4g32_gemv_list.hip: the generated code touches in-flight ring registers:\n  " + "\n  ".join(errs[:20]))
+def main(hipcc="/opt/rocm/bin/hipcc", flags=(), sources=SOURCES):
+    for name in sources:
+        with tempfile.TemporaryDirectory() as td:
+            out = os.path.join(td, "k.s")
+            subprocess.check_call([hipcc, *flags, "-S", "--cuda-device-only", os.path.join(HERE, "csrc", name), "-o", out],
+                                  stderr=subprocess.DEVNULL)
+            errs = check(open(out).read())
+        if errs:
+            raise RuntimeError(f"{name}: the generated code touches in-flight ring registers:\n  " + "\n  ".join(errs[:20]))
     return True
 
 

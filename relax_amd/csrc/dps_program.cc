@@ -53,6 +53,7 @@ struct FusedGroup {
 struct DecodeLinear {
   int W, S, x, bias, residual, y;  // registers; bias / residual -1 when absent
   int64_t N, K;
+  int64_t M;  // rows of x: 1 .. WQ_GEMV_LIST_MAX_M
 };
 
 }  // namespace
@@ -217,7 +218,7 @@ static bool as_decode_linear(const wq_program* p, const Instr& in, DecodeLinear*
   for (size_t i = 0; i < in.regs.size(); ++i)
     if (in.regs[i] < 0 && !(in.codes[i] == kTVMNullptr)) return false;
   DecodeLinear d{in.regs[0], in.regs[1], in.regs[2], kind >= 1 ? in.regs[3] : -1, kind >= 2 ? in.regs[4] : -1,
-                 in.regs[3 + kind], 0, 0};
+                 in.regs[3 + kind], 0, 0, 0};
   if (d.W < 0 || d.S < 0 || d.x < 0 || d.y < 0 || (kind >= 1 && d.bias < 0) || (kind >= 2 && d.residual < 0)) return false;
   auto numel = [&](int r) {
     int64_t n = 1;
@@ -234,11 +235,13 @@ static bool as_decode_linear(const wq_program* p, const Instr& in, DecodeLinear*
   d.N = W.shape[0];
   d.K = W.shape[1] * 8;
   if (d.N <= 0 || d.K <= 0 || d.K > WQ_GEMV_LIST_MAX_K || S.shape[0] != d.N || S.shape[1] * 32 != d.K) return false;
-  // one row of x: the decode case
-  if (p->regs[d.x].shape.empty() || p->regs[d.x].shape.back() != d.K || numel(d.x) != d.K) return false;
-  if (p->regs[d.y].shape.empty() || p->regs[d.y].shape.back() != d.N || numel(d.y) != d.N) return false;
+  // one row of x (the decode case) or a few (a small decode batch, which the list kernel takes for K % 256 == 0)
+  if (p->regs[d.x].shape.empty() || p->regs[d.x].shape.back() != d.K) return false;
+  d.M = numel(d.x) / d.K;
+  if (d.M < 1 || d.M > WQ_GEMV_LIST_MAX_M || (d.M > 1 && d.K % 256 != 0)) return false;
+  if (p->regs[d.y].shape.empty() || p->regs[d.y].shape.back() != d.N || numel(d.y) != d.M * d.N) return false;
   if (d.bias >= 0 && (!is(d.bias, kDLFloat, 16) || numel(d.bias) != d.N)) return false;
-  if (d.residual >= 0 && (!is(d.residual, kDLFloat, 16) || numel(d.residual) != d.N)) return false;
+  if (d.residual >= 0 && (!is(d.residual, kDLFloat, 16) || numel(d.residual) != d.M * d.N)) return false;
   *out = d;
   return true;
 }
@@ -311,7 +314,8 @@ static void find_groups(wq_program* p) {
     std::vector<DecodeLinear> lin;
     DecodeLinear d;
     int j = i;
-    while (j < n && (int)lin.size() < WQ_GEMV_LIST_MAX && as_decode_linear(p, p->instrs[j], &d)) {
+    while (j < n && (int)lin.size() < WQ_GEMV_LIST_MAX && as_decode_linear(p, p->instrs[j], &d) &&
+           (lin.empty() || d.M == lin[0].M)) {  // one list, one batch size
       lin.push_back(d);
       ++j;
     }
@@ -426,16 +430,18 @@ static int build_lists(wq_program* p, hipStream_t stream) {
   for (FusedGroup& g : p->groups) {
     if (g.list || g.failed) continue;
     std::vector<wq_q4g32_gemv_desc> descs;
+    int64_t rows = 1;
     for (int k : g.order) {
       DecodeLinear d;
       if (!as_decode_linear(p, p->instrs[k], &d)) return wq::fail(WQ_EINVAL, "instruction %d no longer qualifies for its fused group", k);
       auto ptr = [&](int r) { return r < 0 ? nullptr : static_cast<char*>(p->regs[r].dl.data) + p->regs[r].dl.byte_offset; };
       descs.push_back({(const uint32_t*)ptr(d.W), (const uint16_t*)ptr(d.S), (const uint16_t*)ptr(d.x),
                        (const uint16_t*)ptr(d.bias), (const uint16_t*)ptr(d.residual), (uint16_t*)ptr(d.y), d.N, d.K});
+      rows = d.M;
     }
     char* ws = static_cast<char*>(p->workspace) + g.ws_offset;
-    g.list = wq_q4g32_gemv_list_create(descs.data(), (int)descs.size(), ws,
-                                       wq_q4g32_gemv_list_workspace_bytes((int)descs.size()), stream);
+    g.list = wq_q4g32_gemv_list_create_batched(descs.data(), (int)descs.size(), (int)rows, ws,
+                                               wq_q4g32_gemv_list_workspace_bytes((int)descs.size()), stream);
     // operands that alias in a way the list kernel cannot order (or pointers it cannot take): the
     // group runs instruction by instruction, which is always valid
     if (!g.list) g.failed = true;

@@ -1,0 +1,99 @@
+// Definitions shared by the two kernels that run a list of format-A linears in one launch
+// (q4g32_gemv_list.hip: one activation row; q4g32_batch_list.hip: 2 .. 16 rows): the descriptor
+// table, the device-side completion counters, and the host object behind wq_gemv_list_t.
+#ifndef RELAX_AMD_CSRC_GEMV_LIST_COMMON_H_
+#define RELAX_AMD_CSRC_GEMV_LIST_COMMON_H_
+
+#include <vector>
+
+#include "wq_device.h"
+#include "wq_host.h"
+
+namespace wq {
+
+struct GemvListDesc {  // 128 bytes, device memory
+  const char* W;       // uint32 [N, K/8]
+  const char* S;       // fp16   [N, K/32]
+  const half_t* x;     // fp16   [M, K]   (M: a property of the list, 1 .. 16)
+  const half_t* bias;  // fp16   [N] or null
+  const half_t* residual;  // fp16 [M, N] or null
+  half_t* y;           // fp16   [M, N]
+  int32_t N;
+  int32_t q;           // row groups / workgroups  (a row group is 2^gs consecutive rows)
+  uint32_t g_dep;      // bits 0..15: K / 32; bits 16..30: 1 + the linear of this list that writes x (0: none);
+                       // bit 31: a later linear reads y
+  uint16_t rem;        // row groups % workgroups
+  uint16_t off;        // rotation: workgroup b owns the row groups local * workgroups + ((b - off) mod workgroups)
+  // words 16 ..: the batch kernel only.  A linear is run by ONE group of workgroups, those with
+  // b mod 2^gmod_log2 == gidx (member c = b >> gmod_log2 of workgroups >> gmod_log2); q, rem and off
+  // then count within the group.
+  uint8_t gmod_log2, gidx;
+  uint8_t pad[62];
+};
+static_assert(sizeof(GemvListDesc) == 128, "descriptor layout");
+constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y
+
+typedef const GemvListDesc __attribute__((address_space(4)))* gemv_desc_ptr;  // scalar loads
+
+constexpr int kCounterStride = 16;   // ints between two counters (64 bytes: one cache line each)
+constexpr int kCountersPerLinear = 8;
+constexpr int kBufferFlags = 0x00020000;  // buffer resource word 3: 32-bit data format, no swizzle
+constexpr int kDeviceScope = 16;          // cache policy bit sc1: the access is coherent over the whole device
+
+// error word: 1 + the linear a consumer waited for in vain, or kBatchInternalWait + a code: a hand-over
+// inside a workgroup of the batch kernel that did not come
+constexpr int kBatchInternalWait = 1 << 20;
+
+// sync layout (ints): [lin][8] counters at stride kCounterStride, then `finished`, then `error`
+__host__ __device__ inline int sync_counter_index(int lin, int k) { return (lin * kCountersPerLinear + k) * kCounterStride; }
+__host__ __device__ inline int sync_finished_index(int nlin) { return sync_counter_index(nlin, 0); }
+__host__ __device__ inline int sync_error_index(int nlin) { return sync_counter_index(nlin, 1); }
+__host__ __device__ inline int sync_ints(int nlin) { return sync_counter_index(nlin, 2); }
+
+__device__ __forceinline__ void lds_done_then_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+__device__ __forceinline__ void lds_spin_until(const int* flag, int target) {
+  while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) __builtin_amdgcn_s_sleep(1);
+  asm volatile("" ::: "memory");  // LDS is served in order: what was written before the flag is visible now
+}
+
+}  // namespace wq
+
+struct wq_gemv_list {
+  std::vector<wq::GemvListDesc> descs;
+  int n = 0;
+  void* table = nullptr;  // device: descriptors
+  int* sync = nullptr;    // device: counters
+  int blocks = 0, threads = 0;
+  size_t lds = 0;
+  int xbuf_bytes = 0, ybuf_floats = 0;
+  int late = 0, deps = 0;
+  int nb = 2;
+  int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
+  long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
+  int M = 1;               // activation rows; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
+  int batch_u = 0;         // chunks per tile and wavefront (4: panels of 4096 k, M <= 8; 2: 2048 k)
+  int batch_groups = 1;    // groups of workgroups that run different linears side by side
+  int batch_nxb = 0;       // panels of activations in LDS
+  int batch_ring = 0;      // items the compute wavefronts may spread over (slots of scales and of partial sums)
+  int batch_acc_tiles = 0; // most tiles a workgroup holds of a linear that spans several panels
+};
+
+namespace wq {
+
+constexpr size_t kListAlign = 256;
+
+inline size_t list_table_bytes(int n) { return ((size_t)n * sizeof(GemvListDesc) + kListAlign - 1) / kListAlign * kListAlign; }
+
+
+// q4g32_batch_list.hip: launch shape and LDS plan of a list with 2 .. 16 activation rows (fills
+// l->blocks, threads, lds, batch_*; the descriptors' q / rem / off), and its launch
+int batch_list_plan(wq_gemv_list* l);
+int batch_list_launch(wq_gemv_list* l, hipStream_t stream);
+
+}  // namespace wq
+#endif  // RELAX_AMD_CSRC_GEMV_LIST_COMMON_H_

@@ -1,0 +1,639 @@
+// A list of format-A (q4f16_1) linears with 2 .. 16 activation rows each, in ONE launch.
+//
+// The counterpart of q4g32_gemv_list.hip for a small batch: the same persistent grid (one workgroup
+// per CU walks the list, device-side counters order dependent linears), but the products are done by
+// the matrix cores so that all M rows share one pass over the weights, and the weights go from
+// memory straight into the registers that feed them.
+//
+// Work.  The unit is a TILE of 16 consecutive rows of W times a PANEL of K (4096 k for M <= 8, else
+// 2048 k).  A linear is run by one GROUP of workgroups (see batch_assign_groups), its tiles dealt to them
+// round-robin, with a rotation that continues from linear to linear.  Inside a workgroup the 8 compute
+// wavefronts split a panel along K: wavefront w owns the 4 U scale groups w * 4U .. of every panel
+// (U = 4 or 2), i.e. U chunks per tile; a chunk is one 16-byte load per lane: lane (i, kq) takes scale
+// group 4u + kq of row i, the 32 codes that the four v_mfma_f32_16x16x32_f16 of the chunk consume as A
+// operands (one dword, 8 codes, each).
+// Unpacking is exact: OR the code into 0x6400 (1024 + q, or 1024 + 16 q), subtract 1031 (1136),
+// multiply by the scale, all in packed fp16: 13 VALU instructions per 8 weights and lane, whatever M.
+// The B operands (the activations of the wavefront's K slice, in the k order of the unpack, the
+// 16 q positions pre-divided by 16) live in registers for the whole panel.
+//
+// The other four wavefronts keep everything irregular away from that loop, through LDS:
+//   * 2 x wavefronts wait for a producer linear (bounded spin), load a panel of activations,
+//     rearrange it and leave it in one of 2 .. 4 LDS buffers, that many panels ahead (under load a round
+//     trip to L2 takes several microseconds); the compute wavefronts copy their slice into registers
+//     when they reach the panel, which frees the buffer at once.
+//   * the scale wavefront streams the tile's scales (16 rows x 256 contiguous bytes: fetched per
+//     lane they cost more than the codes) into a ring of LDS slots, a few tiles ahead.
+//   * the y wavefront adds the 8 partial sums of a tile in a fixed order, keeps the sum in LDS while
+//     further panels of the same rows follow, and at the last panel applies bias / cast / residual,
+//     stores y with device-scope stores and signals the linear's completion counter.
+// Codes in flight per CU: 8 wavefronts x (NT - 1) tiles x U KiB.
+#include <algorithm>
+#include <cmath>
+#include <vector>
+
+#include "gemv_list_common.h"
+
+namespace wq {
+
+constexpr int kBW = 8;     // compute wavefronts: K slices of a panel
+constexpr int kBXW = 2;    // wavefronts that stage activations
+constexpr int kBRing = 4;  // LDS slots of scales and of partial sums: how far the compute wavefronts may spread
+constexpr int kBNT = 3;    // tile buffers per compute wavefront (NT - 1 tiles of loads in flight)
+constexpr int kBThreads = 64 * (kBW + kBXW + 2);
+
+// LDS words that hand the buffers over inside a workgroup (items = (linear, panel, tile) in the
+// order the workgroup walks them; panels counted over all linears)
+constexpr int kBMaxXBuf = 4;
+struct BatchFlags {
+  int x_ready[kBMaxXBuf];  // [panel mod buffers] = panel + 1 once that panel's activations are staged
+  int x_taken[kBMaxXBuf];  // [panel mod buffers] += 1 by each compute wavefront that has copied the panel
+                           // (per buffer: with two buffers a wavefront may be a panel ahead of another)
+  int s_ready;       // items whose scales are staged
+  int y_done;        // items whose partial sums have been added up
+  int abort;         // a wait of this workgroup ran into the spin limit: nobody waits any more
+  int pad;
+  int done[kBRing];  // += 1 by each compute wavefront per item finished, by slot (item mod ring)
+};
+static_assert(sizeof(BatchFlags) == 64, "flags layout");
+
+// Waits inside a workgroup are bounded like the waits between workgroups: a hand-over that never comes
+// (a defect, or a wavefront that died) ends as an error word and a launch that finishes, not as a hang.
+struct BatchWait {
+  BatchFlags* flags;
+  int* error;  // the list's error word
+  long long limit;
+  __device__ __forceinline__ void until(const int* flag, int target, int code) const {
+    if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) {
+      asm volatile("" ::: "memory");
+      return;
+    }
+    const long long t0 = wall_clock64();
+    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
+      if (__hip_atomic_load(&flags->abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) break;
+      if (wall_clock64() - t0 > limit) {
+        __hip_atomic_store(&flags->abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_store(error, kBatchInternalWait + code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    asm volatile("" ::: "memory");  // LDS is served in order: what was written before the flag is visible now
+  }
+};
+
+__host__ __device__ constexpr int batch_panel_groups(int U) { return kBW * 4 * U; }
+__host__ __device__ constexpr int batch_scale_row_bytes(int U) { return batch_panel_groups(U) * 2 + 16; }  // + 16: rows on different banks
+__host__ __device__ constexpr int batch_scale_slot_bytes(int U) { return 16 * batch_scale_row_bytes(U); }
+__host__ __device__ constexpr int batch_partial_slot_bytes() { return kBW * 1024; }
+
+// ---- the walk of a workgroup over its items.  All fields are wavefront-uniform.
+struct ItemCursor {
+  int lin;           // current linear (nlin: past the end)
+  int panel, lt;     // panel of K, local tile (tile = lt * ncu + rb)
+  int T, P;          // tiles of this workgroup in the linear (> 0), panels
+  int ncu, rb;       // workgroups in the linear's group; (member - off) mod ncu
+  int N, G, row_w;   // rows, scale groups per row, bytes per row of W
+  const char* W;
+  const char* S;
+};
+
+// positions the cursor on the first linear >= c.lin in which this workgroup holds a tile
+template <int U>
+__device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg) {
+  typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
+  while (c.lin < nlin) {
+    const words_ptr p = (words_ptr)(descs + c.lin);
+    const uint32_t grp = p[16];
+    const int gl = (int)(grp & 0xffu);
+    if ((b & ((1 << gl) - 1)) == (int)((grp >> 8) & 0xffu)) {  // this workgroup's group runs the linear
+      uint32_t w[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) w[i] = p[i];
+      const int ncu = nwg >> gl;
+      int rb = (b >> gl) - (int)(w[15] >> 16);
+      if (rb < 0) rb += ncu;
+      const int T = (int)w[13] + (rb < (int)(w[15] & 0xffffu) ? 1 : 0);
+      if (T > 0) {
+        const int G = (int)(w[14] & 0xffffu);
+        c.T = T;
+        c.rb = rb;
+        c.ncu = ncu;
+        c.G = G;
+        c.P = (G + batch_panel_groups(U) - 1) / batch_panel_groups(U);
+        c.N = (int)w[12];
+        c.row_w = G << 4;
+        c.W = reinterpret_cast<const char*>(((uint64_t)w[1] << 32) | w[0]);
+        c.S = reinterpret_cast<const char*>(((uint64_t)w[3] << 32) | w[2]);
+        c.panel = 0;
+        c.lt = 0;
+        return;
+      }
+    }
+    ++c.lin;
+  }
+}
+
+template <int U>
+__device__ __forceinline__ void item_next_panel(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg) {
+  c.lt = 0;
+  if (++c.panel == c.P) {
+    ++c.lin;
+    item_seek<U>(c, descs, nlin, b, nwg);
+  }
+}
+
+template <int U>
+__device__ __forceinline__ void item_next(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg) {
+  if (++c.lt == c.T) item_next_panel<U>(c, descs, nlin, b, nwg);
+}
+
+template <int U>
+__global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvListDesc* __restrict__ descs_, int nlin,
+                                                                     int* __restrict__ sync, long long spin_limit,
+                                                                     int M, int nxb, int ring, int use_sync) {
+  constexpr int PG = batch_panel_groups(U);  // scale groups per panel
+  constexpr int NT = kBNT;
+  constexpr int SROW = batch_scale_row_bytes(U), SSLOT = batch_scale_slot_bytes(U);
+  extern __shared__ uint4_t smem[];
+  const gemv_desc_ptr descs = (gemv_desc_ptr)descs_;
+  char* lds = reinterpret_cast<char*>(smem);
+  // flags | nxb panels of activations, M x PG x 64 bytes each | `ring` scale slots | `ring` partial-sum slots |
+  // sums kept between panels.  `ring` (2 or 4) is how many items the compute wavefronts may spread over.
+  BatchFlags* flags = reinterpret_cast<BatchFlags*>(lds);
+  char* const xbuf = lds + sizeof(BatchFlags);
+  const int xbuf_bytes = M * (PG * 64);
+  char* const sbuf = xbuf + nxb * xbuf_bytes;
+  char* const pbuf = sbuf + ring * SSLOT;
+  char* const abuf = pbuf + ring * batch_partial_slot_bytes();
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nwg = gridDim.x;
+  const int b = blockIdx.x;
+  const BatchWait wait{flags, sync + sync_error_index(nlin), spin_limit > 0 ? spin_limit : 1000000};
+
+  if (tid < (int)(sizeof(BatchFlags) / sizeof(int))) reinterpret_cast<int*>(flags)[tid] = 0;
+  lds_done_then_barrier();  // LDS starts undefined: the flags are cleared before anyone looks
+
+  if (wave < kBW) {
+    // =========================== compute wavefront ===========================
+    const int i = lane & 15, kq = lane >> 4;
+    // The tile buffers are loaded in assembly and waited for by hand (loads retire in order and a
+    // compute wavefront issues no other vector memory operation).  `magic` (0x6400 in both halves,
+    // OR-ed under every code) doubles as the token that orders the reads of a buffer behind the wait
+    // for it: the wait "modifies" magic, every first read of a buffer register takes magic as an
+    // operand, and the registers appear in no other statement (checked in the generated code at
+    // build time).
+    uint4_t tb[NT][U];
+    uint32_t magic = 0x64006400u;
+    int ahead = 0;  // items issued and not yet consumed
+    ItemCursor ic, cc;
+    ic.lin = 0;
+    item_seek<U>(ic, descs, nlin, b, nwg);
+    cc = ic;
+    int k = 0;    // items consumed
+    int pk = -1;  // panels taken
+    half8_t xb[U][4];
+    const int gi0 = wave * (4 * U) + kq;  // the lane's scale group within the panel, chunk 0
+
+    auto issue = [&](uint4_t (&buf)[U]) {
+      if (ic.lin >= nlin) return;
+      const int n0 = (ic.lt * ic.ncu + ic.rb) << 4;
+      const int rows = min(16, ic.N - n0);                // >= 1
+      const int pg = min(PG, ic.G - ic.panel * PG);       // scale groups of this panel (the last may be short)
+      const char* base = ic.W + (int64_t)n0 * ic.row_w + ic.panel * (PG * 16);
+      const uint32_t roff = __umul24((uint32_t)min(i, rows - 1), (uint32_t)ic.row_w);
+      // rows past N repeat the last row (never stored); groups past K repeat the last group (their
+      // activations and scales are staged as zeros)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t voff = roff + (uint32_t)min(gi0 + 4 * u, pg - 1) * 16u;
+        asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(buf[u]) : "v"(voff), "s"(base));
+      }
+      ++ahead;
+      item_next<U>(ic, descs, nlin, b, nwg);
+    };
+
+    const half2_t k1031 = {(half_t)-1031.0f, (half_t)-1031.0f};
+    const half2_t k1136 = {(half_t)-1136.0f, (half_t)-1136.0f};
+    auto ring_shr8 = [&](uint32_t word) {
+      uint32_t r;
+      asm("v_lshrrev_b32 %0, 8, %1 ; %2" : "=v"(r) : "v"(word), "v"(magic));
+      return r;
+    };
+    // (t + c) * s with s taken from the low half of `s16` for both results: two roundings, as the format defines
+    auto unpack = [&](uint32_t t, half2_t c, uint32_t s16) {
+      const half2_t d = as_half2(t) + c;
+      uint32_t r;
+      asm("v_pk_mul_f16 %0, %1, %2 op_sel_hi:[1,0]" : "=v"(r) : "v"(d), "v"(s16));
+      return r;
+    };
+
+    auto consume = [&](uint4_t (&buf)[U]) {
+      if (cc.lt == 0) {
+        // a new panel: its activations are staged (or will be); this wavefront's K slice goes to registers
+        ++pk;
+        const int xslot = pk % nxb;
+        wait.until(&flags->x_ready[xslot], pk + 1, 1);
+        const char* xs = xbuf + xslot * xbuf_bytes + (wave * U * 16 * M + kq * M + min(i, M - 1)) * 16;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) xb[u][d] = *reinterpret_cast<const half8_t*>(xs + ((u * 4 + d) * 4 * M) * 16);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) __hip_atomic_fetch_add(&flags->x_taken[xslot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      wait.until(&flags->s_ready, k + 1, 2);
+      const int slot = k & (ring - 1);
+      const char* sb = sbuf + slot * SSLOT + i * SROW + gi0 * 2;
+      float4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t s16 = *reinterpret_cast<const uint16_t*>(sb + u * 8);
+        if (ahead == NT) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"((NT - 1) * U + (U - 1 - u)));
+        else asm volatile("s_waitcnt vmcnt(0)" : "+v"(magic));
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t word = d == 0 ? buf[u].x : d == 1 ? buf[u].y : d == 2 ? buf[u].z : buf[u].w;
+          const uint32_t w8 = ring_shr8(word);
+          const uint32_t a0 = unpack(and_or(word, 0x000F000Fu, magic), k1031, s16);  // (q0, q4)
+          const uint32_t a1 = unpack(and_or(word, 0x00F000F0u, magic), k1136, s16);  // 16 (q1, q5)
+          const uint32_t a2 = unpack(and_or(w8, 0x000F000Fu, magic), k1031, s16);    // (q2, q6)
+          const uint32_t a3 = unpack(and_or(w8, 0x00F000F0u, magic), k1136, s16);    // 16 (q3, q7)
+          const half8_t aop = __builtin_bit_cast(half8_t, uint4_t{a0, a1, a2, a3});
+          if (d & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, xb[u][d], acc1, 0, 0, 0);
+          else acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, xb[u][d], acc0, 0, 0, 0);
+        }
+      }
+      --ahead;
+      const float4_t part = acc0 + acc1;
+      if (k >= ring) wait.until(&flags->y_done, k - ring + 1, 3);
+      *reinterpret_cast<float4_t*>(pbuf + (slot * kBW + wave) * 1024 + lane * 16) = part;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      if (lane == 0) __hip_atomic_fetch_add(&flags->done[slot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      ++k;
+      item_next<U>(cc, descs, nlin, b, nwg);
+    };
+
+#pragma unroll
+    for (int t = 0; t < NT - 1; ++t) issue(tb[t]);
+    while (cc.lin < nlin) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        issue(tb[(t + NT - 1) % NT]);
+        if (cc.lin < nlin) consume(tb[t]);
+      }
+    }
+    return;
+  }
+
+  bool aborted = false;
+
+  if (wave < kBW + kBXW) {
+    // ====================== x wavefronts: a panel of activations -> LDS ======================
+    const int xw = wave - kBW;
+    // until every workgroup has signalled linear `dep`, or the spin limit passes
+    auto wait_for = [&](int dep) {
+      if (aborted) return;
+      const long long t0 = wall_clock64();
+      while (true) {
+        // read-modify-write (+ 0): performed where the counter lives, never served from a stale cache line
+        int v = 0;
+        if (lane < kCountersPerLinear)
+          v = __hip_atomic_fetch_add(sync + sync_counter_index(dep, lane), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 4, 64);
+        if (__builtin_amdgcn_readfirstlane(v) >= (nwg >> descs[dep].gmod_log2)) break;  // every member of its group
+        if (wall_clock64() - t0 > spin_limit) {
+          aborted = true;
+          if (lane == 0)
+            __hip_atomic_store(sync + sync_error_index(nlin), dep + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      // whatever this XCD's L2 still holds of an earlier content of x (the addresses are reused
+      // from launch to launch) must not serve the loads that follow
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    };
+
+    const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+    constexpr int PPR = PG * 4;  // 16-byte pieces (8 activations) per row and panel; a power of two
+    constexpr int UX = 32;       // loads in flight per lane: one round trip for a panel of 8 rows x 2048 k
+    ItemCursor xc;
+    xc.lin = 0;
+    item_seek<U>(xc, descs, nlin, b, nwg);
+    // the x wavefronts take whole panels by turns (panel pk belongs to wavefront pk mod kBXW) and run up
+    // to nxb panels ahead of the compute wavefronts: under load a round trip to L2 takes several microseconds
+    int pk = 0;
+    int confirmed = -1;  // the latest producer linear this wavefront has seen complete
+    while (xc.lin < nlin) {
+      if (pk % kBXW == xw) {
+        const int xslot = pk % nxb;
+        // the buffer is free once every compute wavefront has copied the panel that used it before
+        if (pk >= nxb) wait.until(&flags->x_taken[xslot], kBW * (pk / nxb), 4);
+        const int j = xc.lin;
+        const int dep = (int)((descs[j].g_dep >> 16) & 0x7fffu) - 1;
+        if (dep >= 0 && dep != confirmed) {
+          wait_for(dep);
+          confirmed = dep;
+        }
+        const int K = xc.G << 5;
+        const int K8 = K >> 3;
+        // an x that other workgroups of this launch have written is read with device-scope loads (sc1)
+        const __amdgpu_buffer_rsrc_t xr =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(descs[j].x), 0, M * K * 2, kBufferFlags);
+        char* const xdst = xbuf + xslot * xbuf_bytes;
+        const int total = M * PPR;
+        for (int base = 0; base < total; base += 64 * UX) {
+          uint4_t v[UX];
+#pragma unroll
+          for (int t = 0; t < UX; ++t) {
+            const int idx = base + t * 64 + lane;
+            const int row = idx / PPR, o = idx & (PPR - 1);
+            const int go = xc.panel * PPR + o;  // the piece's place in the row
+            v[t] = uint4_t{0, 0, 0, 0};
+            if (idx < total && go < K8)
+              v[t] = dep >= 0 ? __builtin_amdgcn_raw_buffer_load_b128(xr, (row * K8 + go) * 16, 0, kDeviceScope)
+                              : __builtin_amdgcn_raw_buffer_load_b128(xr, (row * K8 + go) * 16, 0, 0);
+          }
+#pragma unroll
+          for (int t = 0; t < UX; ++t) {
+            const int idx = base + t * 64 + lane;
+            if (idx < total) {
+              const int row = idx / PPR, o = idx & (PPR - 1);
+              const uint32_t in[4] = {v[t].x, v[t].y, v[t].z, v[t].w};
+              uint32_t p[4];
+              pair_i_i4(in, p);  // p[e] = (x_e, x_{e+4})
+              // piece o: scale group g = o / 4, dword d = o % 4 of it; the group belongs to wavefront
+              // g / 4U, chunk (g / 4) % U, lane quarter g % 4
+              const int g = o >> 2, d = o & 3;
+              const int cw = g / (4 * U), cu = (g >> 2) & (U - 1), ckq = g & 3;
+              char* dst = xdst + ((((cw * U + cu) * 4 + d) * 4 + ckq) * M + row) * 16;
+              *reinterpret_cast<uint4_t*>(dst) =
+                  uint4_t{p[0], as_u32(as_half2(p[1]) * sixteenth), p[2], as_u32(as_half2(p[3]) * sixteenth)};
+            }
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) __hip_atomic_store(&flags->x_ready[xslot], pk + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      ++pk;
+      item_next_panel<U>(xc, descs, nlin, b, nwg);
+    }
+    return;
+  }
+
+  if (wave == kBW + kBXW) {
+    // ====================== scale wavefront: the scales of a tile -> LDS ======================
+    constexpr int PD = 3;            // items in flight in registers
+    constexpr int PPR = PG / 8;      // 16-byte pieces (8 scales) per row and panel
+    constexpr int LP = 16 * PPR / 64;  // pieces per lane and item
+    uint4_t sv[PD][LP];
+    ItemCursor ic, cc;
+    ic.lin = 0;
+    item_seek<U>(ic, descs, nlin, b, nwg);
+    cc = ic;
+    int k = 0;
+    auto issue = [&](uint4_t (&buf)[LP]) {
+      if (ic.lin >= nlin) return;
+      const int n0 = (ic.lt * ic.ncu + ic.rb) << 4;
+      const int pg = min(PG, ic.G - ic.panel * PG);
+      const char* base = ic.S + ic.panel * (PG * 2);
+#pragma unroll
+      for (int t = 0; t < LP; ++t) {
+        const int idx = t * 64 + lane;
+        const int r = idx / PPR, pc = idx % PPR;
+        buf[t] = uint4_t{0, 0, 0, 0};  // groups past K: a zero scale
+        if (pc * 8 < pg)
+          buf[t] = __builtin_nontemporal_load(
+              reinterpret_cast<const uint4_t*>(base + (int64_t)min(n0 + r, ic.N - 1) * (ic.G * 2) + pc * 16));
+      }
+      item_next<U>(ic, descs, nlin, b, nwg);
+    };
+    auto consume = [&](uint4_t (&buf)[LP]) {
+      const int slot = k & (ring - 1);
+      // the slot is free once every compute wavefront has finished the item that used it before
+      if (k >= ring) wait.until(&flags->done[slot], kBW * (k / ring), 5);
+#pragma unroll
+      for (int t = 0; t < LP; ++t) {
+        const int idx = t * 64 + lane;
+        const int r = idx / PPR, pc = idx % PPR;
+        *reinterpret_cast<uint4_t*>(sbuf + slot * SSLOT + r * SROW + pc * 16) = buf[t];
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      ++k;
+      if (lane == 0) __hip_atomic_store(&flags->s_ready, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      item_next<U>(cc, descs, nlin, b, nwg);
+    };
+#pragma unroll
+    for (int t = 0; t < PD - 1; ++t) issue(sv[t]);
+    while (cc.lin < nlin) {
+#pragma unroll
+      for (int t = 0; t < PD; ++t) {
+        issue(sv[(t + PD - 1) % PD]);
+        if (cc.lin < nlin) consume(sv[t]);
+      }
+    }
+    return;
+  }
+
+  // ================== y wavefront: partial sums -> y, completion signals ==================
+  {
+    const int j16 = lane & 15, rq = lane >> 4;
+    int k = 0;
+    for (int lin = 0; lin < nlin; ++lin) {
+      const uint32_t g_dep = descs[lin].g_dep;
+      const int gl = descs[lin].gmod_log2;
+      if ((b & ((1 << gl) - 1)) != (int)descs[lin].gidx) continue;  // another group's linear
+      const int ncu = nwg >> gl;
+      int rb = (b >> gl) - (int)descs[lin].off;
+      if (rb < 0) rb += ncu;
+      const int T = descs[lin].q + (rb < (int)descs[lin].rem ? 1 : 0);
+      const int N = descs[lin].N;
+      const int P = ((int)(g_dep & 0xffffu) + PG - 1) / PG;
+      const half_t* bias = descs[lin].bias;
+      const half_t* residual = descs[lin].residual;
+      const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[lin].y, 0, M * N * 2, kBufferFlags);
+      for (int panel = 0; panel < (T > 0 ? P : 0); ++panel) {
+        for (int lt = 0; lt < T; ++lt, ++k) {
+          const int slot = k & (ring - 1);
+          wait.until(&flags->done[slot], kBW * (k / ring + 1), 6);
+          const char* pb = pbuf + slot * batch_partial_slot_bytes() + lane * 16;
+          float4_t sum = *reinterpret_cast<const float4_t*>(pb);
+#pragma unroll
+          for (int w = 1; w < kBW; ++w) sum += *reinterpret_cast<const float4_t*>(pb + w * 1024);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          if (lane == 0) __hip_atomic_store(&flags->y_done, k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if (P > 1) {
+            float4_t* keep = reinterpret_cast<float4_t*>(abuf + lt * 1024 + lane * 16);
+            if (panel > 0) sum += *keep;
+            if (panel < P - 1) {
+              *keep = sum;
+              continue;
+            }
+          }
+          // lane (j, rq) holds rows n0 + 4 rq .. + 3 of activation row j
+          const int n0 = ((lt * ncu + rb) << 4) + 4 * rq;
+          if (j16 < M) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int n = n0 + r;
+              if (n < N) {
+                float v = sum[r];
+                if (bias) v += (float)bias[n];
+                half_t h = (half_t)v;
+                if (residual) h = h + residual[(int64_t)j16 * N + n];
+                // device-scope store: written through, so that a counter update after it publishes it
+                __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (j16 * N + n) * 2, 0, kDeviceScope);
+              }
+            }
+          }
+        }
+      }
+      if (g_dep & kSignal) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores of this workgroup have been written through
+        if (lane == 0)
+          __hip_atomic_fetch_add(sync + sync_counter_index(lin, b & (kCountersPerLinear - 1)), 1, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (!use_sync) return;
+    // the last workgroup to get here clears the counters for the next launch
+    int last = 0;
+    if (lane == 0)
+      last = __hip_atomic_fetch_add(sync + sync_finished_index(nlin), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+             nwg - 1;
+    if (__builtin_amdgcn_readfirstlane(last)) {
+      for (int i = lane; i < nlin * kCountersPerLinear; i += 64)
+        __hip_atomic_store(sync + i * kCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0)
+        __hip_atomic_store(sync + sync_finished_index(nlin), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ host side
+static size_t batch_lds_bytes(int U, int M, int nxb, int ring, int acc_tiles) {
+  return sizeof(BatchFlags) + (size_t)nxb * M * batch_panel_groups(U) * 64 + (size_t)ring * batch_scale_slot_bytes(U) +
+         (size_t)ring * batch_partial_slot_bytes() + (size_t)acc_tiles * 1024;
+}
+
+// Which group of workgroups runs which linear.  Every workgroup needs all M x K activations of a linear
+// it takes part in, and those bytes cost what weight bytes cost (they pass the same memory pipeline of the
+// CU): with 256 workgroups on a 4096-row linear that is twice the weights at M = 8.  So a list is run by 2^g
+// groups side by side, each linear by one group (group = workgroup index mod 2^g, which is one XCD for
+// g = 3: the activations then stay in that XCD's L2): a workgroup sees 1 / 2^g of the linears and 2^g times
+// as many rows of each.  Linears go, in list order, to the group that can start them first (a consumer
+// not before its producer has ended), with the duration of a linear estimated from the bytes a workgroup
+// moves for it; g is the best of 0 .. 3 by that estimate.
+struct BatchGroupPlan {
+  std::vector<int> group;
+  double makespan = 0.0;
+};
+
+static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl) {
+  const int groups = 1 << gl, ncu = l->blocks >> gl;
+  BatchGroupPlan plan;
+  plan.group.resize(l->n);
+  std::vector<double> free_at(groups, 0.0), end(l->n, 0.0);
+  for (int i = 0; i < l->n; ++i) {
+    const GemvListDesc& g = l->descs[i];
+    const double K = (double)(g.g_dep & 0xffffu) * 32.0;
+    const double tiles = ((double)g.N + 15.0) / 16.0;
+    // bytes through one workgroup: its tiles' codes and scales, and all activations
+    const double dur = std::ceil(tiles / ncu) * 16.0 * K * (0.5 + 1.0 / 16.0) + l->M * K * 2.0 + 4096.0;
+    const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
+    const double ready = dep >= 0 ? end[dep] : 0.0;
+    int best = 0;
+    for (int c = 1; c < groups; ++c) {
+      const double sb = std::max(free_at[best], ready), sc = std::max(free_at[c], ready);
+      if (sc < sb || (sc == sb && free_at[c] > free_at[best])) best = c;  // earliest start, then least idle time
+    }
+    plan.group[i] = best;
+    end[i] = std::max(free_at[best], ready) + dur;
+    free_at[best] = end[i];
+  }
+  for (double f : free_at) plan.makespan = std::max(plan.makespan, f);
+  return plan;
+}
+
+int batch_list_plan(wq_gemv_list* l) {
+  const int U = l->M <= 8 ? 4 : 2;  // panels of 4096 k (M <= 8) or 2048 k: 64 KiB of activations at most
+  l->batch_u = U;
+  l->gs = 4;
+  l->threads = kBThreads;
+  l->blocks = std::min(cu_count(), 32768);
+  const size_t budget = 160 * 1024;
+  int best_gl = -1;
+  BatchGroupPlan best;
+  int best_acc = 0;
+  for (int gl = 0; gl <= 3; ++gl) {
+    if (l->blocks % (1 << gl) != 0 || (l->blocks >> gl) < 1) break;
+    const int ncu = l->blocks >> gl;
+    int acc_tiles = 0;
+    for (int i = 0; i < l->n; ++i) {
+      const GemvListDesc& g = l->descs[i];
+      const int64_t tiles = ((int64_t)g.N + 15) >> 4;
+      if ((int)(g.g_dep & 0xffffu) > batch_panel_groups(U)) acc_tiles = std::max<int>(acc_tiles, (int)((tiles + ncu - 1) / ncu));
+    }
+    if (batch_lds_bytes(U, l->M, 1, 2, acc_tiles) > budget) continue;  // sums kept between panels do not fit
+    BatchGroupPlan p = batch_assign_groups(l, gl);
+    if (best_gl < 0 || p.makespan < best.makespan * 0.98) {
+      best_gl = gl;
+      best = std::move(p);
+      best_acc = acc_tiles;
+    }
+  }
+  if (best_gl < 0)
+    return fail(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: %d rows of activations do not fit the LDS", l->M);
+  const int groups = 1 << best_gl, ncu = l->blocks >> best_gl;
+  std::vector<int64_t> off(groups, 0);
+  for (int i = 0; i < l->n; ++i) {
+    GemvListDesc& g = l->descs[i];
+    const int c = best.group[i];
+    const int64_t tiles = ((int64_t)g.N + 15) >> 4;
+    g.q = (int32_t)(tiles / ncu);
+    g.rem = (uint16_t)(tiles % ncu);
+    g.off = (uint16_t)off[c];
+    off[c] = (off[c] + tiles) % ncu;
+    g.gmod_log2 = (uint8_t)best_gl;
+    g.gidx = (uint8_t)c;
+  }
+  l->batch_groups = groups;
+  l->batch_acc_tiles = best_acc;
+  // a ring of 4 items and up to 2 panels of activations in LDS if they fit, else a ring of 2
+  l->batch_ring = 4;
+  l->batch_nxb = batch_lds_bytes(U, l->M, 2, 4, best_acc) <= budget ? 2 : batch_lds_bytes(U, l->M, 1, 4, best_acc) <= budget ? 1 : 0;
+  if (!l->batch_nxb) {
+    l->batch_ring = 2;
+    l->batch_nxb = batch_lds_bytes(U, l->M, 2, 2, best_acc) <= budget ? 2 : 1;
+  }
+  l->lds = batch_lds_bytes(U, l->M, l->batch_nxb, l->batch_ring, best_acc);
+  const void* kern = U == 4 ? reinterpret_cast<const void*>(q4g32_batch_list_kernel<4>)
+                            : reinterpret_cast<const void*>(q4g32_batch_list_kernel<2>);
+  if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l->lds) != hipSuccess)
+    return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
+  int resident = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
+    return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: the workgroup does not fit a CU (%zu bytes of LDS)", l->lds);
+  return WQ_OK;
+}
+
+int batch_list_launch(wq_gemv_list* l, hipStream_t stream) {
+  const GemvListDesc* table = (const GemvListDesc*)l->table;
+  const int use_sync = l->deps > 0 ? 1 : 0;
+  if (l->batch_u == 4) {
+    WQ_LAUNCH("wq_q4g32_gemv_list_run", q4g32_batch_list_kernel<4>, dim3((unsigned)l->blocks), dim3((unsigned)l->threads),
+              l->lds, stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, use_sync);
+  } else {
+    WQ_LAUNCH("wq_q4g32_gemv_list_run", q4g32_batch_list_kernel<2>, dim3((unsigned)l->blocks), dim3((unsigned)l->threads),
+              l->lds, stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, use_sync);
+  }
+  return WQ_OK;
+}
+
+}  // namespace wq

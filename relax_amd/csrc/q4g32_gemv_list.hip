@@ -39,47 +39,13 @@
 #include <memory>
 #include <vector>
 
+#include "gemv_list_common.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
 namespace wq {
 
-struct GemvListDesc {  // 64 bytes, device memory
-  const char* W;       // uint32 [N, K/8]
-  const char* S;       // fp16   [N, K/32]
-  const half_t* x;     // fp16   [K]
-  const half_t* bias;  // fp16   [N] or null
-  const half_t* residual;  // fp16 [N] or null
-  half_t* y;           // fp16   [N]
-  int32_t N;
-  int32_t q;           // row groups / workgroups  (a row group is 2^gs consecutive rows)
-  uint32_t g_dep;      // bits 0..15: K / 32; bits 16..30: 1 + the linear of this list that writes x (0: none);
-                       // bit 31: a later linear reads y
-  uint16_t rem;        // row groups % workgroups
-  uint16_t off;        // rotation: workgroup b owns the row groups local * workgroups + ((b - off) mod workgroups)
-};
-static_assert(sizeof(GemvListDesc) == 64, "descriptor layout");
-constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y
-
-typedef const GemvListDesc __attribute__((address_space(4)))* gemv_desc_ptr;  // scalar loads
-
-constexpr int kCounterStride = 16;   // ints between two counters (64 bytes: one cache line each)
-constexpr int kCountersPerLinear = 8;
-constexpr int kChunkBytes = 4096 + 256;
-constexpr int kBufferFlags = 0x00020000;  // buffer resource word 3: 32-bit data format, no swizzle
-constexpr int kDeviceScope = 16;          // cache policy bit sc1: the access is coherent over the whole device  // LDS bytes per chunk of x: 4 x 64 uint4 + 64 floats
-
-// sync layout (ints): [lin][8] counters at stride kCounterStride, then `finished`, then `error`
-__host__ __device__ inline int sync_counter_index(int lin, int k) { return (lin * kCountersPerLinear + k) * kCounterStride; }
-__host__ __device__ inline int sync_finished_index(int nlin) { return sync_counter_index(nlin, 0); }
-__host__ __device__ inline int sync_error_index(int nlin) { return sync_counter_index(nlin, 1); }
-__host__ __device__ inline int sync_ints(int nlin) { return sync_counter_index(nlin, 2); }
-
-__device__ __forceinline__ void lds_done_then_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
+constexpr int kChunkBytes = 4096 + 256;  // LDS bytes per chunk of x: 4 x 64 uint4 + 64 floats
 
 // ---- where a workgroup's rows are: its rows of all linears, in list order, form one sequence of
 // ---- positions 0, 1, 2, ...; a cursor maps a position to (linear, local row).  Forward only.
@@ -151,11 +117,6 @@ struct ListFlags {
   int next_x;    // the next linear whose activations no x wavefront has taken
   int pad[5];
 };
-
-__device__ __forceinline__ void lds_spin_until(const int* flag, int target) {
-  while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) __builtin_amdgcn_s_sleep(1);
-  asm volatile("" ::: "memory");  // LDS is served in order: what was written before the flag is visible now
-}
 
 #ifdef WQ_LIST_TRACE
 __device__ long long* g_list_trace = nullptr;  // [workgroup 0 | workgroup 100][64] wall-clock stamps
@@ -532,30 +493,12 @@ static bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
 
 }  // namespace wq
 
-struct wq_gemv_list {
-  std::vector<wq::GemvListDesc> descs;
-  int n = 0;
-  void* table = nullptr;  // device: descriptors
-  int* sync = nullptr;    // device: counters
-  int blocks = 0, threads = 0;
-  size_t lds = 0;
-  int xbuf_bytes = 0, ybuf_floats = 0;
-  int late = 0, deps = 0;
-  int nb = 2;
-  int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
-  long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
-};
-
 namespace wq {
 
 constexpr int kListNC = 13;    // compute wavefronts per workgroup
 constexpr int kListXW = 2;     // wavefronts that stage activations
 constexpr int kListDepth = 4;  // ring slots (KiB of codes in flight) per compute wavefront: 52 KiB per CU
                                // (2, 3, 4 and 6 slots measure the same within 2 %)
-constexpr size_t kListAlign = 256;
-
-static size_t list_table_bytes(int n) { return ((size_t)n * sizeof(GemvListDesc) + kListAlign - 1) / kListAlign * kListAlign; }
-
 }  // namespace wq
 
 extern "C" size_t wq_q4g32_gemv_list_workspace_bytes(int n) {
@@ -566,10 +509,17 @@ extern "C" size_t wq_q4g32_gemv_list_workspace_bytes(int n) {
 extern "C" void wq_q4g32_gemv_list_destroy(wq_gemv_list_t* l) { delete l; }
 
 extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d, int n, void* workspace,
-                                                     size_t workspace_bytes, wq_stream_t stream_) {
+                                                     size_t workspace_bytes, wq_stream_t stream) {
+  return wq_q4g32_gemv_list_create_batched(d, n, 1, workspace, workspace_bytes, stream);
+}
+
+extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv_desc* d, int n, int M, void* workspace,
+                                                             size_t workspace_bytes, wq_stream_t stream_) {
   using namespace wq;
   hipStream_t stream = (hipStream_t)stream_;
 #define bad(code, ...) ((void)fail(code, __VA_ARGS__), (wq_gemv_list_t*)nullptr)
+  if (M < 1 || M > WQ_GEMV_LIST_MAX_M)
+    return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: 1 .. %d rows of activations, got %d", WQ_GEMV_LIST_MAX_M, M);
   if (!d || n <= 0 || n > WQ_GEMV_LIST_MAX) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: need 1 .. %d linears, got %d", WQ_GEMV_LIST_MAX, n);
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & (kListAlign - 1)) ||
       workspace_bytes < wq_q4g32_gemv_list_workspace_bytes(n))
@@ -577,6 +527,7 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
                wq_q4g32_gemv_list_workspace_bytes(n));
   std::unique_ptr<wq_gemv_list> l(new wq_gemv_list());
   l->n = n;
+  l->M = M;
   l->descs.resize(n);
   int cmax = 1;
   for (int i = 0; i < n; ++i) {
@@ -587,6 +538,9 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
     if (!s.W || !s.S || !s.x || !s.y) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: null pointer", i);
     if (!aligned16(s.W) || !aligned16(s.x))
       return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: W and x must be 16-byte aligned", i);
+    // several rows: the scales travel in 16-byte pieces of 8, and rows of x and y are addressed with 32-bit offsets
+    if (M > 1 && (s.K % 256 != 0 || !aligned16(s.S) || (int64_t)M * s.N >= (1ll << 30) || s.K / 32 > 0xffff))
+      return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d: with %d rows of activations K=%lld must be a multiple of 256, S 16-byte aligned and M * N < 2^30", i, M, (long long)s.K);
     GemvListDesc& g = l->descs[i];
     g.W = reinterpret_cast<const char*>(s.W);
     g.S = reinterpret_cast<const char*>(s.S);
@@ -607,16 +561,16 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
     const wq_q4g32_gemv_desc& a = d[i];
     for (int j = i - 1; j >= 0; --j) {
       const wq_q4g32_gemv_desc& b = d[j];
-      const size_t yb = (size_t)b.N * 2, ya = (size_t)a.N * 2;
-      if (((l->descs[i].g_dep >> 16) & 0x7fffu) == 0 && ranges_overlap(a.x, (size_t)a.K * 2, b.y, yb))
+      const size_t yb = (size_t)b.N * 2 * M, ya = (size_t)a.N * 2 * M;
+      if (((l->descs[i].g_dep >> 16) & 0x7fffu) == 0 && ranges_overlap(a.x, (size_t)a.K * 2 * M, b.y, yb))
         l->descs[i].g_dep |= (uint32_t)(j + 1) << 16;
-      if (ranges_overlap(a.residual, ya, b.y, yb) || ranges_overlap(a.bias, ya, b.y, yb))
+      if (ranges_overlap(a.residual, ya, b.y, yb) || ranges_overlap(a.bias, (size_t)a.N * 2, b.y, yb))
         return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i, j);
-      if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, (size_t)b.K * 2) ||
-          ranges_overlap(a.y, ya, b.residual, yb) || ranges_overlap(a.y, ya, b.bias, yb))
+      if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, (size_t)b.K * 2 * M) ||
+          ranges_overlap(a.y, ya, b.residual, yb) || ranges_overlap(a.y, ya, b.bias, (size_t)b.N * 2))
         return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the output of linear %d overlaps an operand of linear %d", i, j);
     }
-    if (ranges_overlap(a.y, (size_t)a.N * 2, a.x, (size_t)a.K * 2))
+    if (ranges_overlap(a.y, (size_t)a.N * 2 * M, a.x, (size_t)a.K * 2 * M))
       return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: y overlaps x", i);
     const int dep = (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1;
     if (dep >= 0) {
@@ -625,6 +579,9 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
       if (dep == i - 1) ++l->late;
     }
   }
+  if (M > 1) {
+    if (batch_list_plan(l.get()) != WQ_OK) return nullptr;
+  } else {
   // launch shape: one workgroup of 16 wavefronts per CU.  Workgroup b owns the rows
   // n = local * workgroups + ((b - off) mod workgroups); `off` continues the round-robin where the
   // previous linear ended, so that the remainders of all linears spread over the workgroups.
@@ -656,6 +613,7 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
     return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: the workgroup does not fit a CU (%zu bytes of LDS)", l->lds);
+  }
   l->table = workspace;
   l->sync = reinterpret_cast<int*>(static_cast<char*>(workspace) + list_table_bytes(n));
   if (hipMemcpyAsync(l->table, l->descs.data(), (size_t)n * sizeof(GemvListDesc), hipMemcpyHostToDevice, stream) != hipSuccess ||
@@ -669,6 +627,7 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
 extern "C" int wq_q4g32_gemv_list_run(wq_gemv_list_t* l, wq_stream_t stream) {
   using namespace wq;
   WQ_REQUIRE(l && l->table, "wq_q4g32_gemv_list_run: null list");
+  if (l->M > 1) return batch_list_launch(l, (hipStream_t)stream);
   WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>), dim3((unsigned)l->blocks),
             dim3((unsigned)l->threads), l->lds, (hipStream_t)stream, (const GemvListDesc*)l->table, l->n, l->sync,
             l->spin_limit, l->xbuf_bytes, l->ybuf_floats, l->nb == 4 ? 2 : 1, l->gs, l->deps > 0 ? 1 : 0);
@@ -686,6 +645,9 @@ extern "C" int wq_q4g32_gemv_list_status(wq_gemv_list_t* l, wq_stream_t stream) 
   // the counters may be mid-count after an abandoned wait: start clean
   WQ_HIP(hipMemsetAsync(l->sync, 0, (size_t)sync_ints(l->n) * sizeof(int), (hipStream_t)stream));
   WQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+  if (err > kBatchInternalWait)
+    return fail(WQ_EDEVICE, "wq_q4g32_gemv_list: a hand-over inside a workgroup (kind %d) timed out; results of that launch are undefined",
+                err - kBatchInternalWait);
   return fail(WQ_EDEVICE,
               "wq_q4g32_gemv_list: a wait for linear %d timed out (the grid was not resident at once?); "
               "results of that launch are undefined",

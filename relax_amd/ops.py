@@ -148,9 +148,10 @@ class Q4G32GemvList:
     ``linears``: sequence of ``(W, S, x, y)`` or ``(W, S, x, y, bias, residual)`` device tensors; a linear
     whose ``x`` is the ``y`` of an earlier one waits for it on the device.  The tensors are kept alive by
     this object; the descriptor table and the counters live in a workspace allocated here, once.
+    ``M`` (1 .. 16): rows of activations of every linear of the list (x ``[M, K]``, y and residual ``[M, N]``).
     """
 
-    def __init__(self, linears):
+    def __init__(self, linears, M: int = 1):
         self._l = _lib.lib()
         n = len(linears)
         arr = (GemvDesc * max(1, n))()
@@ -167,17 +168,18 @@ class Q4G32GemvList:
             K = kw * 8
             if K % 32 or tuple(S.shape) != (N, K // 32):
                 raise ValueError(f"linear {i}: S must be [N, K/32] = [{N}, {K // 32}], got {tuple(S.shape)}")
-            if x.numel() != K or y.numel() != N:
-                raise ValueError(f"linear {i}: x must hold K={K} and y N={N} elements (one row each)")
-            for t, name in ((bias, "bias"), (residual, "residual")):
-                if t is not None and _dev(t, torch.float16, name).numel() != N:
-                    raise ValueError(f"linear {i}: {name} must hold N={N} elements")
+            if x.numel() != M * K or y.numel() != M * N:
+                raise ValueError(f"linear {i}: x must hold M*K={M * K} and y M*N={M * N} elements")
+            for t, name, want in ((bias, "bias", N), (residual, "residual", M * N)):
+                if t is not None and _dev(t, torch.float16, name).numel() != want:
+                    raise ValueError(f"linear {i}: {name} must hold {want} elements")
             arr[i] = GemvDesc(_ptr(W), _ptr(S), _ptr(x), _ptr(bias), _ptr(residual), _ptr(y), N, K)
             self._keep.append((W, S, x, y, bias, residual))
         need = self._l.wq_q4g32_gemv_list_workspace_bytes(n)
         self._workspace = torch.zeros(max(int(need), 256), dtype=torch.uint8, device="cuda")
-        self._h = self._l.wq_q4g32_gemv_list_create(arr, n, self._workspace.data_ptr(), self._workspace.numel(),
-                                                    _stream())
+        self.M = M
+        self._h = self._l.wq_q4g32_gemv_list_create_batched(arr, n, M, self._workspace.data_ptr(),
+                                                            self._workspace.numel(), _stream())
         if not self._h:
             raise _lib.WqError("wq_q4g32_gemv_list_create failed: " + self._l.wq_last_error().decode())
 

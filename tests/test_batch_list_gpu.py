@@ -1,0 +1,147 @@
+"""wq_q4g32_gemv_list_create_batched: a list of linears with 2 .. 16 rows of activations in one launch (matrix
+cores), against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need a GPU"
+    from relax_amd import ops
+    from tests import gpu_util
+
+    return ops, gpu_util, torch
+
+
+def _linear(oracle, u, N, K, M, seed):
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed)
+    return dict(W=W, S=S, x=x, dW=u.dev(W), dS=u.dev(S), N=N, K=K)
+
+
+# K = 256: one short panel; 4096: exactly one panel at M <= 8, two at M > 8; 11008: three panels, the last one short;
+# N = 1, 7, 130: fewer rows than a tile / a partial last tile; 40000: ten tiles per workgroup
+SHAPES = [(4096, 4096), (12288, 4096), (22016, 4096), (4096, 11008), (1, 256), (7, 512), (130, 11008), (1001, 2304),
+          (40000, 256), (48, 16384)]
+
+
+@pytest.mark.parametrize("M", [2, 5, 8, 9, 16])
+def test_independent_linears_match_oracle(env, oracle, M):
+    ops, u, torch = env
+    lins = []
+    for i, (N, K) in enumerate(SHAPES):
+        l = _linear(oracle, u, N, K, M, seed=200 + i)
+        l["dx"] = u.dev(l["x"])
+        l["y"] = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+        lins.append(l)
+    gl = ops.Q4G32GemvList([(l["dW"], l["dS"], l["dx"], l["y"]) for l in lins], M=M)
+    assert gl.info() == (0, 0)
+    print(f"batch list: independent linears, M = {M}", flush=True)
+    gl.run()
+    gl.status()
+    first = [l["y"].clone() for l in lins]
+    for l in lins:
+        u.assert_close(u.host(l["y"]), oracle.q4g32_linear(l["W"], l["S"], l["x"], nthreads=8), f"batch list M={M} {l['N']}x{l['K']}")
+    # launches repeat bit for bit: the partial sums are added in a fixed order
+    for rep in range(2):
+        for l in lins:
+            l["y"].zero_()
+        gl.run()
+        gl.status()
+        for l, f in zip(lins, first):
+            assert torch.equal(l["y"], f), (rep, l["N"], l["K"], float((l["y"].float() - f.float()).abs().max()),
+                                            int((l["y"] != f).sum()))
+
+
+def test_epilogue_and_one_hot(env, oracle):
+    ops, u, torch = env
+    M, N, K = 6, 520, 1024
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=7)
+    rng = np.random.default_rng(3)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    y2 = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    xh = np.zeros((M, K), np.float16)
+    cols = [0, 37, 260, 511, 777, 1023]
+    for m, c in enumerate(cols):
+        xh[m, c] = 1
+    dW, dS = u.dev(W), u.dev(S)
+    gl = ops.Q4G32GemvList([(dW, dS, u.dev(x), y, u.dev(bias), u.dev(res)), (dW, dS, u.dev(xh), y2)], M=M)
+    gl.run()
+    gl.status()
+    u.assert_close(u.host(y), oracle.q4g32_linear(W, S, x, bias=bias, residual=res), "batch list epilogue")
+    # a one-hot row of x selects a dequantized column exactly (every position of the 8-weight unpack is hit)
+    B = oracle.q4g32_dequant(W, S)
+    got = u.host(y2)
+    for m, c in enumerate(cols):
+        assert np.array_equal(got[m].view(np.uint16), B[:, c].view(np.uint16)), (m, c)
+
+
+@pytest.mark.parametrize("M", [4, 12])
+def test_dependent_chain_matches_oracle(env, oracle, M):
+    """x of a linear is the y of an earlier one: directly in front, one apart, two consumers of one producer; a
+    producer with several panels (K = 11008)."""
+    ops, u, torch = env
+    rng = np.random.default_rng(11)
+    a = _linear(oracle, u, 4096, 4096, M, seed=1)    # 0: x0 -> t0
+    b = _linear(oracle, u, 11008, 4096, M, seed=2)   # 1: t0 -> t1   (directly behind its producer)
+    c = _linear(oracle, u, 4096, 11008, M, seed=3)   # 2: t1 -> t2   (again directly behind, three panels)
+    d = _linear(oracle, u, 12288, 4096, M, seed=4)   # 3: t0 -> t3   (second consumer of t0)
+    e = _linear(oracle, u, 1024, 4096, M, seed=5)    # 4: t2 -> t4   (producer two in front)
+    x0 = rng.standard_normal((M, 4096)).astype(np.float16)
+    t = [torch.zeros((M, n), dtype=torch.float16, device="cuda") for n in (4096, 11008, 4096, 12288, 1024)]
+    gl = ops.Q4G32GemvList([(a["dW"], a["dS"], u.dev(x0), t[0]), (b["dW"], b["dS"], t[0], t[1]),
+                            (c["dW"], c["dS"], t[1], t[2]), (d["dW"], d["dS"], t[0], t[3]),
+                            (e["dW"], e["dS"], t[2], t[4])], M=M)
+    assert gl.info() == (4, 2)
+    print(f"batch list: dependent chain, M = {M}", flush=True)
+    r0 = oracle.q4g32_linear(a["W"], a["S"], x0, nthreads=8)
+    r1 = oracle.q4g32_linear(b["W"], b["S"], r0, nthreads=8)
+    r2 = oracle.q4g32_linear(c["W"], c["S"], r1, nthreads=8)
+    r3 = oracle.q4g32_linear(d["W"], d["S"], r0, nthreads=8)
+    r4 = oracle.q4g32_linear(e["W"], e["S"], r2, nthreads=8)
+    for rep in range(3):
+        for y in t:
+            y.zero_()
+        gl.run()
+        gl.status()
+        for got, ref, name in zip(t, (r0, r1, r2, r3, r4), "abcde"):
+            u.assert_close(u.host(got), ref, f"batch chain {name} rep {rep}")
+    # the same list inside a HIP graph, replayed with eager work in between
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        gl.run()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            gl.run()
+    keep = [y.clone() for y in t]
+    for rep in range(3):
+        for y in t:
+            y.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for y, k in zip(t, keep):
+            assert torch.equal(y, k), rep
+    gl.status()
+
+
+def test_argument_errors(env, oracle):
+    ops, u, torch = env
+    from relax_amd._lib import WqError
+
+    a = _linear(oracle, u, 64, 128, 4, seed=1)
+    y = torch.zeros((4, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(WqError, match="multiple of 256"):
+        ops.Q4G32GemvList([(a["dW"], a["dS"], u.dev(a["x"]), y)], M=4)
+    b = _linear(oracle, u, 64, 256, 17, seed=1)
+    with pytest.raises(WqError, match="rows of activations"):
+        ops.Q4G32GemvList([(b["dW"], b["dS"], u.dev(b["x"]), torch.zeros((17, 64), dtype=torch.float16, device="cuda"))], M=17)
+    c = _linear(oracle, u, 64, 256, 4, seed=1)
+    with pytest.raises(ValueError):
+        ops.Q4G32GemvList([(c["dW"], c["dS"], u.dev(c["x"])[:2], y)], M=4)
