@@ -18,7 +18,7 @@ step; `roofline` describes the decode GEMV kernel, `gemm` the M=2048 prefill
 GEMM of the same quantization scheme, `cpu_baseline` the CPU restatement of the
 reference's path timed on this machine's host cores.  Further objects on the same
 line: `stack` (32 decoder layers' linears run as one captured instruction list at
-M = 1, 8, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
+M = 1, 8, 16, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
 128, 512) and `calibration` (measured pure-read and MFMA-only ceilings).
 """
 from __future__ import annotations
@@ -151,7 +151,7 @@ def _measure(torch, stream, fn, min_ms=None, samples=None):
                  "min": round(t[0], 6), "max": round(t[-1], 6)}
 
 
-def bench_stack(torch, layers=32, batches=(1, 8, 32)):
+def bench_stack(torch, layers=32, batches=(1, 8, 16, 32)):
     """The four quantized linears of `layers` Llama-2-7B decoder layers (3.6 GB of codes and scales,
     so every step is cache-cold) as one instruction list of PackedFunc calls, planned and replayed
     as one HIP graph by the library's executor."""
@@ -169,7 +169,8 @@ def bench_stack(torch, layers=32, batches=(1, 8, 32)):
         weights.append(layer)
     stream = torch.cuda.Stream()
     res = {"layers": layers, "instructions_per_step": 4 * layers,
-           "launch": "hip_graph of PackedFunc calls; runs of decode linears (M = 1) fused into one launch", "batches": []}
+           "launch": "hip_graph of PackedFunc calls; runs of decode linears (M <= 32) fused into one launch "
+                     "(M = 1: VALU list kernel; 2 .. 16: MFMA list kernel; 17 .. 32: the same as two halves)", "batches": []}
     for M in batches:
         hidden = torch.randn((M, 4096), device="cuda", dtype=torch.float16)
         attn = torch.randn((M, 4096), device="cuda", dtype=torch.float16)

@@ -28,7 +28,8 @@ struct GemvListDesc {  // 128 bytes, device memory
   // b mod 2^gmod_log2 == gidx (member c = b >> gmod_log2 of workgroups >> gmod_log2); q, rem and off
   // then count within the group.
   uint8_t gmod_log2, gidx;
-  uint8_t pad[62];
+  uint8_t rows;  // rows of x and y of this entry (<= the M of the launch: a list of more than 16 rows is run as two halves)
+  uint8_t pad[61];
 };
 static_assert(sizeof(GemvListDesc) == 128, "descriptor layout");
 constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y
@@ -75,7 +76,8 @@ struct wq_gemv_list {
   int nb = 2;
   int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
   long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
-  int M = 1;               // activation rows; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
+  int halves = 1;          // entries of the list per linear of the caller (2: more than 16 rows)
+  int M = 1;               // activation rows of the launch; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
   int batch_u = 0;         // chunks per tile and wavefront (4: panels of 4096 k, M <= 8; 2: 2048 k)
   int batch_groups = 1;    // groups of workgroups that run different linears side by side
   int batch_nxb = 0;       // panels of activations in LDS

@@ -33,6 +33,7 @@
 #include <vector>
 
 #include "gemv_list_common.h"
+#include "tuning.h"
 
 namespace wq {
 
@@ -97,6 +98,13 @@ struct ItemCursor {
   const char* W;
   const char* S;
 };
+
+// word 16 of a descriptor: gmod_log2 | gidx << 8 | rows << 16 (read as one word: a scalar load; single
+// bytes would come through a vector load and end up in vector registers)
+__device__ __forceinline__ uint32_t desc_group_word(gemv_desc_ptr descs, int lin) {
+  typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
+  return ((words_ptr)(descs + lin))[16];
+}
 
 // positions the cursor on the first linear >= c.lin in which this workgroup holds a tile
 template <int U>
@@ -306,7 +314,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         v += __shfl_xor(v, 1, 64);
         v += __shfl_xor(v, 2, 64);
         v += __shfl_xor(v, 4, 64);
-        if (__builtin_amdgcn_readfirstlane(v) >= (nwg >> descs[dep].gmod_log2)) break;  // every member of its group
+        if (__builtin_amdgcn_readfirstlane(v) >= (nwg >> (desc_group_word(descs, dep) & 0xffu))) break;  // every member of its group
         if (wall_clock64() - t0 > spin_limit) {
           aborted = true;
           if (lane == 0)
@@ -343,9 +351,10 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         }
         const int K = xc.G << 5;
         const int K8 = K >> 3;
+        const int xrows = (int)((desc_group_word(descs, j) >> 16) & 0xffu);
         // an x that other workgroups of this launch have written is read with device-scope loads (sc1)
         const __amdgpu_buffer_rsrc_t xr =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(descs[j].x), 0, M * K * 2, kBufferFlags);
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(descs[j].x), 0, xrows * K * 2, kBufferFlags);
         char* const xdst = xbuf + xslot * xbuf_bytes;
         const int total = M * PPR;
         for (int base = 0; base < total; base += 64 * UX) {
@@ -356,9 +365,10 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
             const int row = idx / PPR, o = idx & (PPR - 1);
             const int go = xc.panel * PPR + o;  // the piece's place in the row
             v[t] = uint4_t{0, 0, 0, 0};
+            const int src = min(row, xrows - 1);  // rows past the entry's repeat its last row (never stored)
             if (idx < total && go < K8)
-              v[t] = dep >= 0 ? __builtin_amdgcn_raw_buffer_load_b128(xr, (row * K8 + go) * 16, 0, kDeviceScope)
-                              : __builtin_amdgcn_raw_buffer_load_b128(xr, (row * K8 + go) * 16, 0, 0);
+              v[t] = dep >= 0 ? __builtin_amdgcn_raw_buffer_load_b128(xr, (src * K8 + go) * 16, 0, kDeviceScope)
+                              : __builtin_amdgcn_raw_buffer_load_b128(xr, (src * K8 + go) * 16, 0, 0);
           }
 #pragma unroll
           for (int t = 0; t < UX; ++t) {
@@ -389,7 +399,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
 
   if (wave == kBW + kBXW) {
     // ====================== scale wavefront: the scales of a tile -> LDS ======================
-    constexpr int PD = 3;            // items in flight in registers
+    constexpr int PD = 6;            // items in flight in registers (a round trip under load is several items long)
     constexpr int PPR = PG / 8;      // 16-byte pieces (8 scales) per row and panel
     constexpr int LP = 16 * PPR / 64;  // pieces per lane and item
     uint4_t sv[PD][LP];
@@ -447,8 +457,9 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     int k = 0;
     for (int lin = 0; lin < nlin; ++lin) {
       const uint32_t g_dep = descs[lin].g_dep;
-      const int gl = descs[lin].gmod_log2;
-      if ((b & ((1 << gl) - 1)) != (int)descs[lin].gidx) continue;  // another group's linear
+      const uint32_t grp = desc_group_word(descs, lin);
+      const int gl = (int)(grp & 0xffu);
+      if ((b & ((1 << gl) - 1)) != (int)((grp >> 8) & 0xffu)) continue;  // another group's linear
       const int ncu = nwg >> gl;
       int rb = (b >> gl) - (int)descs[lin].off;
       if (rb < 0) rb += ncu;
@@ -457,7 +468,8 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       const int P = ((int)(g_dep & 0xffffu) + PG - 1) / PG;
       const half_t* bias = descs[lin].bias;
       const half_t* residual = descs[lin].residual;
-      const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[lin].y, 0, M * N * 2, kBufferFlags);
+      const int yrows = (int)((grp >> 16) & 0xffu);
+      const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[lin].y, 0, yrows * N * 2, kBufferFlags);
       for (int panel = 0; panel < (T > 0 ? P : 0); ++panel) {
         for (int lt = 0; lt < T; ++lt, ++k) {
           const int slot = k & (ring - 1);
@@ -478,7 +490,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
           }
           // lane (j, rq) holds rows n0 + 4 rq .. + 3 of activation row j
           const int n0 = ((lt * ncu + rb) << 4) + 4 * rq;
-          if (j16 < M) {
+          if (j16 < yrows) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const int n = n0 + r;
@@ -529,7 +541,8 @@ static size_t batch_lds_bytes(int U, int M, int nxb, int ring, int acc_tiles) {
 // g = 3: the activations then stay in that XCD's L2): a workgroup sees 1 / 2^g of the linears and 2^g times
 // as many rows of each.  Linears go, in list order, to the group that can start them first (a consumer
 // not before its producer has ended), with the duration of a linear estimated from the bytes a workgroup
-// moves for it; g is the best of 0 .. 3 by that estimate.
+// moves for it; g is the best of 0 .. 4 by that estimate (32-layer Llama-2-7B stack, M = 8: 1.25 ms with one
+// group, 0.89 ms with 8, 0.85 ms with 16).
 struct BatchGroupPlan {
   std::vector<int> group;
   double makespan = 0.0;
@@ -571,7 +584,7 @@ int batch_list_plan(wq_gemv_list* l) {
   int best_gl = -1;
   BatchGroupPlan best;
   int best_acc = 0;
-  for (int gl = 0; gl <= 3; ++gl) {
+  for (int gl = 0; gl <= 4; ++gl) {
     if (l->blocks % (1 << gl) != 0 || (l->blocks >> gl) < 1) break;
     const int ncu = l->blocks >> gl;
     int acc_tiles = 0;
@@ -615,7 +628,9 @@ int batch_list_plan(wq_gemv_list* l) {
   l->lds = batch_lds_bytes(U, l->M, l->batch_nxb, l->batch_ring, best_acc);
   const void* kern = U == 4 ? reinterpret_cast<const void*>(q4g32_batch_list_kernel<4>)
                             : reinterpret_cast<const void*>(q4g32_batch_list_kernel<2>);
-  if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l->lds) != hipSuccess)
+  // several lists share a kernel: the limit only ever grows
+  static DynamicLdsLimit limit4, limit2;
+  if ((U == 4 ? limit4 : limit2).ensure(kern, (int)l->lds) != hipSuccess)
     return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)

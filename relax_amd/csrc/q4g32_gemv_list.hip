@@ -40,6 +40,7 @@
 #include <vector>
 
 #include "gemv_list_common.h"
+#include "tuning.h"
 #include "wq_device.h"
 #include "wq_host.h"
 
@@ -503,7 +504,8 @@ constexpr int kListDepth = 4;  // ring slots (KiB of codes in flight) per comput
 
 extern "C" size_t wq_q4g32_gemv_list_workspace_bytes(int n) {
   if (n <= 0) return 0;
-  return wq::list_table_bytes(n) + (size_t)wq::sync_ints(n) * sizeof(int);
+  // room for two entries per linear (lists with more than 16 rows of activations)
+  return wq::list_table_bytes(2 * n) + (size_t)wq::sync_ints(2 * n) * sizeof(int);
 }
 
 extern "C" void wq_q4g32_gemv_list_destroy(wq_gemv_list_t* l) { delete l; }
@@ -525,11 +527,13 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
       workspace_bytes < wq_q4g32_gemv_list_workspace_bytes(n))
     return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: workspace must be 256-byte aligned device memory of %zu bytes",
                wq_q4g32_gemv_list_workspace_bytes(n));
-  std::unique_ptr<wq_gemv_list> l(new wq_gemv_list());
-  l->n = n;
-  l->M = M;
-  l->descs.resize(n);
-  int cmax = 1;
+  // More than 16 rows: every linear becomes two entries of the list, one per half of the rows (the kernel
+  // holds 16 rows of activations; the two halves read the same weights at about the same time on different
+  // groups of workgroups, so the second read is served by the memory-side cache).
+  const int halves = M > 16 ? 2 : 1;
+  const int Mk = halves == 2 ? (M + 1) / 2 : M;  // rows the kernel is launched for
+  std::vector<wq_q4g32_gemv_desc> e;
+  std::vector<int> rows;
   for (int i = 0; i < n; ++i) {
     const wq_q4g32_gemv_desc& s = d[i];
     if (s.N <= 0 || s.K <= 0 || s.K % 32 != 0 || s.K > WQ_GEMV_LIST_MAX_K || s.N >= (1ll << 30))
@@ -541,6 +545,25 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
     // several rows: the scales travel in 16-byte pieces of 8, and rows of x and y are addressed with 32-bit offsets
     if (M > 1 && (s.K % 256 != 0 || !aligned16(s.S) || (int64_t)M * s.N >= (1ll << 30) || s.K / 32 > 0xffff))
       return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d: with %d rows of activations K=%lld must be a multiple of 256, S 16-byte aligned and M * N < 2^30", i, M, (long long)s.K);
+    for (int h = 0; h < halves; ++h) {
+      wq_q4g32_gemv_desc t = s;
+      const int64_t r0 = (int64_t)h * Mk;
+      t.x = s.x + r0 * s.K;
+      t.y = s.y + r0 * s.N;
+      if (s.residual) t.residual = s.residual + r0 * s.N;
+      e.push_back(t);
+      rows.push_back(h == 0 ? Mk : M - Mk);
+    }
+  }
+  const int ne = (int)e.size();
+  std::unique_ptr<wq_gemv_list> l(new wq_gemv_list());
+  l->n = ne;
+  l->M = Mk;
+  l->halves = halves;
+  l->descs.resize(ne);
+  int cmax = 1;
+  for (int i = 0; i < ne; ++i) {
+    const wq_q4g32_gemv_desc& s = e[i];
     GemvListDesc& g = l->descs[i];
     g.W = reinterpret_cast<const char*>(s.W);
     g.S = reinterpret_cast<const char*>(s.S);
@@ -553,25 +576,27 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
     g.g_dep = (uint32_t)(s.K / 32);
     g.rem = 0;
     g.off = 0;
+    g.rows = (uint8_t)rows[i];
     cmax = std::max(cmax, (int)((s.K / 32 + 63) / 64));
   }
   // Who reads what an earlier linear of the list wrote.  Writing over something an earlier linear
   // still reads or wrote is refused: workgroups are not synchronised except through `dep`.
-  for (int i = 0; i < n; ++i) {
-    const wq_q4g32_gemv_desc& a = d[i];
+  for (int i = 0; i < ne; ++i) {
+    const wq_q4g32_gemv_desc& a = e[i];
+    const size_t ya = (size_t)a.N * 2 * rows[i], xa = (size_t)a.K * 2 * rows[i];
     for (int j = i - 1; j >= 0; --j) {
-      const wq_q4g32_gemv_desc& b = d[j];
-      const size_t yb = (size_t)b.N * 2 * M, ya = (size_t)a.N * 2 * M;
-      if (((l->descs[i].g_dep >> 16) & 0x7fffu) == 0 && ranges_overlap(a.x, (size_t)a.K * 2 * M, b.y, yb))
+      const wq_q4g32_gemv_desc& b = e[j];
+      const size_t yb = (size_t)b.N * 2 * rows[j], xb = (size_t)b.K * 2 * rows[j];
+      if (((l->descs[i].g_dep >> 16) & 0x7fffu) == 0 && ranges_overlap(a.x, xa, b.y, yb))
         l->descs[i].g_dep |= (uint32_t)(j + 1) << 16;
       if (ranges_overlap(a.residual, ya, b.y, yb) || ranges_overlap(a.bias, (size_t)a.N * 2, b.y, yb))
-        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i, j);
-      if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, (size_t)b.K * 2 * M) ||
+        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i / halves, j / halves);
+      if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, xb) ||
           ranges_overlap(a.y, ya, b.residual, yb) || ranges_overlap(a.y, ya, b.bias, (size_t)b.N * 2))
-        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the output of linear %d overlaps an operand of linear %d", i, j);
+        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the output of linear %d overlaps an operand of linear %d", i / halves, j / halves);
     }
-    if (ranges_overlap(a.y, (size_t)a.N * 2 * M, a.x, (size_t)a.K * 2 * M))
-      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: y overlaps x", i);
+    if (ranges_overlap(a.y, ya, a.x, xa))
+      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: y overlaps x", i / halves);
     const int dep = (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1;
     if (dep >= 0) {
       l->descs[dep].g_dep |= kSignal;
@@ -589,9 +614,9 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
   l->blocks = std::min(cu_count(), 32768);
   int64_t turns = 1;
   int64_t off = 0;
-  for (int i = 0; i < n; ++i) {
+  for (int i = 0; i < ne; ++i) {
     GemvListDesc& g = l->descs[i];
-    const int64_t groups = (d[i].N + (1 << l->gs) - 1) >> l->gs;
+    const int64_t groups = (e[i].N + (1 << l->gs) - 1) >> l->gs;
     g.q = (int32_t)(groups / l->blocks);
     g.rem = (uint16_t)(groups % l->blocks);
     g.off = (uint16_t)off;
@@ -607,17 +632,17 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
   if (l->nb < 2) return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations and row sums do not fit the LDS");
   l->lds = fixed + (size_t)l->nb * l->xbuf_bytes;
   auto kern = q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>;
-  if (l->lds > 48 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)l->lds) != hipSuccess)
+  static DynamicLdsLimit limit;  // several lists share the kernel: the limit only ever grows
+  if (l->lds > 48 * 1024 && limit.ensure(reinterpret_cast<const void*>(kern), (int)l->lds) != hipSuccess)
     return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
     return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: the workgroup does not fit a CU (%zu bytes of LDS)", l->lds);
   }
   l->table = workspace;
-  l->sync = reinterpret_cast<int*>(static_cast<char*>(workspace) + list_table_bytes(n));
-  if (hipMemcpyAsync(l->table, l->descs.data(), (size_t)n * sizeof(GemvListDesc), hipMemcpyHostToDevice, stream) != hipSuccess ||
-      hipMemsetAsync(l->sync, 0, (size_t)sync_ints(n) * sizeof(int), stream) != hipSuccess ||
+  l->sync = reinterpret_cast<int*>(static_cast<char*>(workspace) + list_table_bytes(ne));
+  if (hipMemcpyAsync(l->table, l->descs.data(), (size_t)ne * sizeof(GemvListDesc), hipMemcpyHostToDevice, stream) != hipSuccess ||
+      hipMemsetAsync(l->sync, 0, (size_t)sync_ints(ne) * sizeof(int), stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: could not upload the descriptor table");
   return l.release();
@@ -651,7 +676,7 @@ extern "C" int wq_q4g32_gemv_list_status(wq_gemv_list_t* l, wq_stream_t stream) 
   return fail(WQ_EDEVICE,
               "wq_q4g32_gemv_list: a wait for linear %d timed out (the grid was not resident at once?); "
               "results of that launch are undefined",
-              err - 1);
+              (err - 1) / l->halves);
 }
 
 extern "C" int wq_q4g32_gemv_list_info(const wq_gemv_list_t* l, int* dependencies, int* adjacent) {

@@ -148,7 +148,7 @@ class Q4G32GemvList:
     ``linears``: sequence of ``(W, S, x, y)`` or ``(W, S, x, y, bias, residual)`` device tensors; a linear
     whose ``x`` is the ``y`` of an earlier one waits for it on the device.  The tensors are kept alive by
     this object; the descriptor table and the counters live in a workspace allocated here, once.
-    ``M`` (1 .. 16): rows of activations of every linear of the list (x ``[M, K]``, y and residual ``[M, N]``).
+    ``M`` (1 .. 32): rows of activations of every linear of the list (x ``[M, K]``, y and residual ``[M, N]``).
     """
 
     def __init__(self, linears, M: int = 1):

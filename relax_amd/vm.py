@@ -91,6 +91,8 @@ class DpsProgram:
         need = self._l.wq_program_plan(self._p)
         check(min(need, 0), "wq_program_plan")
         self._workspace = torch.zeros(max(need, 256), dtype=torch.uint8, device=device)
+        # the fill runs on torch's current stream, the program on whatever stream run / capture are given
+        torch.cuda.current_stream().synchronize()
         check(self._l.wq_program_set_workspace(self._p, self._workspace.data_ptr(), self._workspace.numel()),
               "wq_program_set_workspace")
         return int(need)

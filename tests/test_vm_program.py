@@ -277,7 +277,7 @@ def test_llama7b_stack_full_size_matches_oracle(oracle):
         prog.run(stream)
         stream.synchronize()
         prog.status(stream)
-        assert prog.num_fused_groups == (1 if M <= 16 else 0)  # up to 16 rows: one launch for the whole stack
+        assert prog.num_fused_groups == 1  # one launch for the whole stack
         check("eager")
         eager = [t.clone() for t in (out, tap_gu, tap_qkv)]
         prog.capture(stream)
