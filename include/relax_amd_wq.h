@@ -257,6 +257,23 @@ int wq_gptq_prepare(const uint32_t* qweight, const uint32_t* qzeros, const uint1
                     const int32_t* g_idx, uint32_t* W_nk, uint16_t* SZ, int32_t* perm,
                     int32_t* status_scratch, int* needs_perm, int64_t K, int64_t N, int64_t G,
                     wq_stream_t stream);
+/* The same for ANY g_idx (groups of unequal size, in any order; entries must lie in [0, G)): each group's rows,
+ * in ascending k, are padded to a multiple of 32, so the prepared layer has K_padded >= K rows in sub-groups of
+ * exactly 32 (K_padded <= wq_gptq_padded_k_bound(K, G), which is what the caller sizes the buffers by:
+ * W_nk uint32 [N, capacity/8], SZ fp16 [N, capacity/32, 2], perm int32 [capacity]).  *K_padded receives the
+ * row count; perm[k'] is the checkpoint row at position k' or -1 for padding.  A load-time call: sorts on the
+ * host, allocates a temporary, synchronises the stream.  Only K % 8 == 0 and N % 8 == 0 are required. */
+int64_t wq_gptq_padded_k_bound(int64_t K, int64_t G);
+int wq_gptq_prepare_padded(const uint32_t* qweight, const uint32_t* qzeros, const uint16_t* scales,
+                           const int32_t* g_idx, uint32_t* W_nk, uint16_t* SZ, int32_t* perm, int64_t capacity,
+                           int64_t* K_padded, int64_t K, int64_t N, int64_t G, wq_stream_t stream);
+/* The linear over operands prepared by wq_gptq_prepare_padded: x fp16 [M, K] is gathered into the workspace
+ * (M * K_padded * 2 bytes, 16-byte aligned; zeros at the padding), then the kernels of wq_gptq_linear run with
+ * K_padded rows in groups of 32.  K_padded <= 32768. */
+size_t wq_gptq_padded_workspace_bytes(int64_t M, int64_t K_padded);
+int wq_gptq_linear_padded(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
+                          const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
+                          int64_t K, int64_t K_padded, void* workspace, size_t workspace_bytes, wq_stream_t stream);
 /* Bytes of workspace wq_gptq_linear needs: M*K*2 for the gathered activations when a row
  * order is given, else 0. */
 size_t wq_gptq_workspace_bytes(int64_t M, int64_t K, int has_perm);

@@ -17,6 +17,7 @@
 // (mfma_gemm_lds.h) all take it.
 // A g_idx whose groups do not all have K/G members is rejected by the preparation.
 #include <mutex>
+#include <vector>
 
 #include "mfma_gemm_lds.h"
 #include "q4_gemv.h"
@@ -134,6 +135,62 @@ __global__ __launch_bounds__(256) void gptq_gather_x_direct_kernel(const half_t*
   if (i < (K >> 1)) {
     const int2 p = reinterpret_cast<const int2*>(perm)[i];
     reinterpret_cast<half2_t*>(xp + m * K)[i] = half2_t{x[m * K + p.x], x[m * K + p.y]};
+  }
+}
+
+// ---- any g_idx: groups of unequal size ------------------------------------------------------
+// The rows of a group, in ascending k, are padded to a multiple of 32 and the whole layer becomes
+// K' / 32 sub-groups of exactly 32 rows (sub-group -> group map `sub2grp`); perm'[k'] is the row of
+// the checkpoint at position k', or -1 for padding.  Padding contributes nothing because its
+// ACTIVATION is gathered as zero (a zero weight cannot be encoded when zero + 1 = 16).
+__global__ __launch_bounds__(256) void gptq_repack_padded_kernel(const uint32_t* __restrict__ qweight,
+                                                                 const int* __restrict__ perm,
+                                                                 uint32_t* __restrict__ W_nk, int KW, int N) {
+  __shared__ uint32_t tile[64][65];
+  const int kw0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = 0; i < 16; ++i) {
+    const int kw = kw0 + ty * 16 + i, n = n0 + tx;
+    if (kw < KW && n < N) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int k = perm[kw * 8 + c];
+        if (k >= 0) word |= ((qweight[(int64_t)(k >> 3) * N + n] >> (4 * (k & 7))) & 15u) << (4 * c);
+      }
+      tile[ty * 16 + i][tx] = word;
+    }
+  }
+  __syncthreads();
+  for (int i = 0; i < 16; ++i) {
+    const int n = n0 + ty * 16 + i, kw = kw0 + tx;
+    if (kw < KW && n < N) W_nk[(int64_t)n * KW + kw] = tile[tx][ty * 16 + i];
+  }
+}
+
+// SZ[n][sub] = (scales[g][n], fp16(zero[g][n] + 1)) with g = sub2grp[sub]
+__global__ __launch_bounds__(256) void gptq_sz_mapped_kernel(const uint32_t* __restrict__ qzeros,
+                                                             const half_t* __restrict__ scales,
+                                                             const int* __restrict__ sub2grp,
+                                                             half2_t* __restrict__ SZ, int N, int GS) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  const int sub = blockIdx.y;
+  if (n >= N) return;
+  const int g = sub2grp[sub];
+  const uint32_t zero = (qzeros[(int64_t)g * (N >> 3) + (n >> 3)] >> (4 * (n & 7))) & 15u;
+  SZ[(int64_t)n * GS + sub] = half2_t{scales[(int64_t)g * N + n], (half_t)(float)(zero + 1u)};
+}
+
+// xp[m][k'] = perm'[k'] >= 0 ? x[m][perm'[k']] : 0; rows of x are K long, rows of xp KP
+__global__ __launch_bounds__(256) void gptq_gather_x_padded_kernel(const half_t* __restrict__ x,
+                                                                   const int* __restrict__ perm,
+                                                                   half_t* __restrict__ xp, int K, int KP) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int64_t m = blockIdx.y;
+  if (i < (KP >> 1)) {
+    const int2 p = reinterpret_cast<const int2*>(perm)[i];
+    const half_t zero = (half_t)0.0f;
+    reinterpret_cast<half2_t*>(xp + m * KP)[i] = half2_t{p.x >= 0 ? x[m * K + p.x] : zero, p.y >= 0 ? x[m * K + p.y] : zero};
   }
 }
 
@@ -302,6 +359,68 @@ extern "C" int wq_gptq_prepare(const uint32_t* qweight, const uint32_t* qzeros, 
   return WQ_OK;
 }
 
+extern "C" int64_t wq_gptq_padded_k_bound(int64_t K, int64_t G) {
+  if (K <= 0 || G <= 0) return 0;
+  return (K + 31 * G + 63) / 64 * 64;
+}
+
+extern "C" int wq_gptq_prepare_padded(const uint32_t* qweight, const uint32_t* qzeros, const uint16_t* scales,
+                                      const int32_t* g_idx, uint32_t* W_nk, uint16_t* SZ, int32_t* perm,
+                                      int64_t capacity, int64_t* K_padded, int64_t K, int64_t N, int64_t G,
+                                      wq_stream_t stream_) {
+  using namespace wq;
+  hipStream_t stream = (hipStream_t)stream_;
+  WQ_REQUIRE(K >= 0 && N >= 0 && G >= 0 && K_padded, "wq_gptq_prepare_padded: negative dimension or null K_padded");
+  *K_padded = 0;
+  if (K == 0 || N == 0) return WQ_OK;
+  WQ_REQUIRE(G > 0 && K % 8 == 0 && N % 8 == 0, "wq_gptq_prepare_padded: K=%lld and N=%lld must be multiples of 8",
+             (long long)K, (long long)N);
+  WQ_REQUIRE(qweight && qzeros && scales && g_idx && W_nk && SZ && perm, "wq_gptq_prepare_padded: null pointer");
+  WQ_REQUIRE(N < (1ll << 30) && K < (1ll << 24) && G < 65536, "wq_gptq_prepare_padded: too large");
+  // a load-time step: the row -> group map is sorted on the host
+  std::vector<int32_t> gi((size_t)K);
+  WQ_HIP(hipMemcpyAsync(gi.data(), g_idx, (size_t)K * 4, hipMemcpyDeviceToHost, stream));
+  WQ_HIP(hipStreamSynchronize(stream));
+  std::vector<int64_t> count((size_t)G, 0);
+  for (int64_t k = 0; k < K; ++k) {
+    WQ_REQUIRE(gi[k] >= 0 && gi[k] < G, "wq_gptq_prepare_padded: g_idx[%lld] = %d is outside [0, %lld)", (long long)k,
+               gi[k], (long long)G);
+    ++count[gi[k]];
+  }
+  std::vector<int64_t> start((size_t)G + 1, 0);
+  for (int64_t g = 0; g < G; ++g) start[g + 1] = start[g] + (count[g] + 31) / 32 * 32;
+  const int64_t KP = (start[G] + 63) / 64 * 64;  // the small-batch kernel walks K in steps of 64
+  WQ_REQUIRE(KP <= capacity, "wq_gptq_prepare_padded: the padded layer has %lld rows, the buffers hold %lld "
+             "(wq_gptq_padded_k_bound gives the most it can be)", (long long)KP, (long long)capacity);
+  std::vector<int32_t> hperm((size_t)KP, -1), sub2grp((size_t)(KP / 32), 0);
+  std::vector<int64_t> fill(start.begin(), start.end() - 1);
+  for (int64_t k = 0; k < K; ++k) hperm[fill[gi[k]]++] = (int32_t)k;
+  for (int64_t g = 0; g < G; ++g)
+    for (int64_t sub = start[g] / 32; sub < start[g + 1] / 32; ++sub) sub2grp[sub] = (int32_t)g;
+  // the sub-group -> group map is only needed by the kernel below: a temporary device allocation
+  int32_t* d_map = nullptr;
+  WQ_HIP(hipMalloc(&d_map, sub2grp.size() * 4));
+  hipError_t e = hipMemcpyAsync(perm, hperm.data(), (size_t)KP * 4, hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(d_map, sub2grp.data(), sub2grp.size() * 4, hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess) {
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((KP / 8 + 63) / 64));
+    hipLaunchKernelGGL(gptq_repack_padded_kernel, grid, dim3(256), 0, stream, qweight, (const int*)perm, W_nk,
+                       (int)(KP / 8), (int)N);
+    hipLaunchKernelGGL(gptq_sz_mapped_kernel, dim3((unsigned)((N + 255) / 256), (unsigned)(KP / 32)), dim3(256), 0,
+                       stream, qzeros, (const half_t*)scales, (const int*)d_map, (half2_t*)SZ, (int)N, (int)(KP / 32));
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);  // the host vectors and d_map are in use until here
+  (void)hipFree(d_map);
+  if (e != hipSuccess) return fail(WQ_EDEVICE, "wq_gptq_prepare_padded: %s", hipGetErrorString(e));
+  *K_padded = KP;
+  return WQ_OK;
+}
+
+extern "C" size_t wq_gptq_padded_workspace_bytes(int64_t M, int64_t K_padded) {
+  return (M > 0 && K_padded > 0) ? (size_t)M * (size_t)K_padded * 2 : 0;
+}
+
 extern "C" size_t wq_gptq_workspace_bytes(int64_t M, int64_t K, int has_perm) {
   return (has_perm && M > 0 && K > 0) ? (size_t)M * (size_t)K * 2 : 0;
 }
@@ -317,6 +436,29 @@ extern "C" int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const in
                               int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream) {
   return wq::gptq_linear_impl(W_nk, SZ, perm, x, bias, residual, y, M, N, K, G, workspace, workspace_bytes,
                               (hipStream_t)stream);
+}
+
+extern "C" int wq_gptq_linear_padded(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
+                                     const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M,
+                                     int64_t N, int64_t K, int64_t K_padded, void* workspace, size_t workspace_bytes,
+                                     wq_stream_t stream_) {
+  using namespace wq;
+  hipStream_t stream = (hipStream_t)stream_;
+  WQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && K_padded >= 0, "wq_gptq_linear_padded: negative dimension");
+  if (M == 0 || N == 0) return WQ_OK;
+  WQ_REQUIRE(K > 0 && K_padded >= K && K_padded % 64 == 0 && K_padded <= 32768,
+             "wq_gptq_linear_padded: K_padded=%lld must be a multiple of 64, at least K=%lld and at most 32768",
+             (long long)K_padded, (long long)K);
+  WQ_REQUIRE(W_nk && SZ && perm && x && y, "wq_gptq_linear_padded: null pointer");
+  WQ_REQUIRE(aligned16(perm) && M < (1ll << 16), "wq_gptq_linear_padded: perm must be 16-byte aligned, M < 65536");
+  const size_t need = wq_gptq_padded_workspace_bytes(M, K_padded);
+  WQ_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
+             "wq_gptq_linear_padded: needs a 16-byte aligned workspace of M*K_padded*2 = %zu bytes (got %zu)", need,
+             workspace_bytes);
+  WQ_LAUNCH("wq_gptq_linear_padded", gptq_gather_x_padded_kernel, dim3((unsigned)((K_padded / 2 + 255) / 256), (unsigned)M),
+            dim3(256), 0, stream, (const half_t*)x, perm, (half_t*)workspace, (int)K, (int)K_padded);
+  return gptq_linear_impl(W_nk, SZ, nullptr, (const uint16_t*)workspace, bias, residual, y, M, N, K_padded,
+                          K_padded / 32, nullptr, 0, stream);
 }
 
 // ---- the same linear for callers that cannot allocate: the gathered activations live in a

@@ -403,6 +403,27 @@ def gptq_prepare(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tens
     return GptqWeight(W_nk, SZ, perm if needs.value else None, K, N, G)
 
 
+def gptq_prepare_padded(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, g_idx: torch.Tensor) -> GptqWeight:
+    """:func:`gptq_prepare` for ANY ``g_idx`` (groups of unequal size): every group padded to a multiple of 32
+    rows (``wq_gptq_prepare_padded``); the result carries ``K_padded`` and is run by :func:`gptq_linear`."""
+    qweight, qzeros, scales, g_idx, K, N, G = _gptq_dims(qweight, qzeros, scales, g_idx)
+    dev = qweight.device
+    cap = int(_lib.lib().wq_gptq_padded_k_bound(K, G))
+    W_nk = torch.empty((N, cap // 8), dtype=qweight.dtype, device=dev)
+    SZ = torch.empty((N, cap // 32, 2), dtype=torch.float16, device=dev)
+    perm = torch.empty((cap,), dtype=torch.int32, device=dev)
+    kp = ctypes.c_int64(0)
+    check(_lib.lib().wq_gptq_prepare_padded(_ptr(qweight), _ptr(qzeros), _ptr(scales), _ptr(g_idx), _ptr(W_nk),
+                                            _ptr(SZ), _ptr(perm), cap, ctypes.byref(kp), K, N, G, _stream()),
+          "wq_gptq_prepare_padded")
+    KP = int(kp.value)
+    # the prepared operands are compact for K_padded rows (they occupy the front of the buffers)
+    w = GptqWeight(W_nk.view(-1)[: N * (KP // 8)].view(N, KP // 8), SZ.view(-1)[: N * (KP // 32) * 2].view(N, KP // 32, 2),
+                   perm[:KP], K, N, G)
+    w.K_padded = KP
+    return w
+
+
 def gptq_linear(w: GptqWeight, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
                 residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                 workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -422,6 +443,16 @@ def gptq_linear(w: GptqWeight, x: torch.Tensor, bias: Optional[torch.Tensor] = N
         out = torch.empty((*x.shape[:-1], w.N), dtype=torch.float16, device=x.device)
     elif not out.is_contiguous() or out.numel() != M * w.N or out.dtype != torch.float16:
         raise ValueError("out must be a contiguous fp16 tensor of M*N elements")
+    KP = getattr(w, "K_padded", 0)
+    if KP:
+        need = _lib.lib().wq_gptq_padded_workspace_bytes(M, KP)
+        if workspace is None:
+            workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=x.device)
+        check(_lib.lib().wq_gptq_linear_padded(_ptr(w.W_nk), _ptr(w.SZ), _ptr(w.perm), _ptr(x), _ptr(bias),
+                                               _ptr(residual), _ptr(out), M, w.N, w.K, KP, _ptr(workspace),
+                                               workspace.numel() * workspace.element_size(), _stream()),
+              "wq_gptq_linear_padded")
+        return out
     need = _lib.lib().wq_gptq_workspace_bytes(M, w.K, 1 if w.perm is not None else 0)
     if need and workspace is None:
         workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)

@@ -181,3 +181,65 @@ def test_linear_argument_errors(ops, u, oracle):
     rc = _lib.lib().wq_gptq_linear(w.W_nk.data_ptr(), w.SZ.data_ptr(), 0, u.dev(x).data_ptr(), 0, 0, y.data_ptr(),
                                    16, 64, 256, 3, 0, 0, 0)
     assert rc != 0 and b"groups" in _lib.lib().wq_last_error()
+
+
+# ---- any g_idx: groups of unequal size (wq_gptq_prepare_padded / wq_gptq_linear_padded) ----
+def _unequal_g_idx(K, G, seed, kind):
+    rng = np.random.default_rng(seed)
+    if kind == "random":        # every row picks a group at random: sizes differ, some may be empty
+        return rng.integers(0, G, size=K).astype(np.int32)
+    if kind == "runs":          # contiguous runs of different lengths, not multiples of 32
+        cuts = np.sort(rng.choice(np.arange(1, K), size=G - 1, replace=False))
+        return np.repeat(np.arange(G), np.diff(np.concatenate([[0], cuts, [K]]))).astype(np.int32)
+    if kind == "one_big":       # one group holds nearly everything, one is empty
+        g = np.zeros(K, np.int32)
+        g[:5] = 1
+        g[-3:] = G - 1
+        return g
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["random", "runs", "one_big"])
+@pytest.mark.parametrize("M,N,K,G", [(1, 256, 1024, 8), (2, 64, 4096, 32), (5, 520, 2048, 16), (40, 128, 1024, 4), (200, 256, 512, 4)])
+def test_unequal_groups_linear_matches_oracle(ops, u, oracle, kind, M, N, K, G):
+    x, qw, qz, s, _ = oracle.make_gptq_inputs(M, N, K, K // G, seed=M + N + K)
+    g_idx = _unequal_g_idx(K, G, seed=K + G, kind=kind)
+    sizes = np.bincount(g_idx, minlength=G)
+    assert len(set(sizes.tolist())) > 1  # really unequal
+    w = ops.gptq_prepare_padded(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
+    assert w.K_padded % 64 == 0 and w.K_padded >= int(((sizes + 31) // 32 * 32).sum())
+    # layout: position k' holds row perm[k'] of the checkpoint, rows of a group in ascending k, padding = -1
+    perm = u.host(w.perm)
+    real = perm[perm >= 0]
+    assert np.array_equal(np.sort(real), np.arange(K))
+    assert np.array_equal(g_idx[real], np.sort(g_idx, kind="stable")) and np.array_equal(real, np.argsort(g_idx, kind="stable"))
+    rng = np.random.default_rng(3)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    got = u.host(ops.gptq_linear(w, u.dev(x), bias=u.dev(bias), residual=u.dev(res)))
+    u.assert_close(got, _ref_linear(oracle, qw, qz, s, g_idx, x, bias, res), f"gptq unequal {kind} {M}x{N}x{K} G={G}")
+
+
+def test_unequal_groups_one_hot_rows_reproduce_the_dequantized_weight(ops, u, oracle):
+    N, K, G = 64, 512, 8
+    _, qw, qz, s, _ = oracle.make_gptq_inputs(1, N, K, K // G, seed=5)
+    g_idx = _unequal_g_idx(K, G, seed=9, kind="random")
+    B = oracle.gptq_dequant(qw, qz, s, g_idx)  # [K, N]
+    rows = [0, 1, 31, 32, 100, 255, 256, 511]
+    x = np.zeros((len(rows), K), np.float16)
+    for m, k in enumerate(rows):
+        x[m, k] = 1
+    w = ops.gptq_prepare_padded(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
+    got = u.host(ops.gptq_linear(w, u.dev(x)))
+    for m, k in enumerate(rows):
+        assert np.array_equal(_bits(got[m]), _bits(B[k])), (m, k)
+
+
+def test_prepare_padded_errors(ops, u, oracle):
+    from relax_amd._lib import WqError
+
+    _, qw, qz, s, g_idx = oracle.make_gptq_inputs(1, 64, 256, 64, seed=1)
+    bad = g_idx.copy()
+    bad[3] = 4  # outside [0, G)
+    with pytest.raises(WqError, match="outside"):
+        ops.gptq_prepare_padded(u.dev(qw), u.dev(qz), u.dev(s), u.dev(bad))
