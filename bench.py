@@ -482,8 +482,8 @@ def main():
     }
 
     if not args.no_gemm:
-        gem = []
-        tot_flops, tot_ms = 0.0, 0.0
+        gem, vendor = [], []
+        tot_flops, tot_ms, vendor_ms = 0.0, 0.0, 0.0
         cur = torch.cuda.current_stream()
         for N, K in PREFILL_SHAPES:
             g = torch.Generator(device="cuda")
@@ -501,7 +501,15 @@ def main():
                         "samples": sp["samples"], "calls_per_sample": sp["calls_per_sample"]})
             tot_flops += fl
             tot_ms += ms
-            del W, S, x, y
+            # for scale: the vendor library's plain fp16 GEMM (no dequantization) on the same shape, weights
+            # as an fp16 [N, K] tensor (torch.matmul -> hipBLASLt / rocBLAS); not part of `value`
+            Wf = torch.randn((N, K), device="cuda", dtype=torch.float16)
+            for _ in range(3):
+                torch.matmul(x, Wf.t(), out=y)
+            vms, _ = _measure(torch, cur, lambda: torch.matmul(x, Wf.t(), out=y), min_ms=MIN_SAMPLE_MS / 4, samples=3)
+            vendor.append({"N": N, "K": K, "us": round(vms * 1e3, 2), "tflops": round(fl / vms / 1e9, 1)})
+            vendor_ms += vms
+            del W, S, x, y, Wf
         tf = tot_flops / tot_ms / 1e9
         gtraffic, gsrc = offline_traffic("gemm_lds_kernel")
         out["gemm"] = {
@@ -512,6 +520,10 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": gtraffic, "traffic_source": gsrc},
+            "vendor_fp16_gemm_same_shapes": {"what": "torch.matmul(x, W_fp16.T): the library's dense fp16 GEMM, no dequantization",
+                                             "value": round(tot_flops / vendor_ms / 1e9, 1), "unit": "TFLOP/s",
+                                             "frac_of_mfma_peak": round(tot_flops / vendor_ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                                             "shapes": vendor},
         }
 
     del lists
