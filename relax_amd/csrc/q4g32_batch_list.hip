@@ -1,4 +1,5 @@
-// A list of format-A (q4f16_1) linears with 2 .. 16 activation rows each, in ONE launch.
+// A list of format-A (q4f16_1) linears with 2 .. 16 activation rows each, in ONE launch
+// (17 .. 32 rows: the host enters every linear twice, once per half of the rows).
 //
 // The counterpart of q4g32_gemv_list.hip for a small batch: the same persistent grid (one workgroup
 // per CU walks the list, device-side counters order dependent linears), but the products are done by
@@ -19,9 +20,9 @@
 //
 // The other four wavefronts keep everything irregular away from that loop, through LDS:
 //   * 2 x wavefronts wait for a producer linear (bounded spin), load a panel of activations,
-//     rearrange it and leave it in one of 2 .. 4 LDS buffers, that many panels ahead (under load a round
-//     trip to L2 takes several microseconds); the compute wavefronts copy their slice into registers
-//     when they reach the panel, which frees the buffer at once.
+//     rearrange it and leave it in one of 1 or 2 LDS buffers (under load a round trip to L2 takes several
+//     microseconds); the compute wavefronts copy their slice into registers when they reach the panel,
+//     which frees the buffer at once, so even one buffer keeps the next panel ready in time.
 //   * the scale wavefront streams the tile's scales (16 rows x 256 contiguous bytes: fetched per
 //     lane they cost more than the codes) into a ring of LDS slots, a few tiles ahead.
 //   * the y wavefront adds the 8 partial sums of a tile in a fixed order, keeps the sum in LDS while
@@ -45,7 +46,7 @@ constexpr int kBThreads = 64 * (kBW + kBXW + 2);
 
 // LDS words that hand the buffers over inside a workgroup (items = (linear, panel, tile) in the
 // order the workgroup walks them; panels counted over all linears)
-constexpr int kBMaxXBuf = 4;
+constexpr int kBMaxXBuf = 4;  // room in the flags; the host uses 1 or 2
 struct BatchFlags {
   int x_ready[kBMaxXBuf];  // [panel mod buffers] = panel + 1 once that panel's activations are staged
   int x_taken[kBMaxXBuf];  // [panel mod buffers] += 1 by each compute wavefront that has copied the panel

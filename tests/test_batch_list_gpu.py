@@ -145,3 +145,35 @@ def test_argument_errors(env, oracle):
     c = _linear(oracle, u, 64, 256, 4, seed=1)
     with pytest.raises(ValueError):
         ops.Q4G32GemvList([(c["dW"], c["dS"], u.dev(c["x"])[:2], y)], M=4)
+
+
+def test_a_wait_that_runs_out_is_reported_and_every_wavefront_exits(env, oracle):
+    """Spin limit 0: the consumer's first look at the producer's counters comes before the producer's group has
+    finished, so the wait gives up at once; the launch still ends, status() reports it, and the next launch
+    with the normal limit is correct."""
+    ops, u, torch = env
+    M = 6
+    a = _linear(oracle, u, 22016, 4096, M, seed=21)
+    b = _linear(oracle, u, 512, 4096, M, seed=22)
+    t0 = torch.zeros((M, 22016), dtype=torch.float16, device="cuda")
+    t1 = torch.zeros((M, 512), dtype=torch.float16, device="cuda")
+    mid = torch.zeros((M, 4096), dtype=torch.float16, device="cuda")
+    c = _linear(oracle, u, 4096, 4096, M, seed=23)
+    # c writes `mid`, which b reads: b waits for c; a keeps the other workgroups busy
+    gl = ops.Q4G32GemvList([(a["dW"], a["dS"], u.dev(a["x"]), t0), (c["dW"], c["dS"], u.dev(c["x"]), mid),
+                            (b["dW"], b["dS"], mid, t1)], M=M)
+    assert gl.info()[0] == 1
+    from relax_amd._lib import WqError
+
+    gl.set_spin_limit(0)
+    print("batch list: spin limit 0", flush=True)
+    gl.run()
+    with pytest.raises(WqError, match="timed out"):
+        gl.status()
+    gl.set_spin_limit(200_000_000)
+    gl.run()
+    gl.status()
+    r_mid = oracle.q4g32_linear(c["W"], c["S"], c["x"], nthreads=8)
+    u.assert_close(u.host(t0), oracle.q4g32_linear(a["W"], a["S"], a["x"], nthreads=8), "bystander after a reported time-out")
+    u.assert_close(u.host(mid), r_mid, "producer after a reported time-out")
+    u.assert_close(u.host(t1), oracle.q4g32_linear(b["W"], b["S"], r_mid, nthreads=8), "consumer after a reported time-out")
