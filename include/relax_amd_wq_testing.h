@@ -26,7 +26,7 @@ extern "C" {
 #endif
 
 /* Tile configuration of the MFMA GEMMs (format A and B): 1..4 the register-staged kernel
- * (256x256, 128x256, 64x128, 128x128), 11..17 the LDS-staged kernel; 0 = from the shape. */
+ * (256x256, 128x256, 64x128, 128x128), 11..18 the LDS-staged kernel; 0 = from the shape. */
 void wq_debug_set_gemm_config(int cfg);
 /* Split the tiles of the last, partly filled round into row slices (default 1). */
 void wq_debug_set_gemm_tail_split(int on);

@@ -3,7 +3,8 @@
 //
 // Every operand of a K-step (64 k) travels global -> LDS with the direct
 // global_load_lds_dwordx4 path: no staging registers, no VALU work, and the loads
-// of the next two to three steps are in flight while a step is multiplied (3-slot ring).  Per slot:
+// of the next two or more steps are in flight while a step is multiplied (a ring of 3 slots, or of up to 6
+// where one workgroup per CU leaves room in LDS; what pays is a 4-slot ring under 256 x 128 tiles).  Per slot:
 //   A   BM rows x 128 B of activations, 16-byte chunk c of row r at slot position
 //       c ^ ((r >> 1) & 7) (the swizzle is applied to the GLOBAL address each lane fetches,
 //       because the LDS side of a direct load is fixed: lane l writes 16 bytes at
@@ -54,17 +55,20 @@
 
 namespace wq {
 
-template <class Policy, int TM, int TN, int WM, int WN>
+template <class Policy, int TM, int TN, int WM, int WN, int WPE>
 struct LdsGemmCfg {
   static_assert(WM * WN == 4, "four wavefronts per workgroup");
   static constexpr int kThreads = 256;
   static constexpr int BM = 32 * TM * WM;
   static constexpr int BN = 32 * TN * WN;
-  static constexpr int kStages = 3;
   static constexpr int kAOff = 0;
   static constexpr int kBOff = BM * 128;
   static constexpr int kSOff = kBOff + BN * Policy::kColBytes;
   static constexpr int kStageBytes = kSOff + BN * Policy::kScaleBytes;
+  // ring slots: loads of kStages - 1 steps are in flight while a step is multiplied; four where a
+  // single workgroup per CU leaves room for them in the 160 KiB of LDS
+  static constexpr int kFit = (158 * 1024) / kStageBytes;
+  static constexpr int kStages = WPE == 1 ? (kFit >= 6 ? 6 : kFit >= 4 ? kFit : 3) : 3;
   static constexpr int kLdsBytes = kStages * kStageBytes;
   static constexpr int kALoads = BM / 32;   // direct loads per wavefront per step (64 chunks each)
   static constexpr int kBLoads = BN * Policy::kColBytes / 4096;
@@ -99,15 +103,15 @@ typedef void __attribute__((address_space(3))) * wq_lptr_t;
 //               and s_barrier (everyone's have); then, between its MFMAs, the packed
 //               weights, the first activation fragments and the first weight pairs of
 //               step ks+1, so that step ks+1 starts multiplying at once.
-// One barrier per K-step suffices: slot (ks+2)%3 = (ks-1)%3 is refilled by loads issued after
+// One barrier per K-step suffices (three slots shown): slot (ks+2)%3 = (ks-1)%3 is refilled by loads issued after
 // the barrier of step ks-1, and every wavefront has waited for its last LDS reads of that slot
 // (the phase-3 fragments of step ks-1) before that barrier.
-template <class Policy, class Epilogue, int TM, int TN, int WM, int WN, int TME>
+template <class Policy, class Epilogue, int TM, int TN, int WM, int WN, int WPE, int TME>
 __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs,
                                               const half_t* __restrict__ X, half_t* __restrict__ Y,
                                               const Epilogue& epilogue, int M, int N, int K, int m0,
                                               int n0, unsigned char* lds) {
-  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN>;
+  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN, WPE>;
   constexpr int kALoadsE = Cfg::kALoads * TME / TM;  // direct A loads per wavefront per step
   constexpr int L = kALoadsE + Cfg::kBLoads + Cfg::kSLoads;  // direct loads per wavefront per step
   constexpr int NSLOT = TME * TN;                    // MFMAs per phase
@@ -186,14 +190,27 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
     }
   };
 
-  // ---- prologue: steps 0 and 1 in flight, operands of step 0 ready ----
+  // ---- prologue: steps 0 .. kStages - 2 in flight, operands of step 0 ready ----
+  constexpr int AHEAD = Cfg::kStages - 1;  // steps of loads in flight while a step is multiplied
 #pragma unroll
-  for (int idx = 0; idx < L; ++idx) issue_one(0, idx);
-  if (ksteps > 1) {
+  for (int st = 0; st < AHEAD; ++st) {
+    if (st < ksteps) {
 #pragma unroll
-    for (int idx = 0; idx < L; ++idx) issue_one(1, idx);
+      for (int idx = 0; idx < L; ++idx) issue_one(st, idx);
+    }
   }
-  if (ksteps > 1) {
+  // loads retire in order: step 0 has landed once at most the loads of the later steps are outstanding
+  static_assert(AHEAD * L <= 63, "vmcnt holds 6 bits");
+  const int first_later = min(AHEAD, ksteps) - 1;
+  if (first_later >= 5) {
+    WQ_WAITCNT_VM(5 * L);
+  } else if (first_later == 4) {
+    WQ_WAITCNT_VM(4 * L);
+  } else if (first_later == 3) {
+    WQ_WAITCNT_VM(3 * L);
+  } else if (first_later == 2) {
+    WQ_WAITCNT_VM(2 * L);
+  } else if (ksteps >= 2) {
     WQ_WAITCNT_VM(L);
   } else {
     WQ_WAITCNT_VM(0);
@@ -215,7 +232,8 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
   for (int ks = 0; ks < ksteps; ++ks) {
     const unsigned char* slot = lds + (ks % Cfg::kStages) * Cfg::kStageBytes;
     const unsigned char* next_slot = lds + ((ks + 1) % Cfg::kStages) * Cfg::kStageBytes;
-    const bool ahead2 = ks + 2 < ksteps;
+    const bool ahead2 = ks + AHEAD < ksteps;  // there is a step to request in this one
+    const int later = min(AHEAD - 1, ksteps - 2 - ks);  // steps requested beyond ks + 1 when phase 3 waits
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       const int cur = kk & 1, nxt = cur ^ 1;
@@ -223,7 +241,13 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
       const int a_kk = kk == 3 ? 0 : kk + 1;
       if (kk == 3) {
         // loads of step ks+1 landed (those of ks+2 may be in flight), own LDS reads done
-        if (ahead2) {
+        if (later >= 4) {
+          WQ_WAITCNT_VM_LGKM0(4 * L);
+        } else if (later == 3) {
+          WQ_WAITCNT_VM_LGKM0(3 * L);
+        } else if (later == 2) {
+          WQ_WAITCNT_VM_LGKM0(2 * L);
+        } else if (later == 1) {
           WQ_WAITCNT_VM_LGKM0(L);
         } else {
           WQ_WAITCNT_VM_LGKM0(0);
@@ -254,13 +278,13 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
           if (sl == first + p * half / NPAIR) pb[p] = Policy::pair_bits(bw[tt], (kk + 1) & 3, j);
           if (sl == first + half + p * (usable - half) / NPAIR) dq[tt][j] = Policy::pair_finish(pb[p], bs[tt]);
         }
-        // direct loads of step ks+2, all in phase 0 (into the slot of step ks-1, free since the
+        // direct loads of step ks+AHEAD, all in phase 0 (into the slot of step ks-1, free since the
         // barrier of its phase 3): timed on the GPU, one phase with loads and three without beat
         // the same loads spread over two phases (by 1-2 %) or over all four (by 15 %)
         if (kk == 0 && ahead2) {
           const int l0 = sl * L / NSLOT, l1 = (sl + 1) * L / NSLOT;
 #pragma unroll
-          for (int idx = l0; idx < l1; ++idx) issue_one(ks + 2, idx);
+          for (int idx = l0; idx < l1; ++idx) issue_one(ks + AHEAD, idx);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -306,7 +330,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WAVES_PER_E
 void gemm_lds_kernel(typename Policy::Args wargs, const half_t* __restrict__ X, half_t* __restrict__ Y,
                      Epilogue epilogue, int M, int N, int K, int tiles_m, int tiles_n, int n_full,
                      int split) {
-  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN>;
+  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN, WAVES_PER_EU>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   int pid = blockIdx.x;
   if (pid < n_full) {
@@ -315,7 +339,7 @@ void gemm_lds_kernel(typename Policy::Args wargs, const half_t* __restrict__ X, 
     const int xcd = pid & 7, idx = pid >> 3;
     pid = xcd * per + min(xcd, rem) + idx;
     const int tile_m = pid % tiles_m, tile_n = pid / tiles_m;
-    gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM>(wargs, X, Y, epilogue, M, N, K,
+    gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, WAVES_PER_EU, TM>(wargs, X, Y, epilogue, M, N, K,
                                                         tile_m * Cfg::BM, tile_n * Cfg::BN, lds);
     return;
   }
@@ -325,12 +349,12 @@ void gemm_lds_kernel(typename Policy::Args wargs, const half_t* __restrict__ X, 
   if (m0 >= M) return;  // a slice that lies entirely past the last row
   if (split == 2) {
     if constexpr (TM % 2 == 0)
-      gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM / 2>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
+      gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, WAVES_PER_EU, TM / 2>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   } else if (split == 4) {
     if constexpr (TM % 4 == 0)
-      gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM / 4>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
+      gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, WAVES_PER_EU, TM / 4>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   } else {
-    gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, TM>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
+    gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, WAVES_PER_EU, TM>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   }
 }
 
@@ -338,7 +362,7 @@ template <class Policy, class Epilogue, int TM, int TN, int WM, int WN, int WPE>
 static int launch_gemm_lds(const char* who, const typename Policy::Args& wargs, const uint16_t* x,
                            uint16_t* y, const Epilogue& ep, int64_t M, int64_t N, int64_t K,
                            hipStream_t stream) {
-  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN>;
+  using Cfg = LdsGemmCfg<Policy, TM, TN, WM, WN, WPE>;
   const int tiles_m = (int)((M + Cfg::BM - 1) / Cfg::BM);
   const int tiles_n = (int)((N + Cfg::BN - 1) / Cfg::BN);
   auto kern = gemm_lds_kernel<Policy, Epilogue, TM, TN, WM, WN, WPE>;

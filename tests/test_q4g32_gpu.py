@@ -123,7 +123,7 @@ GEMM_SMALL = [  # (M, N, K) edge shapes: ragged M/N, odd number of groups
 ]
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 13, 14, 17])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 13, 14, 17, 18])
 @pytest.mark.parametrize("M,N,K", GEMM_SMALL)
 def test_gemm_small_vs_oracle(ops, u, oracle, cfg, M, N, K):
     from relax_amd import _lib
