@@ -68,10 +68,19 @@ WQ_PACKED(relax_amd_fpA_intB_encode);
  *                                perm_out i32[K], scratch i32[1]) -> int               load time; 1 = pass
  *                                perm_out to the matmul, 0 = rows already in group order
  *   relax_amd.autogptq_matmul   (W_nk, SZ, perm | null, x f16[..,K], residual | null, out f16[..,N]
- *                                [, workspace u8 >= M*K*2 bytes, needed with perm])    matmul + T_add */
+ *                                [, workspace u8 >= M*K*2 bytes, needed with perm])    matmul + T_add
+ * autogptq_prepare wants groups of equal size; the PrimFunc reads scales[g_idx[k], n] for ANY g_idx (:645-648),
+ * which the padded pair serves (each group's rows padded to a multiple of 32):
+ *   relax_amd.autogptq_prepare_padded (qweight, qzeros, scales, g_idx, W_out u32[N*cap/8], SZ_out f16[N*cap/32*2],
+ *                                perm_out i32[cap]) -> int K_padded        load time; cap = len(perm_out)
+ *                                >= wq_gptq_padded_k_bound(K, G); outputs compact for K_padded
+ *   relax_amd.autogptq_matmul_padded  (W_nk, SZ, perm, K_padded, x f16[..,K], residual | null, out f16[..,N],
+ *                                workspace u8 >= wq_gptq_padded_workspace_bytes(M, K_padded)) */
 WQ_PACKED(relax_amd_autogptq_decode);
 WQ_PACKED(relax_amd_autogptq_prepare);
 WQ_PACKED(relax_amd_autogptq_matmul);
+WQ_PACKED(relax_amd_autogptq_prepare_padded);
+WQ_PACKED(relax_amd_autogptq_matmul_padded);
 
 /* Format B composites, one per pattern name of
  * python/tvm/relax/backend/contrib/cutlass.py:305-312, 344-372.  Arguments are the

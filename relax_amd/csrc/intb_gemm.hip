@@ -155,6 +155,7 @@ static int intb_gemm_lds(int cfg, const char* who, const int8_t* B, const uint16
     case 11: return launch_gemm_lds<P, IntbGemmEpilogue, 8, 2, 1, 4, 1>(who, largs, A, C, gep, m, n, k, stream);
     case 12: return launch_gemm_lds<P, IntbGemmEpilogue, 4, 2, 1, 4, 2>(who, largs, A, C, gep, m, n, k, stream);
     case 17: return launch_gemm_lds<P, IntbGemmEpilogue, 4, 1, 1, 4, 2>(who, largs, A, C, gep, m, n, k, stream);
+    case 18: return launch_gemm_lds<P, IntbGemmEpilogue, 8, 1, 1, 4, 1>(who, largs, A, C, gep, m, n, k, stream);
     default: return fail(WQ_EINVAL, "%s: unknown tile configuration %d", who, cfg);
   }
 }
@@ -194,15 +195,21 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
       return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
   }
   const IntbGemmEpilogue gep{ep, (int)n};
-  // the fully LDS-staged kernel (11, 12, 17) except between M = 320 and 1536, where the 128x256
-  // register-staged tiles fill the CUs better (timings at K = 8192, N = 28672); fine-grained
-  // scales whose pairs are not 4-byte aligned: the register-staged kernel (1..4)
+  // the fully LDS-staged kernel under the tile shape (11, 17 or 18) whose rounds of the machine come out
+  // shortest; fine-grained scales whose pairs are not 4-byte aligned: the register-staged kernel (1..4).
+  // silu / gelu run the element-wise epilogue, whose inlined exp / erf code does not fit next to the 256
+  // accumulator registers of the 256x256 tile (11): they choose between the other two
   const bool lds_ok = !group || (reinterpret_cast<uintptr_t>(scales) & 3u) == 0;
   int cfg = wq_gemm_cfg_override();
-  if (!cfg) cfg = !lds_ok ? choose_gemm_cfg(m, n, false) : (m <= 320 ? 17 : m <= 1536 ? 2 : 11);
-  // silu / gelu run the element-wise epilogue, whose inlined exp / erf code does not fit next to
-  // the 256 accumulator registers of the 256x256 tile: stay with 128-row tiles
-  if (!wq_gemm_cfg_override() && activation >= WQ_ACT_SILU && cfg == 11) cfg = 2;
+  if (!cfg && !lds_ok) cfg = choose_gemm_cfg(m, n, false);
+  if (!cfg) {
+    double best = 0;
+    for (int c : {17, 18, 11}) {
+      if (c == 11 && activation >= WQ_ACT_SILU) continue;
+      const double t = lds_cfg_cost(c, m, n, cu_count());
+      if (!cfg || t < best) cfg = c, best = t;
+    }
+  }
   if (cfg >= 11 && lds_ok) {
     if (group)
       return nbit == 8 ? intb_gemm_lds<8, true>(cfg, who, B, scales, A, C, gep, m, n, k, stream)

@@ -321,6 +321,40 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
   }
 }
 
+// Row slices (1, 2 or 4) that the tiles of the last, partially filled round are cut into: as many as
+// still run all at once.  A rest that already has a CU per tile is only cut if every slice gets a
+// CU of its own: two slices sharing a CU take as long as the whole tile, and read its weights twice.
+inline int lds_tail_split(int rest, int slots, int cus, int TM, int a_loads) {
+  const int room = rest <= cus ? cus : slots;
+  for (int sp : {4, 2})
+    if (TM % sp == 0 && a_loads % sp == 0 && rest * sp <= room) return sp;
+  return 1;
+}
+
+// Relative duration of the LDS-staged GEMM on an M x N problem under tile configuration 11 (256 x 256
+// tiles), 17 (128 x 128, two workgroups per CU) or 18 (256 x 128): rounds of the machine times tile
+// area over the rate one CU sustains on such tiles.  The rates are tile areas per microsecond measured
+// at K = 8192, N = 28672 with int8 weights (128 x 128 alone on its CU 193, two per CU 243 together;
+// 256 x 128: 254; 256 x 256: 294); row slices of a cut tile run at 0.85 (halves) and 0.75 (quarters) of
+// them.  The model reproduces the measured times at M = 65 .. 2048 within 6 %.
+inline double lds_cfg_cost(int cfg, int64_t M, int64_t N, int cus) {
+  const int BM = cfg == 17 ? 128 : 256, BN = cfg == 11 ? 256 : 128, per_cu = cfg == 17 ? 2 : 1;
+  const double rate_alone = cfg == 17 ? 193.0 : cfg == 18 ? 254.0 : 294.0;
+  const double rate_full = cfg == 17 ? 243.0 : rate_alone;  // per CU, every slot taken
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const int slots = cus * per_cu;
+  const int rest = (int)(tiles % slots);
+  const double area = (double)BM * BN;
+  double t = (double)(tiles / slots) * per_cu * area / rate_full;
+  if (rest) {
+    const int split = lds_tail_split(rest, slots, cus, BM / 32, BM / 32);
+    const bool alone = rest * split <= cus;
+    const double slice = split == 4 ? 0.75 : split == 2 ? 0.85 : 1.0;
+    t += area / split * (alone ? 1 : per_cu) / ((alone ? rate_alone : rate_full) * slice);
+  }
+  return t;
+}
+
 // Workgroup -> work item.  The first n_full workgroups compute whole tiles (as many
 // as fill complete rounds of the machine); the tiles of the last, partially filled
 // round are cut into `split` row slices of TM/split sub-tiles so that the round is
@@ -375,15 +409,7 @@ static int launch_gemm_lds(const char* who, const typename Policy::Args& wargs, 
   const int total = tiles_m * tiles_n;
   const int n_full = (total / slots) * slots;
   const int rest = total - n_full;
-  int split = 1;
-  if (tuning().gemm_tail_split) {
-    for (int sp : {4, 2}) {
-      if (TM % sp == 0 && Cfg::kALoads % sp == 0 && rest * sp <= slots) {
-        split = sp;
-        break;
-      }
-    }
-  }
+  const int split = tuning().gemm_tail_split ? lds_tail_split(rest, slots, cu_count(), TM, Cfg::kALoads) : 1;
   WQ_LAUNCH(who, kern, dim3((unsigned)(n_full + rest * split)), dim3(256), Cfg::kLdsBytes, stream, wargs,
             (const half_t*)x, (half_t*)y, ep, (int)M, (int)N, (int)K, tiles_m, tiles_n, n_full, split);
   return WQ_OK;

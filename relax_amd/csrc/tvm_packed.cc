@@ -577,6 +577,80 @@ WQ_PACKED(relax_amd_autogptq_matmul) {
   return rc == WQ_OK ? 0 : packed_fail();
 }
 
+// (qweight, qzeros, scales, g_idx, W_out uint32 [N * capacity/8], SZ_out fp16 [N * capacity/32 * 2],
+//  perm_out int32 [capacity]) -> int: K_padded.  Any g_idx (groups of unequal size, in any order: the
+// PrimFunc indexes scales[g_idx[k], n] without restriction); capacity = perm_out's length, at least
+// wq_gptq_padded_k_bound(K, G).  The outputs are filled compactly for K_padded: W [N, K_padded/8] and so on.
+WQ_PACKED(relax_amd_autogptq_prepare_padded) {
+  (void)resource_handle;
+  const char* who = "relax_amd.autogptq_prepare_padded";
+  Tensor qw, qz, sc, gi, Wo, SZ, perm;
+  int64_t K, N, G;
+  if (num_args != 7) {
+    fail(WQ_EINVAL, "%s: expected (qweight, qzeros, scales, g_idx, W_out, SZ_out, perm_out)", who);
+    return packed_fail();
+  }
+  if (!gptq_checkpoint_args(who, args, type_codes, num_args, &qw, &qz, &sc, &gi, &K, &N, &G) ||
+      !get_tensor(who, args, type_codes, num_args, 4, kDLUInt, 32, "W_out", &Wo) ||
+      !get_tensor(who, args, type_codes, num_args, 5, kDLFloat, 16, "SZ_out", &SZ) ||
+      !get_tensor(who, args, type_codes, num_args, 6, kDLInt, 32, "perm_out", &perm))
+    return packed_fail();
+  const int64_t capacity = perm.numel;
+  if (capacity % 32 != 0 || Wo.numel < N * (capacity / 8) || SZ.numel < N * (capacity / 32) * 2) {
+    fail(WQ_EINVAL, "%s: outputs must hold W [N, capacity/8], SZ [N, capacity/32, 2] for capacity = len(perm_out), a multiple of 32", who);
+    return packed_fail();
+  }
+  int64_t k_padded = 0;
+  const int rc = wq_gptq_prepare_padded((const uint32_t*)qw.ptr, (const uint32_t*)qz.ptr, (const uint16_t*)sc.ptr,
+                                        (const int32_t*)gi.ptr, (uint32_t*)Wo.ptr, (uint16_t*)SZ.ptr,
+                                        (int32_t*)perm.ptr, capacity, &k_padded, K, N, G, current_stream());
+  if (rc != WQ_OK) return packed_fail();
+  if (out_ret_value && out_ret_tcode) {
+    out_ret_value->v_int64 = k_padded;
+    *out_ret_tcode = kTVMArgInt;
+  }
+  return 0;
+}
+
+// (W_nk, SZ, perm, K_padded, x fp16 [.., K], residual | null, out fp16 [.., N], workspace uint8): the matmul and
+// the add over operands prepared by relax_amd.autogptq_prepare_padded (N follows from out, K from x).
+WQ_PACKED(relax_amd_autogptq_matmul_padded) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.autogptq_matmul_padded";
+  Tensor W, SZ, perm, x, res, out, ws;
+  int64_t k_padded = 0;
+  if (num_args != 8) {
+    fail(WQ_EINVAL, "%s: expected (W_nk, SZ, perm, K_padded, x, residual|null, out, workspace)", who);
+    return packed_fail();
+  }
+  const bool has_res = type_codes[5] != kTVMNullptr;
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W_nk", &W) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "SZ", &SZ) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLInt, 32, "perm", &perm) ||
+      !get_int(who, args, type_codes, num_args, 3, "K_padded", &k_padded) ||
+      !get_tensor(who, args, type_codes, num_args, 4, kDLFloat, 16, "x", &x) ||
+      (has_res && !get_tensor(who, args, type_codes, num_args, 5, kDLFloat, 16, "residual", &res)) ||
+      !get_tensor(who, args, type_codes, num_args, 6, kDLFloat, 16, "out", &out) ||
+      !get_tensor(who, args, type_codes, num_args, 7, kDLUInt, 8, "workspace", &ws))
+    return packed_fail();
+  if (x.t->ndim < 1 || out.t->ndim < 1) {
+    fail(WQ_EINVAL, "%s: x and out need at least one dimension", who);
+    return packed_fail();
+  }
+  const int64_t K = x.t->shape[x.t->ndim - 1], N = out.t->shape[out.t->ndim - 1];
+  const int64_t m = leading(x.t);
+  if (k_padded <= 0 || k_padded % 32 != 0 || perm.numel < k_padded || W.numel < N * (k_padded / 8) ||
+      SZ.numel < N * (k_padded / 32) * 2 || out.numel != m * N || (has_res && res.numel != m * N)) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (m=%lld n=%lld k=%lld k_padded=%lld)", who, (long long)m, (long long)N,
+         (long long)K, (long long)k_padded);
+    return packed_fail();
+  }
+  const int rc = wq_gptq_linear_padded((const uint32_t*)W.ptr, (const uint16_t*)SZ.ptr, (const int32_t*)perm.ptr,
+                                       (const uint16_t*)x.ptr, nullptr, (const uint16_t*)res.ptr, (uint16_t*)out.ptr, m,
+                                       N, K, k_padded, ws.ptr, (size_t)ws.numel, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
 // (A fp16 [N, K]) -> (w int8 [K, N] | [K, N/2], scales fp16 [N] | [K/64, N], scratch fp32 [N]): the
 // reference fixtures' `encode`; int4 and the group size follow from the output shapes.
 WQ_PACKED(relax_amd_fpA_intB_encode) {
@@ -683,6 +757,8 @@ const std::vector<Entry>& table() {
     v.push_back({"relax_amd.autogptq_decode", "relax_amd_autogptq_decode", relax_amd_autogptq_decode});
     v.push_back({"relax_amd.autogptq_prepare", "relax_amd_autogptq_prepare", relax_amd_autogptq_prepare});
     v.push_back({"relax_amd.autogptq_matmul", "relax_amd_autogptq_matmul", relax_amd_autogptq_matmul});
+    v.push_back({"relax_amd.autogptq_prepare_padded", "relax_amd_autogptq_prepare_padded", relax_amd_autogptq_prepare_padded});
+    v.push_back({"relax_amd.autogptq_matmul_padded", "relax_amd_autogptq_matmul_padded", relax_amd_autogptq_matmul_padded});
 #define WQ_ENTRY(sym, op) v.push_back({std::string("relax_amd.") + op, #sym, sym});
     WQ_DECODE_MATMUL_LIST(WQ_ENTRY)
 #undef WQ_ENTRY

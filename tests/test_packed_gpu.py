@@ -241,6 +241,55 @@ def test_autogptq_family(env, oracle):
     assert rc == -1 and b"inconsistent" in lib.wq_last_error()
 
 
+@pytest.mark.parametrize("M", [1, 3, 40])
+def test_autogptq_padded_pair(env, oracle, M):
+    """relax_amd.autogptq_prepare_padded / autogptq_matmul_padded: a g_idx whose groups differ in size
+    (tests/python/dlight/test_gpu_gemv.py:645-648 index scales[g_idx[k], n] without restriction)."""
+    lib, u, T, torch = env
+    N, K, G = 136, 1024, 8
+    x, qw, qz, s, _ = oracle.make_gptq_inputs(M, N, K, K // G, seed=30 + M)
+    g_idx = np.random.default_rng(31).integers(0, G, size=K).astype(np.int32)
+    assert len(set(np.bincount(g_idx, minlength=G).tolist())) > 1
+    res = np.random.default_rng(32).standard_normal((M, N)).astype(np.float16)
+    d = {k: u.dev(v) for k, v in dict(qw=qw, qz=qz, s=s, g=g_idx, x=x, r=res).items()}
+    tqw, _ = T.from_torch(d["qw"], "uint32")
+    tqz, _ = T.from_torch(d["qz"], "uint32")
+    ts, _ = T.from_torch(d["s"])
+    tg, _ = T.from_torch(d["g"])
+    tx, _ = T.from_torch(d["x"])
+    tr, _ = T.from_torch(d["r"])
+    cap = int(lib.wq_gptq_padded_k_bound(K, G))
+    assert cap >= K and cap % 32 == 0
+    W = torch.empty((N * cap // 8,), dtype=torch.int32, device="cuda")
+    SZ = torch.empty((N * cap // 32 * 2,), dtype=torch.float16, device="cuda")
+    perm = torch.empty((cap,), dtype=torch.int32, device="cuda")
+    tW, _ = T.from_torch(W, "uint32")
+    tSZ, _ = T.from_torch(SZ)
+    tp, _ = T.from_torch(perm)
+    rc, rv, rcode = T.call(lib.relax_amd_autogptq_prepare_padded, tqw, tqz, ts, tg, tW, tSZ, tp)
+    assert rc == 0, lib.wq_last_error()
+    kp = rv.v_int64
+    assert rcode == T.kTVMArgInt and K <= kp <= cap and kp % 32 == 0
+    order = u.host(perm)[:kp]
+    assert np.array_equal(order[order >= 0], np.argsort(g_idx, kind="stable"))
+    y = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    ty, _ = T.from_torch(y)
+    ws = torch.empty((int(lib.wq_gptq_padded_workspace_bytes(M, kp)),), dtype=torch.uint8, device="cuda")
+    tws, _ = T.from_torch(ws)
+    Bref = oracle.gptq_dequant(qw, qz, s, g_idx)
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul_padded, tW, tSZ, tp, int(kp), tx, tr, ty, tws)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y), oracle.nt_matmul_f32acc(np.ascontiguousarray(Bref.T), x, None, res), "padded matmul + add")
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul_padded, tW, tSZ, tp, int(kp), tx, None, ty, tws)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y), oracle.nt_matmul_f32acc(np.ascontiguousarray(Bref.T), x), "padded matmul")
+    # errors: a K_padded that the buffers cannot hold; too few arguments
+    rc, _, _ = T.call(lib.relax_amd_autogptq_matmul_padded, tW, tSZ, tp, cap + 32, tx, None, ty, tws)
+    assert rc == -1 and b"inconsistent" in lib.wq_last_error()
+    rc, _, _ = T.call(lib.relax_amd_autogptq_prepare_padded, tqw, tqz, ts, tg, tW, tSZ)
+    assert rc == -1
+
+
 @pytest.mark.parametrize("case,nbit,group,M", [("int8_percol", 8, -1, 40), ("int8_nobias", 8, -1, 1),
                                                ("int8_percol", 8, -1, 300), ("int4_fine", 4, 64, 24),
                                                ("int4_fine", 4, 64, 260)])
