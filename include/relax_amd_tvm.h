@@ -59,6 +59,10 @@ WQ_PACKED(relax_amd_q4f16_1_decode);
  *                                (tests/python/relax/test_codegen_cutlass.py:1392-1457, 1631-1676, 2044-2109) */
 WQ_PACKED(relax_amd_q4f16_1_encode);
 WQ_PACKED(relax_amd_q4f16_1_kn_to_nk);
+/* "relax_amd.q4f16_1_kn_matmul"(W_kn u32[K/8,N], S_kn f16[K/32,N], x f16[..,K], out f16[..,N][, workspace u8]):
+ * the decode linear over a K-major checkpoint in place (tests/python/dlight/test_gpu_reduction.py:102-165), up to
+ * WQ_KN_GEMV_MAX_M rows; workspace >= wq_q4g32_kn_gemv_workspace_bytes(M, N, K) bytes where that is not 0. */
+WQ_PACKED(relax_amd_q4f16_1_kn_matmul);
 WQ_PACKED(relax_amd_fpA_intB_encode);
 
 /* AutoGPTQ layers (tests/python/dlight/test_gpu_gemv.py:636-665: qweight u32[K/8,N], qzeros u32[G,N/8],

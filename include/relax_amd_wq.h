@@ -227,6 +227,17 @@ int wq_q4g32_encode(const uint16_t* A, uint32_t* W, uint16_t* S, int64_t N, int6
  * time.  Not in place. */
 int wq_q4g32_kn_to_nk(const uint32_t* W_kn, const uint16_t* S_kn, uint32_t* W_nk, uint16_t* S_nk,
                       int64_t N, int64_t K, wq_stream_t stream);
+/* The decode linear over a K-major checkpoint IN PLACE (no transposed copy): y fp16 [M, N] =
+ * epilogue(x fp16 [M, K] . w) for M <= WQ_KN_GEMV_MAX_M rows, 4 rows per pass over the weights (what the
+ * reference's reduction rule schedules for this layout, test_gpu_reduction.py:102-165; epilogue as
+ * wq_q4g32_linear).  N % 4 == 0.  K is cut into slices over workgroups; their partial sums go through
+ * `workspace` (wq_q4g32_kn_gemv_workspace_bytes, 16-byte aligned; 0 bytes when one slice covers K).  More rows
+ * are refused with WQ_EUNSUPPORTED: convert once with wq_q4g32_kn_to_nk and use wq_q4g32_linear. */
+#define WQ_KN_GEMV_MAX_M 16
+size_t wq_q4g32_kn_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int wq_q4g32_kn_gemv(const uint32_t* W_kn, const uint16_t* S_kn, const uint16_t* x, const uint16_t* bias,
+                     const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K, void* workspace,
+                     size_t workspace_bytes, wq_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * AutoGPTQ checkpoints (tests/python/dlight/test_gpu_gemv.py:636-665):

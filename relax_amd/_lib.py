@@ -39,6 +39,8 @@ SIGNATURES = {
     "wq_fpA_intB_gemm": [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
     "wq_fpA_intB_gemm_residual": [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp],
     "wq_q4g32_kn_to_nk": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
+    "wq_q4g32_kn_gemv_workspace_bytes": [_i64, _i64, _i64],
+    "wq_q4g32_kn_gemv": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp],
     "wq_gptq_dequantize": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_gptq_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_int), _i64, _i64, _i64, _vp],
     "wq_gptq_workspace_bytes": [_i64, _i64, _int],
@@ -73,7 +75,7 @@ SIGNATURES = {
 }
 _RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p, "wq_program_create": _vp,
              "wq_program_destroy": None, "wq_program_plan": _i64, "wq_program_unplanned_bytes": _i64,
-             "wq_gptq_workspace_bytes": _sz, "wq_gptq_padded_workspace_bytes": _sz, "wq_gptq_padded_k_bound": _i64, "wq_q4g32_gemv_list_workspace_bytes": _sz,
+             "wq_gptq_workspace_bytes": _sz, "wq_q4g32_kn_gemv_workspace_bytes": _sz, "wq_gptq_padded_workspace_bytes": _sz, "wq_gptq_padded_k_bound": _i64, "wq_q4g32_gemv_list_workspace_bytes": _sz,
              "wq_q4g32_gemv_list_create": _vp, "wq_q4g32_gemv_list_create_batched": _vp, "wq_q4g32_gemv_list_destroy": None}
 
 # include/relax_amd_wq_testing.h: the work-split overrides of the calling thread (all return void)

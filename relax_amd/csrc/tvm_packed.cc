@@ -405,6 +405,39 @@ WQ_PACKED(relax_amd_q4f16_1_decode) {
   return rc == WQ_OK ? 0 : packed_fail();
 }
 
+// (W_kn uint32 [K/8, N], S_kn fp16 [K/32, N], x fp16 [.., K], out fp16 [.., N][, workspace uint8]): the decode
+// linear over a K-major checkpoint in place (buffer order of tests/python/dlight/test_gpu_reduction.py:102-107:
+// weights, scales, activations, result), up to WQ_KN_GEMV_MAX_M rows.
+WQ_PACKED(relax_amd_q4f16_1_kn_matmul) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.q4f16_1_kn_matmul";
+  Tensor W, S, x, out, ws;
+  if (num_args != 4 && num_args != 5) {
+    fail(WQ_EINVAL, "%s: expected (W_kn, S_kn, x, out[, workspace])", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W_kn", &W) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "S_kn", &S) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLFloat, 16, "x", &x) ||
+      !get_tensor(who, args, type_codes, num_args, 3, kDLFloat, 16, "out", &out) ||
+      (num_args == 5 && !get_tensor(who, args, type_codes, num_args, 4, kDLUInt, 8, "workspace", &ws)))
+    return packed_fail();
+  if (W.t->ndim != 2 || S.t->ndim != 2 || x.t->ndim < 1 || S.t->shape[1] != W.t->shape[1] ||
+      S.t->shape[0] * 4 != W.t->shape[0] || x.t->shape[x.t->ndim - 1] != W.t->shape[0] * 8) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (W_kn [K/8,N], S_kn [K/32,N], x [..,K])", who);
+    return packed_fail();
+  }
+  const int64_t N = W.t->shape[1], K = W.t->shape[0] * 8, m = leading(x.t);
+  if (out.numel != m * N) {
+    fail(WQ_EINVAL, "%s: out must have %lld x %lld elements", who, (long long)m, (long long)N);
+    return packed_fail();
+  }
+  const int rc = wq_q4g32_kn_gemv((const uint32_t*)W.ptr, (const uint16_t*)S.ptr, (const uint16_t*)x.ptr, nullptr, nullptr,
+                                  (uint16_t*)out.ptr, m, N, K, ws.ptr, num_args == 5 ? (size_t)ws.numel : 0,
+                                  current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
 // (A fp16 [N, K]) -> (W uint32 [N, K/8], S fp16 [N, K/32]): the q4f16_1 quantizer.
 WQ_PACKED(relax_amd_q4f16_1_encode) {
   (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
@@ -753,6 +786,7 @@ const std::vector<Entry>& table() {
     v.push_back({"relax_amd.q4f16_1_decode", "relax_amd_q4f16_1_decode", relax_amd_q4f16_1_decode});
     v.push_back({"relax_amd.q4f16_1_encode", "relax_amd_q4f16_1_encode", relax_amd_q4f16_1_encode});
     v.push_back({"relax_amd.q4f16_1_kn_to_nk", "relax_amd_q4f16_1_kn_to_nk", relax_amd_q4f16_1_kn_to_nk});
+    v.push_back({"relax_amd.q4f16_1_kn_matmul", "relax_amd_q4f16_1_kn_matmul", relax_amd_q4f16_1_kn_matmul});
     v.push_back({"relax_amd.fpA_intB_encode", "relax_amd_fpA_intB_encode", relax_amd_fpA_intB_encode});
     v.push_back({"relax_amd.autogptq_decode", "relax_amd_autogptq_decode", relax_amd_autogptq_decode});
     v.push_back({"relax_amd.autogptq_prepare", "relax_amd_autogptq_prepare", relax_amd_autogptq_prepare});

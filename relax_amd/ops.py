@@ -353,6 +353,49 @@ def q4g32_kn_to_nk(W_kn: torch.Tensor, S_kn: torch.Tensor):
     return W, S
 
 
+KN_GEMV_MAX_M = 16
+
+
+def q4g32_kn_gemv(W_kn: torch.Tensor, S_kn: torch.Tensor, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                  residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                  workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The decode linear over a K-major q4f16_1 checkpoint used in place (``W [K/8, N]``, ``S [K/32, N]``;
+    tests/python/dlight/test_gpu_reduction.py:102-165), ``M <= 16`` rows.  ``workspace`` (uint8, see
+    ``wq_q4g32_kn_gemv_workspace_bytes``) is allocated here when not given."""
+    W_kn = _w32(W_kn)
+    S_kn = _dev(S_kn, torch.float16, "S_kn")
+    x = _dev(x, torch.float16, "x")
+    k8, N = W_kn.shape
+    K = k8 * 8
+    if K % 32 or tuple(S_kn.shape) != (K // 32, N):
+        raise ValueError(f"S_kn must be [K/32, N] = [{K // 32}, {N}], got {tuple(S_kn.shape)}")
+    if x.shape[-1] != K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {K}")
+    M = x.numel() // K if K else 0
+    if bias is not None:
+        bias = _dev(bias, torch.float16, "bias")
+        if bias.numel() != N:
+            raise ValueError("bias must have N elements")
+    if residual is not None:
+        residual = _dev(residual, torch.float16, "residual")
+        if residual.numel() != M * N:
+            raise ValueError("residual must have M*N elements")
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (N,), dtype=torch.float16, device=x.device)
+    else:
+        out = _dev(out, torch.float16, "out")
+        if out.numel() != M * N:
+            raise ValueError("out must have M*N elements")
+    L = _lib.lib()
+    need = int(L.wq_q4g32_kn_gemv_workspace_bytes(M, N, K))
+    if workspace is None and need:
+        workspace = torch.empty((need,), dtype=torch.uint8, device=x.device)
+    check(L.wq_q4g32_kn_gemv(_ptr(W_kn), _ptr(S_kn), _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), M, N, K,
+                             _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream()),
+          "wq_q4g32_kn_gemv")
+    return out
+
+
 # ------------------------------------------------------------------ AutoGPTQ checkpoints
 
 

@@ -241,6 +241,33 @@ def test_autogptq_family(env, oracle):
     assert rc == -1 and b"inconsistent" in lib.wq_last_error()
 
 
+def test_q4f16_1_kn_matmul(env, oracle):
+    """relax_amd.q4f16_1_kn_matmul: the K-major layout of tests/python/dlight/test_gpu_reduction.py:102-120 in place."""
+    lib, u, T, torch = env
+    M, N, K = 3, 520, 4096
+    rng = np.random.default_rng(40)
+    W_kn = rng.integers(0, 2**32, size=(K // 8, N), dtype=np.uint64).astype(np.uint32)
+    S_kn = rng.uniform(0.005, 0.02, size=(K // 32, N)).astype(np.float16)
+    x = rng.standard_normal((M, 1, K)).astype(np.float16)
+    dW, dS, dx = u.dev(W_kn), u.dev(S_kn), u.dev(x)
+    y = torch.empty((M, 1, N), dtype=torch.float16, device="cuda")
+    ws = torch.empty((int(lib.wq_q4g32_kn_gemv_workspace_bytes(M, N, K)),), dtype=torch.uint8, device="cuda")
+    assert ws.numel() > 0
+    tW, _ = T.from_torch(dW, "uint32")
+    tS, _ = T.from_torch(dS)
+    tx, _ = T.from_torch(dx)
+    ty, _ = T.from_torch(y)
+    tws, _ = T.from_torch(ws)
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_kn_matmul, tW, tS, tx, ty, tws)
+    assert rc == 0, lib.wq_last_error()
+    B = oracle.q4g32_kn_dequant(W_kn, S_kn)
+    u.assert_close(u.host(y).reshape(M, N), oracle.nt_matmul_f32acc(np.ascontiguousarray(B.T), x.reshape(M, K)), "kn matmul")
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_kn_matmul, tW, tS, tx, ty)   # K is sliced here: the workspace is needed
+    assert rc == -1 and b"workspace" in lib.wq_last_error()
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_kn_matmul, tS, tS, tx, ty, tws)
+    assert rc == -1
+
+
 @pytest.mark.parametrize("M", [1, 3, 40])
 def test_autogptq_padded_pair(env, oracle, M):
     """relax_amd.autogptq_prepare_padded / autogptq_matmul_padded: a g_idx whose groups differ in size
