@@ -170,7 +170,7 @@ def bench_stack(torch, layers=32, batches=(1, 8, 16, 32)):
     stream = torch.cuda.Stream()
     res = {"layers": layers, "instructions_per_step": 4 * layers,
            "launch": "hip_graph of PackedFunc calls; runs of decode linears (M <= 32) fused into one launch "
-                     "(M = 1: VALU list kernel; 2 .. 16: MFMA list kernel; 17 .. 32: the same as two halves)", "batches": []}
+                     "(M = 1: VALU list kernel; 2 .. 32: MFMA list kernel)", "batches": []}
     for M in batches:
         hidden = torch.randn((M, 4096), device="cuda", dtype=torch.float16)
         attn = torch.randn((M, 4096), device="cuda", dtype=torch.float16)

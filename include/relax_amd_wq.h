@@ -134,8 +134,9 @@ wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* descs, int n
                                           size_t workspace_bytes, wq_stream_t stream);
 /* The same for M rows of activations per linear, 1 <= M <= WQ_GEMV_LIST_MAX_M (a small decode batch): x is
  * fp16 [M, K], y and residual fp16 [M, N], all contiguous; one launch runs the list on the matrix cores, one pass
- * over the weights for up to 16 rows (17 .. 32 rows run as two halves side by side).  M > 1 needs K % 256 == 0 and S 16-byte aligned (WQ_EUNSUPPORTED otherwise:
- * run such a list linear by linear with wq_q4g32_linear). */
+ * over the weights for every M (more than 16 rows: each unpacked weight feeds two matrix-core tiles of 16
+ * rows).  M > 1 needs K % 256 == 0 and S 16-byte aligned (WQ_EUNSUPPORTED otherwise: run such a list linear by
+ * linear with wq_q4g32_linear). */
 #define WQ_GEMV_LIST_MAX_M 32
 wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv_desc* descs, int n, int M, void* workspace,
                                                   size_t workspace_bytes, wq_stream_t stream);

@@ -1,5 +1,5 @@
 // Definitions shared by the two kernels that run a list of format-A linears in one launch
-// (q4g32_gemv_list.hip: one activation row; q4g32_batch_list.hip: 2 .. 16 rows): the descriptor
+// (q4g32_gemv_list.hip: one activation row; q4g32_batch_list.hip: 2 .. 32 rows): the descriptor
 // table, the device-side completion counters, and the host object behind wq_gemv_list_t.
 #ifndef RELAX_AMD_CSRC_GEMV_LIST_COMMON_H_
 #define RELAX_AMD_CSRC_GEMV_LIST_COMMON_H_
@@ -14,7 +14,7 @@ namespace wq {
 struct GemvListDesc {  // 128 bytes, device memory
   const char* W;       // uint32 [N, K/8]
   const char* S;       // fp16   [N, K/32]
-  const half_t* x;     // fp16   [M, K]   (M: a property of the list, 1 .. 16)
+  const half_t* x;     // fp16   [M, K]   (M: a property of the list, 1 .. 32)
   const half_t* bias;  // fp16   [N] or null
   const half_t* residual;  // fp16 [M, N] or null
   half_t* y;           // fp16   [M, N]
@@ -28,7 +28,7 @@ struct GemvListDesc {  // 128 bytes, device memory
   // b mod 2^gmod_log2 == gidx (member c = b >> gmod_log2 of workgroups >> gmod_log2); q, rem and off
   // then count within the group.
   uint8_t gmod_log2, gidx;
-  uint8_t rows;  // rows of x and y of this entry (<= the M of the launch: a list of more than 16 rows is run as two halves)
+  uint8_t rows;  // rows of x and y of this entry (the M of the launch)
   uint8_t pad[61];
 };
 static_assert(sizeof(GemvListDesc) == 128, "descriptor layout");
@@ -76,13 +76,13 @@ struct wq_gemv_list {
   int nb = 2;
   int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
   long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
-  int halves = 1;          // entries of the list per linear of the caller (2: more than 16 rows)
   int M = 1;               // activation rows of the launch; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
-  int batch_u = 0;         // chunks per tile and wavefront (4: panels of 4096 k, M <= 8; 2: 2048 k)
+  int batch_u = 0;         // chunks per tile and wavefront (4: panels of 4096 k, M <= 8; 2: 2048 k, M <= 16; 1: 1024 k)
   int batch_groups = 1;    // groups of workgroups that run different linears side by side
   int batch_nxb = 0;       // panels of activations in LDS
   int batch_ring = 0;      // items the compute wavefronts may spread over (slots of scales and of partial sums)
-  int batch_acc_tiles = 0; // most tiles a workgroup holds of a linear that spans several panels
+  int batch_acc_tiles = 0; // tiles whose sums LDS keeps between the panels of a linear: a chunk of the workgroup's tiles
+  bool batch_chunked = false;  // some linear is walked in several chunks
 };
 
 namespace wq {
@@ -92,7 +92,7 @@ constexpr size_t kListAlign = 256;
 inline size_t list_table_bytes(int n) { return ((size_t)n * sizeof(GemvListDesc) + kListAlign - 1) / kListAlign * kListAlign; }
 
 
-// q4g32_batch_list.hip: launch shape and LDS plan of a list with 2 .. 16 activation rows (fills
+// q4g32_batch_list.hip: launch shape and LDS plan of a list with 2 .. 32 activation rows (fills
 // l->blocks, threads, lds, batch_*; the descriptors' q / rem / off), and its launch
 int batch_list_plan(wq_gemv_list* l);
 int batch_list_launch(wq_gemv_list* l, hipStream_t stream);

@@ -1,18 +1,18 @@
-// A list of format-A (q4f16_1) linears with 2 .. 16 activation rows each, in ONE launch
-// (17 .. 32 rows: the host enters every linear twice, once per half of the rows).
+// A list of format-A (q4f16_1) linears with 2 .. 32 activation rows each, in ONE launch.
 //
 // The counterpart of q4g32_gemv_list.hip for a small batch: the same persistent grid (one workgroup
 // per CU walks the list, device-side counters order dependent linears), but the products are done by
 // the matrix cores so that all M rows share one pass over the weights, and the weights go from
 // memory straight into the registers that feed them.
 //
-// Work.  The unit is a TILE of 16 consecutive rows of W times a PANEL of K (4096 k for M <= 8, else
-// 2048 k).  A linear is run by one GROUP of workgroups (see batch_assign_groups), its tiles dealt to them
-// round-robin, with a rotation that continues from linear to linear.  Inside a workgroup the 8 compute
-// wavefronts split a panel along K: wavefront w owns the 4 U scale groups w * 4U .. of every panel
-// (U = 4 or 2), i.e. U chunks per tile; a chunk is one 16-byte load per lane: lane (i, kq) takes scale
-// group 4u + kq of row i, the 32 codes that the four v_mfma_f32_16x16x32_f16 of the chunk consume as A
-// operands (one dword, 8 codes, each).
+// Work.  The unit is a TILE of 16 consecutive rows of W times a PANEL of K (4096 k for M <= 8, 2048 k
+// for M <= 16, 1024 k beyond: a panel of activations is at most 64 KiB).  A linear is run by one GROUP of
+// workgroups (see batch_assign_groups), its tiles dealt to them round-robin, with a rotation that continues
+// from linear to linear.  Inside a workgroup the 8 compute wavefronts split a panel along K: wavefront w
+// owns the 4 U scale groups w * 4U .. of every panel (U = 4, 2 or 1), i.e. U chunks per tile; a chunk is
+// one 16-byte load per lane: lane (i, kq) takes scale group 4u + kq of row i, the 32 codes that the four
+// v_mfma_f32_16x16x32_f16 of the chunk consume as A operands (one dword, 8 codes, each).  With more than
+// 16 activation rows every unpacked A operand feeds R = 2 MFMAs, one per set of 16 rows.
 // Unpacking is exact: OR the code into 0x6400 (1024 + q, or 1024 + 16 q), subtract 1031 (1136),
 // multiply by the scale, all in packed fp16: 13 VALU instructions per 8 weights and lane, whatever M.
 // The B operands (the activations of the wavefront's K slice, in the k order of the unpack, the
@@ -22,12 +22,17 @@
 //   * 2 x wavefronts wait for a producer linear (bounded spin), load a panel of activations,
 //     rearrange it and leave it in one of 1 or 2 LDS buffers (under load a round trip to L2 takes several
 //     microseconds); the compute wavefronts copy their slice into registers when they reach the panel,
-//     which frees the buffer at once, so even one buffer keeps the next panel ready in time.
+//     which frees the buffer at once, so even one buffer keeps the next panel ready in time.  The two take
+//     whole panels by turns: while one waits for a producer the other already fetches the panel after it
+//     (sharing every panel between them instead was slower at every M).
 //   * the scale wavefront streams the tile's scales (16 rows x 256 contiguous bytes: fetched per
 //     lane they cost more than the codes) into a ring of LDS slots, a few tiles ahead.
 //   * the y wavefront adds the 8 partial sums of a tile in a fixed order, keeps the sum in LDS while
 //     further panels of the same rows follow, and at the last panel applies bias / cast / residual,
 //     stores y with device-scope stores and signals the linear's completion counter.
+// A linear of several panels whose kept sums would not fit the LDS is walked in CHUNKS of its tiles (all
+// panels of a chunk, then the next chunk; template parameter CH): the activations are then loaded once
+// per chunk, which the host weighs against fewer, larger groups when it plans the list.
 // Codes in flight per CU: 8 wavefronts x (NT - 1) tiles x U KiB.
 #include <algorithm>
 #include <cmath>
@@ -87,12 +92,15 @@ struct BatchWait {
 __host__ __device__ constexpr int batch_panel_groups(int U) { return kBW * 4 * U; }
 __host__ __device__ constexpr int batch_scale_row_bytes(int U) { return batch_panel_groups(U) * 2 + 16; }  // + 16: rows on different banks
 __host__ __device__ constexpr int batch_scale_slot_bytes(int U) { return 16 * batch_scale_row_bytes(U); }
-__host__ __device__ constexpr int batch_partial_slot_bytes() { return kBW * 1024; }
+__host__ __device__ constexpr int batch_partial_slot_bytes(int R) { return kBW * R * 1024; }  // R sets of 16 activation rows
 
 // ---- the walk of a workgroup over its items.  All fields are wavefront-uniform.
 struct ItemCursor {
   int lin;           // current linear (nlin: past the end)
   int panel, lt;     // panel of K, local tile (tile = lt * ncu + rb)
+  int lt0, ltend;    // the current chunk of local tiles: a linear of several panels is walked chunk by chunk, all
+                     // panels of a chunk before the next chunk, so that LDS holds the sums of one chunk only
+  int csize;         // tiles per chunk of this linear
   int T, P;          // tiles of this workgroup in the linear (> 0), panels
   int ncu, rb;       // workgroups in the linear's group; (member - off) mod ncu
   int N, G, row_w;   // rows, scale groups per row, bytes per row of W
@@ -108,8 +116,8 @@ __device__ __forceinline__ uint32_t desc_group_word(gemv_desc_ptr descs, int lin
 }
 
 // positions the cursor on the first linear >= c.lin in which this workgroup holds a tile
-template <int U>
-__device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg) {
+template <int U, bool CH>
+__device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg, int chunk) {
   typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
   while (c.lin < nlin) {
     const words_ptr p = (words_ptr)(descs + c.lin);
@@ -136,6 +144,16 @@ __device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, in
         c.S = reinterpret_cast<const char*>(((uint64_t)w[3] << 32) | w[2]);
         c.panel = 0;
         c.lt = 0;
+        if constexpr (CH) {
+          c.lt0 = 0;
+          // chunks of equal size, at most `chunk` tiles (one panel: no sums are kept, one chunk)
+          c.csize = T;
+          if (c.P > 1 && T > chunk) {
+            const int nch = (T + chunk - 1) / chunk;
+            c.csize = (T + nch - 1) / nch;
+          }
+          c.ltend = c.csize;
+        }
         return;
       }
     }
@@ -143,24 +161,38 @@ __device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, in
   }
 }
 
-template <int U>
-__device__ __forceinline__ void item_next_panel(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg) {
-  c.lt = 0;
-  if (++c.panel == c.P) {
-    ++c.lin;
-    item_seek<U>(c, descs, nlin, b, nwg);
+template <int U, bool CH>
+__device__ __forceinline__ void item_next_panel(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg, int chunk) {
+  if constexpr (CH) {
+    if (++c.panel == c.P) {
+      c.panel = 0;
+      c.lt0 = c.ltend;
+      if (c.lt0 >= c.T) {
+        ++c.lin;
+        item_seek<U, CH>(c, descs, nlin, b, nwg, chunk);
+        return;
+      }
+      c.ltend = min(c.T, c.lt0 + c.csize);
+    }
+    c.lt = c.lt0;
+  } else {
+    c.lt = 0;
+    if (++c.panel == c.P) {
+      ++c.lin;
+      item_seek<U, CH>(c, descs, nlin, b, nwg, chunk);
+    }
   }
 }
 
-template <int U>
-__device__ __forceinline__ void item_next(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg) {
-  if (++c.lt == c.T) item_next_panel<U>(c, descs, nlin, b, nwg);
+template <int U, bool CH>
+__device__ __forceinline__ void item_next(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg, int chunk) {
+  if (++c.lt == (CH ? c.ltend : c.T)) item_next_panel<U, CH>(c, descs, nlin, b, nwg, chunk);
 }
 
-template <int U>
+template <int U, int R, bool CH>
 __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvListDesc* __restrict__ descs_, int nlin,
                                                                      int* __restrict__ sync, long long spin_limit,
-                                                                     int M, int nxb, int ring, int use_sync) {
+                                                                     int M, int nxb, int ring, int chunk, int use_sync) {
   constexpr int PG = batch_panel_groups(U);  // scale groups per panel
   constexpr int NT = kBNT;
   constexpr int SROW = batch_scale_row_bytes(U), SSLOT = batch_scale_slot_bytes(U);
@@ -174,7 +206,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
   const int xbuf_bytes = M * (PG * 64);
   char* const sbuf = xbuf + nxb * xbuf_bytes;
   char* const pbuf = sbuf + ring * SSLOT;
-  char* const abuf = pbuf + ring * batch_partial_slot_bytes();
+  char* const abuf = pbuf + ring * batch_partial_slot_bytes(R);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -200,11 +232,11 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     int ahead = 0;  // items issued and not yet consumed
     ItemCursor ic, cc;
     ic.lin = 0;
-    item_seek<U>(ic, descs, nlin, b, nwg);
+    item_seek<U, CH>(ic, descs, nlin, b, nwg, chunk);
     cc = ic;
     int k = 0;    // items consumed
     int pk = -1;  // panels taken
-    half8_t xb[U][4];
+    half8_t xb[R][U][4];
     const int gi0 = wave * (4 * U) + kq;  // the lane's scale group within the panel, chunk 0
 
     auto issue = [&](uint4_t (&buf)[U]) {
@@ -222,7 +254,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(buf[u]) : "v"(voff), "s"(base));
       }
       ++ahead;
-      item_next<U>(ic, descs, nlin, b, nwg);
+      item_next<U, CH>(ic, descs, nlin, b, nwg, chunk);
     };
 
     const half2_t k1031 = {(half_t)-1031.0f, (half_t)-1031.0f};
@@ -241,23 +273,28 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     };
 
     auto consume = [&](uint4_t (&buf)[U]) {
-      if (cc.lt == 0) {
+      if (cc.lt == (CH ? cc.lt0 : 0)) {
         // a new panel: its activations are staged (or will be); this wavefront's K slice goes to registers
         ++pk;
         const int xslot = pk % nxb;
         wait.until(&flags->x_ready[xslot], pk + 1, 1);
-        const char* xs = xbuf + xslot * xbuf_bytes + (wave * U * 16 * M + kq * M + min(i, M - 1)) * 16;
 #pragma unroll
-        for (int u = 0; u < U; ++u)
+        for (int r = 0; r < R; ++r) {
+          const char* xs = xbuf + xslot * xbuf_bytes + (wave * U * 16 * M + kq * M + min(i + 16 * r, M - 1)) * 16;
 #pragma unroll
-          for (int d = 0; d < 4; ++d) xb[u][d] = *reinterpret_cast<const half8_t*>(xs + ((u * 4 + d) * 4 * M) * 16);
+          for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) xb[r][u][d] = *reinterpret_cast<const half8_t*>(xs + ((u * 4 + d) * 4 * M) * 16);
+        }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (lane == 0) __hip_atomic_fetch_add(&flags->x_taken[xslot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
       wait.until(&flags->s_ready, k + 1, 2);
       const int slot = k & (ring - 1);
       const char* sb = sbuf + slot * SSLOT + i * SROW + gi0 * 2;
-      float4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+      float4_t acc0[R], acc1[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc0[r] = acc1[r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint32_t s16 = *reinterpret_cast<const uint16_t*>(sb + u * 8);
@@ -272,18 +309,22 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
           const uint32_t a2 = unpack(and_or(w8, 0x000F000Fu, magic), k1031, s16);    // (q2, q6)
           const uint32_t a3 = unpack(and_or(w8, 0x00F000F0u, magic), k1136, s16);    // 16 (q3, q7)
           const half8_t aop = __builtin_bit_cast(half8_t, uint4_t{a0, a1, a2, a3});
-          if (d & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, xb[u][d], acc1, 0, 0, 0);
-          else acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, xb[u][d], acc0, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            if (d & 1) acc1[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, xb[r][u][d], acc1[r], 0, 0, 0);
+            else acc0[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, xb[r][u][d], acc0[r], 0, 0, 0);
+          }
         }
       }
       --ahead;
-      const float4_t part = acc0 + acc1;
       if (k >= ring) wait.until(&flags->y_done, k - ring + 1, 3);
-      *reinterpret_cast<float4_t*>(pbuf + (slot * kBW + wave) * 1024 + lane * 16) = part;
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        *reinterpret_cast<float4_t*>(pbuf + ((slot * kBW + wave) * R + r) * 1024 + lane * 16) = acc0[r] + acc1[r];
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       if (lane == 0) __hip_atomic_fetch_add(&flags->done[slot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       ++k;
-      item_next<U>(cc, descs, nlin, b, nwg);
+      item_next<U, CH>(cc, descs, nlin, b, nwg, chunk);
     };
 
 #pragma unroll
@@ -334,7 +375,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     constexpr int UX = 32;       // loads in flight per lane: one round trip for a panel of 8 rows x 2048 k
     ItemCursor xc;
     xc.lin = 0;
-    item_seek<U>(xc, descs, nlin, b, nwg);
+    item_seek<U, CH>(xc, descs, nlin, b, nwg, chunk);
     // the x wavefronts take whole panels by turns (panel pk belongs to wavefront pk mod kBXW) and run up
     // to nxb panels ahead of the compute wavefronts: under load a round trip to L2 takes several microseconds
     int pk = 0;
@@ -393,7 +434,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         if (lane == 0) __hip_atomic_store(&flags->x_ready[xslot], pk + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
       ++pk;
-      item_next_panel<U>(xc, descs, nlin, b, nwg);
+      item_next_panel<U, CH>(xc, descs, nlin, b, nwg, chunk);
     }
     return;
   }
@@ -406,7 +447,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     uint4_t sv[PD][LP];
     ItemCursor ic, cc;
     ic.lin = 0;
-    item_seek<U>(ic, descs, nlin, b, nwg);
+    item_seek<U, CH>(ic, descs, nlin, b, nwg, chunk);
     cc = ic;
     int k = 0;
     auto issue = [&](uint4_t (&buf)[LP]) {
@@ -423,7 +464,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
           buf[t] = __builtin_nontemporal_load(
               reinterpret_cast<const uint4_t*>(base + (int64_t)min(n0 + r, ic.N - 1) * (ic.G * 2) + pc * 16));
       }
-      item_next<U>(ic, descs, nlin, b, nwg);
+      item_next<U, CH>(ic, descs, nlin, b, nwg, chunk);
     };
     auto consume = [&](uint4_t (&buf)[LP]) {
       const int slot = k & (ring - 1);
@@ -438,7 +479,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       ++k;
       if (lane == 0) __hip_atomic_store(&flags->s_ready, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      item_next<U>(cc, descs, nlin, b, nwg);
+      item_next<U, CH>(cc, descs, nlin, b, nwg, chunk);
     };
 #pragma unroll
     for (int t = 0; t < PD - 1; ++t) issue(sv[t]);
@@ -467,41 +508,61 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       const int T = descs[lin].q + (rb < (int)descs[lin].rem ? 1 : 0);
       const int N = descs[lin].N;
       const int P = ((int)(g_dep & 0xffffu) + PG - 1) / PG;
+      int csize = T;
+      if (CH && P > 1 && T > chunk) {
+        const int nch = (T + chunk - 1) / chunk;
+        csize = (T + nch - 1) / nch;
+      }
       const half_t* bias = descs[lin].bias;
       const half_t* residual = descs[lin].residual;
       const int yrows = (int)((grp >> 16) & 0xffu);
       const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[lin].y, 0, yrows * N * 2, kBufferFlags);
-      for (int panel = 0; panel < (T > 0 ? P : 0); ++panel) {
-        for (int lt = 0; lt < T; ++lt, ++k) {
-          const int slot = k & (ring - 1);
-          wait.until(&flags->done[slot], kBW * (k / ring + 1), 6);
-          const char* pb = pbuf + slot * batch_partial_slot_bytes() + lane * 16;
-          float4_t sum = *reinterpret_cast<const float4_t*>(pb);
+      for (int lt0 = 0; lt0 < T; lt0 += csize) {
+        const int ltend = min(T, lt0 + csize);
+        for (int panel = 0; panel < P; ++panel) {
+          for (int lt = lt0; lt < ltend; ++lt, ++k) {
+            const int slot = k & (ring - 1);
+            wait.until(&flags->done[slot], kBW * (k / ring + 1), 6);
+            const char* pb = pbuf + slot * batch_partial_slot_bytes(R) + lane * 16;
+            float4_t sum[R];
 #pragma unroll
-          for (int w = 1; w < kBW; ++w) sum += *reinterpret_cast<const float4_t*>(pb + w * 1024);
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          if (lane == 0) __hip_atomic_store(&flags->y_done, k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          if (P > 1) {
-            float4_t* keep = reinterpret_cast<float4_t*>(abuf + lt * 1024 + lane * 16);
-            if (panel > 0) sum += *keep;
-            if (panel < P - 1) {
-              *keep = sum;
-              continue;
+            for (int r = 0; r < R; ++r) {
+              sum[r] = *reinterpret_cast<const float4_t*>(pb + r * 1024);
+#pragma unroll
+              for (int w = 1; w < kBW; ++w) sum[r] += *reinterpret_cast<const float4_t*>(pb + (w * R + r) * 1024);
             }
-          }
-          // lane (j, rq) holds rows n0 + 4 rq .. + 3 of activation row j
-          const int n0 = ((lt * ncu + rb) << 4) + 4 * rq;
-          if (j16 < yrows) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (lane == 0) __hip_atomic_store(&flags->y_done, k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (P > 1) {
+              float4_t* keep = reinterpret_cast<float4_t*>(abuf + (lt - lt0) * (R * 1024) + lane * 16);
+              if (panel > 0) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int n = n0 + r;
-              if (n < N) {
-                float v = sum[r];
-                if (bias) v += (float)bias[n];
-                half_t h = (half_t)v;
-                if (residual) h = h + residual[(int64_t)j16 * N + n];
-                // device-scope store: written through, so that a counter update after it publishes it
-                __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (j16 * N + n) * 2, 0, kDeviceScope);
+                for (int r = 0; r < R; ++r) sum[r] += keep[r * 64];
+              }
+              if (panel < P - 1) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) keep[r * 64] = sum[r];
+                continue;
+              }
+            }
+            // lane (j, rq) holds rows n0 + 4 rq .. + 3 of activation rows j, j + 16, ..
+            const int n0 = ((lt * ncu + rb) << 4) + 4 * rq;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const int j = j16 + 16 * r;
+              if (j < yrows) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  const int n = n0 + e;
+                  if (n < N) {
+                    float v = sum[r][e];
+                    if (bias) v += (float)bias[n];
+                    half_t h = (half_t)v;
+                    if (residual) h = h + residual[(int64_t)j * N + n];
+                    // device-scope store: written through, so that a counter update after it publishes it
+                    __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (j * N + n) * 2, 0, kDeviceScope);
+                  }
+                }
               }
             }
           }
@@ -530,9 +591,9 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
 }
 
 // ------------------------------------------------------------------ host side
-static size_t batch_lds_bytes(int U, int M, int nxb, int ring, int acc_tiles) {
+static size_t batch_lds_bytes(int U, int R, int M, int nxb, int ring, int acc_tiles) {
   return sizeof(BatchFlags) + (size_t)nxb * M * batch_panel_groups(U) * 64 + (size_t)ring * batch_scale_slot_bytes(U) +
-         (size_t)ring * batch_partial_slot_bytes() + (size_t)acc_tiles * 1024;
+         (size_t)ring * batch_partial_slot_bytes(R) + (size_t)acc_tiles * R * 1024;
 }
 
 // Which group of workgroups runs which linear.  Every workgroup needs all M x K activations of a linear
@@ -549,17 +610,22 @@ struct BatchGroupPlan {
   double makespan = 0.0;
 };
 
-static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl) {
+// chunks a workgroup with `tiles` tiles of a linear walks them in (each chunk loads every panel of activations again)
+static int batch_chunks(int tiles, int panels, int chunk) { return panels > 1 && tiles > chunk ? (tiles + chunk - 1) / chunk : 1; }
+
+static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, int chunk) {
   const int groups = 1 << gl, ncu = l->blocks >> gl;
   BatchGroupPlan plan;
   plan.group.resize(l->n);
   std::vector<double> free_at(groups, 0.0), end(l->n, 0.0);
   for (int i = 0; i < l->n; ++i) {
     const GemvListDesc& g = l->descs[i];
-    const double K = (double)(g.g_dep & 0xffffu) * 32.0;
-    const double tiles = ((double)g.N + 15.0) / 16.0;
-    // bytes through one workgroup: its tiles' codes and scales, and all activations
-    const double dur = std::ceil(tiles / ncu) * 16.0 * K * (0.5 + 1.0 / 16.0) + l->M * K * 2.0 + 4096.0;
+    const int G = (int)(g.g_dep & 0xffffu);
+    const double K = (double)G * 32.0;
+    const double tiles = (double)((((int64_t)g.N + 15) / 16 + ncu - 1) / ncu);  // of one workgroup
+    const int panels = (G + batch_panel_groups(U) - 1) / batch_panel_groups(U);
+    // bytes through one workgroup: its tiles' codes and scales, and all activations once per chunk
+    const double dur = tiles * 16.0 * K * (0.5 + 1.0 / 16.0) + batch_chunks((int)tiles, panels, chunk) * l->M * K * 2.0 + 4096.0;
     const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
     const double ready = dep >= 0 ? end[dep] : 0.0;
     int best = 0;
@@ -575,8 +641,18 @@ static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl) {
   return plan;
 }
 
+// the kernel that walks the tiles of a linear in chunks carries more loop state: only where a list needs it
+typedef void (*batch_kernel_t)(const GemvListDesc*, int, int*, long long, int, int, int, int, int);
+static batch_kernel_t batch_kernel(int U, bool chunked) {
+  if (U == 4) return chunked ? q4g32_batch_list_kernel<4, 1, true> : q4g32_batch_list_kernel<4, 1, false>;
+  if (U == 2) return chunked ? q4g32_batch_list_kernel<2, 1, true> : q4g32_batch_list_kernel<2, 1, false>;
+  return chunked ? q4g32_batch_list_kernel<1, 2, true> : q4g32_batch_list_kernel<1, 2, false>;
+}
+
 int batch_list_plan(wq_gemv_list* l) {
-  const int U = l->M <= 8 ? 4 : 2;  // panels of 4096 k (M <= 8) or 2048 k: 64 KiB of activations at most
+  // panels of 4096 k (M <= 8), 2048 k (M <= 16) or 1024 k (two sets of 16 rows): 64 KiB of activations at most
+  const int U = l->M <= 8 ? 4 : l->M <= 16 ? 2 : 1;
+  const int R = l->M <= 16 ? 1 : 2;
   l->batch_u = U;
   l->gs = 4;
   l->threads = kBThreads;
@@ -585,21 +661,28 @@ int batch_list_plan(wq_gemv_list* l) {
   int best_gl = -1;
   BatchGroupPlan best;
   int best_acc = 0;
+  bool best_chunked = false;
   for (int gl = 0; gl <= 4; ++gl) {
     if (l->blocks % (1 << gl) != 0 || (l->blocks >> gl) < 1) break;
     const int ncu = l->blocks >> gl;
-    int acc_tiles = 0;
+    int acc_tiles = 0;  // most tiles a workgroup holds of a linear that spans several panels
     for (int i = 0; i < l->n; ++i) {
       const GemvListDesc& g = l->descs[i];
       const int64_t tiles = ((int64_t)g.N + 15) >> 4;
       if ((int)(g.g_dep & 0xffffu) > batch_panel_groups(U)) acc_tiles = std::max<int>(acc_tiles, (int)((tiles + ncu - 1) / ncu));
     }
-    if (batch_lds_bytes(U, l->M, 1, 2, acc_tiles) > budget) continue;  // sums kept between panels do not fit
-    BatchGroupPlan p = batch_assign_groups(l, gl);
+    // the sums kept between panels must fit beside one panel of activations and a ring of 2: else the tiles of
+    // a linear are walked in chunks of what fits, at the price of loading the activations once per chunk
+    const size_t base = batch_lds_bytes(U, R, l->M, 1, 2, 0);
+    if (base + 4 * R * 1024 > budget) continue;
+    const int fit = (int)((budget - base) / ((size_t)R * 1024));
+    const int chunk = std::min(acc_tiles, fit);
+    BatchGroupPlan p = batch_assign_groups(l, gl, U, std::max(chunk, 1));
     if (best_gl < 0 || p.makespan < best.makespan * 0.98) {
       best_gl = gl;
       best = std::move(p);
-      best_acc = acc_tiles;
+      best_acc = chunk;
+      best_chunked = chunk < acc_tiles;
     }
   }
   if (best_gl < 0)
@@ -619,19 +702,19 @@ int batch_list_plan(wq_gemv_list* l) {
   }
   l->batch_groups = groups;
   l->batch_acc_tiles = best_acc;
+  l->batch_chunked = best_chunked;
   // a ring of 4 items and up to 2 panels of activations in LDS if they fit, else a ring of 2
   l->batch_ring = 4;
-  l->batch_nxb = batch_lds_bytes(U, l->M, 2, 4, best_acc) <= budget ? 2 : batch_lds_bytes(U, l->M, 1, 4, best_acc) <= budget ? 1 : 0;
+  l->batch_nxb = batch_lds_bytes(U, R, l->M, 2, 4, best_acc) <= budget ? 2 : batch_lds_bytes(U, R, l->M, 1, 4, best_acc) <= budget ? 1 : 0;
   if (!l->batch_nxb) {
     l->batch_ring = 2;
-    l->batch_nxb = batch_lds_bytes(U, l->M, 2, 2, best_acc) <= budget ? 2 : 1;
+    l->batch_nxb = batch_lds_bytes(U, R, l->M, 2, 2, best_acc) <= budget ? 2 : 1;
   }
-  l->lds = batch_lds_bytes(U, l->M, l->batch_nxb, l->batch_ring, best_acc);
-  const void* kern = U == 4 ? reinterpret_cast<const void*>(q4g32_batch_list_kernel<4>)
-                            : reinterpret_cast<const void*>(q4g32_batch_list_kernel<2>);
+  l->lds = batch_lds_bytes(U, R, l->M, l->batch_nxb, l->batch_ring, best_acc);
+  const void* kern = reinterpret_cast<const void*>(batch_kernel(U, best_chunked));
   // several lists share a kernel: the limit only ever grows
-  static DynamicLdsLimit limit4, limit2;
-  if ((U == 4 ? limit4 : limit2).ensure(kern, (int)l->lds) != hipSuccess)
+  static DynamicLdsLimit limits[3][2];
+  if (limits[U == 4 ? 0 : U == 2 ? 1 : 2][best_chunked ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
     return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
@@ -642,13 +725,10 @@ int batch_list_plan(wq_gemv_list* l) {
 int batch_list_launch(wq_gemv_list* l, hipStream_t stream) {
   const GemvListDesc* table = (const GemvListDesc*)l->table;
   const int use_sync = l->deps > 0 ? 1 : 0;
-  if (l->batch_u == 4) {
-    WQ_LAUNCH("wq_q4g32_gemv_list_run", q4g32_batch_list_kernel<4>, dim3((unsigned)l->blocks), dim3((unsigned)l->threads),
-              l->lds, stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, use_sync);
-  } else {
-    WQ_LAUNCH("wq_q4g32_gemv_list_run", q4g32_batch_list_kernel<2>, dim3((unsigned)l->blocks), dim3((unsigned)l->threads),
-              l->lds, stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, use_sync);
-  }
+  // chunk: at least 1 (a list without a linear of several panels keeps no sums)
+  WQ_LAUNCH("wq_q4g32_gemv_list_run", batch_kernel(l->batch_u, l->batch_chunked), dim3((unsigned)l->blocks), dim3((unsigned)l->threads), l->lds,
+            stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, std::max(l->batch_acc_tiles, 1),
+            use_sync);
   return WQ_OK;
 }
 

@@ -35,6 +35,7 @@
 // loaded) until the producer has finished everywhere; callers order lists so that this is rare.
 // The last workgroup to finish clears the counters for the next launch.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <vector>
@@ -504,8 +505,7 @@ constexpr int kListDepth = 4;  // ring slots (KiB of codes in flight) per comput
 
 extern "C" size_t wq_q4g32_gemv_list_workspace_bytes(int n) {
   if (n <= 0) return 0;
-  // room for two entries per linear (lists with more than 16 rows of activations)
-  return wq::list_table_bytes(2 * n) + (size_t)wq::sync_ints(2 * n) * sizeof(int);
+  return wq::list_table_bytes(n) + (size_t)wq::sync_ints(n) * sizeof(int);
 }
 
 extern "C" void wq_q4g32_gemv_list_destroy(wq_gemv_list_t* l) { delete l; }
@@ -527,11 +527,6 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
       workspace_bytes < wq_q4g32_gemv_list_workspace_bytes(n))
     return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: workspace must be 256-byte aligned device memory of %zu bytes",
                wq_q4g32_gemv_list_workspace_bytes(n));
-  // More than 16 rows: every linear becomes two entries of the list, one per half of the rows (the kernel
-  // holds 16 rows of activations; the two halves read the same weights at about the same time on different
-  // groups of workgroups, so the second read is served by the memory-side cache).
-  const int halves = M > 16 ? 2 : 1;
-  const int Mk = halves == 2 ? (M + 1) / 2 : M;  // rows the kernel is launched for
   std::vector<wq_q4g32_gemv_desc> e;
   std::vector<int> rows;
   for (int i = 0; i < n; ++i) {
@@ -545,21 +540,13 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
     // several rows: the scales travel in 16-byte pieces of 8, and rows of x and y are addressed with 32-bit offsets
     if (M > 1 && (s.K % 256 != 0 || !aligned16(s.S) || (int64_t)M * s.N >= (1ll << 30) || s.K / 32 > 0xffff))
       return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d: with %d rows of activations K=%lld must be a multiple of 256, S 16-byte aligned and M * N < 2^30", i, M, (long long)s.K);
-    for (int h = 0; h < halves; ++h) {
-      wq_q4g32_gemv_desc t = s;
-      const int64_t r0 = (int64_t)h * Mk;
-      t.x = s.x + r0 * s.K;
-      t.y = s.y + r0 * s.N;
-      if (s.residual) t.residual = s.residual + r0 * s.N;
-      e.push_back(t);
-      rows.push_back(h == 0 ? Mk : M - Mk);
-    }
+    e.push_back(s);
+    rows.push_back(M);
   }
   const int ne = (int)e.size();
   std::unique_ptr<wq_gemv_list> l(new wq_gemv_list());
   l->n = ne;
-  l->M = Mk;
-  l->halves = halves;
+  l->M = M;
   l->descs.resize(ne);
   int cmax = 1;
   for (int i = 0; i < ne; ++i) {
@@ -590,13 +577,13 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
       if (((l->descs[i].g_dep >> 16) & 0x7fffu) == 0 && ranges_overlap(a.x, xa, b.y, yb))
         l->descs[i].g_dep |= (uint32_t)(j + 1) << 16;
       if (ranges_overlap(a.residual, ya, b.y, yb) || ranges_overlap(a.bias, (size_t)a.N * 2, b.y, yb))
-        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i / halves, j / halves);
+        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i, j);
       if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, xb) ||
           ranges_overlap(a.y, ya, b.residual, yb) || ranges_overlap(a.y, ya, b.bias, (size_t)b.N * 2))
-        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the output of linear %d overlaps an operand of linear %d", i / halves, j / halves);
+        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the output of linear %d overlaps an operand of linear %d", i, j);
     }
     if (ranges_overlap(a.y, ya, a.x, xa))
-      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: y overlaps x", i / halves);
+      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: y overlaps x", i);
     const int dep = (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1;
     if (dep >= 0) {
       l->descs[dep].g_dep |= kSignal;
@@ -677,7 +664,7 @@ extern "C" int wq_q4g32_gemv_list_status(wq_gemv_list_t* l, wq_stream_t stream) 
   return fail(WQ_EDEVICE,
               "wq_q4g32_gemv_list: a wait for linear %d timed out (the grid was not resident at once?); "
               "results of that launch are undefined",
-              (err - 1) / l->halves);
+              err - 1);
 }
 
 extern "C" int wq_q4g32_gemv_list_info(const wq_gemv_list_t* l, int* dependencies, int* adjacent) {

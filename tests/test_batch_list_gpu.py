@@ -1,5 +1,5 @@
 """wq_q4g32_gemv_list_create_batched: a list of linears with 2 .. 32 rows of activations in one launch (matrix
-cores; more than 16 rows as two halves), against the CPU oracle, through the C ABI."""
+cores; more than 16 rows as two sets of 16 per weight tile), against the CPU oracle, through the C ABI."""
 import numpy as np
 import pytest
 
@@ -97,7 +97,7 @@ def test_dependent_chain_matches_oracle(env, oracle, M):
     gl = ops.Q4G32GemvList([(a["dW"], a["dS"], u.dev(x0), t[0]), (b["dW"], b["dS"], t[0], t[1]),
                             (c["dW"], c["dS"], t[1], t[2]), (d["dW"], d["dS"], t[0], t[3]),
                             (e["dW"], e["dS"], t[2], t[4])], M=M)
-    assert gl.info()[0] == (4 if M <= 16 else 8)  # more than 16 rows: two halves per linear, each with its own waits
+    assert gl.info()[0] == 4  # dependent linears
     print(f"batch list: dependent chain, M = {M}", flush=True)
     r0 = oracle.q4g32_linear(a["W"], a["S"], x0, nthreads=8)
     r1 = oracle.q4g32_linear(b["W"], b["S"], r0, nthreads=8)
