@@ -144,10 +144,10 @@ def test_small_batch_work_splits(ops, u, oracle, nbit, group_size, nw, stages, w
         _lib.lib().wq_debug_set_skinny_config(0, 0, 0)
 
 
-@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 17])
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 17, 18])
 @pytest.mark.parametrize("nbit", [8, 4])
 def test_gemm_tile_configurations(ops, u, oracle, nbit, cfg):
-    """every tile shape of the register-staged (1-4) and the LDS-staged (11, 12, 17) kernel, ragged M,
+    """every tile shape of the register-staged (1-4) and the LDS-staged (11, 12, 17, 18) kernel, ragged M,
     N smaller than a tile, with and without the row-wise epilogue (bias stride not a multiple of 8)."""
     from relax_amd import _lib
 
@@ -168,7 +168,7 @@ def test_gemm_tile_configurations(ops, u, oracle, nbit, cfg):
         _lib.lib().wq_debug_set_gemm_config(0)
 
 
-@pytest.mark.parametrize("M", [1, 16, 128, 512])
+@pytest.mark.parametrize("M", [1, 16, 128, 256, 512])
 def test_int8_full_size_sampled(ops, u, oracle, M):
     """K=8192, N=28672 int8 per-channel.  The oracle checks a sample of output columns
     (columns are independent given x), the one-hot test checks the layout end to end."""
@@ -184,7 +184,7 @@ def test_int8_full_size_sampled(ops, u, oracle, M):
     got = u.host(ops.fpA_intB_gemm(u.dev(x), P, u.dev(s), weight_nbit=8))
     cols = np.concatenate([np.arange(0, 64), np.arange(14000, 14064), np.arange(N - 64, N)])
     A_cols = u.host(dA[:, torch.from_numpy(cols).cuda()].contiguous())
-    # rows from every row tile of the kernels that serve these M (tiles of 128 and 256 rows)
+    # rows from every row tile of the kernels that serve these M (128 x 128, 256 x 128 and 256 x 256 tiles by M)
     rows = np.unique(np.clip(np.array([0, 7, 8, 15, 31, 32, 63, 64, 127, 128, 129, 255, 256, 300, 383, 384, 511]), 0, M - 1))
     ref = oracle.intb_linear(x[rows], A_cols, s[cols], 8, nthreads=8)
     u.assert_close(got[rows][:, cols], ref, f"int8 full M={M}")
