@@ -8,8 +8,9 @@ spill of a ring register inserted between load and wait would read it too early)
 compiles the file to assembly and verifies, in the kernel's text, that
 
 * every ring register (destination of a ``global_load_* ... nt`` instruction) is read only by the
-  three unpack instructions the source uses (``v_and_or_b32``, ``v_lshrrev_b32 .., 8, ..``,
-  ``v_cvt_f32_f16``), never by a move, a store or anything else, and
+  instructions the source uses for it (``v_and_or_b32``, ``v_lshrrev_b32 .., 8, ..``, ``v_cvt_f32_f16``,
+  and the cross-lane ``v_mov_b32_dpp`` of the batch kernel's lane exchange, which the compiler never
+  generates by itself), never by a plain move, a store or anything else, and
 * each ring slot keeps one register in the prologue and in the loop (no renaming copies).
 
 Registers that the compiler also uses for short-lived temporaries while a slot is empty are
@@ -25,7 +26,7 @@ import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ("q4g32_gemv_list.hip", "q4g32_batch_list.hip")
-ALLOWED_READERS = ("v_and_or_b32", "v_lshrrev_b32", "v_cvt_f32_f16")
+ALLOWED_READERS = ("v_and_or_b32", "v_lshrrev_b32", "v_cvt_f32_f16", "v_mov_b32_dpp")
 
 
 def _regs(tok: str):

@@ -245,13 +245,29 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       const int rows = min(16, ic.N - n0);                // >= 1
       const int pg = min(PG, ic.G - ic.panel * PG);       // scale groups of this panel (the last may be short)
       const char* base = ic.W + (int64_t)n0 * ic.row_w + ic.panel * (PG * 16);
-      const uint32_t roff = __umul24((uint32_t)min(i, rows - 1), (uint32_t)ic.row_w);
       // rows past N repeat the last row (never stored); groups past K repeat the last group (their
       // activations and scales are staged as zeros)
+      if constexpr (U >= 2) {
+        // Whole 128-byte lines: the two loads of a pair of chunks take 8 rows each, lane (i, kq) the 16 bytes of
+        // group 4 (i / 8) + kq of row i mod 8 (+ 8 for the second load), so a row contributes 128 contiguous
+        // bytes to an instruction instead of 64 (measured on a 1 GiB stream with the full unpack + MFMA work:
+        // 7.1 against 5.7 TB/s).  consume() puts the halves back where the MFMA wants them.
+        const uint32_t roff_lo = __umul24((uint32_t)min(i & 7, rows - 1), (uint32_t)ic.row_w);
+        const uint32_t roff_hi = __umul24((uint32_t)min(8 + (i & 7), rows - 1), (uint32_t)ic.row_w);
+        const int gpair = wave * (4 * U) + (i >> 3) * 4 + kq;
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const uint32_t voff = roff + (uint32_t)min(gi0 + 4 * u, pg - 1) * 16u;
-        asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(buf[u]) : "v"(voff), "s"(base));
+        for (int u = 0; u < U; u += 2) {
+          const uint32_t goff = (uint32_t)min(gpair + 4 * u, pg - 1) * 16u;
+          asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(buf[u]) : "v"(roff_lo + goff), "s"(base));
+          asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(buf[u + 1]) : "v"(roff_hi + goff), "s"(base));
+        }
+      } else {
+        const uint32_t roff = __umul24((uint32_t)min(i, rows - 1), (uint32_t)ic.row_w);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t voff = roff + (uint32_t)min(gi0 + 4 * u, pg - 1) * 16u;
+          asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(buf[u]) : "v"(voff), "s"(base));
+        }
       }
       ++ahead;
       item_next<U, CH>(ic, descs, nlin, b, nwg, chunk);
@@ -264,13 +280,11 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       asm("v_lshrrev_b32 %0, 8, %1 ; %2" : "=v"(r) : "v"(word), "v"(magic));
       return r;
     };
-    // (t + c) * s with s taken from the low half of `s16` for both results: two roundings, as the format defines
-    auto unpack = [&](uint32_t t, half2_t c, uint32_t s16) {
-      const half2_t d = as_half2(t) + c;
-      uint32_t r;
-      asm("v_pk_mul_f16 %0, %1, %2 op_sel_hi:[1,0]" : "=v"(r) : "v"(d), "v"(s16));
-      return r;
-    };
+    // (t + c) * s: two roundings, as the format defines.  Plain C++ on purpose: the products are the MFMA's A operand, and
+    // the compiler only keeps the wait states between a VALU result and the MFMA that reads it for instructions
+    // it has issued itself (written as inline assembly, v_pk_mul_f16 two instructions in front of the MFMA was
+    // read before it had been written: the weights came out unscaled)
+    auto unpack = [&](uint32_t t, half2_t c, half2_t s2) { return as_u32((as_half2(t) + c) * s2); };
 
     auto consume = [&](uint4_t (&buf)[U]) {
       if (cc.lt == (CH ? cc.lt0 : 0)) {
@@ -295,15 +309,45 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       float4_t acc0[R], acc1[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) acc0[r] = acc1[r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      uint32_t cw[2][4];  // the chunks of a pair after the exchange
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint32_t s16 = *reinterpret_cast<const uint16_t*>(sb + u * 8);
-        if (ahead == NT) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"((NT - 1) * U + (U - 1 - u)));
-        else asm volatile("s_waitcnt vmcnt(0)" : "+v"(magic));
+        const half_t sh = *reinterpret_cast<const half_t*>(sb + u * 8);
+        const half2_t s16 = {sh, sh};
+        if constexpr (U >= 2) {
+          if ((u & 1) == 0) {
+            // both loads of the pair have landed; lanes 8 .. 15 of every 16 take their half of chunk u from the second
+            // load 8 lanes below, lanes 0 .. 7 their half of chunk u + 1 from the first load 8 lanes above (row_ror:8
+            // turns a row of 16 lanes by 8).
+            if (ahead == NT) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"((NT - 1) * U + (U - 2 - u)));
+            else asm volatile("s_waitcnt vmcnt(0)" : "+v"(magic));
+            // every ring register is first copied by a statement that depends on the wait (a cross-lane move with the
+            // identity pattern: not an instruction the compiler would put there by itself), the exchange is the compiler's
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const uint32_t lo_in = d == 0 ? buf[u].x : d == 1 ? buf[u].y : d == 2 ? buf[u].z : buf[u].w;
+              const uint32_t hi_in = d == 0 ? buf[u | 1].x : d == 1 ? buf[u | 1].y : d == 2 ? buf[u | 1].z : buf[u | 1].w;
+              uint32_t lo, hi;
+              asm("v_mov_b32_dpp %0, %1 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf ; %2" : "=v"(lo) : "v"(lo_in), "v"(magic));
+              asm("v_mov_b32_dpp %0, %1 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf ; %2" : "=v"(hi) : "v"(hi_in), "v"(magic));
+              cw[0][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)hi, 0x128 /* row_ror:8 */, 0xf, 0xc, false);
+              cw[1][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)lo, 0x128, 0xf, 0x3, false);
+            }
+          }
+        } else {
+          if (ahead == NT) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"((NT - 1) * U + (U - 1 - u)));
+          else asm volatile("s_waitcnt vmcnt(0)" : "+v"(magic));
+        }
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const uint32_t word = d == 0 ? buf[u].x : d == 1 ? buf[u].y : d == 2 ? buf[u].z : buf[u].w;
-          const uint32_t w8 = ring_shr8(word);
+          uint32_t word, w8;
+          if constexpr (U >= 2) {
+            word = cw[u & 1][d];
+            w8 = word >> 8;
+          } else {
+            word = d == 0 ? buf[u].x : d == 1 ? buf[u].y : d == 2 ? buf[u].z : buf[u].w;
+            w8 = ring_shr8(word);
+          }
           const uint32_t a0 = unpack(and_or(word, 0x000F000Fu, magic), k1031, s16);  // (q0, q4)
           const uint32_t a1 = unpack(and_or(word, 0x00F000F0u, magic), k1136, s16);  // 16 (q1, q5)
           const uint32_t a2 = unpack(and_or(w8, 0x000F000Fu, magic), k1031, s16);    // (q2, q6)
