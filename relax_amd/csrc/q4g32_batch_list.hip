@@ -328,8 +328,13 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
               const uint32_t lo_in = d == 0 ? buf[u].x : d == 1 ? buf[u].y : d == 2 ? buf[u].z : buf[u].w;
               const uint32_t hi_in = d == 0 ? buf[u | 1].x : d == 1 ? buf[u | 1].y : d == 2 ? buf[u | 1].z : buf[u | 1].w;
               uint32_t lo, hi;
-              asm("v_mov_b32_dpp %0, %1 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf ; %2" : "=v"(lo) : "v"(lo_in), "v"(magic));
-              asm("v_mov_b32_dpp %0, %1 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf ; %2" : "=v"(hi) : "v"(hi_in), "v"(magic));
+              // (the s_nop: a DPP instruction must not read a register a VALU instruction wrote in the two cycles before it,
+              // and the compiler does not count inline assembly as one)
+              asm("v_mov_b32_dpp %0, %2 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf\n\t"
+                  "v_mov_b32_dpp %1, %3 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf\n\t"
+                  "s_nop 1 ; %4"
+                  : "=&v"(lo), "=&v"(hi)
+                  : "v"(lo_in), "v"(hi_in), "v"(magic));
               cw[0][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)hi, 0x128 /* row_ror:8 */, 0xf, 0xc, false);
               cw[1][d] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)lo, 0x128, 0xf, 0x3, false);
             }
