@@ -19,7 +19,8 @@ GEMM of the same quantization scheme, `cpu_baseline` the CPU restatement of the
 reference's path timed on this machine's host cores.  Further objects on the same
 line: `stack` (32 decoder layers' linears run as one captured instruction list at
 M = 1, 8, 16, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
-128, 512) and `calibration` (measured pure-read and MFMA-only ceilings).
+128, 512), `autogptq` and `kn_gemv` (the neighbouring checkpoint layouts at decode) and
+`calibration` (measured pure-read and MFMA-only ceilings).
 """
 from __future__ import annotations
 
@@ -275,6 +276,44 @@ def bench_autogptq(torch, ops, K=4096, N=4096, group=128, batches=(1, 8), copies
                                  "GB/s": round(nbytes / ms / 1e6, 1),
                                  "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)})
         del layers
+    return res
+
+
+def bench_kn_gemv(torch, ops, copies=24):
+    """The decode linear over K-major (KN) q4f16_1 weights used in place (`wq_q4g32_kn_gemv`), M = 1, the
+    four Llama-2-7B shapes; `copies` weight copies (more than the last-level cache) are cycled inside one
+    captured graph.  Bytes = codes + scales + x + y."""
+    from relax_amd import _lib
+
+    L = _lib.lib()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(13)
+    res = {"weight": "q4f16_1, K-major [K/8, N]", "M": 1, "shapes": []}
+    for N, K in ((12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)):
+        Ws = [torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device="cuda", generator=g)
+              for _ in range(copies)]
+        S = (torch.rand((K // 32, N), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+        x = torch.randn((1, K), device="cuda", dtype=torch.float16)
+        y = torch.empty((1, N), device="cuda", dtype=torch.float16)
+        ws = torch.empty((max(16, int(L.wq_q4g32_kn_gemv_workspace_bytes(1, N, K))),), dtype=torch.uint8, device="cuda")
+
+        def step():
+            for W in Ws:
+                ops.q4g32_kn_gemv(W, S, x, out=y, workspace=ws)
+
+        step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        graph.replay()
+        ms, _ = _measure(torch, torch.cuda.current_stream(), graph.replay, min_ms=MIN_SAMPLE_MS / 4, samples=3)
+        ms /= copies
+        nbytes = N * K // 2 + N * (K // 32) * 2 + K * 2 + N * 2
+        res["shapes"].append({"N": N, "K": K, "us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+                              "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)})
+        del Ws
+        torch.cuda.empty_cache()
     return res
 
 
@@ -540,6 +579,7 @@ def main():
         torch.cuda.empty_cache()
     if not args.no_autogptq:
         out["autogptq"] = bench_autogptq(torch, ops)
+        out["kn_gemv"] = bench_kn_gemv(torch, ops)
     if not args.no_calibration:
         out["calibration"] = bench_calibration(torch)
 
