@@ -56,6 +56,31 @@ def test_independent_linears_match_oracle(env, oracle, M):
                                             int((l["y"] != f).sum()))
 
 
+@pytest.mark.parametrize("M", [2, 8, 9, 16, 17, 32])
+def test_every_nibble_position_carries_its_scale(env, oracle, M):
+    """All codes 8 (weight = scale), a different power-of-two-free scale per (row, group), activations that pick
+    ONE of the 8 nibble positions of every word: y[m, n] = sum over groups of scale[n, g] * (sum of the x at that
+    position), exactly representable.  Catches a scale applied to some positions only (one-hot activations and
+    uniform scales both hide that), on a single tile and on a matrix of several panels."""
+    ops, u, torch = env
+    for N, K in [(16, 256), (48, 4096)]:
+        G = K // 32
+        W = np.full((N, K // 8), 0x88888888, dtype=np.uint32)
+        S = (1.0 + (np.arange(N)[:, None] * 7 + np.arange(G)[None, :] * 3) % 29).astype(np.float16)
+        dW, dS = u.dev(W), u.dev(S)
+        for p in range(8):
+            x = np.zeros((M, K), np.float16)
+            x[:, p::8] = (1 + np.arange(M)[:, None] % 3).astype(np.float16)      # 4 weights per group and row of x
+            y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+            gl = ops.Q4G32GemvList([(dW, dS, u.dev(x), y)], M=M)
+            gl.run()
+            gl.status()
+            want = (4.0 * (1 + np.arange(M) % 3))[:, None] * S.astype(np.float64).sum(axis=1)[None, :]
+            assert want.max() < 65504
+            got = u.host(y).astype(np.float64)
+            assert np.array_equal(got, want.astype(np.float16).astype(np.float64)), (M, N, K, p, np.abs(got - want).max())
+
+
 def test_epilogue_and_one_hot(env, oracle):
     ops, u, torch = env
     M, N, K = 6, 520, 1024
