@@ -15,6 +15,10 @@ compiles the file to assembly and verifies, in the kernel's text, that
 
 Registers that the compiler also uses for short-lived temporaries while a slot is empty are
 recognised by being written by another instruction first.
+
+A second check (``check_asm_results``) covers what inline assembly costs besides: the compiler does
+not keep the hardware's wait states between an inline-assembly VALU result and an MFMA or DPP
+instruction that reads it.
 """
 from __future__ import annotations
 
@@ -72,6 +76,50 @@ def _check_function(body: list[str]) -> list[str]:
     return errors
 
 
+HAZARD_WINDOW = 3  # instructions: the hardware wants up to 2 wait states, one instruction may be a zero-cycle s_nop
+
+
+def check_asm_results(asm_text: str) -> list[str]:
+    """The compiler inserts the wait states between a VALU result and an MFMA or DPP instruction that reads it
+    only when it issued the VALU instruction itself: the text of an inline-assembly statement is opaque to its
+    hazard recognizer.  So no register written inside an ASMSTART / ASMEND block may be read by a v_mfma* or
+    *_dpp instruction within the next HAZARD_WINDOW instructions, unless an s_nop of the block itself follows
+    the write (loads are exempt: their results are waited for with s_waitcnt)."""
+    errors = []
+    recent = []  # (instructions ago, set of registers) written by inline assembly
+    in_asm = False
+    for raw in asm_text.splitlines():
+        t = raw.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        l = t.split(";")[0].strip()
+        if not l or l.startswith(".") or l.endswith(":"):
+            if l.endswith(":") and not l.startswith("."):
+                recent = []
+            continue
+        parts = l.replace(",", " ").split()
+        op, ops = parts[0], parts[1:]
+        if in_asm and op.startswith("s_nop"):
+            recent = []  # the statement brings its own wait states
+            continue
+        reads_all = set()
+        for tok in ops[1:] if ops else []:
+            reads_all |= _regs(tok)
+        if (op.startswith("v_mfma") or op.endswith("_dpp") or "_dpp " in l) and not in_asm:
+            for age, regs in recent:
+                hit = regs & (reads_all | (_regs(ops[0]) if op.endswith("_dpp") else set()))
+                if hit:
+                    errors.append(f"`{l}` reads v{sorted(hit)} written by inline assembly {age} instruction(s) before")
+        recent = [(a + 1, r) for a, r in recent if a + 1 < HAZARD_WINDOW]
+        if in_asm and ops and op.startswith("v_") and not op.startswith("v_cmp"):
+            recent.append((0, _regs(ops[0])))
+    return errors
+
+
 def check(asm_text: str) -> list[str]:
     """Checks every kernel of the file on its own (register names mean nothing across kernels)."""
     lines = [l.split(";")[0].strip() for l in asm_text.splitlines()]
@@ -102,9 +150,14 @@ def main(hipcc="/opt/rocm/bin/hipcc", flags=(), sources=SOURCES):
             out = os.path.join(td, "k.s")
             subprocess.check_call([hipcc, *flags, "-S", "--cuda-device-only", os.path.join(HERE, "csrc", name), "-o", out],
                                   stderr=subprocess.DEVNULL)
-            errs = check(open(out).read())
+            text = open(out).read()
+            errs = check(text)
+            hazards = check_asm_results(text)
         if errs:
             raise RuntimeError(f"{name}: the generated code touches in-flight ring registers:\n  " + "\n  ".join(errs[:20]))
+        if hazards:
+            raise RuntimeError(f"{name}: an inline-assembly result reaches an MFMA / DPP instruction without wait states:\n  "
+                               + "\n  ".join(hazards[:20]))
     return True
 
 
