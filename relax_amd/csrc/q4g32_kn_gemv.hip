@@ -147,8 +147,15 @@ __global__ __launch_bounds__(256) void q4g32_kn_finish_kernel(const float* __res
                                                               half_t* __restrict__ y, int rows, int N, int slices) {
   const int col = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
   if (col >= N) return;
-  float v = partial[(int64_t)m * N + col];
-  for (int s = 1; s < slices; ++s) v += partial[((int64_t)s * rows + m) * N + col];
+  // eight loads in flight at a time, added in slice order
+  float v = 0.0f;
+  for (int s0 = 0; s0 < slices; s0 += 8) {
+    float p[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p[j] = s0 + j < slices ? partial[((int64_t)(s0 + j) * rows + m) * N + col] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v += p[j];
+  }
   if (bias) v += (float)bias[col];
   half_t h = (half_t)v;
   if (residual) h = h + residual[(int64_t)m * N + col];
