@@ -566,6 +566,9 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       const half_t* residual = descs[lin].residual;
       const int yrows = (int)((grp >> 16) & 0xffu);
       const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[lin].y, 0, yrows * N * 2, kBufferFlags);
+      // the four outputs of a lane are adjacent in a row of y: one 8-byte store where the addresses allow it
+      // (a store instruction waits its turn behind the weight loads of the whole workgroup)
+      const bool wide = (N & 3) == 0 && (((uintptr_t)descs[lin].y | (uintptr_t)bias | (uintptr_t)residual) & 7) == 0;
       for (int lt0 = 0; lt0 < T; lt0 += csize) {
         const int ltend = min(T, lt0 + csize);
         for (int panel = 0; panel < P; ++panel) {
@@ -599,7 +602,19 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
 #pragma unroll
             for (int r = 0; r < R; ++r) {
               const int j = j16 + 16 * r;
-              if (j < yrows) {
+              if (j < yrows && wide) {
+                if (n0 < N) {
+                  float4_t v = sum[r];
+                  if (bias) {
+                    const half4_t bv = *reinterpret_cast<const half4_t*>(bias + n0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
+                  }
+                  half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                  if (residual) h = h + *reinterpret_cast<const half4_t*>(residual + (int64_t)j * N + n0);
+                  __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2_t, h), yr, (j * N + n0) * 2, 0, kDeviceScope);
+                }
+              } else if (j < yrows) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                   const int n = n0 + e;
@@ -625,7 +640,9 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       }
     }
     if (!use_sync) return;
-    // the last workgroup to get here clears the counters for the next launch
+    // the last workgroup to get here clears the counters for the next launch (its own counter updates
+    // have arrived by then: nothing of this launch may land on a cleared counter)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     int last = 0;
     if (lane == 0)
       last = __hip_atomic_fetch_add(sync + sync_finished_index(nlin), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==

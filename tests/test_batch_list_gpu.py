@@ -81,9 +81,12 @@ def test_every_nibble_position_carries_its_scale(env, oracle, M):
             assert np.array_equal(got, want.astype(np.float16).astype(np.float64)), (M, N, K, p, np.abs(got - want).max())
 
 
-def test_epilogue_and_one_hot(env, oracle):
+# N = 520 with aligned operands: the four outputs of a lane go out as one 8-byte store; N = 522 / 1001 or a bias that
+# starts 2 bytes past an 8-byte boundary: one 2-byte store per output
+@pytest.mark.parametrize("M,N,shift", [(6, 520, 0), (20, 520, 0), (6, 522, 0), (20, 1001, 0), (6, 520, 1), (32, 520, 1)])
+def test_epilogue_and_one_hot(env, oracle, M, N, shift):
     ops, u, torch = env
-    M, N, K = 6, 520, 1024
+    K = 1024
     x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=7)
     rng = np.random.default_rng(3)
     bias = rng.standard_normal(N).astype(np.float16)
@@ -91,11 +94,13 @@ def test_epilogue_and_one_hot(env, oracle):
     y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
     y2 = torch.zeros((M, N), dtype=torch.float16, device="cuda")
     xh = np.zeros((M, K), np.float16)
-    cols = [0, 37, 260, 511, 777, 1023]
+    cols = ([0, 37, 260, 511, 777, 1023] * 6)[:M]
     for m, c in enumerate(cols):
         xh[m, c] = 1
     dW, dS = u.dev(W), u.dev(S)
-    gl = ops.Q4G32GemvList([(dW, dS, u.dev(x), y, u.dev(bias), u.dev(res)), (dW, dS, u.dev(xh), y2)], M=M)
+    dbias = u.dev(np.concatenate([np.zeros(shift, np.float16), bias]))[shift:]
+    assert dbias.data_ptr() % 8 == 2 * shift
+    gl = ops.Q4G32GemvList([(dW, dS, u.dev(x), y, dbias, u.dev(res)), (dW, dS, u.dev(xh), y2)], M=M)
     gl.run()
     gl.status()
     u.assert_close(u.host(y), oracle.q4g32_linear(W, S, x, bias=bias, residual=res), "batch list epilogue")
