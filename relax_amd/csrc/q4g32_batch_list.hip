@@ -89,10 +89,15 @@ struct BatchWait {
   }
 };
 
-__host__ __device__ constexpr int batch_panel_groups(int U) { return kBW * 4 * U; }
-__host__ __device__ constexpr int batch_scale_row_bytes(int U) { return batch_panel_groups(U) * 2 + 16; }  // + 16: rows on different banks
-__host__ __device__ constexpr int batch_scale_slot_bytes(int U) { return 16 * batch_scale_row_bytes(U); }
-__host__ __device__ constexpr int batch_partial_slot_bytes(int R) { return kBW * R * 1024; }  // R sets of 16 activation rows
+// R = 1: a tile is 16 rows of W and the 8 compute wavefronts split the panel 8 ways along K.  R = 2 (more than 16
+// activation rows): a tile is 32 rows, wavefronts 0 .. 3 split the panel 4 ways for its rows 0 .. 15, wavefronts
+// 4 .. 7 for rows 16 .. 31, and every wavefront holds two sets of 16 activation rows.
+__host__ __device__ constexpr int batch_k_ways(int R) { return kBW / R; }
+__host__ __device__ constexpr int batch_panel_groups(int U, int R) { return batch_k_ways(R) * 4 * U; }
+__host__ __device__ constexpr int batch_scale_row_bytes(int U, int R) { return batch_panel_groups(U, R) * 2 + 16; }  // + 16: rows on different banks
+__host__ __device__ constexpr int batch_scale_slot_bytes(int U, int R) { return 16 * R * batch_scale_row_bytes(U, R); }
+__host__ __device__ constexpr int batch_partial_slot_bytes(int R) { return kBW * R * 1024; }  // per wavefront R sets of 16 activation rows
+__host__ __device__ constexpr int batch_kept_bytes(int R) { return R * R * 1024; }            // sums of a tile kept between panels
 
 // ---- the walk of a workgroup over its items.  All fields are wavefront-uniform.
 struct ItemCursor {
@@ -116,7 +121,7 @@ __device__ __forceinline__ uint32_t desc_group_word(gemv_desc_ptr descs, int lin
 }
 
 // positions the cursor on the first linear >= c.lin in which this workgroup holds a tile
-template <int U, bool CH>
+template <int PG, bool CH>
 __device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg, int chunk) {
   typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
   while (c.lin < nlin) {
@@ -137,7 +142,7 @@ __device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, in
         c.rb = rb;
         c.ncu = ncu;
         c.G = G;
-        c.P = (G + batch_panel_groups(U) - 1) / batch_panel_groups(U);
+        c.P = (G + PG - 1) / PG;
         c.N = (int)w[12];
         c.row_w = G << 4;
         c.W = reinterpret_cast<const char*>(((uint64_t)w[1] << 32) | w[0]);
@@ -161,7 +166,7 @@ __device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, in
   }
 }
 
-template <int U, bool CH>
+template <int PG, bool CH>
 __device__ __forceinline__ void item_next_panel(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg, int chunk) {
   if constexpr (CH) {
     if (++c.panel == c.P) {
@@ -169,7 +174,7 @@ __device__ __forceinline__ void item_next_panel(ItemCursor& c, gemv_desc_ptr des
       c.lt0 = c.ltend;
       if (c.lt0 >= c.T) {
         ++c.lin;
-        item_seek<U, CH>(c, descs, nlin, b, nwg, chunk);
+        item_seek<PG, CH>(c, descs, nlin, b, nwg, chunk);
         return;
       }
       c.ltend = min(c.T, c.lt0 + c.csize);
@@ -179,23 +184,24 @@ __device__ __forceinline__ void item_next_panel(ItemCursor& c, gemv_desc_ptr des
     c.lt = 0;
     if (++c.panel == c.P) {
       ++c.lin;
-      item_seek<U, CH>(c, descs, nlin, b, nwg, chunk);
+      item_seek<PG, CH>(c, descs, nlin, b, nwg, chunk);
     }
   }
 }
 
-template <int U, bool CH>
+template <int PG, bool CH>
 __device__ __forceinline__ void item_next(ItemCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg, int chunk) {
-  if (++c.lt == (CH ? c.ltend : c.T)) item_next_panel<U, CH>(c, descs, nlin, b, nwg, chunk);
+  if (++c.lt == (CH ? c.ltend : c.T)) item_next_panel<PG, CH>(c, descs, nlin, b, nwg, chunk);
 }
 
 template <int U, int R, bool CH>
 __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvListDesc* __restrict__ descs_, int nlin,
                                                                      int* __restrict__ sync, long long spin_limit,
                                                                      int M, int nxb, int ring, int chunk, int use_sync) {
-  constexpr int PG = batch_panel_groups(U);  // scale groups per panel
+  constexpr int PG = batch_panel_groups(U, R);  // scale groups per panel
+  constexpr int KW = batch_k_ways(R);          // wavefronts that share a panel along K
   constexpr int NT = kBNT;
-  constexpr int SROW = batch_scale_row_bytes(U), SSLOT = batch_scale_slot_bytes(U);
+  constexpr int SROW = batch_scale_row_bytes(U, R), SSLOT = batch_scale_slot_bytes(U, R);
   extern __shared__ uint4_t smem[];
   const gemv_desc_ptr descs = (gemv_desc_ptr)descs_;
   char* lds = reinterpret_cast<char*>(smem);
@@ -221,6 +227,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
   if (wave < kBW) {
     // =========================== compute wavefront ===========================
     const int i = lane & 15, kq = lane >> 4;
+    const int ks = wave & (KW - 1), rt = wave / KW;  // K slice of the panel; which 16 rows of the tile
     // The tile buffers are loaded in assembly and waited for by hand (loads retire in order and a
     // compute wavefront issues no other vector memory operation).  `magic` (0x6400 in both halves,
     // OR-ed under every code) doubles as the token that orders the reads of a buffer behind the wait
@@ -232,16 +239,16 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     int ahead = 0;  // items issued and not yet consumed
     ItemCursor ic, cc;
     ic.lin = 0;
-    item_seek<U, CH>(ic, descs, nlin, b, nwg, chunk);
+    item_seek<PG, CH>(ic, descs, nlin, b, nwg, chunk);
     cc = ic;
     int k = 0;    // items consumed
     int pk = -1;  // panels taken
     half8_t xb[R][U][4];
-    const int gi0 = wave * (4 * U) + kq;  // the lane's scale group within the panel, chunk 0
+    const int gi0 = ks * (4 * U) + kq;  // the lane's scale group within the panel, chunk 0
 
     auto issue = [&](uint4_t (&buf)[U]) {
       if (ic.lin >= nlin) return;
-      const int n0 = (ic.lt * ic.ncu + ic.rb) << 4;
+      const int n0 = min(((ic.lt * ic.ncu + ic.rb) * R + rt) << 4, ic.N - 1);  // (the second 16 rows of the last tile may lie past N)
       const int rows = min(16, ic.N - n0);                // >= 1
       const int pg = min(PG, ic.G - ic.panel * PG);       // scale groups of this panel (the last may be short)
       const char* base = ic.W + (int64_t)n0 * ic.row_w + ic.panel * (PG * 16);
@@ -254,7 +261,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         // 7.1 against 5.7 TB/s).  consume() puts the halves back where the MFMA wants them.
         const uint32_t roff_lo = __umul24((uint32_t)min(i & 7, rows - 1), (uint32_t)ic.row_w);
         const uint32_t roff_hi = __umul24((uint32_t)min(8 + (i & 7), rows - 1), (uint32_t)ic.row_w);
-        const int gpair = wave * (4 * U) + (i >> 3) * 4 + kq;
+        const int gpair = ks * (4 * U) + (i >> 3) * 4 + kq;
 #pragma unroll
         for (int u = 0; u < U; u += 2) {
           const uint32_t goff = (uint32_t)min(gpair + 4 * u, pg - 1) * 16u;
@@ -270,7 +277,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         }
       }
       ++ahead;
-      item_next<U, CH>(ic, descs, nlin, b, nwg, chunk);
+      item_next<PG, CH>(ic, descs, nlin, b, nwg, chunk);
     };
 
     const half2_t k1031 = {(half_t)-1031.0f, (half_t)-1031.0f};
@@ -294,7 +301,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         wait.until(&flags->x_ready[xslot], pk + 1, 1);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          const char* xs = xbuf + xslot * xbuf_bytes + (wave * U * 16 * M + kq * M + min(i + 16 * r, M - 1)) * 16;
+          const char* xs = xbuf + xslot * xbuf_bytes + (ks * U * 16 * M + kq * M + min(i + 16 * r, M - 1)) * 16;
 #pragma unroll
           for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -305,7 +312,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       }
       wait.until(&flags->s_ready, k + 1, 2);
       const int slot = k & (ring - 1);
-      const char* sb = sbuf + slot * SSLOT + i * SROW + gi0 * 2;
+      const char* sb = sbuf + slot * SSLOT + (rt * 16 + i) * SROW + gi0 * 2;
       float4_t acc0[R], acc1[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) acc0[r] = acc1[r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -373,7 +380,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       if (lane == 0) __hip_atomic_fetch_add(&flags->done[slot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       ++k;
-      item_next<U, CH>(cc, descs, nlin, b, nwg, chunk);
+      item_next<PG, CH>(cc, descs, nlin, b, nwg, chunk);
     };
 
 #pragma unroll
@@ -424,7 +431,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     constexpr int UX = 32;       // loads in flight per lane: one round trip for a panel of 8 rows x 2048 k
     ItemCursor xc;
     xc.lin = 0;
-    item_seek<U, CH>(xc, descs, nlin, b, nwg, chunk);
+    item_seek<PG, CH>(xc, descs, nlin, b, nwg, chunk);
     // the x wavefronts take whole panels by turns (panel pk belongs to wavefront pk mod kBXW) and run up
     // to nxb panels ahead of the compute wavefronts: under load a round trip to L2 takes several microseconds
     int pk = 0;
@@ -483,7 +490,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         if (lane == 0) __hip_atomic_store(&flags->x_ready[xslot], pk + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
       ++pk;
-      item_next_panel<U, CH>(xc, descs, nlin, b, nwg, chunk);
+      item_next_panel<PG, CH>(xc, descs, nlin, b, nwg, chunk);
     }
     return;
   }
@@ -492,16 +499,16 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     // ====================== scale wavefront: the scales of a tile -> LDS ======================
     constexpr int PD = 6;            // items in flight in registers (a round trip under load is several items long)
     constexpr int PPR = PG / 8;      // 16-byte pieces (8 scales) per row and panel
-    constexpr int LP = 16 * PPR / 64;  // pieces per lane and item
+    constexpr int LP = 16 * R * PPR / 64;  // pieces per lane and item
     uint4_t sv[PD][LP];
     ItemCursor ic, cc;
     ic.lin = 0;
-    item_seek<U, CH>(ic, descs, nlin, b, nwg, chunk);
+    item_seek<PG, CH>(ic, descs, nlin, b, nwg, chunk);
     cc = ic;
     int k = 0;
     auto issue = [&](uint4_t (&buf)[LP]) {
       if (ic.lin >= nlin) return;
-      const int n0 = (ic.lt * ic.ncu + ic.rb) << 4;
+      const int n0 = (ic.lt * ic.ncu + ic.rb) * (16 * R);
       const int pg = min(PG, ic.G - ic.panel * PG);
       const char* base = ic.S + ic.panel * (PG * 2);
 #pragma unroll
@@ -513,7 +520,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
           buf[t] = __builtin_nontemporal_load(
               reinterpret_cast<const uint4_t*>(base + (int64_t)min(n0 + r, ic.N - 1) * (ic.G * 2) + pc * 16));
       }
-      item_next<U, CH>(ic, descs, nlin, b, nwg, chunk);
+      item_next<PG, CH>(ic, descs, nlin, b, nwg, chunk);
     };
     auto consume = [&](uint4_t (&buf)[LP]) {
       const int slot = k & (ring - 1);
@@ -528,7 +535,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       ++k;
       if (lane == 0) __hip_atomic_store(&flags->s_ready, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      item_next<U, CH>(cc, descs, nlin, b, nwg, chunk);
+      item_next<PG, CH>(cc, descs, nlin, b, nwg, chunk);
     };
 #pragma unroll
     for (int t = 0; t < PD - 1; ++t) issue(sv[t]);
@@ -575,56 +582,66 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
           for (int lt = lt0; lt < ltend; ++lt, ++k) {
             const int slot = k & (ring - 1);
             wait.until(&flags->done[slot], kBW * (k / ring + 1), 6);
+            // sum[t][r]: rows 16 t .. of the tile, activation rows 16 r ..; the K slices in a fixed order
             const char* pb = pbuf + slot * batch_partial_slot_bytes(R) + lane * 16;
-            float4_t sum[R];
+            float4_t sum[R][R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-              sum[r] = *reinterpret_cast<const float4_t*>(pb + r * 1024);
+            for (int t = 0; t < R; ++t)
 #pragma unroll
-              for (int w = 1; w < kBW; ++w) sum[r] += *reinterpret_cast<const float4_t*>(pb + (w * R + r) * 1024);
-            }
+              for (int r = 0; r < R; ++r) {
+                sum[t][r] = *reinterpret_cast<const float4_t*>(pb + ((t * KW) * R + r) * 1024);
+#pragma unroll
+                for (int w = 1; w < KW; ++w) sum[t][r] += *reinterpret_cast<const float4_t*>(pb + ((t * KW + w) * R + r) * 1024);
+              }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             if (lane == 0) __hip_atomic_store(&flags->y_done, k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (P > 1) {
-              float4_t* keep = reinterpret_cast<float4_t*>(abuf + (lt - lt0) * (R * 1024) + lane * 16);
+              float4_t* keep = reinterpret_cast<float4_t*>(abuf + (lt - lt0) * batch_kept_bytes(R) + lane * 16);
               if (panel > 0) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) sum[r] += keep[r * 64];
+                for (int t = 0; t < R; ++t)
+#pragma unroll
+                  for (int r = 0; r < R; ++r) sum[t][r] += keep[(t * R + r) * 64];
               }
               if (panel < P - 1) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) keep[r * 64] = sum[r];
+                for (int t = 0; t < R; ++t)
+#pragma unroll
+                  for (int r = 0; r < R; ++r) keep[(t * R + r) * 64] = sum[t][r];
                 continue;
               }
             }
-            // lane (j, rq) holds rows n0 + 4 rq .. + 3 of activation rows j, j + 16, ..
-            const int n0 = ((lt * ncu + rb) << 4) + 4 * rq;
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-              const int j = j16 + 16 * r;
-              if (j < yrows && wide) {
-                if (n0 < N) {
-                  float4_t v = sum[r];
-                  if (bias) {
-                    const half4_t bv = *reinterpret_cast<const half4_t*>(bias + n0);
+            for (int t = 0; t < R; ++t) {
+              // lane (j, rq) holds rows n0 + 4 rq .. + 3 of activation rows j, j + 16
+              const int n0 = (((lt * ncu + rb) * R + t) << 4) + 4 * rq;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
-                  }
-                  half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                  if (residual) h = h + *reinterpret_cast<const half4_t*>(residual + (int64_t)j * N + n0);
-                  __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2_t, h), yr, (j * N + n0) * 2, 0, kDeviceScope);
-                }
-              } else if (j < yrows) {
+              for (int r = 0; r < R; ++r) {
+                const int j = j16 + 16 * r;
+                if (j < yrows && wide) {
+                  if (n0 < N) {
+                    float4_t v = sum[t][r];
+                    if (bias) {
+                      const half4_t bv = *reinterpret_cast<const half4_t*>(bias + n0);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                  const int n = n0 + e;
-                  if (n < N) {
-                    float v = sum[r][e];
-                    if (bias) v += (float)bias[n];
-                    half_t h = (half_t)v;
-                    if (residual) h = h + residual[(int64_t)j * N + n];
+                      for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
+                    }
+                    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                    if (residual) h = h + *reinterpret_cast<const half4_t*>(residual + (int64_t)j * N + n0);
                     // device-scope store: written through, so that a counter update after it publishes it
-                    __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (j * N + n) * 2, 0, kDeviceScope);
+                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2_t, h), yr, (j * N + n0) * 2, 0, kDeviceScope);
+                  }
+                } else if (j < yrows) {
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) {
+                    const int n = n0 + e;
+                    if (n < N) {
+                      float v = sum[t][r][e];
+                      if (bias) v += (float)bias[n];
+                      half_t h = (half_t)v;
+                      if (residual) h = h + residual[(int64_t)j * N + n];
+                      __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (j * N + n) * 2, 0, kDeviceScope);
+                    }
                   }
                 }
               }
@@ -658,8 +675,8 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
 
 // ------------------------------------------------------------------ host side
 static size_t batch_lds_bytes(int U, int R, int M, int nxb, int ring, int acc_tiles) {
-  return sizeof(BatchFlags) + (size_t)nxb * M * batch_panel_groups(U) * 64 + (size_t)ring * batch_scale_slot_bytes(U) +
-         (size_t)ring * batch_partial_slot_bytes(R) + (size_t)acc_tiles * R * 1024;
+  return sizeof(BatchFlags) + (size_t)nxb * M * batch_panel_groups(U, R) * 64 + (size_t)ring * batch_scale_slot_bytes(U, R) +
+         (size_t)ring * batch_partial_slot_bytes(R) + (size_t)acc_tiles * batch_kept_bytes(R);
 }
 
 // Which group of workgroups runs which linear.  Every workgroup needs all M x K activations of a linear
@@ -679,7 +696,7 @@ struct BatchGroupPlan {
 // chunks a workgroup with `tiles` tiles of a linear walks them in (each chunk loads every panel of activations again)
 static int batch_chunks(int tiles, int panels, int chunk) { return panels > 1 && tiles > chunk ? (tiles + chunk - 1) / chunk : 1; }
 
-static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, int chunk) {
+static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, int R, int chunk) {
   const int groups = 1 << gl, ncu = l->blocks >> gl;
   BatchGroupPlan plan;
   plan.group.resize(l->n);
@@ -688,10 +705,11 @@ static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, 
     const GemvListDesc& g = l->descs[i];
     const int G = (int)(g.g_dep & 0xffffu);
     const double K = (double)G * 32.0;
-    const double tiles = (double)((((int64_t)g.N + 15) / 16 + ncu - 1) / ncu);  // of one workgroup
-    const int panels = (G + batch_panel_groups(U) - 1) / batch_panel_groups(U);
+    const int trows = 16 * R;
+    const double tiles = (double)((((int64_t)g.N + trows - 1) / trows + ncu - 1) / ncu);  // of one workgroup
+    const int panels = (G + batch_panel_groups(U, R) - 1) / batch_panel_groups(U, R);
     // bytes through one workgroup: its tiles' codes and scales, and all activations once per chunk
-    const double dur = tiles * 16.0 * K * (0.5 + 1.0 / 16.0) + batch_chunks((int)tiles, panels, chunk) * l->M * K * 2.0 + 4096.0;
+    const double dur = tiles * trows * K * (0.5 + 1.0 / 16.0) + batch_chunks((int)tiles, panels, chunk) * l->M * K * 2.0 + 4096.0;
     const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
     const double ready = dep >= 0 ? end[dep] : 0.0;
     int best = 0;
@@ -709,16 +727,18 @@ static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, 
 
 // the kernel that walks the tiles of a linear in chunks carries more loop state: only where a list needs it
 typedef void (*batch_kernel_t)(const GemvListDesc*, int, int*, long long, int, int, int, int, int);
-static batch_kernel_t batch_kernel(int U, bool chunked) {
+static int batch_rows_sets(int M) { return M <= 16 ? 1 : 2; }
+static batch_kernel_t batch_kernel(int U, int R, bool chunked) {
+  if (R == 2) return chunked ? q4g32_batch_list_kernel<2, 2, true> : q4g32_batch_list_kernel<2, 2, false>;
   if (U == 4) return chunked ? q4g32_batch_list_kernel<4, 1, true> : q4g32_batch_list_kernel<4, 1, false>;
-  if (U == 2) return chunked ? q4g32_batch_list_kernel<2, 1, true> : q4g32_batch_list_kernel<2, 1, false>;
-  return chunked ? q4g32_batch_list_kernel<1, 2, true> : q4g32_batch_list_kernel<1, 2, false>;
+  return chunked ? q4g32_batch_list_kernel<2, 1, true> : q4g32_batch_list_kernel<2, 1, false>;
 }
 
 int batch_list_plan(wq_gemv_list* l) {
   // panels of 4096 k (M <= 8), 2048 k (M <= 16) or 1024 k (two sets of 16 rows): 64 KiB of activations at most
-  const int U = l->M <= 8 ? 4 : l->M <= 16 ? 2 : 1;
-  const int R = l->M <= 16 ? 1 : 2;
+  const int U = l->M <= 8 ? 4 : 2;
+  const int R = batch_rows_sets(l->M);
+  const int trows = 16 * R;
   l->batch_u = U;
   l->gs = 4;
   l->threads = kBThreads;
@@ -734,16 +754,16 @@ int batch_list_plan(wq_gemv_list* l) {
     int acc_tiles = 0;  // most tiles a workgroup holds of a linear that spans several panels
     for (int i = 0; i < l->n; ++i) {
       const GemvListDesc& g = l->descs[i];
-      const int64_t tiles = ((int64_t)g.N + 15) >> 4;
-      if ((int)(g.g_dep & 0xffffu) > batch_panel_groups(U)) acc_tiles = std::max<int>(acc_tiles, (int)((tiles + ncu - 1) / ncu));
+      const int64_t tiles = ((int64_t)g.N + trows - 1) / trows;
+      if ((int)(g.g_dep & 0xffffu) > batch_panel_groups(U, R)) acc_tiles = std::max<int>(acc_tiles, (int)((tiles + ncu - 1) / ncu));
     }
     // the sums kept between panels must fit beside one panel of activations and a ring of 2: else the tiles of
     // a linear are walked in chunks of what fits, at the price of loading the activations once per chunk
     const size_t base = batch_lds_bytes(U, R, l->M, 1, 2, 0);
-    if (base + 4 * R * 1024 > budget) continue;
-    const int fit = (int)((budget - base) / ((size_t)R * 1024));
+    if (base + 4 * batch_kept_bytes(R) > budget) continue;
+    const int fit = (int)((budget - base) / (size_t)batch_kept_bytes(R));
     const int chunk = std::min(acc_tiles, fit);
-    BatchGroupPlan p = batch_assign_groups(l, gl, U, std::max(chunk, 1));
+    BatchGroupPlan p = batch_assign_groups(l, gl, U, R, std::max(chunk, 1));
     if (best_gl < 0 || p.makespan < best.makespan * 0.98) {
       best_gl = gl;
       best = std::move(p);
@@ -758,7 +778,7 @@ int batch_list_plan(wq_gemv_list* l) {
   for (int i = 0; i < l->n; ++i) {
     GemvListDesc& g = l->descs[i];
     const int c = best.group[i];
-    const int64_t tiles = ((int64_t)g.N + 15) >> 4;
+    const int64_t tiles = ((int64_t)g.N + trows - 1) / trows;
     g.q = (int32_t)(tiles / ncu);
     g.rem = (uint16_t)(tiles % ncu);
     g.off = (uint16_t)off[c];
@@ -777,10 +797,10 @@ int batch_list_plan(wq_gemv_list* l) {
     l->batch_nxb = batch_lds_bytes(U, R, l->M, 2, 2, best_acc) <= budget ? 2 : 1;
   }
   l->lds = batch_lds_bytes(U, R, l->M, l->batch_nxb, l->batch_ring, best_acc);
-  const void* kern = reinterpret_cast<const void*>(batch_kernel(U, best_chunked));
+  const void* kern = reinterpret_cast<const void*>(batch_kernel(U, R, best_chunked));
   // several lists share a kernel: the limit only ever grows
   static DynamicLdsLimit limits[3][2];
-  if (limits[U == 4 ? 0 : U == 2 ? 1 : 2][best_chunked ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
+  if (limits[R == 2 ? 2 : U == 4 ? 0 : 1][best_chunked ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
     return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
@@ -792,7 +812,7 @@ int batch_list_launch(wq_gemv_list* l, hipStream_t stream) {
   const GemvListDesc* table = (const GemvListDesc*)l->table;
   const int use_sync = l->deps > 0 ? 1 : 0;
   // chunk: at least 1 (a list without a linear of several panels keeps no sums)
-  WQ_LAUNCH("wq_q4g32_gemv_list_run", batch_kernel(l->batch_u, l->batch_chunked), dim3((unsigned)l->blocks), dim3((unsigned)l->threads), l->lds,
+  WQ_LAUNCH("wq_q4g32_gemv_list_run", batch_kernel(l->batch_u, batch_rows_sets(l->M), l->batch_chunked), dim3((unsigned)l->blocks), dim3((unsigned)l->threads), l->lds,
             stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, std::max(l->batch_acc_tiles, 1),
             use_sync);
   return WQ_OK;
