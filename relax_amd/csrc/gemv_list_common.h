@@ -77,7 +77,7 @@ struct wq_gemv_list {
   int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
   long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
   int M = 1;               // activation rows of the launch; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
-  int batch_u = 0;         // chunks per tile and wavefront (4: panels of 4096 k, M <= 8; 2: 2048 k, M <= 16; 1: 1024 k)
+  int batch_u = 0;         // chunks per tile and wavefront (4: M <= 16; 2: beyond)
   int batch_groups = 1;    // groups of workgroups that run different linears side by side
   int batch_nxb = 0;       // panels of activations in LDS
   int batch_ring = 0;      // items the compute wavefronts may spread over (slots of scales and of partial sums)

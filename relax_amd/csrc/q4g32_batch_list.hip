@@ -5,11 +5,13 @@
 // the matrix cores so that all M rows share one pass over the weights, and the weights go from
 // memory straight into the registers that feed them.
 //
-// Work.  The unit is a TILE of 16 consecutive rows of W times a PANEL of K (4096 k for M <= 8, 2048 k
-// for M <= 16, 1024 k beyond: a panel of activations is at most 64 KiB).  A linear is run by one GROUP of
+// Work.  The unit is a TILE of rows of W times a PANEL of K: 16 rows x 4096 k for M <= 8, 32 rows x 2048 k for
+// M <= 16, 32 rows x 1024 k beyond (a panel of activations is at most 64 KiB; an item is 32, 32 or 16 KiB of codes:
+// what a workgroup spends per item on hand-overs does not depend on its size).  A linear is run by one GROUP of
 // workgroups (see batch_assign_groups), its tiles dealt to them round-robin, with a rotation that continues
-// from linear to linear.  Inside a workgroup the 8 compute wavefronts split a panel along K: wavefront w
-// owns the 4 U scale groups w * 4U .. of every panel (U = 4, 2 or 1), i.e. U chunks per tile; a chunk is
+// from linear to linear.  Inside a workgroup the 8 compute wavefronts split a tile: 16 rows x an eighth of the
+// panel each, or, with tiles of 32 rows, wavefronts 0 .. 3 a quarter of the panel of rows 0 .. 15 each and
+// wavefronts 4 .. 7 of rows 16 .. 31.  A wavefront's share is U chunks (U = 4 or 2); a chunk is
 // one 16-byte load per lane: lane (i, kq) takes scale group 4u + kq of row i, the 32 codes that the four
 // v_mfma_f32_16x16x32_f16 of the chunk consume as A operands (one dword, 8 codes, each).  With more than
 // 16 activation rows every unpacked A operand feeds R = 2 MFMAs, one per set of 16 rows.
@@ -25,10 +27,10 @@
 //     which frees the buffer at once, so even one buffer keeps the next panel ready in time.  The two take
 //     whole panels by turns: while one waits for a producer the other already fetches the panel after it
 //     (sharing every panel between them instead was slower at every M).
-//   * the scale wavefront streams the tile's scales (16 rows x 256 contiguous bytes: fetched per
+//   * the scale wavefront streams the tile's scales (per row up to 256 contiguous bytes: fetched per
 //     lane they cost more than the codes) into a ring of LDS slots, a few tiles ahead.
-//   * the y wavefront adds the 8 partial sums of a tile in a fixed order, keeps the sum in LDS while
-//     further panels of the same rows follow, and at the last panel applies bias / cast / residual,
+//   * the y wavefront adds the 8 partial sums of a tile (4 per 16 rows of a 32-row tile) in a fixed order, keeps the
+//     sum in LDS while further panels of the same rows follow, and at the last panel applies bias / cast / residual,
 //     stores y with device-scope stores and signals the linear's completion counter.
 // A linear of several panels whose kept sums would not fit the LDS is walked in CHUNKS of its tiles (all
 // panels of a chunk, then the next chunk; template parameter CH): the activations are then loaded once
@@ -89,15 +91,16 @@ struct BatchWait {
   }
 };
 
-// R = 1: a tile is 16 rows of W and the 8 compute wavefronts split the panel 8 ways along K.  R = 2 (more than 16
-// activation rows): a tile is 32 rows, wavefronts 0 .. 3 split the panel 4 ways for its rows 0 .. 15, wavefronts
-// 4 .. 7 for rows 16 .. 31, and every wavefront holds two sets of 16 activation rows.
-__host__ __device__ constexpr int batch_k_ways(int R) { return kBW / R; }
-__host__ __device__ constexpr int batch_panel_groups(int U, int R) { return batch_k_ways(R) * 4 * U; }
-__host__ __device__ constexpr int batch_scale_row_bytes(int U, int R) { return batch_panel_groups(U, R) * 2 + 16; }  // + 16: rows on different banks
-__host__ __device__ constexpr int batch_scale_slot_bytes(int U, int R) { return 16 * R * batch_scale_row_bytes(U, R); }
+// TW = 1: a tile is 16 rows of W and the 8 compute wavefronts split the panel 8 ways along K.  TW = 2: a tile is
+// 32 rows, wavefronts 0 .. 3 split the panel 4 ways for its rows 0 .. 15, wavefronts 4 .. 7 for rows 16 .. 31 (half
+// as many hand-overs per byte of weights, twice the activations in a wavefront's registers).
+// R: sets of 16 activation rows every wavefront holds.
+__host__ __device__ constexpr int batch_k_ways(int TW) { return kBW / TW; }
+__host__ __device__ constexpr int batch_panel_groups(int U, int TW) { return batch_k_ways(TW) * 4 * U; }
+__host__ __device__ constexpr int batch_scale_row_bytes(int U, int TW) { return batch_panel_groups(U, TW) * 2 + 16; }  // + 16: rows on different banks
+__host__ __device__ constexpr int batch_scale_slot_bytes(int U, int TW) { return 16 * TW * batch_scale_row_bytes(U, TW); }
 __host__ __device__ constexpr int batch_partial_slot_bytes(int R) { return kBW * R * 1024; }  // per wavefront R sets of 16 activation rows
-__host__ __device__ constexpr int batch_kept_bytes(int R) { return R * R * 1024; }            // sums of a tile kept between panels
+__host__ __device__ constexpr int batch_kept_bytes(int R, int TW) { return TW * R * 1024; }   // sums of a tile kept between panels
 
 // ---- the walk of a workgroup over its items.  All fields are wavefront-uniform.
 struct ItemCursor {
@@ -194,14 +197,14 @@ __device__ __forceinline__ void item_next(ItemCursor& c, gemv_desc_ptr descs, in
   if (++c.lt == (CH ? c.ltend : c.T)) item_next_panel<PG, CH>(c, descs, nlin, b, nwg, chunk);
 }
 
-template <int U, int R, bool CH>
+template <int U, int R, int TW, bool CH>
 __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvListDesc* __restrict__ descs_, int nlin,
                                                                      int* __restrict__ sync, long long spin_limit,
                                                                      int M, int nxb, int ring, int chunk, int use_sync) {
-  constexpr int PG = batch_panel_groups(U, R);  // scale groups per panel
-  constexpr int KW = batch_k_ways(R);          // wavefronts that share a panel along K
+  constexpr int PG = batch_panel_groups(U, TW);  // scale groups per panel
+  constexpr int KW = batch_k_ways(TW);          // wavefronts that share a panel along K
   constexpr int NT = kBNT;
-  constexpr int SROW = batch_scale_row_bytes(U, R), SSLOT = batch_scale_slot_bytes(U, R);
+  constexpr int SROW = batch_scale_row_bytes(U, TW), SSLOT = batch_scale_slot_bytes(U, TW);
   extern __shared__ uint4_t smem[];
   const gemv_desc_ptr descs = (gemv_desc_ptr)descs_;
   char* lds = reinterpret_cast<char*>(smem);
@@ -248,7 +251,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
 
     auto issue = [&](uint4_t (&buf)[U]) {
       if (ic.lin >= nlin) return;
-      const int n0 = min(((ic.lt * ic.ncu + ic.rb) * R + rt) << 4, ic.N - 1);  // (the second 16 rows of the last tile may lie past N)
+      const int n0 = min(((ic.lt * ic.ncu + ic.rb) * TW + rt) << 4, ic.N - 1);  // (the second 16 rows of the last tile may lie past N)
       const int rows = min(16, ic.N - n0);                // >= 1
       const int pg = min(PG, ic.G - ic.panel * PG);       // scale groups of this panel (the last may be short)
       const char* base = ic.W + (int64_t)n0 * ic.row_w + ic.panel * (PG * 16);
@@ -499,7 +502,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     // ====================== scale wavefront: the scales of a tile -> LDS ======================
     constexpr int PD = 6;            // items in flight in registers (a round trip under load is several items long)
     constexpr int PPR = PG / 8;      // 16-byte pieces (8 scales) per row and panel
-    constexpr int LP = 16 * R * PPR / 64;  // pieces per lane and item
+    constexpr int LP = 16 * TW * PPR / 64;  // pieces per lane and item
     uint4_t sv[PD][LP];
     ItemCursor ic, cc;
     ic.lin = 0;
@@ -508,7 +511,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     int k = 0;
     auto issue = [&](uint4_t (&buf)[LP]) {
       if (ic.lin >= nlin) return;
-      const int n0 = (ic.lt * ic.ncu + ic.rb) * (16 * R);
+      const int n0 = (ic.lt * ic.ncu + ic.rb) * (16 * TW);
       const int pg = min(PG, ic.G - ic.panel * PG);
       const char* base = ic.S + ic.panel * (PG * 2);
 #pragma unroll
@@ -584,9 +587,9 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
             wait.until(&flags->done[slot], kBW * (k / ring + 1), 6);
             // sum[t][r]: rows 16 t .. of the tile, activation rows 16 r ..; the K slices in a fixed order
             const char* pb = pbuf + slot * batch_partial_slot_bytes(R) + lane * 16;
-            float4_t sum[R][R];
+            float4_t sum[TW][R];
 #pragma unroll
-            for (int t = 0; t < R; ++t)
+            for (int t = 0; t < TW; ++t)
 #pragma unroll
               for (int r = 0; r < R; ++r) {
                 sum[t][r] = *reinterpret_cast<const float4_t*>(pb + ((t * KW) * R + r) * 1024);
@@ -596,25 +599,25 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             if (lane == 0) __hip_atomic_store(&flags->y_done, k + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (P > 1) {
-              float4_t* keep = reinterpret_cast<float4_t*>(abuf + (lt - lt0) * batch_kept_bytes(R) + lane * 16);
+              float4_t* keep = reinterpret_cast<float4_t*>(abuf + (lt - lt0) * batch_kept_bytes(R, TW) + lane * 16);
               if (panel > 0) {
 #pragma unroll
-                for (int t = 0; t < R; ++t)
+                for (int t = 0; t < TW; ++t)
 #pragma unroll
                   for (int r = 0; r < R; ++r) sum[t][r] += keep[(t * R + r) * 64];
               }
               if (panel < P - 1) {
 #pragma unroll
-                for (int t = 0; t < R; ++t)
+                for (int t = 0; t < TW; ++t)
 #pragma unroll
                   for (int r = 0; r < R; ++r) keep[(t * R + r) * 64] = sum[t][r];
                 continue;
               }
             }
 #pragma unroll
-            for (int t = 0; t < R; ++t) {
+            for (int t = 0; t < TW; ++t) {
               // lane (j, rq) holds rows n0 + 4 rq .. + 3 of activation rows j, j + 16
-              const int n0 = (((lt * ncu + rb) * R + t) << 4) + 4 * rq;
+              const int n0 = (((lt * ncu + rb) * TW + t) << 4) + 4 * rq;
 #pragma unroll
               for (int r = 0; r < R; ++r) {
                 const int j = j16 + 16 * r;
@@ -674,9 +677,19 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
 }
 
 // ------------------------------------------------------------------ host side
-static size_t batch_lds_bytes(int U, int R, int M, int nxb, int ring, int acc_tiles) {
-  return sizeof(BatchFlags) + (size_t)nxb * M * batch_panel_groups(U, R) * 64 + (size_t)ring * batch_scale_slot_bytes(U, R) +
-         (size_t)ring * batch_partial_slot_bytes(R) + (size_t)acc_tiles * batch_kept_bytes(R);
+// the kernel a list of M activation rows runs: chunks per wavefront and tile, sets of 16 activation rows, tile rows / 16
+struct BatchShape {
+  int U, R, TW;
+};
+static BatchShape batch_shape(int M) {
+  if (M <= 8) return {4, 1, 1};   // tiles of 16 rows, panels of 4096 k (tiles of 32 rows x 2048 k: the same time at M = 8, slower at M = 4)
+  if (M <= 16) return {4, 1, 2};  // 32 rows, 2048 k (16 rows x 2048 k, chunks of 2: 0.90 instead of 0.81 ms for the Llama-2-7B stack)
+  return {2, 2, 2};               // 32 rows, 1024 k: a panel of activations is 64 KiB at most (16 rows x 1024 k: 1.36 instead of 1.11 ms)
+}
+
+static size_t batch_lds_bytes(BatchShape s, int M, int nxb, int ring, int acc_tiles) {
+  return sizeof(BatchFlags) + (size_t)nxb * M * batch_panel_groups(s.U, s.TW) * 64 + (size_t)ring * batch_scale_slot_bytes(s.U, s.TW) +
+         (size_t)ring * batch_partial_slot_bytes(s.R) + (size_t)acc_tiles * batch_kept_bytes(s.R, s.TW);
 }
 
 // Which group of workgroups runs which linear.  Every workgroup needs all M x K activations of a linear
@@ -696,7 +709,7 @@ struct BatchGroupPlan {
 // chunks a workgroup with `tiles` tiles of a linear walks them in (each chunk loads every panel of activations again)
 static int batch_chunks(int tiles, int panels, int chunk) { return panels > 1 && tiles > chunk ? (tiles + chunk - 1) / chunk : 1; }
 
-static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, int R, int chunk) {
+static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, BatchShape s, int chunk) {
   const int groups = 1 << gl, ncu = l->blocks >> gl;
   BatchGroupPlan plan;
   plan.group.resize(l->n);
@@ -705,9 +718,9 @@ static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, 
     const GemvListDesc& g = l->descs[i];
     const int G = (int)(g.g_dep & 0xffffu);
     const double K = (double)G * 32.0;
-    const int trows = 16 * R;
+    const int trows = 16 * s.TW;
     const double tiles = (double)((((int64_t)g.N + trows - 1) / trows + ncu - 1) / ncu);  // of one workgroup
-    const int panels = (G + batch_panel_groups(U, R) - 1) / batch_panel_groups(U, R);
+    const int panels = (G + batch_panel_groups(s.U, s.TW) - 1) / batch_panel_groups(s.U, s.TW);
     // bytes through one workgroup: its tiles' codes and scales, and all activations once per chunk
     const double dur = tiles * trows * K * (0.5 + 1.0 / 16.0) + batch_chunks((int)tiles, panels, chunk) * l->M * K * 2.0 + 4096.0;
     const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
@@ -727,18 +740,19 @@ static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, int U, 
 
 // the kernel that walks the tiles of a linear in chunks carries more loop state: only where a list needs it
 typedef void (*batch_kernel_t)(const GemvListDesc*, int, int*, long long, int, int, int, int, int);
-static int batch_rows_sets(int M) { return M <= 16 ? 1 : 2; }
-static batch_kernel_t batch_kernel(int U, int R, bool chunked) {
-  if (R == 2) return chunked ? q4g32_batch_list_kernel<2, 2, true> : q4g32_batch_list_kernel<2, 2, false>;
-  if (U == 4) return chunked ? q4g32_batch_list_kernel<4, 1, true> : q4g32_batch_list_kernel<4, 1, false>;
-  return chunked ? q4g32_batch_list_kernel<2, 1, true> : q4g32_batch_list_kernel<2, 1, false>;
+static int batch_kernel_index(BatchShape s) { return s.R == 2 ? 2 : s.TW == 2 ? 1 : 0; }
+static batch_kernel_t batch_kernel(BatchShape s, bool chunked) {
+  switch (batch_kernel_index(s)) {
+    case 2: return chunked ? q4g32_batch_list_kernel<2, 2, 2, true> : q4g32_batch_list_kernel<2, 2, 2, false>;
+    case 1: return chunked ? q4g32_batch_list_kernel<4, 1, 2, true> : q4g32_batch_list_kernel<4, 1, 2, false>;
+    default: return chunked ? q4g32_batch_list_kernel<4, 1, 1, true> : q4g32_batch_list_kernel<4, 1, 1, false>;
+  }
 }
 
 int batch_list_plan(wq_gemv_list* l) {
-  // panels of 4096 k (M <= 8), 2048 k (M <= 16) or 1024 k (two sets of 16 rows): 64 KiB of activations at most
-  const int U = l->M <= 8 ? 4 : 2;
-  const int R = batch_rows_sets(l->M);
-  const int trows = 16 * R;
+  const BatchShape s = batch_shape(l->M);
+  const int U = s.U;
+  const int trows = 16 * s.TW;
   l->batch_u = U;
   l->gs = 4;
   l->threads = kBThreads;
@@ -755,15 +769,15 @@ int batch_list_plan(wq_gemv_list* l) {
     for (int i = 0; i < l->n; ++i) {
       const GemvListDesc& g = l->descs[i];
       const int64_t tiles = ((int64_t)g.N + trows - 1) / trows;
-      if ((int)(g.g_dep & 0xffffu) > batch_panel_groups(U, R)) acc_tiles = std::max<int>(acc_tiles, (int)((tiles + ncu - 1) / ncu));
+      if ((int)(g.g_dep & 0xffffu) > batch_panel_groups(s.U, s.TW)) acc_tiles = std::max<int>(acc_tiles, (int)((tiles + ncu - 1) / ncu));
     }
     // the sums kept between panels must fit beside one panel of activations and a ring of 2: else the tiles of
     // a linear are walked in chunks of what fits, at the price of loading the activations once per chunk
-    const size_t base = batch_lds_bytes(U, R, l->M, 1, 2, 0);
-    if (base + 4 * batch_kept_bytes(R) > budget) continue;
-    const int fit = (int)((budget - base) / (size_t)batch_kept_bytes(R));
+    const size_t base = batch_lds_bytes(s, l->M, 1, 2, 0);
+    if (base + 4 * batch_kept_bytes(s.R, s.TW) > budget) continue;
+    const int fit = (int)((budget - base) / (size_t)batch_kept_bytes(s.R, s.TW));
     const int chunk = std::min(acc_tiles, fit);
-    BatchGroupPlan p = batch_assign_groups(l, gl, U, R, std::max(chunk, 1));
+    BatchGroupPlan p = batch_assign_groups(l, gl, s, std::max(chunk, 1));
     if (best_gl < 0 || p.makespan < best.makespan * 0.98) {
       best_gl = gl;
       best = std::move(p);
@@ -791,16 +805,16 @@ int batch_list_plan(wq_gemv_list* l) {
   l->batch_chunked = best_chunked;
   // a ring of 4 items and up to 2 panels of activations in LDS if they fit, else a ring of 2
   l->batch_ring = 4;
-  l->batch_nxb = batch_lds_bytes(U, R, l->M, 2, 4, best_acc) <= budget ? 2 : batch_lds_bytes(U, R, l->M, 1, 4, best_acc) <= budget ? 1 : 0;
+  l->batch_nxb = batch_lds_bytes(s, l->M, 2, 4, best_acc) <= budget ? 2 : batch_lds_bytes(s, l->M, 1, 4, best_acc) <= budget ? 1 : 0;
   if (!l->batch_nxb) {
     l->batch_ring = 2;
-    l->batch_nxb = batch_lds_bytes(U, R, l->M, 2, 2, best_acc) <= budget ? 2 : 1;
+    l->batch_nxb = batch_lds_bytes(s, l->M, 2, 2, best_acc) <= budget ? 2 : 1;
   }
-  l->lds = batch_lds_bytes(U, R, l->M, l->batch_nxb, l->batch_ring, best_acc);
-  const void* kern = reinterpret_cast<const void*>(batch_kernel(U, R, best_chunked));
+  l->lds = batch_lds_bytes(s, l->M, l->batch_nxb, l->batch_ring, best_acc);
+  const void* kern = reinterpret_cast<const void*>(batch_kernel(s, best_chunked));
   // several lists share a kernel: the limit only ever grows
   static DynamicLdsLimit limits[3][2];
-  if (limits[R == 2 ? 2 : U == 4 ? 0 : 1][best_chunked ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
+  if (limits[batch_kernel_index(s)][best_chunked ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
     return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
@@ -812,7 +826,7 @@ int batch_list_launch(wq_gemv_list* l, hipStream_t stream) {
   const GemvListDesc* table = (const GemvListDesc*)l->table;
   const int use_sync = l->deps > 0 ? 1 : 0;
   // chunk: at least 1 (a list without a linear of several panels keeps no sums)
-  WQ_LAUNCH("wq_q4g32_gemv_list_run", batch_kernel(l->batch_u, batch_rows_sets(l->M), l->batch_chunked), dim3((unsigned)l->blocks), dim3((unsigned)l->threads), l->lds,
+  WQ_LAUNCH("wq_q4g32_gemv_list_run", batch_kernel(batch_shape(l->M), l->batch_chunked), dim3((unsigned)l->blocks), dim3((unsigned)l->threads), l->lds,
             stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, std::max(l->batch_acc_tiles, 1),
             use_sync);
   return WQ_OK;
