@@ -111,6 +111,23 @@ def test_epilogue_and_one_hot(env, oracle, M, N, shift):
         assert np.array_equal(got[m].view(np.uint16), B[:, c].view(np.uint16)), (m, c)
 
 
+def test_tiles_walked_in_chunks_with_a_ragged_end(env, oracle):
+    """One linear of two panels (M = 20: panels of 1024 k) with more tiles per workgroup than LDS keeps sums for: the
+    tiles are walked in chunks.  N is odd (2-byte stores) and ends 7 rows into a 32-row tile (its second 16 rows
+    lie past N)."""
+    ops, u, torch = env
+    M, N, K = 20, 150007, 2048
+    l = _linear(oracle, u, N, K, M, seed=77)
+    rng = np.random.default_rng(5)
+    bias = rng.standard_normal(N).astype(np.float16)
+    y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    gl = ops.Q4G32GemvList([(l["dW"], l["dS"], u.dev(l["x"]), y, u.dev(bias))], M=M)
+    print("batch list: chunks", flush=True)
+    gl.run()
+    gl.status()
+    u.assert_close(u.host(y), oracle.q4g32_linear(l["W"], l["S"], l["x"], bias=bias, nthreads=8), "batch list in chunks")
+
+
 @pytest.mark.parametrize("M", [4, 12, 27])
 def test_dependent_chain_matches_oracle(env, oracle, M):
     """x of a linear is the y of an earlier one: directly in front, one apart, two consumers of one producer; a
