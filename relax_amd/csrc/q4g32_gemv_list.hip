@@ -120,17 +120,6 @@ struct ListFlags {
   int pad[13];
 };
 
-#ifdef WQ_LIST_TRACE
-__device__ long long* g_list_trace = nullptr;  // [workgroup 0 | workgroup 100][64] wall-clock stamps
-#define WQ_TR(i)                                                                                   \
-  do {                                                                                             \
-    if (g_list_trace && (blockIdx.x == 0 || blockIdx.x == 100) && (threadIdx.x & 63) == 0 && (i) < 64) \
-      g_list_trace[(blockIdx.x ? 64 : 0) + (i)] = wall_clock64();                                  \
-  } while (0)
-#else
-#define WQ_TR(i) do { } while (0)
-#endif
-
 template <int NC, int XW, int D>
 __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(const GemvListDesc* __restrict__ descs_,
                                                                         int nlin, int* __restrict__ sync,
@@ -343,16 +332,6 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         v += __shfl_xor(v, 4, 64);
         if (__builtin_amdgcn_readfirstlane(v) >= nwg) break;
         if (wall_clock64() - t0 > spin_limit) {
-#ifdef WQ_LIST_TRACE
-          // first time-out of the launch: who waited for what, and the state of its workgroup
-          if (g_list_trace && lane == 0 && atomicCAS((unsigned long long*)&g_list_trace[128], 0ull, 1ull) == 0ull) {
-            long long* t = g_list_trace + 129;
-            t[0] = blockIdx.x; t[1] = cur_j; t[2] = dep; t[3] = nwg;
-            for (int k = 0; k < 8; ++k) t[4 + k] = __hip_atomic_load(sync + sync_counter_index(dep, k), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            for (int k = 0; k < 4; ++k) { t[12 + k] = flags->x_ready[k]; t[16 + k] = flags->left[k]; }
-            t[20] = flags->flushed; t[21] = flags->next_pos; t[22] = flags->next_x;
-          }
-#endif
           aborted = true;
           if (lane == 0)
             __hip_atomic_store(sync + sync_error_index(nlin), dep + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -383,7 +362,6 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       const int dep = (int)((descs[j].g_dep >> 16) & 0x7fffu) - 1;
       cur_j = j;
       if (dep >= 0) wait_for(dep);
-      if (j < 16) WQ_TR(32 + j);
       const int K = (int)(descs[j].g_dep & 0xffffu) << 5;
       // an x that other workgroups of this launch have written is read with device-scope loads
       // (sc1), which see what device-scope stores followed by the counter update have published,
@@ -425,7 +403,6 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       if (lane == 0) __hip_atomic_store(&flags->x_ready[slot], j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      if (j < 16) WQ_TR(48 + j);
     }
     return;
   }
@@ -434,7 +411,6 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
   for (int j = 0; j < nlin; ++j) {
     const int slot = j & (nb - 1);
     lds_spin_until(&flags->left[slot], NC * ((j >> nb_log2) + 1));
-    if (j < 16) WQ_TR(j);
     const half_t* bias = descs[j].bias;
     const half_t* residual = descs[j].residual;
     const float* yb = ybuf + (j & (kYSlots - 1)) * ybuf_floats;
@@ -463,11 +439,11 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         __hip_atomic_fetch_add(sync + sync_counter_index(j, blockIdx.x & (kCountersPerLinear - 1)), 1,
                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (j < 16) WQ_TR(16 + j);
   }
   if (!use_sync) return;
   // the last workgroup to get here clears the counters for the next launch (every wait of this
   // workgroup lies behind it: its last row sums could only be stored after all its activations were staged)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this workgroup's own counter updates have arrived: none may land on a cleared counter
   int last = 0;
   if (lane == 0)
     last = __hip_atomic_fetch_add(sync + sync_finished_index(nlin), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
@@ -682,8 +658,3 @@ extern "C" int wq_q4g32_gemv_list_set_spin_limit(wq_gemv_list_t* l, long long ti
   return WQ_OK;
 }
 
-#ifdef WQ_LIST_TRACE
-extern "C" __attribute__((visibility("default"))) int wq_debug_list_trace(long long* device_buffer) {
-  return hipMemcpyToSymbol(HIP_SYMBOL(wq::g_list_trace), &device_buffer, sizeof(device_buffer)) == hipSuccess ? 0 : -1;
-}
-#endif
