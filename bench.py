@@ -146,6 +146,12 @@ def _measure(torch, stream, fn, min_ms=None, samples=None):
     fn()
     one = max(_time_on_stream(torch, stream, fn, 2), 1e-4)
     reps = max(1, int(np.ceil(min_ms / one)))
+    # the first calls are slower than the steady state: size the sample from a sample
+    for _ in range(3):
+        one = max(_time_on_stream(torch, stream, fn, reps), 1e-4)
+        if one * reps >= min_ms:
+            break
+        reps = int(np.ceil(1.03 * min_ms / one))
     t = sorted(_time_on_stream(torch, stream, fn, reps) for _ in range(samples))
     med = t[len(t) // 2] if len(t) % 2 else 0.5 * (t[len(t) // 2 - 1] + t[len(t) // 2])
     return med, {"samples": samples, "calls_per_sample": reps, "sample_ms": round(med * reps, 1),
