@@ -91,7 +91,9 @@ def test_epilogue_and_one_hot(env, oracle, M, N, shift):
     rng = np.random.default_rng(3)
     bias = rng.standard_normal(N).astype(np.float16)
     res = rng.standard_normal((M, N)).astype(np.float16)
-    y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    # (shift = 1: y, like the bias below, starts 2 bytes past an 8-byte boundary)
+    y = torch.zeros((M * N + shift,), dtype=torch.float16, device="cuda")[shift:].view(M, N)
+    assert y.data_ptr() % 8 == 2 * shift
     y2 = torch.zeros((M, N), dtype=torch.float16, device="cuda")
     xh = np.zeros((M, K), np.float16)
     cols = ([0, 37, 260, 511, 777, 1023] * 6)[:M]
