@@ -322,11 +322,14 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
   }
 }
 
-// Row slices (1, 2 or 4) that the tiles of the last, partially filled round are cut into: as many as
-// still run all at once.  A rest that already has a CU per tile is only cut if every slice gets a
+// Row slices (1, 2 or 4; 8 where the policy carries the extra copy of the tile body, `fine`) that the tiles of
+// the last, partially filled round are cut into: as many as still run all at once.  (Every slice unpacks all
+// columns of its tile, so slices get less efficient as they get lower: eight only pay on 32 tiles or fewer:
+// M = 256, N = 4096, K = 11008 format A 73.6 -> 68.6 us.)  A rest that already has a CU per tile is only cut if every slice gets a
 // CU of its own: two slices sharing a CU take as long as the whole tile, and read its weights twice.
-inline int lds_tail_split(int rest, int slots, int cus, int TM, int a_loads) {
+inline int lds_tail_split(int rest, int slots, int cus, int TM, int a_loads, bool fine = false) {
   const int room = rest <= cus ? cus : slots;
+  if (fine && TM % 8 == 0 && a_loads % 8 == 0 && rest * 8 <= room) return 8;
   for (int sp : {4, 2})
     if (TM % sp == 0 && a_loads % sp == 0 && rest * sp <= room) return sp;
   return 1;
@@ -355,6 +358,12 @@ inline double lds_cfg_cost(int cfg, int64_t M, int64_t N, int cus) {
   }
   return t;
 }
+
+// Policy::kFineTail = true: the kernels of that policy also hold the tile body for slices of TM / 8 sub-tiles.
+template <class P, class = void>
+struct FineTail : std::false_type {};
+template <class P>
+struct FineTail<P, std::void_t<decltype(P::kFineTail)>> : std::bool_constant<P::kFineTail> {};
 
 // Workgroup -> work item.  The first n_full workgroups compute whole tiles (as many
 // as fill complete rounds of the machine); the tiles of the last, partially filled
@@ -404,6 +413,9 @@ void gemm_lds_kernel(typename Policy::Args wargs, const half_t* __restrict__ X, 
   } else if (split == 4) {
     if constexpr (TM % 4 == 0)
       gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, WAVES_PER_EU, TM / 4>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
+  } else if (split == 8) {
+    if constexpr (TM % 8 == 0 && FineTail<Policy>::value)
+      gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, WAVES_PER_EU, TM / 8>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   } else {
     gemm_lds_tile<Policy, Epilogue, TM, TN, WM, WN, WAVES_PER_EU, TM>(wargs, X, Y, epilogue, M, N, K, m0, n0, lds);
   }
@@ -426,7 +438,7 @@ static int launch_gemm_lds(const char* who, const typename Policy::Args& wargs, 
   const int total = tiles_m * tiles_n;
   const int n_full = (total / slots) * slots;
   const int rest = total - n_full;
-  const int split = tuning().gemm_tail_split ? lds_tail_split(rest, slots, cu_count(), TM, Cfg::kALoads) : 1;
+  const int split = tuning().gemm_tail_split ? lds_tail_split(rest, slots, cu_count(), TM, Cfg::kALoads, FineTail<Policy>::value) : 1;
   // height of the block of tiles an XCD runs at one time: the activation rows of a tile against its weight
   // columns, in bytes per step of K, decide how a block of slots / 8 tiles is best shaped
   const double ratio = (double)(Cfg::BN * Policy::kColBytes) / (double)(Cfg::BM * 128);

@@ -56,6 +56,7 @@ struct Q4G32Loader {
 // column is 32 bytes of codes (chunk (n, h) of the B tile = 16 bytes = one scale group) and two
 // scales (4 bytes, staged in LDS with the codes).
 struct Q4G32LdsPolicy {
+  static constexpr bool kFineTail = true;  // a last round of few tiles may be cut into eight row slices
   static constexpr int kColBytes = 32;
   static constexpr int kScaleBytes = 4;
   static constexpr int kStepStride = 32;
