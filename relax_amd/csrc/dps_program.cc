@@ -305,6 +305,13 @@ static std::vector<int> schedule_group(const std::vector<DecodeLinear>& lin) {
   return order;
 }
 
+// Shortest run worth one launch of the list kernel, by rows of x.  With several rows every workgroup of a
+// linear's group loads all of that linear's activations, which a long list spreads over many small groups and a
+// short one cannot: four Llama-2-7B linears (one decoder layer) take 48 / 78 / 100 us as a list against
+// 43 / 52 / 71 us call by call at M = 8 / 16 / 32; eight linears 40 / 61 / 56 against 45 / 52 / 71; sixteen
+// 37 / 39 / 54 against 44 / 52 / 71.  At M <= 4 the list wins from the first layer on (30 against 42 us).
+static size_t min_fused_run(int64_t M) { return M <= 4 ? 2 : M <= 8 ? 8 : M <= 16 ? 16 : 8; }
+
 static void find_groups(wq_program* p) {
   drop_lists(p);
   p->groups.clear();
@@ -319,7 +326,7 @@ static void find_groups(wq_program* p) {
       lin.push_back(d);
       ++j;
     }
-    if (lin.size() >= 2) {
+    if (!lin.empty() && lin.size() >= min_fused_run(lin[0].M)) {
       FusedGroup g;
       g.first = i;
       g.last = j - 1;

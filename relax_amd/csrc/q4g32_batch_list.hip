@@ -754,7 +754,6 @@ int batch_list_plan(wq_gemv_list* l) {
   const int U = s.U;
   const int trows = 16 * s.TW;
   l->batch_u = U;
-  l->gs = 4;
   l->threads = kBThreads;
   l->blocks = std::min(cu_count(), 32768);
   const size_t budget = 160 * 1024;

@@ -143,6 +143,32 @@ def test_fused_group_order_keeps_dependences_and_separates_producers_from_consum
         l.wq_program_destroy(p)
 
 
+@pytest.mark.parametrize("M,n,fused", [(1, 2, 1), (4, 2, 1), (4, 1, 0), (8, 4, 0), (8, 8, 1), (16, 8, 0), (16, 16, 1),
+                                       (32, 4, 0), (32, 8, 1)])
+def test_short_runs_of_batched_linears_are_not_fused(M, n, fused):
+    """Planning alone (no GPU): with several rows of x a run only becomes one launch of the list kernel from the
+    length at which that launch is faster than the calls one by one."""
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        addr = [0x100000]
+
+        def ext(code, bits, *shape):
+            addr[0] += 0x100000
+            return l.wq_program_add_external(p, code, bits, len(shape), _shape(*shape), addr[0], 10)
+
+        x = ext(2, 16, M, 256)
+        for _ in range(n):
+            W, S, y = ext(1, 32, 64, 32), ext(2, 16, 64, 8), ext(2, 16, M, 64)
+            assert _call(l, p, "relax_amd.q4f16_1_matmul", [W, S, x, y]) == 0
+        assert l.wq_program_plan(p) >= 0
+        buf = (ctypes.c_int * n)()
+        got = l.wq_program_fused_order(p, 0, buf, n)  # the first run, if there is one
+        assert (got == n) if fused else (got < 0), got
+    finally:
+        l.wq_program_destroy(p)
+
+
 SMALL_LINEARS = (("qkv_proj", 384, 128), ("o_proj", 128, 128), ("gate_up_proj", 512, 128), ("down_proj", 128, 256))
 
 
