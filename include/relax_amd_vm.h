@@ -79,10 +79,13 @@ int wq_program_replay(wq_program_t* p, wq_stream_t stream);
 
 int wq_program_num_instructions(const wq_program_t* p);
 
-/* Fused decode linears.  A run of two or more consecutive relax_amd.q4f16_1_matmul[_bias[_residual]]
- * instructions with one row of x each (the decode step of a stack of quantized linears) is
- * executed as ONE launch of the list kernel (wq_q4g32_gemv_list_* of relax_amd_wq.h) instead of
- * one kernel per instruction, which is what the reference's VM does with the generated kernels
+/* Fused decode linears.  A run of consecutive relax_amd.q4f16_1_matmul[_bias[_residual]]
+ * instructions with the same number M <= 32 of rows of x (the decode step of a stack of quantized
+ * linears; K % 256 == 0 where M > 1) is executed as ONE launch of the list kernel if it is long
+ * enough for that to be the faster way: 2 instructions at M <= 4, 8 at M <= 8, 16 at M <= 16, 8 beyond
+ * (a short list with several rows of x cannot spread the loads of the activations over small groups
+ * of workgroups).  The list kernel is wq_q4g32_gemv_list_* of relax_amd_wq.h; one kernel per
+ * instruction is what the reference's VM does with the generated kernels
  * of python/tvm/dlight/gpu/gemv.py.  Inside such a run, independent linears are moved between a
  * producer and its consumer (results are unchanged: every true, anti and output dependence
  * between the instructions is kept), and the planned tensors of the run do not share storage.
