@@ -7,11 +7,14 @@ statement that depends on the wait; what is left to chance is register allocatio
 spill of a ring register inserted between load and wait would read it too early).  This script
 compiles the file to assembly and verifies, in the kernel's text, that
 
-* every ring register (destination of a ``global_load_* ... nt`` instruction) is read only by the
+* every ring register (destination of a ``global_load_* ... nt`` or ``buffer_load_* ... nt`` instruction) is read only by the
   instructions the source uses for it (``v_and_or_b32``, ``v_lshrrev_b32 .., 8, ..``, ``v_cvt_f32_f16``,
   and the cross-lane ``v_mov_b32_dpp`` of the batch kernel's lane exchange, which the compiler never
   generates by itself), never by a plain move, a store or anything else, and
-* each ring slot keeps one register in the prologue and in the loop (no renaming copies).
+* each ring slot keeps one register in the prologue and in the loop (no renaming copies), and
+* behind the last ring load of the kernel's text (the way out of the loop), no ring register is
+  written by anything else before an instruction of the consumer read it or an ``s_waitcnt vmcnt(0)``
+  passed: a slot abandoned on the way out would otherwise receive its data on top of a new value.
 
 Registers that the compiler also uses for short-lived temporaries while a slot is empty are
 recognised by being written by another instruction first.
@@ -33,6 +36,11 @@ SOURCES = ("q4g32_gemv_list.hip", "q4g32_batch_list.hip")
 ALLOWED_READERS = ("v_and_or_b32", "v_lshrrev_b32", "v_cvt_f32_f16", "v_mov_b32_dpp")
 
 
+def _is_ring_load(l: str) -> bool:
+    """A load of the weight stream: the only non-temporal loads of these kernels."""
+    return l.startswith(("global_load_", "buffer_load_")) and l.endswith(" nt")
+
+
 def _regs(tok: str):
     """'v[4:7]' -> {4,5,6,7}; 'v12' -> {12}; anything else -> empty."""
     m = re.fullmatch(r"v\[(\d+):(\d+)\]", tok)
@@ -46,18 +54,23 @@ def _check_function(body: list[str]) -> list[str]:
     errors = []
     ring = set()
     for l in body:
-        if l.startswith("global_load_") and l.endswith(" nt"):
+        if _is_ring_load(l):
             ring |= _regs(l.split()[1].rstrip(","))
     if not ring:
         return []
     # walk the text; a ring register is "loaded" after a ring load wrote it and until something else writes it
     loaded = set()
-    for l in body:
+    unread = set()  # loaded, and neither read by the consumer nor covered by a wait for all loads since
+    last_load = max(i for i, l in enumerate(body) if _is_ring_load(l))
+    for i, l in enumerate(body):
         parts = l.replace(",", " ").split()
         op, ops = parts[0], parts[1:]
-        if op.startswith("global_load_") and l.endswith(" nt"):
+        if _is_ring_load(l):
             loaded |= _regs(ops[0])
+            unread |= _regs(ops[0])
             continue
+        if op == "s_waitcnt" and "vmcnt(0)" in l:
+            unread = set()
         if not ops:
             continue
         stores = ("global_store", "ds_write", "buffer_store", "scratch_store", "global_atomic", "ds_add")
@@ -70,6 +83,13 @@ def _check_function(body: list[str]) -> list[str]:
         hit = reads & loaded
         if hit and not op.startswith(ALLOWED_READERS):
             errors.append(f"ring register(s) {sorted(hit)} read by `{l}`")
+        unread -= reads
+        late = writes & unread if i > last_load else set()  # (text order says nothing about in flight inside the loops)
+        if late:
+            # the compiler took a register whose load may still be in flight (a slot abandoned on the way
+            # out of the loop): the data would land on top of the new value
+            errors.append(f"ring register(s) {sorted(late)} written by `{l}` before their load was consumed or waited for")
+            unread -= late
         if op.startswith("v_lshrrev_b32") and hit and ops[1] != "8":
             errors.append(f"unexpected shift of a ring register: `{l}`")
         loaded -= writes  # now a temporary of the compiler
@@ -136,11 +156,11 @@ def check(asm_text: str) -> list[str]:
             cur.append(l)
     errors, with_ring = [], 0
     for body in functions:
-        if any(l.startswith("global_load_") and l.endswith(" nt") for l in body):
+        if any(_is_ring_load(l) for l in body):
             with_ring += 1
             errors += _check_function(body)
     if with_ring == 0:
-        return ["no ring loads found (expected global_load_* ... nt in the kernel)"]
+        return ["no ring loads found (expected global_load_* / buffer_load_* ... nt in the kernel)"]
     return errors
 
 

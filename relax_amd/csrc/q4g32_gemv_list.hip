@@ -57,7 +57,7 @@ struct RowCursor {
   int R;            // positions of it that belong to this workgroup (whole row groups)
   int rb;           // (b - off) mod workgroups: row group = local group * workgroups + rb
   int N;            // rows of the linear (positions of a last, partial row group beyond N are empty)
-  int C, glast;     // chunks per row, groups in the last chunk (1..64)
+  int C;            // chunks per row
   int row_w, row_s; // bytes per row of W and S
   const char* W;
   const char* S;
@@ -82,7 +82,6 @@ __device__ __forceinline__ void row_cursor_load(RowCursor& cu, gemv_desc_ptr des
   cu.N = (int)w[12];
   cu.R = ((int)w[13] + (rb < (int)(w[15] & 0xffffu) ? 1 : 0)) << gs;
   cu.C = (G + 63) >> 6;
-  cu.glast = G - (cu.C - 1) * 64;
   cu.row_w = K >> 1;
   cu.row_s = G * 2;
   cu.W = reinterpret_cast<const char*>(((uint64_t)w[1] << 32) | w[0]);
@@ -143,91 +142,103 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
     // =========================== compute wavefront ===========================
     // Rows are taken one at a time from the workgroup's sequence (an LDS counter), so the NC
     // wavefronts stay balanced whatever the row lengths; the next position is fetched one row ahead.
+    //
+    // The ring.  Its loads are written in assembly and waited for by hand.  Every turn of a slot issues
+    // exactly two loads (16 bytes of codes and one scale per lane), also when the list has run out
+    // (then from an empty buffer: nothing is fetched), and no other path of a compute wavefront
+    // issues a vector memory operation: loads retire in order, so "at most 2 (D - 1) outstanding"
+    // says that the oldest slot has landed.  (Left to the compiler, the wait of the first slot of the
+    // unrolled loop comes out as "all but one".)  The loads are buffer loads over ONE ROW (base = the row, size = its
+    // bytes): lanes beyond the end of a row whose K is not a multiple of 2048 receive zeros for codes
+    // and scale, and the x wavefronts zero the activations of those groups, so a partial last chunk
+    // needs no code of its own.
+    // A wavefront issues one instruction every four cycles, so what a chunk costs is its instruction
+    // count: what the consumer needs (where the activations are, whether the row ends) is packed into
+    // two scalars per slot when the chunk is issued; everything per row or per linear is off the path.
     const int b = blockIdx.x;
     const uint32_t lane16 = lane * 16;
     if (tid < (int)(sizeof(ListFlags) / sizeof(int))) reinterpret_cast<int*>(flags)[tid] = 0;
     lds_done_then_barrier();  // LDS starts undefined: the flags are cleared before anyone looks
 
-    auto take_position = [&]() {
-      int p = 0;
-      if (lane == 0) p = __hip_atomic_fetch_add(&flags->next_pos, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      return p;  // valid in lane 0; read with readfirstlane where it is used
-    };
-
-    // The ring.  Its loads are written in assembly and waited for by hand: loads retire in order and
-    // a compute wavefront issues no other vector memory operation, so with all D slots in flight the
-    // oldest one has landed when at most 2 (D - 1) loads are outstanding.  (Left to the compiler, the
-    // counts come out right only as long as every path through the loop issues the same loads.)
-    // A wavefront issues one instruction every four cycles, so what a chunk costs is its instruction
-    // count: everything a chunk needs when it is consumed (where its activations are, where its row
-    // sum goes) is worked out when it is issued, once per row where possible, and kept per slot.
+    constexpr int kLast = 1, kNewLinear = 2, kDead = 4;  // slot flags (bits 0..7 of slot_meta; the rest: LDS offset of x)
     uint4_t rw[D];
     uint32_t rs[D];
-    int slot_lin[D];    // linear of the chunk in the slot; -1: the slot is empty
-    int slot_x[D];      // LDS byte offset of the chunk's activations
-    int slot_y[D];      // LDS byte offset of the row sum if this is the row's last chunk, else -1
-    int slot_gl[D];     // groups in the chunk (64, or fewer in a partial last chunk)
-    int inflight = 0;   // slots issued and not yet consumed
+    int slot_meta[D];   // flags | LDS byte offset of the chunk's activations << 8
+    int slot_yl[D];     // LDS byte offset of the row sum | linear << 18
     const int xbuf0 = (int)sizeof(ListFlags);
     const int ybuf0 = xbuf0 + nb * xbuf_bytes;
 
-    // issue side: the row being issued, and the next position (fetched one row ahead)
+    // the position counter: one lane adds, the answer is read one row later
+    int inext;
+    auto take_position = [&]() {
+      if (lane == 0) {
+        int one = 1;
+        asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=v"(inext) : "v"((uint32_t)(uintptr_t)&flags->next_pos), "v"(one) : "memory");
+      }
+    };
+    take_position();
+
+    // issue side: the row being issued
     RowCursor ic;
     ic.lin = 0;
     ic.base = 0;
     row_cursor_load(ic, descs, nlin, b, nwg, gs);
-    int inext = take_position();
-    int i_c = 0, i_xbase = 0, i_ypos = 0;
-    const char* i_wb = nullptr;
-    const char* i_sb = nullptr;
-    uint32_t i_part16 = 0;  // lane offset in a partial last chunk: idle lanes shadow the last group
-    int i_part_lin = -1;
+    int i_left = 0;       // chunks of the row still to issue
+    int i_off = 0;        // byte offset of the next chunk in the row of codes (in the row of scales: / 8)
+    int i_x = 0;          // LDS offset of the next chunk's activations
+    int i_yl = 0;         // slot_yl of the row
+    int i_new = kNewLinear;  // the next chunk is this wavefront's first of a linear
+    // buffer resources of the row: base address, size in bytes, flags (an empty one: every lane reads zero, no memory access)
+    auto row_rsrc = [](const char* p, int bytes) {
+      const uint64_t a = reinterpret_cast<uint64_t>(p);
+      return uint4_t{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)bytes, (uint32_t)kBufferFlags};
+    };
+    uint4_t i_w = row_rsrc(nullptr, 0), i_s = row_rsrc(nullptr, 0);
     auto next_row = [&]() {  // the next position that holds a row (a last, partial row group has empty ones)
       int64_t row;
       int pos;
+      int lin0 = ic.lin;
       do {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(inext)::"memory");  // the counter's answer has arrived
         pos = __builtin_amdgcn_readfirstlane(inext);
-        inext = take_position();
+        take_position();
         row_cursor_seek(ic, pos, descs, nlin, b, nwg, gs);
         row = row_cursor_row(ic, pos, nwg, gs);
       } while (ic.lin < nlin && row >= ic.N);
-      if (ic.lin >= nlin) return;
-      if (i_part_lin != ic.lin) {
-        i_part_lin = ic.lin;
-        i_part16 = min(lane, ic.glast - 1) * 16;
+      if (ic.lin >= nlin) {  // the list has run out: the slots drain
+        // nobody will read the counter's last answer: it must have landed before its register is used for something else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(inext)::"memory");
+        i_left = -1;
+        i_w = row_rsrc(nullptr, 0);
+        i_s = i_w;
+        return;
       }
-      i_c = 0;
-      i_wb = ic.W + row * ic.row_w;
-      i_sb = ic.S + row * ic.row_s;
-      i_xbase = xbuf0 + (ic.lin & (nb - 1)) * xbuf_bytes;
-      i_ypos = ybuf0 + ((ic.lin & (kYSlots - 1)) * ybuf_floats + (pos - ic.base)) * 4;
+      if (ic.lin != lin0) i_new = kNewLinear;
+      i_left = ic.C;
+      i_off = 0;
+      i_w = row_rsrc(ic.W + row * ic.row_w, ic.row_w);
+      i_s = row_rsrc(ic.S + row * ic.row_s, ic.row_s);
+      i_x = xbuf0 + (ic.lin & (nb - 1)) * xbuf_bytes;
+      i_yl = (ybuf0 + ((ic.lin & (kYSlots - 1)) * ybuf_floats + (pos - ic.base)) * 4) | (ic.lin << 18);
     };
-    next_row();
 
-    auto issue = [&](uint4_t& w, uint32_t& s, int& slin, int& sx, int& sy, int& sgl) {
-      slin = -1;
-      if (ic.lin >= nlin) return;
-      const bool last = i_c == ic.C - 1;
-      const bool partial = last && ic.glast < 64;
-      const uint32_t voff = partial ? i_part16 : lane16;
-      const uint32_t soff = voff >> 3;
+    auto issue = [&](uint4_t& w, uint32_t& s, int& meta, int& yl) {
+      if (i_left == 0) next_row();
       asm volatile(
-          "global_load_dwordx4 %0, %2, %3 nt\n\t"
-          "global_load_ushort %1, %4, %5 nt"
+          "buffer_load_dwordx4 %0, %2, %3, %4 offen nt\n\t"
+          "buffer_load_ushort %1, %5, %6, %7 offen nt"
           : "=&v"(w), "=&v"(s)
-          : "v"(voff), "s"(i_wb), "v"(soff), "s"(i_sb));
-      slin = ic.lin;
-      sx = i_xbase + i_c * kChunkBytes;
-      sy = last ? i_ypos : -1;
-      sgl = partial ? ic.glast : 64;
-      ++inflight;
-      if (last) {
-        next_row();
-      } else {
-        ++i_c;
-        i_wb += 1024;
-        i_sb += 128;
+          : "v"(lane16), "s"(i_w), "s"(i_off), "v"(lane16 >> 3), "s"(i_s), "s"(i_off >> 3));
+      if (i_left < 0) {
+        meta = kDead;
+        return;
       }
+      --i_left;
+      meta = (i_x << 8) | i_new | (i_left == 0 ? kLast : 0);
+      yl = i_yl;
+      i_new = 0;
+      i_off += 1024;
+      i_x += kChunkBytes;
     };
 
     // Every compute wavefront passes through every linear, also those in which it takes no row:
@@ -262,19 +273,15 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       asm("v_cvt_f32_f16 %0, %1 ; %2" : "=v"(r) : "v"(s16), "v"(magic));
       return r;
     };
-    auto consume = [&](const uint4_t& w4, const uint32_t& s16, int lin, int sx, int sy, int gl) {
-      if (lin != entered) advance_to(lin);
-      uint32_t lo = lane16;
-      if (gl < 64) lo = min(lane, gl - 1) * 16;
-      const char* xb = lds + sx;
+    auto consume = [&](const uint4_t& w4, const uint32_t& s16, int meta, int yl) {
+      if (meta & kNewLinear) advance_to(yl >> 18);
+      const char* xb = lds + (meta >> 8);
       uint4_t xv[4];
 #pragma unroll
-      for (int ch = 0; ch < 4; ++ch) xv[ch] = *reinterpret_cast<const uint4_t*>(xb + ch * 1024 + lo);
-      float grp = *reinterpret_cast<const float*>(xb + 4096 + (lo >> 2));
-      // this slot is the oldest in flight
-      if (inflight == D) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"(2 * (D - 1)));
-      else asm volatile("s_waitcnt vmcnt(0)" : "+v"(magic));
-      --inflight;
+      for (int ch = 0; ch < 4; ++ch) xv[ch] = *reinterpret_cast<const uint4_t*>(xb + ch * 1024 + lane16);
+      float grp = *reinterpret_cast<const float*>(xb + 4096 + (lane16 >> 2));
+      // every slot is always in flight (the drained ones with loads that fetch nothing): this one is the oldest
+      asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"(2 * (D - 1)));
 #pragma unroll
       for (int ch = 0; ch < 4; ++ch) {
         const uint32_t word = ch == 0 ? w4.x : ch == 1 ? w4.y : ch == 2 ? w4.z : w4.w;
@@ -288,25 +295,31 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         grp = dot2(t2, as_half2(xv[ch].z), grp);
         grp = dot2(t3, as_half2(xv[ch].w), grp);
       }
-      float sf = ring_scale(s16);
-      if (gl < 64 && lane >= gl) sf = 0.0f;
-      acc = fmaf(sf, grp, acc);
-      if (sy >= 0) {
+      acc = fmaf(ring_scale(s16), grp, acc);
+      if (meta & kLast) {
         const float tot = wave_sum_to_lane63(acc);
-        if (lane == 63) *reinterpret_cast<float*>(lds + sy) = tot;
+        if (lane == 63) *reinterpret_cast<float*>(lds + (yl & 0x3ffff)) = tot;
         acc = 0.0f;
       }
     };
 
 #pragma unroll
-    for (int s = 0; s < D; ++s) issue(rw[s], rs[s], slot_lin[s], slot_x[s], slot_y[s], slot_gl[s]);
-    while (inflight > 0) {
+    for (int s = 0; s < D; ++s) issue(rw[s], rs[s], slot_meta[s], slot_yl[s]);
+    bool live = true;
+    while (live) {
 #pragma unroll
       for (int s = 0; s < D; ++s) {
-        if (slot_lin[s] >= 0) consume(rw[s], rs[s], slot_lin[s], slot_x[s], slot_y[s], slot_gl[s]);
-        issue(rw[s], rs[s], slot_lin[s], slot_x[s], slot_y[s], slot_gl[s]);
+        if (slot_meta[s] & kDead) {  // the slots behind it are dead too
+          live = false;
+          break;
+        }
+        consume(rw[s], rs[s], slot_meta[s], slot_yl[s]);
+        issue(rw[s], rs[s], slot_meta[s], slot_yl[s]);
       }
     }
+    // the drained slots still have their (empty) loads in flight: they must have landed before the
+    // ring's registers are used for something else
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     advance_to(nlin);
     return;
   }
@@ -369,7 +382,8 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       const __amdgpu_buffer_rsrc_t xr =
           __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(descs[j].x), 0, K * 2, kBufferFlags);
       char* xb = xbuf + slot * xbuf_bytes;
-      const int nwords = K >> 3;  // 16-byte words of 8 activations; a multiple of 4
+      const int nwords = (((K >> 5) + 63) & ~63) << 2;  // 16-byte words of 8 activations, up to the end of the last chunk
+                                                        // (beyond K the buffer loads return zeros)
       constexpr int U = 16;       // loads in flight per lane: one round trip per 16 KiB of x
       for (int base = 0; base < nwords; base += 64 * U) {
         uint4_t v[U];
