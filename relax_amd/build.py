@@ -84,7 +84,12 @@ def build(verbose: bool = True, incremental: bool = False) -> str:
     ring = [os.path.basename(s) for s in todo if os.path.basename(s) in check_ring_asm.SOURCES]
     if ring:
         # those kernels wait for their inline-assembly loads by hand: verify the generated code
-        check_ring_asm.main(HIPCC, [f for f in FLAGS if f != "-fPIC"], ring)
+        try:
+            check_ring_asm.main(HIPCC, [f for f in FLAGS if f != "-fPIC"], ring)
+        except Exception:
+            for name in ring:  # an incremental build must not take the refused objects for up to date
+                os.remove(os.path.join(OBJDIR, name + ".o"))
+            raise
     for lib, want in ((LIB, False), (CALIBRATE_LIB, True)):
         objs = [os.path.join(OBJDIR, os.path.basename(s) + ".o") for s in srcs
                 if (os.path.basename(s) in CALIBRATE_SOURCES) == want]

@@ -11,10 +11,11 @@ compiles the file to assembly and verifies, in the kernel's text, that
   instructions the source uses for it (``v_and_or_b32``, ``v_lshrrev_b32 .., 8, ..``, ``v_cvt_f32_f16``,
   and the cross-lane ``v_mov_b32_dpp`` of the batch kernel's lane exchange, which the compiler never
   generates by itself), never by a plain move, a store or anything else, and
-* each ring slot keeps one register in the prologue and in the loop (no renaming copies), and
-* behind the last ring load of the kernel's text (the way out of the loop), no ring register is
-  written by anything else before an instruction of the consumer read it or an ``s_waitcnt vmcnt(0)``
-  passed: a slot abandoned on the way out would otherwise receive its data on top of a new value.
+* each ring slot keeps one register in the prologue and in the loop (no renaming copies).
+
+What the text cannot show is a slot abandoned on the way out of the loop: its load is still in flight, and
+a register the compiler reuses behind the loop would receive the data on top of its new value.  The
+sources therefore wait for all loads (``s_waitcnt vmcnt(0)``) where the ring's loop ends.
 
 Registers that the compiler also uses for short-lived temporaries while a slot is empty are
 recognised by being written by another instruction first.
@@ -60,17 +61,12 @@ def _check_function(body: list[str]) -> list[str]:
         return []
     # walk the text; a ring register is "loaded" after a ring load wrote it and until something else writes it
     loaded = set()
-    unread = set()  # loaded, and neither read by the consumer nor covered by a wait for all loads since
-    last_load = max(i for i, l in enumerate(body) if _is_ring_load(l))
-    for i, l in enumerate(body):
+    for l in body:
         parts = l.replace(",", " ").split()
         op, ops = parts[0], parts[1:]
         if _is_ring_load(l):
             loaded |= _regs(ops[0])
-            unread |= _regs(ops[0])
             continue
-        if op == "s_waitcnt" and "vmcnt(0)" in l:
-            unread = set()
         if not ops:
             continue
         stores = ("global_store", "ds_write", "buffer_store", "scratch_store", "global_atomic", "ds_add")
@@ -83,13 +79,6 @@ def _check_function(body: list[str]) -> list[str]:
         hit = reads & loaded
         if hit and not op.startswith(ALLOWED_READERS):
             errors.append(f"ring register(s) {sorted(hit)} read by `{l}`")
-        unread -= reads
-        late = writes & unread if i > last_load else set()  # (text order says nothing about in flight inside the loops)
-        if late:
-            # the compiler took a register whose load may still be in flight (a slot abandoned on the way
-            # out of the loop): the data would land on top of the new value
-            errors.append(f"ring register(s) {sorted(late)} written by `{l}` before their load was consumed or waited for")
-            unread -= late
         if op.startswith("v_lshrrev_b32") and hit and ops[1] != "8":
             errors.append(f"unexpected shift of a ring register: `{l}`")
         loaded -= writes  # now a temporary of the compiler

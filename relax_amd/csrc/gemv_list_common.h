@@ -29,7 +29,11 @@ struct GemvListDesc {  // 128 bytes, device memory
   // then count within the group.
   uint8_t gmod_log2, gidx;
   uint8_t rows;  // rows of x and y of this entry (the M of the launch)
-  uint8_t pad[61];
+  // words 17 ..: the one-row kernel only.
+  uint8_t ts;          // log2 of the rows a compute wavefront takes at a time (0 .. gs)
+  uint32_t x_off;      // LDS byte offset of the linear's activations (the workgroup's LDS is dealt as a ring)
+  int32_t free_after;  // ... which may be written once this many linears of the list have been flushed
+  uint8_t pad[52];
 };
 static_assert(sizeof(GemvListDesc) == 128, "descriptor layout");
 constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y
@@ -72,6 +76,7 @@ struct wq_gemv_list {
   int blocks = 0, threads = 0;
   size_t lds = 0;
   int xbuf_bytes = 0, ybuf_floats = 0;
+  int ybuf0 = 0;  // LDS byte offset of the row-sum buffers (one-row kernel)
   int late = 0, deps = 0;
   int nb = 2;
   int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time

@@ -6,22 +6,29 @@
 // next linear is already in flight while the current one finishes, and a linear that reads what an
 // earlier one wrote waits on a device-side counter instead of a kernel boundary.
 //
-// Workgroup = NC compute wavefronts + 2 service wavefronts, one workgroup per CU.
-//   * A compute wavefront owns whole rows: row r of a linear belongs to wavefront r mod (all
-//     compute wavefronts of the grid).  A row is streamed in chunks of 64 scale groups (2048 k,
-//     1 KiB of codes: one 16-byte load and one scale per lane).  The chunks of all its rows, over
-//     all linears, form one stream that runs through a ring of D register slots: the loads of chunk
-//     f + D are issued when chunk f has been consumed, also across the boundary between two
-//     linears.  Compute wavefronts issue no other vector memory operation, so the compiler's
-//     s_waitcnt vmcnt(2(D-1)) in front of each consume is exact.  Arithmetic per chunk as in the
-//     single-linear kernel (q4_gemv.h): 1 shift + 4 v_and_or + 4 v_dot2 per 8 weights, zero point
-//     and scale applied once per group.  Row sums go to LDS, not to memory.
+// Workgroup = NC compute wavefronts + 2 x wavefronts + 1 y wavefront, one workgroup per CU.
+//   * Work is dealt in ROW GROUPS (2^gs consecutive rows of one linear).  The row groups of a
+//     workgroup, over all linears in list order, form one sequence; a compute wavefront takes the
+//     next one through an LDS counter whenever it has issued the last chunk of its group, so the NC
+//     wavefronts stay balanced whatever the row lengths, and a wavefront only ever looks at the
+//     linears in which it works.  A row is streamed in chunks of 64 scale groups (2048 k, 1 KiB of
+//     codes: one 16-byte load and one scale per lane).  The chunks of all rows of a wavefront form
+//     one stream that runs through a ring of D register slots: the loads of chunk f + D are issued
+//     when chunk f has been consumed, also across rows, groups and linears.  Arithmetic per chunk as
+//     in the single-linear kernel (q4_gemv.h): 1 shift + 4 v_and_or + 4 v_dot2 per 8 weights, zero
+//     point and scale applied once per group.  Row sums go to LDS, not to memory.
+//   * What bounds the kernel is the number of instructions a SIMD can issue (its waves never wait for
+//     memory), the SCALAR ones first: so a chunk costs two scalars of state, everything per row is a
+//     handful of additions, and the arithmetic of a row group (where it is, which linear) is paid once
+//     per group.
 //   * The service wavefronts do everything irregular, each at its own pace, up to NB (2..8) linears
 //     ahead of or behind the compute wavefronts; LDS words (ListFlags) hand the NB buffer slots over.
-//     The x wavefront waits for a producer linear (bounded spin), loads the activations of a coming
+//     An x wavefront waits for a producer linear (bounded spin), loads the activations of a coming
 //     linear, rearranges them to the pairing of the unpack, computes the zero-point constants and
-//     writes both to LDS.  The y wavefront takes the finished row sums of a linear from LDS, applies
-//     bias / cast / residual, stores y, and signals completion.
+//     writes both to LDS.  The y wavefront takes the finished row sums of a linear from LDS (once
+//     the compute wavefronts have counted all of the workgroup's rows of it), applies bias / cast /
+//     residual, stores y, and signals completion.  They run at raised priority: they are the
+//     youngest wavefronts of their SIMDs and would otherwise be starved by the compute wavefronts.
 //
 // Dependencies.  Linear i may read the y of an earlier linear `dep` of the same list.  Each
 // workgroup adds 1 to one of 8 counters of linear `dep` once its stores of y (device scope, written
@@ -31,8 +38,9 @@
 // error word, stops waiting for anything and lets every wavefront run to the end (results are then
 // undefined, the host reads the error word).  The grid is sized so that all workgroups are resident
 // at once; the bounded wait is what keeps a launch that is not (another kernel holding CUs) from
-// hanging.  If dep == i - 1 nothing can overlap: the compute wavefronts idle (their ring stays
-// loaded) until the producer has finished everywhere; callers order lists so that this is rare.
+// hanging.  The waits on LDS words inside a workgroup are not bounded: every party is a wavefront of
+// the same resident workgroup, and an x wavefront that has given up on a producer still stages (then
+// meaningless) activations, so each of those waits ends.
 // The last workgroup to finish clears the counters for the next launch.
 #include <algorithm>
 #include <cstdlib>
@@ -47,74 +55,65 @@
 
 namespace wq {
 
-constexpr int kChunkBytes = 4096 + 256;  // LDS bytes per chunk of x: 4 x 64 uint4 + 64 floats
+// LDS bytes per chunk of x: 4 blocks of 64 x 16 bytes (word ch of the chunk's group g at ch * 1024 + g * 16),
+// then the 64 zero-point constants, one float per 16 bytes (so that one address register serves all five reads)
+constexpr int kChunkBytes = 4096 + 1024;
 
-// ---- where a workgroup's rows are: its rows of all linears, in list order, form one sequence of
-// ---- positions 0, 1, 2, ...; a cursor maps a position to (linear, local row).  Forward only.
-struct RowCursor {
+// ---- where a workgroup's row groups are: its groups of all linears, in list order, form one sequence of
+// ---- positions 0, 1, 2, ...; a cursor maps a position to (linear, local group).  Forward only.
+struct GroupCursor {
   int lin;          // current linear (nlin: past the end)
-  int base;         // position of its first row
-  int R;            // positions of it that belong to this workgroup (whole row groups)
+  int base;         // position of its first group
+  int R;            // positions of it that belong to this workgroup
   int rb;           // (b - off) mod workgroups: row group = local group * workgroups + rb
-  int N;            // rows of the linear (positions of a last, partial row group beyond N are empty)
+  int N;            // rows of the linear
+  int ts;           // log2 of the rows of a position (a position is a whole row group or a part of one)
+  int xoff;         // LDS offset of the linear's activations
   int C;            // chunks per row
   int row_w, row_s; // bytes per row of W and S
   const char* W;
   const char* S;
 };
 
-__device__ __forceinline__ void row_cursor_load(RowCursor& cu, gemv_desc_ptr descs, int nlin, int b, int nwg, int gs) {
+__device__ __forceinline__ void group_cursor_load(GroupCursor& cu, gemv_desc_ptr descs, int nlin, int b, int nwg, int gs) {
   if (cu.lin >= nlin) {
     cu.R = 0x7fffffff;  // every position from here on is "past the end"
     return;
   }
-  // the whole descriptor with one scalar load (W, S: words 0..3; N, q, g_dep, rem | off << 16: 12..15)
+  // (W, S: words 0..3; N, q, g_dep, rem | off << 16: 12..15)
   typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
   const words_ptr p = (words_ptr)(descs + cu.lin);
-  uint32_t w[16];
+  uint32_t w[19];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) w[i] = p[i];
+  for (int i = 0; i < 19; ++i) w[i] = p[i];  // (16: groups of the batch kernel, ts; 17: x_off)
   const int G = (int)(w[14] & 0xffffu);
-  const int K = G << 5;
   int rb = b - (int)(w[15] >> 16);
   if (rb < 0) rb += nwg;
   cu.rb = rb;
   cu.N = (int)w[12];
-  cu.R = ((int)w[13] + (rb < (int)(w[15] & 0xffffu) ? 1 : 0)) << gs;
+  cu.ts = (int)(w[16] >> 24);
+  cu.xoff = (int)w[17];
+  cu.R = ((int)w[13] + (rb < (int)(w[15] & 0xffffu) ? 1 : 0)) << (gs - cu.ts);
   cu.C = (G + 63) >> 6;
-  cu.row_w = K >> 1;
-  cu.row_s = G * 2;
+  cu.row_w = G << 4;
+  cu.row_s = G << 1;
   cu.W = reinterpret_cast<const char*>(((uint64_t)w[1] << 32) | w[0]);
   cu.S = reinterpret_cast<const char*>(((uint64_t)w[3] << 32) | w[2]);
 }
 
-// moves the cursor to the linear that holds position `pos`
-__device__ __forceinline__ void row_cursor_seek(RowCursor& cu, int pos, gemv_desc_ptr descs, int nlin, int b, int nwg, int gs) {
-  while (cu.lin < nlin && pos >= cu.base + cu.R) {
-    cu.base += cu.R;
-    ++cu.lin;
-    row_cursor_load(cu, descs, nlin, b, nwg, gs);
-  }
-}
-
-// row of the linear at position `pos` of the workgroup's sequence (may be >= N in a partial last group)
-__device__ __forceinline__ int64_t row_cursor_row(const RowCursor& cu, int pos, int nwg, int gs) {
-  const int lp = pos - cu.base;
-  return ((((int64_t)(lp >> gs)) * nwg + cu.rb) << gs) + (lp & ((1 << gs) - 1));
-}
-
-// LDS words that hand the buffers over inside a workgroup.  Activations live in NB (2, 4 or 8) slots
-// (slot = linear mod NB), row sums in kYSlots slots (linear mod kYSlots):
-//   x_ready[slot]  = j + 1 once the activations of linear j are staged            (written by an x wavefront)
-//   left[slot]     += 1 by every compute wavefront that is done with a linear of that slot (cumulative)
-//   flushed        = j + 1 once the row sums of linears 0..j have been stored to y (written by the y wavefront)
-constexpr int kMaxSlots = 8;
-constexpr int kYSlots = 8;
+// LDS words that hand the buffers over inside a workgroup:
+//   x_ready[slot]  = j + 1 once the activations of linear j are staged              (written by an x wavefront)
+//   done[slot]     += 1 by a compute wavefront for every row sum it has written; the y wavefront clears it
+//   flushed        = j + 1 once the row sums of linears 0..j have been stored to y   (written by the y wavefront);
+//                    the buffers of linear j are free from then on (every row of it has been consumed)
+// with slot = linear mod kYSlots.  The activations themselves live in a ring of LDS that the host deals out
+// (GemvListDesc::x_off, free_after): a long row takes more of it than a short one.
+constexpr int kYSlots = 16;  // linears in flight at most (flags and row-sum buffers: linear mod kYSlots)
 struct ListFlags {
-  int x_ready[kMaxSlots];
-  int left[kMaxSlots];
+  int x_ready[kYSlots];
+  int done[kYSlots];
   int flushed;
-  int next_pos;  // the next position of the workgroup's row sequence that nobody has taken
+  int next_pos;  // the next position of the workgroup's sequence that nobody has taken
   int next_x;    // the next linear whose activations no x wavefront has taken
   int pad[13];
 };
@@ -122,16 +121,14 @@ struct ListFlags {
 template <int NC, int XW, int D>
 __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(const GemvListDesc* __restrict__ descs_,
                                                                         int nlin, int* __restrict__ sync,
-                                                                        long long spin_limit, int xbuf_bytes,
-                                                                        int ybuf_floats, int nb_log2, int gs, int use_sync) {
-  const int nb = 1 << nb_log2;
+                                                                        long long spin_limit, int ybuf0,
+                                                                        int ybuf_floats, int gs, int use_sync) {
   extern __shared__ uint4_t smem[];
   const gemv_desc_ptr descs = (gemv_desc_ptr)descs_;
   char* lds = reinterpret_cast<char*>(smem);
-  // flags, then nb x buffers of xbuf_bytes each, then kYSlots y buffers of ybuf_floats floats
+  // flags, then the ring of activations, then (at byte ybuf0) kYSlots buffers of ybuf_floats row sums
   ListFlags* flags = reinterpret_cast<ListFlags*>(lds);
-  char* xbuf = lds + sizeof(ListFlags);
-  float* ybuf = reinterpret_cast<float*>(xbuf + nb * xbuf_bytes);
+  float* ybuf = reinterpret_cast<float*>(lds + ybuf0);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -140,120 +137,128 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
 
   if (wave < NC) {
     // =========================== compute wavefront ===========================
-    // Rows are taken one at a time from the workgroup's sequence (an LDS counter), so the NC
-    // wavefronts stay balanced whatever the row lengths; the next position is fetched one row ahead.
-    //
     // The ring.  Its loads are written in assembly and waited for by hand.  Every turn of a slot issues
     // exactly two loads (16 bytes of codes and one scale per lane), also when the list has run out
     // (then from an empty buffer: nothing is fetched), and no other path of a compute wavefront
     // issues a vector memory operation: loads retire in order, so "at most 2 (D - 1) outstanding"
     // says that the oldest slot has landed.  (Left to the compiler, the wait of the first slot of the
-    // unrolled loop comes out as "all but one".)  The loads are buffer loads over ONE ROW (base = the row, size = its
-    // bytes): lanes beyond the end of a row whose K is not a multiple of 2048 receive zeros for codes
-    // and scale, and the x wavefronts zero the activations of those groups, so a partial last chunk
-    // needs no code of its own.
-    // A wavefront issues one instruction every four cycles, so what a chunk costs is its instruction
-    // count: what the consumer needs (where the activations are, whether the row ends) is packed into
-    // two scalars per slot when the chunk is issued; everything per row or per linear is off the path.
+    // unrolled loop comes out as "all but one".)  The loads are buffer loads over ONE ROW (base = the
+    // row, size = its bytes): lanes beyond the end of a row whose K is not a multiple of 2048 receive
+    // zeros for codes and scale, and the x wavefronts zero the activations of those groups, so a
+    // partial last chunk needs no code of its own.
     const int b = blockIdx.x;
     const uint32_t lane16 = lane * 16;
     if (tid < (int)(sizeof(ListFlags) / sizeof(int))) reinterpret_cast<int*>(flags)[tid] = 0;
     lds_done_then_barrier();  // LDS starts undefined: the flags are cleared before anyone looks
 
-    constexpr int kLast = 1, kNewLinear = 2, kDead = 4;  // slot flags (bits 0..7 of slot_meta; the rest: LDS offset of x)
+    // slot state, two scalars.  meta: LDS offset of the chunk's activations (a multiple of 16) + the chunks of the row
+    // that follow this one (0: the row ends here) + kFirst (the group's first chunk: are the activations there?) or
+    // kDead (the list has run out).  yl: LDS offset of the row's sum | linear << 18.
+    constexpr int kFirst = 1 << 24, kDead = 1 << 25;
     uint4_t rw[D];
     uint32_t rs[D];
-    int slot_meta[D];   // flags | LDS byte offset of the chunk's activations << 8
-    int slot_yl[D];     // LDS byte offset of the row sum | linear << 18
-    const int xbuf0 = (int)sizeof(ListFlags);
-    const int ybuf0 = xbuf0 + nb * xbuf_bytes;
+    int slot_meta[D];
+    int slot_yl[D];
 
-    // the position counter: one lane adds, the answer is read one row later
-    int inext;
+    // the position counter: one lane adds.  The statement waits for its own answer: the compiler takes the
+    // output of an asm statement as there when the statement ends (it may copy it at once).
     auto take_position = [&]() {
+      int p = 0;
       if (lane == 0) {
         int one = 1;
-        asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=v"(inext) : "v"((uint32_t)(uintptr_t)&flags->next_pos), "v"(one) : "memory");
+        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                     : "=v"(p)
+                     : "v"((uint32_t)(uintptr_t)&flags->next_pos), "v"(one)
+                     : "memory");
       }
+      return __builtin_amdgcn_readfirstlane(p);
     };
-    take_position();
 
-    // issue side: the row being issued
-    RowCursor ic;
+    // issue side
+    GroupCursor ic;
     ic.lin = 0;
     ic.base = 0;
-    row_cursor_load(ic, descs, nlin, b, nwg, gs);
+    group_cursor_load(ic, descs, nlin, b, nwg, gs);
+    int i_rows = 0;       // rows of the group still to start
     int i_left = 0;       // chunks of the row still to issue
-    int i_off = 0;        // byte offset of the next chunk in the row of codes (in the row of scales: / 8)
+    int i_off = 0;        // byte offset of the next chunk in the row of codes
+    int i_soff = 0;       // ... and in the row of scales
     int i_x = 0;          // LDS offset of the next chunk's activations
+    int i_x0 = 0;         // ... of the row's first chunk
     int i_yl = 0;         // slot_yl of the row
-    int i_new = kNewLinear;  // the next chunk is this wavefront's first of a linear
+    int i_first = 0;      // kFirst until the group's first chunk has been issued
     // buffer resources of the row: base address, size in bytes, flags (an empty one: every lane reads zero, no memory access)
     auto row_rsrc = [](const char* p, int bytes) {
       const uint64_t a = reinterpret_cast<uint64_t>(p);
       return uint4_t{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)bytes, (uint32_t)kBufferFlags};
     };
     uint4_t i_w = row_rsrc(nullptr, 0), i_s = row_rsrc(nullptr, 0);
-    auto next_row = [&]() {  // the next position that holds a row (a last, partial row group has empty ones)
-      int64_t row;
+    auto next_group = [&]() {
       int pos;
-      int lin0 = ic.lin;
-      do {
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(inext)::"memory");  // the counter's answer has arrived
-        pos = __builtin_amdgcn_readfirstlane(inext);
-        take_position();
-        row_cursor_seek(ic, pos, descs, nlin, b, nwg, gs);
-        row = row_cursor_row(ic, pos, nwg, gs);
-      } while (ic.lin < nlin && row >= ic.N);
-      if (ic.lin >= nlin) {  // the list has run out: the slots drain
-        // nobody will read the counter's last answer: it must have landed before its register is used for something else
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(inext)::"memory");
-        i_left = -1;
-        i_w = row_rsrc(nullptr, 0);
-        i_s = i_w;
-        return;
+      uint32_t lp, row;
+      while (true) {
+        pos = take_position();
+        while (ic.lin < nlin && pos >= ic.base + ic.R) {
+          ic.base += ic.R;
+          ++ic.lin;
+          group_cursor_load(ic, descs, nlin, b, nwg, gs);
+        }
+        if (ic.lin >= nlin) {  // the list has run out: the slots drain
+          i_left = -1;
+          i_w = row_rsrc(nullptr, 0);
+          i_s = i_w;
+          return;
+        }
+        // position -> (row group of this workgroup, part of it) -> first row; N < 2^30: 32 bits hold it
+        lp = (uint32_t)(pos - ic.base) << ic.ts;  // first row of the position among the workgroup's rows of the linear
+        row = (((lp >> gs) * (uint32_t)nwg + (uint32_t)ic.rb) << gs) + (lp & ((1u << gs) - 1));
+        if ((int)row < ic.N) break;  // (else a part of the linear's last row group that lies beyond its last row)
       }
-      if (ic.lin != lin0) i_new = kNewLinear;
+      i_rows = min(1 << ic.ts, ic.N - (int)row) - 1;
+      const uint64_t woff = (uint64_t)row * (uint32_t)ic.row_w;  // a row of scales is an eighth of a row of codes
+      i_w = row_rsrc(ic.W + woff, ic.row_w);
+      i_s = row_rsrc(ic.S + (woff >> 3), ic.row_s);
       i_left = ic.C;
-      i_off = 0;
-      i_w = row_rsrc(ic.W + row * ic.row_w, ic.row_w);
-      i_s = row_rsrc(ic.S + row * ic.row_s, ic.row_s);
-      i_x = xbuf0 + (ic.lin & (nb - 1)) * xbuf_bytes;
-      i_yl = (ybuf0 + ((ic.lin & (kYSlots - 1)) * ybuf_floats + (pos - ic.base)) * 4) | (ic.lin << 18);
+      i_off = i_soff = 0;
+      i_x = i_x0 = ic.xoff;
+      i_yl = (ybuf0 + ((ic.lin & (kYSlots - 1)) * ybuf_floats + (int)lp) * 4) | (ic.lin << 18);
+      i_first = kFirst;
+    };
+    auto next_row = [&]() {  // the row behind the one just issued
+      --i_rows;
+      uint64_t a = ((uint64_t)i_w.y << 32 | i_w.x) + (uint32_t)ic.row_w;
+      i_w.x = (uint32_t)a;
+      i_w.y = (uint32_t)(a >> 32);
+      a = ((uint64_t)i_s.y << 32 | i_s.x) + (uint32_t)ic.row_s;
+      i_s.x = (uint32_t)a;
+      i_s.y = (uint32_t)(a >> 32);
+      i_left = ic.C;
+      i_off = i_soff = 0;
+      i_x = i_x0;
+      i_yl += 4;
     };
 
     auto issue = [&](uint4_t& w, uint32_t& s, int& meta, int& yl) {
-      if (i_left == 0) next_row();
+      if (i_left == 0) {
+        if (i_rows > 0) next_row();
+        else next_group();
+      }
       asm volatile(
           "buffer_load_dwordx4 %0, %2, %3, %4 offen nt\n\t"
           "buffer_load_ushort %1, %5, %6, %7 offen nt"
           : "=&v"(w), "=&v"(s)
-          : "v"(lane16), "s"(i_w), "s"(i_off), "v"(lane16 >> 3), "s"(i_s), "s"(i_off >> 3));
+          : "v"(lane16), "s"(i_w), "s"(i_off), "v"(lane16 >> 3), "s"(i_s), "s"(i_soff));
       if (i_left < 0) {
         meta = kDead;
         return;
       }
       --i_left;
-      meta = (i_x << 8) | i_new | (i_left == 0 ? kLast : 0);
+      meta = (i_x + i_left) | i_first;
       yl = i_yl;
-      i_new = 0;
+      i_first = 0;
       i_off += 1024;
+      i_soff += 128;
       i_x += kChunkBytes;
-    };
-
-    // Every compute wavefront passes through every linear, also those in which it takes no row:
-    // leaving linear e says "my row sums of e are in LDS and I no longer read its activations".
-    int entered = -1;
-    auto advance_to = [&](int lin) {
-      while (entered < lin) {
-        if (entered >= 0) {
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          if (lane == 0)
-            __hip_atomic_fetch_add(&flags->left[entered & (nb - 1)], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
-        ++entered;
-        if (entered < nlin) lds_spin_until(&flags->x_ready[entered & (nb - 1)], entered + 1);
-      }
     };
 
     // `magic` (0x6400 in both halves, OR-ed under every code) doubles as the token that orders the
@@ -274,12 +279,15 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       return r;
     };
     auto consume = [&](const uint4_t& w4, const uint32_t& s16, int meta, int yl) {
-      if (meta & kNewLinear) advance_to(yl >> 18);
-      const char* xb = lds + (meta >> 8);
+      if (meta & kFirst) {  // the first chunk of a group: the activations of its linear must be staged
+        const int lin = yl >> 18;
+        lds_spin_until(&flags->x_ready[lin & (kYSlots - 1)], lin + 1);
+      }
+      const char* xb = lds + (meta & 0xfffff0) + lane16;
       uint4_t xv[4];
 #pragma unroll
-      for (int ch = 0; ch < 4; ++ch) xv[ch] = *reinterpret_cast<const uint4_t*>(xb + ch * 1024 + lane16);
-      float grp = *reinterpret_cast<const float*>(xb + 4096 + (lane16 >> 2));
+      for (int ch = 0; ch < 4; ++ch) xv[ch] = *reinterpret_cast<const uint4_t*>(xb + ch * 1024);
+      float grp = *reinterpret_cast<const float*>(xb + 4096);
       // every slot is always in flight (the drained ones with loads that fetch nothing): this one is the oldest
       asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"(2 * (D - 1)));
 #pragma unroll
@@ -296,9 +304,16 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         grp = dot2(t3, as_half2(xv[ch].w), grp);
       }
       acc = fmaf(ring_scale(s16), grp, acc);
-      if (meta & kLast) {
+      if ((meta & 15) == 0) {  // the row ends here
         const float tot = wave_sum_to_lane63(acc);
-        if (lane == 63) *reinterpret_cast<float*>(lds + (yl & 0x3ffff)) = tot;
+        if (lane == 63) {
+          *reinterpret_cast<float*>(lds + (yl & 0x3ffff)) = tot;
+          // LDS is served in order: whoever sees the count sees the sum.  (Written out: the compiler's
+          // own lowering of a one-lane atomic elects a lane and counts the others first.)
+          const uint32_t done_at = (uint32_t)(uintptr_t)&flags->done[0] + (((uint32_t)yl >> 18) & (kYSlots - 1)) * 4;
+          int one = 1;
+          asm volatile("ds_add_u32 %0, %1" ::"v"(done_at), "v"(one) : "memory");
+        }
         acc = 0.0f;
       }
     };
@@ -318,20 +333,20 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       }
     }
     // the drained slots still have their (empty) loads in flight: they must have landed before the
-    // ring's registers are used for something else
+    // ring's registers are used for something else (there is nothing else: the wavefront ends here)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    advance_to(nlin);
     return;
   }
 
   lds_done_then_barrier();  // the flags are cleared
+  // The service wavefronts are the youngest of their SIMDs, and the arbiter serves the oldest first: at equal
+  // priority the compute wavefronts, which never run out of instructions, starve them, and then wait for them.
+  __builtin_amdgcn_s_setprio(3);
   bool aborted = false;
 
   if (wave < NC + XW) {
     // ====================== x wavefronts: activations -> LDS ======================
     // until every workgroup has signalled linear `dep`, or the spin limit passes
-    int cur_j = -1;
-    (void)cur_j;
     auto wait_for = [&](int dep) {
       if (aborted) return;
       const long long t0 = wall_clock64();
@@ -367,13 +382,10 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       if (lane == 0) j = __hip_atomic_fetch_add(&flags->next_x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       j = __builtin_amdgcn_readfirstlane(j);
       if (j >= nlin) break;
-      const int slot = j & (nb - 1);
-      // the slot is free once every compute wavefront has left the linear that used it before; the
-      // row-sum slot of linear j once the sums of linear j - kYSlots have been stored
-      if (j >= nb) lds_spin_until(&flags->left[slot], NC * (((j - nb) >> nb_log2) + 1));
-      if (j >= kYSlots) lds_spin_until(&flags->flushed, j - kYSlots + 1);
+      // its part of the ring (and its flags and row-sum buffer) is free once the linears that used them
+      // before have been flushed: all their rows have been consumed by then
+      lds_spin_until(&flags->flushed, descs[j].free_after);
       const int dep = (int)((descs[j].g_dep >> 16) & 0x7fffu) - 1;
-      cur_j = j;
       if (dep >= 0) wait_for(dep);
       const int K = (int)(descs[j].g_dep & 0xffffu) << 5;
       // an x that other workgroups of this launch have written is read with device-scope loads
@@ -381,7 +393,7 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       // without invalidating any cache; an x from outside the list with ordinary loads
       const __amdgpu_buffer_rsrc_t xr =
           __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(descs[j].x), 0, K * 2, kBufferFlags);
-      char* xb = xbuf + slot * xbuf_bytes;
+      char* xb = lds + descs[j].x_off;
       const int nwords = (((K >> 5) + 63) & ~63) << 2;  // 16-byte words of 8 activations, up to the end of the last chunk
                                                         // (beyond K the buffer loads return zeros)
       constexpr int U = 16;       // loads in flight per lane: one round trip per 16 KiB of x
@@ -411,28 +423,32 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
             char* cb = xb + (grp >> 6) * kChunkBytes;
             *reinterpret_cast<uint4_t*>(cb + ch * 1024 + (grp & 63) * 16) =
                 uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
-            if (ch == 0) *reinterpret_cast<float*>(cb + 4096 + (grp & 63) * 4) = -c;
+            if (ch == 0) *reinterpret_cast<float*>(cb + 4096 + (grp & 63) * 16) = -c;
           }
         }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      if (lane == 0) __hip_atomic_store(&flags->x_ready[slot], j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (lane == 0) __hip_atomic_store(&flags->x_ready[j & (kYSlots - 1)], j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     return;
   }
 
   // ================== y wavefront: row sums -> y, completion signals ==================
   for (int j = 0; j < nlin; ++j) {
-    const int slot = j & (nb - 1);
-    lds_spin_until(&flags->left[slot], NC * ((j >> nb_log2) + 1));
     const half_t* bias = descs[j].bias;
     const half_t* residual = descs[j].residual;
-    const float* yb = ybuf + (j & (kYSlots - 1)) * ybuf_floats;
+    const int yslot = j & (kYSlots - 1);
+    const float* yb = ybuf + yslot * ybuf_floats;
     int rb = (int)blockIdx.x - (int)descs[j].off;
     if (rb < 0) rb += nwg;
     const int N = descs[j].N;
     const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[j].y, 0, N * 2, kBufferFlags);
-    const int R = (descs[j].q + (rb < (int)descs[j].rem ? 1 : 0)) << gs;
+    const int groups = descs[j].q + (rb < (int)descs[j].rem ? 1 : 0);
+    const int R = groups << gs;  // places of this workgroup's rows in the buffer (those of a partial last group beyond N stay empty)
+    // rows of this workgroup: all its groups are whole except the linear's last one
+    const int last_row = (((groups - 1) * nwg + rb) << gs);
+    const int rows = groups == 0 ? 0 : R - max(0, last_row + (1 << gs) - N);
+    lds_spin_until(&flags->done[yslot], rows);
     for (int idx = lane; idx < R; idx += 64) {
       const int64_t n = ((((int64_t)(idx >> gs)) * nwg + rb) << gs) + (idx & ((1 << gs) - 1));
       if (n < N) {
@@ -444,9 +460,12 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (int)n * 2, 0, kDeviceScope);
       }
     }
-    // the row sums are in registers or stored: the slot may be written again
+    // the row sums are in registers or stored: the slots may be written again
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (lane == 0) __hip_atomic_store(&flags->flushed, j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (lane == 0) {
+      __hip_atomic_store(&flags->done[yslot], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_store(&flags->flushed, j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     if (descs[j].g_dep & kSignal) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores of this workgroup have been written through
       if (lane == 0)
@@ -564,8 +583,13 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
     for (int j = i - 1; j >= 0; --j) {
       const wq_q4g32_gemv_desc& b = e[j];
       const size_t yb = (size_t)b.N * 2 * rows[j], xb = (size_t)b.K * 2 * rows[j];
-      if (((l->descs[i].g_dep >> 16) & 0x7fffu) == 0 && ranges_overlap(a.x, xa, b.y, yb))
+      if (ranges_overlap(a.x, xa, b.y, yb)) {
+        // one producer per linear: the consumer waits for a single counter set
+        if (((l->descs[i].g_dep >> 16) & 0x7fffu) != 0)
+          return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations of linear %d are written by more than one linear of the list (%d and %d)",
+                     i, j, (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1);
         l->descs[i].g_dep |= (uint32_t)(j + 1) << 16;
+      }
       if (ranges_overlap(a.residual, ya, b.y, yb) || ranges_overlap(a.bias, (size_t)a.N * 2, b.y, yb))
         return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i, j);
       if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, xb) ||
@@ -600,15 +624,49 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
     off = (off + groups) % l->blocks;
     turns = std::max<int64_t>(turns, ((groups + l->blocks - 1) / l->blocks) << l->gs);
   }
-  l->xbuf_bytes = cmax * kChunkBytes;
   l->ybuf_floats = (int)((turns + 63) / 64 * 64);
-  // 8 buffer slots (linears the service wavefronts may run ahead of or behind the compute wavefronts) if they fit
-  // (a list of 96 linears of 4096 x 4096: 2.2 -> 2.0 us per linear against 4 slots), else 4 or 2
-  const size_t fixed = sizeof(ListFlags) + (size_t)kYSlots * l->ybuf_floats * sizeof(float);
-  const size_t room = fixed < 150 * 1024 ? 150 * 1024 - fixed : 0;
-  l->nb = room / l->xbuf_bytes >= 8 ? 8 : room / l->xbuf_bytes >= 4 ? 4 : room / l->xbuf_bytes >= 2 ? 2 : 0;
-  if (l->nb < 2) return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations and row sums do not fit the LDS");
-  l->lds = fixed + (size_t)l->nb * l->xbuf_bytes;
+  // LDS: flags, the ring of activations, kYSlots buffers of row sums.  A linear takes as much of the ring as its
+  // row is long, from where its predecessor ends (from the start again if it does not fit before the end), and
+  // may be staged once every earlier linear whose part overlaps its own has been flushed, and the linear that
+  // used its flags and row-sum buffer before (kYSlots back).
+  const size_t ysums = (size_t)kYSlots * l->ybuf_floats * sizeof(float);
+  const size_t lds_budget = 150 * 1024;
+  if (sizeof(ListFlags) + ysums + (size_t)cmax * kChunkBytes > lds_budget)
+    return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations and row sums do not fit the LDS");
+  const int ring0 = (int)sizeof(ListFlags), ring1 = (int)(lds_budget - ysums);
+  l->ybuf0 = ring1;
+  l->lds = lds_budget;
+  {
+    int at = ring0;
+    std::vector<int> lo(ne), hi(ne);
+    for (int i = 0; i < ne; ++i) {
+      const int size = (int)((e[i].K / 32 + 63) / 64) * kChunkBytes;
+      if (at + size > ring1) at = ring0;
+      lo[i] = at;
+      hi[i] = at + size;
+      at += size;
+      int after = std::max(0, i - kYSlots + 1);
+      for (int j = i - 1; j >= 0 && j + 1 > after; --j)
+        if (lo[j] < hi[i] && lo[i] < hi[j]) after = j + 1;
+      l->descs[i].x_off = (uint32_t)lo[i];
+      l->descs[i].free_after = after;
+    }
+  }
+  // rows a compute wavefront takes at a time: whole row groups where a workgroup has many rows of the linear
+  // (what a position costs beyond its chunks is paid once), pairs where it has few, single rows at the end of the
+  // list (the launch ends when the last wavefront does).  Measured on the four Llama-2-7B shapes: whole groups
+  // for the 4096-row linears as well cost the 32-layer stack 4 %, single rows everywhere cost the 4-linear
+  // step 4 %.
+  {
+    double tail = 0;  // weights behind the linear: about 2 us of the machine's stream are "the end of the list"
+    for (int i = ne - 1; i >= 0; --i) {
+      const int64_t per_wg = e[i].N / l->blocks;
+      int ts = per_wg >= 32 ? l->gs : per_wg >= 8 ? std::min(1, l->gs) : 0;
+      if (tail < 32e6) ts = 0;
+      tail += (double)e[i].N * e[i].K;
+      l->descs[i].ts = (uint8_t)ts;
+    }
+  }
   auto kern = q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>;
   static DynamicLdsLimit limit;  // several lists share the kernel: the limit only ever grows
   if (l->lds > 48 * 1024 && limit.ensure(reinterpret_cast<const void*>(kern), (int)l->lds) != hipSuccess)
@@ -633,7 +691,7 @@ extern "C" int wq_q4g32_gemv_list_run(wq_gemv_list_t* l, wq_stream_t stream) {
   if (l->M > 1) return batch_list_launch(l, (hipStream_t)stream);
   WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>), dim3((unsigned)l->blocks),
             dim3((unsigned)l->threads), l->lds, (hipStream_t)stream, (const GemvListDesc*)l->table, l->n, l->sync,
-            l->spin_limit, l->xbuf_bytes, l->ybuf_floats, l->nb == 8 ? 3 : l->nb == 4 ? 2 : 1, l->gs, l->deps > 0 ? 1 : 0);
+            l->spin_limit, l->ybuf0, l->ybuf_floats, l->gs, l->deps > 0 ? 1 : 0);
   return WQ_OK;
 }
 

@@ -194,6 +194,13 @@ def test_argument_errors(env, oracle):
     c = _linear(oracle, u, 64, 256, 4, seed=1)
     with pytest.raises(ValueError):
         ops.Q4G32GemvList([(c["dW"], c["dS"], u.dev(c["x"])[:2], y)], M=4)
+    with pytest.raises(WqError, match="more than one linear"):
+        # an x that two earlier linears of the list write: the consumer could only wait for one of them
+        d = _linear(oracle, u, 256, 256, 4, seed=2)
+        xd = u.dev(d["x"])
+        h = torch.zeros((4 * 256,), dtype=torch.float16, device="cuda")   # [4, 256], written in two pieces
+        ops.Q4G32GemvList([(d["dW"][:128], d["dS"][:128], xd, h[:512]), (d["dW"][:128], d["dS"][:128], xd, h[512:]),
+                           (d["dW"], d["dS"], h, torch.zeros((4, 256), dtype=torch.float16, device="cuda"))], M=4)
 
 
 def test_a_wait_that_runs_out_is_reported_and_every_wavefront_exits(env, oracle):

@@ -168,5 +168,11 @@ def test_argument_errors(env, oracle):
     with pytest.raises(WqError, match="bias or residual"):
         y2 = torch.zeros((1, 64), dtype=torch.float16, device="cuda")
         ops.Q4G32GemvList([(a["dW"], a["dS"], x, y), (a["dW"], a["dS"], x, y2, None, y)])
+    with pytest.raises(WqError, match="more than one linear"):
+        # q / k written side by side by two linears and read as one [1, 128] tensor by a third: the
+        # consumer could only wait for one of the producers
+        qk = torch.zeros((1, 128), dtype=torch.float16, device="cuda")
+        y3 = torch.zeros((1, 64), dtype=torch.float16, device="cuda")
+        ops.Q4G32GemvList([(a["dW"], a["dS"], x, qk[:, :64]), (a["dW"], a["dS"], x, qk[:, 64:]), (a["dW"], a["dS"], qk, y3)])
     with pytest.raises(ValueError):
         ops.Q4G32GemvList([(a["dW"], a["dS"], x[:, :64], y)])
