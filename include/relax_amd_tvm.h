@@ -42,7 +42,8 @@ WQ_PACKED(cutlass_ft_preprocess_weight);
 WQ_PACKED(relax_amd_ft_preprocess_weight_dps);
 
 /* Format A (q4f16_1).  Buffer order of the reference's PrimFuncs
- * (tests/python/dlight/test_gpu_gemv.py:189, test_gpu_matmul.py:352):
+ * (tests/python/dlight/test_gpu_gemv.py:189, test_gpu_matmul.py:352; of the latter the argument order and the
+ * epilogue chain :378-401 only: its weights are packed along N, W[k, n/8], which no entry point takes):
  * "relax_amd.q4f16_1_matmul"(W u32[N,K/8], S f16[N,K/32], x f16[..,K], out f16[..,N])
  * "relax_amd.q4f16_1_matmul_bias"(W, S, x, bias f16[N], out)
  * "relax_amd.q4f16_1_matmul_bias_residual"(W, S, x, bias f16[N], residual f16[..,N], out) */

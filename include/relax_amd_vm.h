@@ -91,16 +91,27 @@ int wq_program_num_instructions(const wq_program_t* p);
  * between the instructions is kept), and the planned tensors of the run do not share storage.
  * The descriptor tables live in the workspace (wq_program_plan accounts for them) and are
  * uploaded by the first wq_program_run / wq_program_capture after the plan or a rebind.
- * Option "fuse_decode" (default 1) switches this off; set it before wq_program_plan. */
+ * Option "fuse_decode" (default 1) switches this off; set it before wq_program_plan.
+ * Option "spin_limit_us": the longest a fused run's wait for a producer linear may last, in microseconds
+ * (default: 2 s, the lists' own; wq_q4g32_gemv_list_set_spin_limit); drops a captured graph. */
 int wq_program_set_option(wq_program_t* p, const char* name, int value);
 /* Number of runs that are executed fused (after the first run or capture). */
 int wq_program_num_fused_groups(const wq_program_t* p);
+/* A run that could not be built as a list (operands that alias in a way the list kernel cannot order) is
+ * executed instruction by instruction, which is always valid; this returns what the list kernel said about
+ * run `group` (numbered as found by wq_program_plan, 0 ..), or "" for a run that is fused or unknown. */
+const char* wq_program_unfused_reason(const wq_program_t* p, int group);
 /* The order in which run `group` walks its instructions: writes up to `capacity` instruction
  * indices to `order` and returns how many the run holds. */
 int wq_program_fused_order(const wq_program_t* p, int group, int* order, int capacity);
 /* Synchronises `stream` and reports a device-side wait of a fused run that hit its spin limit
  * (see wq_q4g32_gemv_list_status). */
 int wq_program_status(wq_program_t* p, wq_stream_t stream);
+/* The same check without synchronising (see wq_q4g32_gemv_list_poll): enqueues asynchronous copies of the
+ * error words of the fused runs, one per run in program order, into host_words[0 .. capacity) (pinned host
+ * memory of the caller) and returns the number of fused runs (>= 0; words beyond `capacity` are not copied),
+ * or a negative code.  All words zero once the stream has passed: no wait has run out. */
+int wq_program_poll(wq_program_t* p, int* host_words, int capacity, wq_stream_t stream);
 
 #if defined(__GNUC__)
 #pragma GCC visibility pop

@@ -55,8 +55,12 @@ const char* wq_target_arch(void);
  * Replaces the generated kernels of the TIR functions in
  *   tests/python/dlight/test_gpu_reduction.py:33-51, 400-424     (M = 1)
  *   tests/python/dlight/test_gpu_low_batch_gemv.py:30-57         (small batch)
- *   tests/python/dlight/test_gpu_matmul.py:352-401               (prefill + epilogue)
+ *   tests/python/dlight/test_gpu_matmul.py:378-401               (prefill: the EPILOGUE chain only, see below)
  * which the reference schedules with python/tvm/dlight/gpu/{gemv,low_batch_gemv,matmul}.py.
+ * Not served: the weight layout of that prefill fixture itself.  Its decode block (test_gpu_matmul.py:366-377)
+ * reads W[k, n/8] and S[k, n/32]: the codes are packed along N and a scale covers 32 consecutive n of one k, a
+ * third scheme next to the two of the decode fixtures (rows of 32 k here, K-major words in wq_q4g32_kn_*).  Its
+ * square 4096 x 4096 shape hides the difference; no entry point of this library takes it.
  * Requirements: K % 32 == 0; W, S rows 16-byte aligned (true for K % 32 == 0
  * and 16-byte aligned bases).
  * ------------------------------------------------------------------------- */
@@ -116,6 +120,21 @@ int wq_q4g32_gemv_f16acc(const uint32_t* W, const uint16_t* S, const uint16_t* x
  *   status  synchronises `stream` and reports a wait that ran into the spin limit (WQ_EDEVICE):
  *           this happens only if the grid could not be resident at once, e.g. while another
  *           kernel holds CUs; the results of that launch are undefined.
+ *   poll    the same check without synchronising, for a serving loop that must not stall: enqueues an
+ *           asynchronous copy of the list's error word into `*host_word` (pinned host memory of the caller,
+ *           e.g. from hipHostMalloc) behind the work already on `stream`.  Once the stream has passed that
+ *           point the word is 0, or non-zero if a wait of an earlier launch ran out (then call status, which
+ *           names the linear and resets the counters).  No allocation: capturable.
+ * The kernels rely on two properties of the device that the HIP memory model does not promise.  (1) All
+ * workgroups of a launch are resident at once (one per CU; sized from the occupancy the runtime reports): a
+ * consumer spins on counters that workgroups on other CUs raise.  A kernel of another stream that holds CUs
+ * breaks this; the spin limit turns the resulting dead wait into the error word above instead of a hang.
+ * (2) A producer publishes y with device-scope (sc1) write-through stores, waits for them (vmcnt), then raises
+ * its counter with a relaxed device-scope atomic; the consumer polls the counter with read-modify-write atomics
+ * (performed at the memory side, never served from a stale line), takes a device-scope acquire fence and reads x
+ * with sc1 loads.  There is no release fence (the L2 write-back it implies costs 9 - 17 us per linear on this
+ * part).  This is the gfx950 cache hierarchy's behaviour, checked by the eager-against-replay bit-equality
+ * tests of 32-layer stacks, not a guarantee of the language.
  * NULL from create / non-zero from the others: see wq_last_error(). */
 typedef struct wq_q4g32_gemv_desc {
   const uint32_t* W;        /* uint32 [N, K/8] */
@@ -142,6 +161,7 @@ wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv_desc* desc
                                                   size_t workspace_bytes, wq_stream_t stream);
 int wq_q4g32_gemv_list_run(wq_gemv_list_t* list, wq_stream_t stream);
 int wq_q4g32_gemv_list_status(wq_gemv_list_t* list, wq_stream_t stream);
+int wq_q4g32_gemv_list_poll(wq_gemv_list_t* list, int* host_word, wq_stream_t stream);
 void wq_q4g32_gemv_list_destroy(wq_gemv_list_t* list);
 /* How many linears of the list wait for an earlier one, and how many of those for the linear
  * directly in front of them (those cannot overlap with it; order lists to keep this number low). */
@@ -281,7 +301,8 @@ int wq_gptq_prepare_padded(const uint32_t* qweight, const uint32_t* qzeros, cons
                            int64_t* K_padded, int64_t K, int64_t N, int64_t G, wq_stream_t stream);
 /* The linear over operands prepared by wq_gptq_prepare_padded: x fp16 [M, K] is gathered into the workspace
  * (M * K_padded * 2 bytes, 16-byte aligned; zeros at the padding), then the kernels of wq_gptq_linear run with
- * K_padded rows in groups of 32.  K_padded <= 32768. */
+ * K_padded rows in groups of 32.  K_padded <= 32768.  K is the row length of x: an entry of perm that is not
+ * below K (operands prepared for a wider checkpoint) gathers a zero, it never reads beyond the row. */
 size_t wq_gptq_padded_workspace_bytes(int64_t M, int64_t K_padded);
 int wq_gptq_linear_padded(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
                           const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
@@ -306,7 +327,10 @@ int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm
  * (WQ_GPTQ_NOALLOC_MAX_BYTES of device memory per GPU, held until the process ends), so
  * M*K*2 must not exceed that size; larger problems are refused with WQ_EINVAL.  The call
  * allocates nothing.  Every call on a GPU shares that GPU's buffer: calls that overlap in time
- * on one GPU (different streams) race; calls on one stream are ordered. */
+ * on one GPU (different streams) race; calls on one stream are ordered.
+ * The first call with a row order on a device looks the buffer's address up (hipGetSymbolAddress,
+ * which may load the code object): make that call outside a stream capture.  A call with M = 0
+ * and a non-null perm does the look-up and nothing else. */
 #define WQ_GPTQ_NOALLOC_MAX_BYTES (1u << 20)
 int wq_gptq_linear_noalloc(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm, const uint16_t* x,
                            const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,

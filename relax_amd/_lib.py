@@ -30,6 +30,7 @@ SIGNATURES = {
     "wq_q4g32_gemv_list_create_batched": [_vp, _int, _int, _vp, _sz, _vp],
     "wq_q4g32_gemv_list_run": [_vp, _vp],
     "wq_q4g32_gemv_list_status": [_vp, _vp],
+    "wq_q4g32_gemv_list_poll": [_vp, _vp, _vp],
     "wq_q4g32_gemv_list_destroy": [_vp],
     "wq_q4g32_gemv_list_info": [_vp, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)],
     "wq_q4g32_gemv_list_set_spin_limit": [_vp, ctypes.c_longlong],
@@ -69,11 +70,13 @@ SIGNATURES = {
     "wq_program_num_fused_groups": [_vp],
     "wq_program_fused_order": [_vp, _int, ctypes.POINTER(_int), _int],
     "wq_program_status": [_vp, _vp],
+    "wq_program_unfused_reason": [_vp, _int],
+    "wq_program_poll": [_vp, _vp, _int, _vp],
     "wq_activation_from_string": [ctypes.c_char_p],
     "wq_binary_op_from_string": [ctypes.c_char_p],
     "wq_unary_op_from_string": [ctypes.c_char_p],
 }
-_RESTYPES = {"wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p, "wq_program_create": _vp,
+_RESTYPES = {"wq_program_unfused_reason": ctypes.c_char_p, "wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p, "wq_program_create": _vp,
              "wq_program_destroy": None, "wq_program_plan": _i64, "wq_program_unplanned_bytes": _i64,
              "wq_gptq_workspace_bytes": _sz, "wq_q4g32_kn_gemv_workspace_bytes": _sz, "wq_gptq_padded_workspace_bytes": _sz, "wq_gptq_padded_k_bound": _i64, "wq_q4g32_gemv_list_workspace_bytes": _sz,
              "wq_q4g32_gemv_list_create": _vp, "wq_q4g32_gemv_list_create_batched": _vp, "wq_q4g32_gemv_list_destroy": None}

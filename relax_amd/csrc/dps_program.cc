@@ -47,6 +47,7 @@ struct FusedGroup {
   int64_t ws_offset = 0;       // the list's descriptor table and counters inside the workspace
   wq_gemv_list_t* list = nullptr;
   bool failed = false;         // the list could not be built (aliasing operands): run one by one
+  std::string why;             // ... and what wq_q4g32_gemv_list_create said
 };
 
 // What a q4f16_1_matmul* instruction reads and writes, if it qualifies for a fused group.
@@ -67,6 +68,7 @@ struct wq_program {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
   bool fuse_decode = true;
+  long long spin_limit_ticks = -1;  // of the fused runs' waits, in ticks of the 100 MHz wall clock; < 0: the lists' default
   std::vector<FusedGroup> groups;
   bool lists_stale = true;  // a register moved: the lists must be rebuilt before the next run
 };
@@ -76,6 +78,7 @@ static void drop_lists(wq_program* p) {
     if (g.list) wq_q4g32_gemv_list_destroy(g.list);
     g.list = nullptr;
     g.failed = false;
+    g.why.clear();
   }
   p->lists_stale = true;
 }
@@ -139,6 +142,14 @@ extern "C" int wq_program_set_option(wq_program_t* p, const char* name, int valu
     drop_graph(p);
     drop_lists(p);
     p->groups.clear();
+    return WQ_OK;
+  }
+  if (std::string(name) == "spin_limit_us") {
+    WQ_REQUIRE(value >= 0, "wq_program_set_option: spin_limit_us must not be negative");
+    p->spin_limit_ticks = (long long)value * 100;
+    for (FusedGroup& g : p->groups)
+      if (g.list) (void)wq_q4g32_gemv_list_set_spin_limit(g.list, p->spin_limit_ticks);
+    drop_graph(p);  // a captured launch carries the old limit as a kernel argument
     return WQ_OK;
   }
   return wq::fail(WQ_EINVAL, "wq_program_set_option: unknown option '%s'", name);
@@ -323,6 +334,13 @@ static void find_groups(wq_program* p) {
     int j = i;
     while (j < n && (int)lin.size() < WQ_GEMV_LIST_MAX && as_decode_linear(p, p->instrs[j], &d) &&
            (lin.empty() || d.M == lin[0].M)) {  // one list, one batch size
+      // The list kernel orders a linear behind ONE earlier linear, through its x.  A bias or a residual that an
+      // earlier linear of the run writes (the residual stream: down_proj adds what o_proj produced) is refused
+      // by wq_q4g32_gemv_list_create: the run ends in front of such an instruction, which starts the next one.
+      bool from_run = false;
+      for (const DecodeLinear& e : lin)
+        if ((d.bias >= 0 && d.bias == e.y) || (d.residual >= 0 && d.residual == e.y)) from_run = true;
+      if (from_run) break;
       lin.push_back(d);
       ++j;
     }
@@ -424,6 +442,10 @@ extern "C" int wq_program_set_workspace(wq_program_t* p, void* base, int64_t byt
 
 static int check_ready(wq_program* p, const char* who) {
   WQ_REQUIRE(p, "%s: null program", who);
+  // the descriptor tables and counters of the fused runs live in the workspace, also when every tensor is external
+  if (!p->groups.empty() && !p->workspace)
+    return wq::fail(WQ_EINVAL, "%s: the program has fused runs: plan it and set the workspace (%lld bytes)", who,
+                    (long long)p->workspace_bytes);
   for (const Reg& r : p->regs)
     if (r.first >= 0 && r.bytes > 0 && !r.dl.data)
       return wq::fail(WQ_EINVAL, "%s: a tensor has no storage (%s)", who,
@@ -451,7 +473,10 @@ static int build_lists(wq_program* p, hipStream_t stream) {
                                                wq_q4g32_gemv_list_workspace_bytes((int)descs.size()), stream);
     // operands that alias in a way the list kernel cannot order (or pointers it cannot take): the
     // group runs instruction by instruction, which is always valid
-    if (!g.list) g.failed = true;
+    if (!g.list) {
+      g.failed = true;
+      g.why = wq_last_error();
+    } else if (p->spin_limit_ticks >= 0) (void)wq_q4g32_gemv_list_set_spin_limit(g.list, p->spin_limit_ticks);
   }
   p->lists_stale = false;
   return WQ_OK;
@@ -534,11 +559,28 @@ extern "C" int wq_program_num_fused_groups(const wq_program_t* p) {
   return n;
 }
 
+extern "C" const char* wq_program_unfused_reason(const wq_program_t* p, int group) {
+  if (!p || group < 0 || group >= (int)p->groups.size()) return "";
+  return p->groups[group].why.c_str();
+}
+
 extern "C" int wq_program_fused_order(const wq_program_t* p, int group, int* order, int capacity) {
   WQ_REQUIRE(p && group >= 0 && group < (int)p->groups.size(), "wq_program_fused_order: no such group");
   const FusedGroup& g = p->groups[group];
   for (int i = 0; i < (int)g.order.size() && i < capacity; ++i) order[i] = g.order[i];
   return (int)g.order.size();
+}
+
+extern "C" int wq_program_poll(wq_program_t* p, int* host_words, int capacity, wq_stream_t stream) {
+  WQ_REQUIRE(p && (host_words || capacity == 0) && capacity >= 0, "wq_program_poll: bad argument");
+  int n = 0;
+  for (FusedGroup& g : p->groups) {
+    if (!g.list) continue;
+    if (n < capacity)
+      if (int rc = wq_q4g32_gemv_list_poll(g.list, host_words + n, stream)) return rc;
+    ++n;
+  }
+  return n;
 }
 
 extern "C" int wq_program_status(wq_program_t* p, wq_stream_t stream) {

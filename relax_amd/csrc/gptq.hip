@@ -190,7 +190,9 @@ __global__ __launch_bounds__(256) void gptq_gather_x_padded_kernel(const half_t*
   if (i < (KP >> 1)) {
     const int2 p = reinterpret_cast<const int2*>(perm)[i];
     const half_t zero = (half_t)0.0f;
-    reinterpret_cast<half2_t*>(xp + m * KP)[i] = half2_t{p.x >= 0 ? x[m * K + p.x] : zero, p.y >= 0 ? x[m * K + p.y] : zero};
+    // (an index beyond the row of x, from operands prepared for another K, reads nothing: it gathers a zero)
+    reinterpret_cast<half2_t*>(xp + m * KP)[i] =
+        half2_t{(unsigned)p.x < (unsigned)K ? x[m * K + p.x] : zero, (unsigned)p.y < (unsigned)K ? x[m * K + p.y] : zero};
   }
 }
 
@@ -499,6 +501,9 @@ extern "C" int wq_gptq_linear_noalloc(const uint32_t* W_nk, const uint16_t* SZ, 
   using namespace wq;
   void* ws = nullptr;
   size_t ws_bytes = 0;
+  // (also for M = 0: the way to have the address looked up ahead of a stream capture)
+  if (perm)
+    if (int rc = gptq_scratch_for_current_device(&ws)) return rc;
   if (perm && M > 0 && N > 0 && K > 0) {
     WQ_REQUIRE(M < (1ll << 30) && K <= 32768, "wq_gptq_linear_noalloc: M=%lld K=%lld outside the supported range",
                (long long)M, (long long)K);
@@ -507,7 +512,6 @@ extern "C" int wq_gptq_linear_noalloc(const uint32_t* W_nk, const uint16_t* SZ, 
                "wq_gptq_linear_noalloc: the gathered activations need M*K*2 = %zu bytes, the built-in scratch "
                "buffer holds %zu; use wq_gptq_linear with a workspace",
                need, kGptqScratchBytes);
-    if (int rc = gptq_scratch_for_current_device(&ws)) return rc;
     ws_bytes = kGptqScratchBytes;
   }
   return gptq_linear_impl(W_nk, SZ, perm, x, bias, residual, y, M, N, K, G, ws, ws_bytes, (hipStream_t)stream);

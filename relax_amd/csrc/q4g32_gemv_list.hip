@@ -715,6 +715,14 @@ extern "C" int wq_q4g32_gemv_list_status(wq_gemv_list_t* l, wq_stream_t stream) 
               err - 1);
 }
 
+extern "C" int wq_q4g32_gemv_list_poll(wq_gemv_list_t* l, int* host_word, wq_stream_t stream) {
+  using namespace wq;
+  WQ_REQUIRE(l && l->table && host_word, "wq_q4g32_gemv_list_poll: null argument");
+  // no synchronisation and no allocation: the word arrives when the stream gets here
+  WQ_HIP(hipMemcpyAsync(host_word, l->sync + sync_error_index(l->n), sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  return WQ_OK;
+}
+
 extern "C" int wq_q4g32_gemv_list_info(const wq_gemv_list_t* l, int* dependencies, int* adjacent) {
   using namespace wq;
   WQ_REQUIRE(l, "wq_q4g32_gemv_list_info: null list");

@@ -196,6 +196,14 @@ class Q4G32GemvList:
         """Synchronises and raises if a device-side wait of an earlier launch timed out."""
         check(self._l.wq_q4g32_gemv_list_status(self._h, _stream()), "wq_q4g32_gemv_list_status")
 
+    def poll(self, word: torch.Tensor) -> None:
+        """Enqueues an asynchronous copy of the error word into ``word`` (a pinned int32 host tensor of one
+        element) behind the work on torch's current stream; no synchronisation.  Non-zero once the stream has
+        passed: a wait of an earlier launch ran out (then :meth:`status` says which)."""
+        if word.dtype != torch.int32 or word.numel() != 1 or word.is_cuda or not word.is_pinned():
+            raise ValueError("word must be a pinned int32 host tensor of one element")
+        check(self._l.wq_q4g32_gemv_list_poll(self._h, word.data_ptr(), _stream()), "wq_q4g32_gemv_list_poll")
+
     def info(self):
         """(linears that wait for an earlier one, of which for the one directly in front)."""
         a, b = ctypes.c_int(0), ctypes.c_int(0)

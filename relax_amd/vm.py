@@ -107,7 +107,8 @@ class DpsProgram:
 
     # ---- fused decode linears ----
     def set_option(self, name: str, value: int) -> None:
-        """``fuse_decode`` (default 1): run consecutive decode linears as one launch.  Set before :meth:`plan`."""
+        """``fuse_decode`` (default 1): run consecutive decode linears as one launch; set before :meth:`plan`.
+        ``spin_limit_us``: the longest a fused run may wait for a producer linear (default 2 s)."""
         check(self._l.wq_program_set_option(self._p, name.encode(), int(value)), "wq_program_set_option")
 
     @property
@@ -125,6 +126,17 @@ class DpsProgram:
         """Synchronises and raises if a device-side wait of a fused run timed out."""
         s = (stream or torch.cuda.current_stream()).cuda_stream
         check(self._l.wq_program_status(self._p, s), "wq_program_status")
+
+    def poll(self, words: torch.Tensor, stream: torch.cuda.Stream = None) -> int:
+        """Asynchronous copies of the fused runs' error words into ``words`` (pinned int32 host tensor), no
+        synchronisation; returns the number of fused runs.  All zero once the stream has passed: no wait ran out."""
+        if words.dtype != torch.int32 or words.is_cuda or not words.is_pinned():
+            raise ValueError("words must be a pinned int32 host tensor")
+        s = (stream or torch.cuda.current_stream()).cuda_stream
+        n = int(self._l.wq_program_poll(self._p, words.data_ptr(), int(words.numel()), s))
+        if n < 0:
+            check(n, "wq_program_poll")
+        return n
 
     # ---- execution ----
     def run(self, stream: torch.cuda.Stream = None) -> None:

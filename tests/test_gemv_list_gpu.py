@@ -142,11 +142,18 @@ def test_a_wait_that_runs_out_is_reported_and_every_wavefront_exits(env, oracle)
     gl.set_spin_limit(0)
     print("gemv list: spin limit 0", flush=True)
     gl.run()
+    # the non-blocking check: the word lands in pinned host memory behind the launch, nothing synchronises
+    word = torch.zeros(1, dtype=torch.int32).pin_memory()
+    gl.poll(word)
+    torch.cuda.current_stream().synchronize()
+    assert word.item() != 0
     with pytest.raises(WqError, match="timed out"):
         gl.status()
     gl.set_spin_limit(200_000_000)
     gl.run()
+    gl.poll(word)
     gl.status()
+    assert word.item() == 0
     r0 = oracle.q4g32_linear(a["W"], a["S"], x0, nthreads=8)
     u.assert_close(u.host(t0), r0, "producer after a reported time-out")
     u.assert_close(u.host(t1), oracle.q4g32_linear(b["W"], b["S"], r0[:, :4096], nthreads=8), "consumer after a reported time-out")

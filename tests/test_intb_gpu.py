@@ -195,6 +195,10 @@ def test_int8_full_size_sampled(ops, u, oracle, M):
             yv = u.host(ops.fpA_intB_gemm(u.dev(x[r:r + 1]), P, u.dev(s), weight_nbit=8))
             u.assert_close(got[r:r + 1], yv, f"int8 full M={M} row {r} vs gemv")
     if M == 1:
+        # the reordered layout of the whole matrix (224 MiB), bit for bit against the oracle
+        want_P = oracle.ft_preprocess(u.host(dA), False, 80)
+        assert np.array_equal(u.host(P), want_P)
+        del want_P
         xh = np.zeros((1, K), np.float16)
         xh[0, 4321] = 1
         y = u.host(ops.fpA_intB_gemm(u.dev(xh), P, u.dev(s), weight_nbit=8))

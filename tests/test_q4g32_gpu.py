@@ -202,6 +202,22 @@ def test_small_batch_vs_oracle(ops, u, oracle, nw, waves, stages, M, N, K):
     u.assert_close(got, ref, f"small batch nw{nw} waves{waves} {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M", [1, 4, 5, 8])
+def test_low_batch_fixture_shape(ops, u, oracle, M):
+    """The shape of the reference's low-batch fixture (tests/python/dlight/test_gpu_low_batch_gemv.py:29-34:
+    N = 4096, K = 28672, a dynamic batch) at full size: the automatic dispatch and every kernel that serves it."""
+    N, K = 4096, 28672
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=M + 77)
+    print(f"low-batch fixture shape M={M}", flush=True)
+    ref = oracle.q4g32_linear(W, S, x, nthreads=8)
+    dW, dS, dx = u.dev(W), u.dev(S), u.dev(x)
+    u.assert_close(u.host(ops.q4g32_linear(dW, dS, dx)), ref, f"automatic {M}x{N}x{K}")
+    u.assert_close(u.host(ops.q4g32_linear(dW, dS, dx, kernel="gemv")), ref, f"gemv {M}x{N}x{K}")
+    if M >= 2:
+        u.assert_close(u.host(ops.q4g32_linear(dW, dS, dx, kernel="small_batch")), ref, f"small batch {M}x{N}x{K}")
+    u.assert_close(u.host(ops.q4g32_linear(dW, dS, dx, kernel="gemm")), ref, f"gemm {M}x{N}x{K}")
+
+
 @pytest.mark.parametrize("M", [8, 32])
 @pytest.mark.parametrize("N,K", [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)])
 def test_llama7b_shapes_at_decode_batches(ops, u, oracle, M, N, K):

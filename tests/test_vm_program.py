@@ -169,6 +169,64 @@ def test_short_runs_of_batched_linears_are_not_fused(M, n, fused):
         l.wq_program_destroy(p)
 
 
+def test_a_residual_from_the_run_ends_the_fused_run():
+    """Planning alone: the list kernel orders a linear behind one earlier linear through its x only, so an
+    instruction whose residual (or bias) is the output of an earlier linear of the run starts a new run instead
+    of making the whole run fall back to one launch per instruction."""
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        addr = [0x100000]
+
+        def ext(code, bits, *shape):
+            addr[0] += 0x100000
+            return l.wq_program_add_external(p, code, bits, len(shape), _shape(*shape), addr[0], 10)
+
+        x = ext(2, 16, 1, 256)
+        bias = ext(2, 16, 64)
+        ys = []
+        for i in range(5):
+            W, S, y = ext(1, 32, 64, 32), ext(2, 16, 64, 8), ext(2, 16, 1, 64)
+            if i == 3:  # the residual stream: the output of linear 1 is added to linear 3
+                assert _call(l, p, "relax_amd.q4f16_1_matmul_bias_residual", [W, S, x, bias, ys[1], y]) == 0
+            else:
+                assert _call(l, p, "relax_amd.q4f16_1_matmul", [W, S, x, y]) == 0
+            ys.append(y)
+        assert l.wq_program_plan(p) > 0  # the descriptor tables of the runs
+        buf = (ctypes.c_int * 8)()
+        assert l.wq_program_fused_order(p, 0, buf, 8) == 3 and sorted(buf[:3]) == [0, 1, 2]
+        assert l.wq_program_fused_order(p, 1, buf, 8) == 2 and sorted(buf[:2]) == [3, 4]
+        assert l.wq_program_unfused_reason(p, 0) == b""
+    finally:
+        l.wq_program_destroy(p)
+
+
+def test_options_and_a_program_of_external_tensors_only_needs_its_workspace():
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        assert l.wq_program_set_option(p, b"spin_limit_us", 50) == 0
+        assert l.wq_program_set_option(p, b"spin_limit_us", -1) != 0 and b"negative" in l.wq_last_error()
+        assert l.wq_program_set_option(p, b"no_such_option", 1) != 0 and b"unknown option" in l.wq_last_error()
+        # nothing fused yet: nothing to poll
+        assert l.wq_program_poll(p, None, 0, None) == 0
+        addr = [0x100000]
+
+        def ext(code, bits, *shape):
+            addr[0] += 0x100000
+            return l.wq_program_add_external(p, code, bits, len(shape), _shape(*shape), addr[0], 10)
+
+        x = ext(2, 16, 1, 256)
+        for _ in range(2):
+            assert _call(l, p, "relax_amd.q4f16_1_matmul", [ext(1, 32, 64, 32), ext(2, 16, 64, 8), x, ext(2, 16, 1, 64)]) == 0
+        # every tensor is external, yet the fused run keeps its descriptor table and counters in the workspace
+        assert l.wq_program_plan(p) > 0
+        assert l.wq_program_run(p, None) != 0 and b"set the workspace" in l.wq_last_error()
+        assert l.wq_program_capture(p, 1) != 0 and b"set the workspace" in l.wq_last_error()
+    finally:
+        l.wq_program_destroy(p)
+
+
 SMALL_LINEARS = (("qkv_proj", 384, 128), ("o_proj", 128, 128), ("gate_up_proj", 512, 128), ("down_proj", 128, 256))
 
 
@@ -230,6 +288,27 @@ def test_linear_stack_program_matches_oracle_eager_and_replayed(oracle, M):
         prog.replay(stream)
         stream.synchronize()
         assert np.array_equal(u.host(out).view(np.uint16), eager.view(np.uint16)), rep
+
+    if M == 1:
+        # the non-blocking check of the fused run's error word, and a wait that is made to run out from the host:
+        # with a spin limit of 0 the gate_up linears give up on their producers at once; every launch still ends
+        from relax_amd._lib import WqError
+
+        words = torch.full((4,), -1, dtype=torch.int32).pin_memory()
+        assert prog.poll(words, stream) == 1
+        stream.synchronize()
+        assert words[0].item() == 0
+        prog.set_option("spin_limit_us", 0)
+        prog.run(stream)
+        assert prog.poll(words, stream) == 1
+        stream.synchronize()
+        if words[0].item() != 0:  # (a 3-layer stack this small may finish its producers before anyone looks)
+            with pytest.raises(WqError, match="timed out"):
+                prog.status(stream)
+        prog.set_option("spin_limit_us", 2_000_000)
+        prog.run(stream)
+        prog.status(stream)
+        assert np.array_equal(u.host(out).view(np.uint16), eager.view(np.uint16))
 
     # chain through planned storage: y = gate_up(o_proj(attn)) with both intermediates planned
     p2 = vm.DpsProgram()

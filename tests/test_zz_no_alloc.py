@@ -51,6 +51,26 @@ def test_no_alloc_entry_matches_the_workspace_entry(oracle):
         assert torch.equal(y_ws, y_na), M
         u.assert_close(u.host(y_na), oracle.nt_matmul_f32acc(B, x, None, res, nthreads=4), f"no-alloc M={M}")
 
+    # under stream capture (the address was looked up by the calls above): replays against the eager result
+    M = 3
+    x = np.random.default_rng(33).standard_normal((M, K)).astype(np.float16)
+    dx = u.dev(x)
+    y_eager = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    y_graph = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    _call(lib, "wq_gptq_linear_noalloc", w, dx, y_eager, None, M)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            _call(lib, "wq_gptq_linear_noalloc", w, dx, y_graph, None, M)
+    for rep in range(3):
+        y_graph.zero_()  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, y_eager), rep
+
     # without a row order nothing is gathered and the buffer is not used
     _, qw2, qz2, s2, g2 = oracle.make_gptq_inputs(1, N, K, gs, seed=52)
     w2 = ops.gptq_prepare(u.dev(qw2), u.dev(qz2), u.dev(s2), u.dev(g2))
