@@ -20,7 +20,9 @@ reference's path timed on this machine's host cores.  Further objects on the sam
 line: `stack` (32 decoder layers' linears run as one captured instruction list at
 M = 1, 8, 16, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
 128, 512), `autogptq` and `kn_gemv` (the neighbouring checkpoint layouts at decode) and
-`calibration` (measured pure-read and MFMA-only ceilings).
+`calibration` (measured pure-read and MFMA-only ceilings); `single_gemv_4096x4096` (one linear per launch, with
+its own roofline), `list_steady_state` (the list kernel over 906 MB in one launch) and `f16acc` (the
+fp16-accumulate decode entry point).
 """
 from __future__ import annotations
 
@@ -156,6 +158,55 @@ def _measure(torch, stream, fn, min_ms=None, samples=None):
     med = t[len(t) // 2] if len(t) % 2 else 0.5 * (t[len(t) // 2 - 1] + t[len(t) // 2])
     return med, {"samples": samples, "calls_per_sample": reps, "sample_ms": round(med * reps, 1),
                  "min": round(t[0], 6), "max": round(t[-1], 6)}
+
+
+def bench_list_steady(torch, ops, stream, K=4096, rows_total=131072 * 3, linears=24):
+    """The M = 1 list kernel far from its start and end: ONE launch over `linears` equal linears that together
+    hold 906 MB of codes and scales (three times the last-level cache), so start-up, drain and the hand-over
+    between linears weigh little: the rate the kernel's inner loop sustains."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    W = torch.randint(-2**31, 2**31 - 1, (rows_total, K // 8), dtype=torch.int32, device="cuda", generator=g)
+    S = (torch.rand((rows_total, K // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+    x = torch.randn((1, K), device="cuda", dtype=torch.float16)
+    rows = rows_total // linears
+    y = torch.empty((linears, rows), device="cuda", dtype=torch.float16)
+    gl = ops.Q4G32GemvList([(W[i * rows:(i + 1) * rows], S[i * rows:(i + 1) * rows], x, y[i:i + 1]) for i in range(linears)])
+    gl.run()
+    gl.status()
+    ms, sp = _measure(torch, stream, gl.run, min_ms=MIN_SAMPLE_MS / 4)
+    nbytes = linears * gemv_bytes(1, rows, K)
+    del gl
+    return {"kernel": "q4g32_gemv_list_kernel", "what": f"one launch, {linears} linears of {rows} x {K}, M = 1",
+            "us": round(ms * 1e3, 2), "us_min": round(sp["min"] * 1e3, 2), "us_max": round(sp["max"] * 1e3, 2),
+            "bytes_per_launch": nbytes, "GB/s": round(nbytes / ms / 1e6, 1),
+            "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+
+def bench_f16acc(torch, ops, stream, copies, xs):
+    """The fp16-accumulate decode entry point (wq_q4g32_gemv_f16acc) on the four decode linears, M = 1, one launch
+    each, cycling the weight copies inside one graph like `per_linear`."""
+    res = []
+    for si, (N, K) in enumerate(DECODE_SHAPES):
+        def one(i, si=si):
+            W, S = copies[i % len(copies)][si]
+            ops.q4g32_gemv_f16acc(W, S, xs[si])
+        for i in range(len(copies)):
+            one(i)
+        stream.synchronize()
+        g1 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g1, stream=stream):
+            for i in range(4 * len(copies)):
+                one(i)
+        ms1, sp1 = _measure(torch, stream, g1.replay, min_ms=MIN_SAMPLE_MS / 4)
+        us = ms1 * 1e3 / (4 * len(copies))
+        nb = gemv_bytes(1, N, K)
+        res.append({"N": N, "K": K, "us": round(us, 3), "GB/s": round(nb / us / 1e3, 1),
+                    "frac_of_hbm_peak": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": nb,
+                    "us_min": round(sp1["min"] * 1e3 / (4 * len(copies)), 3),
+                    "us_max": round(sp1["max"] * 1e3 / (4 * len(copies)), 3)})
+        del g1
+    return {"kernel": "q4g32_gemv_f16acc_kernel (wq_q4g32_gemv_f16acc)", "bound": "hbm", "M": 1, "shapes": res}
 
 
 def bench_stack(torch, layers=32, batches=(1, 8, 16, 32)):
@@ -523,8 +574,18 @@ def main():
         # the same four linears one launch each (what a single wq_q4g32_linear call costs), and the
         # 4096 x 4096 linear of the single-GEMV configuration on its own
         "per_linear": per_shape,
-        "single_gemv_4096x4096": next(p for p in per_shape if p["N"] == 4096 and p["K"] == 4096),
     }
+    # the single-GEMV configuration (one 4096 x 4096 linear, one launch of the streaming kernel): its own roofline
+    c1 = dict(next(p for p in per_shape if p["N"] == 4096 and p["K"] == 4096))
+    c1_traffic, c1_src = offline_traffic("q4g32_gemv_kernel")
+    c1["roofline"] = {"kernel": "q4_gemv_kernel<Q4G32Row> (wq_q4g32_gemv)", "bound": "hbm", "achieved": c1["GB/s"],
+                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": c1["frac_of_hbm_peak"],
+                      "avg_launch_us": c1["us"], "bytes_per_launch": c1["bytes"],
+                      "traffic": c1_traffic, "traffic_source": c1_src}
+    out["single_gemv_4096x4096"] = c1
+    with torch.cuda.stream(stream):
+        out["list_steady_state"] = bench_list_steady(torch, ops, stream)
+        out["f16acc"] = bench_f16acc(torch, ops, stream, copies, xs)
 
     if not args.no_gemm:
         gem, vendor = [], []

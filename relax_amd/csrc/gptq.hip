@@ -215,23 +215,23 @@ struct GptqSkinnyPolicy {
     uint32_t inv;
   };
   using Scale = half2_t;  // (scale, zero point)
-  __device__ static void init(Lane& l, const Args& a, int n, int K, int) {
+  __device__ __forceinline__ static void init(Lane& l, const Args& a, int n, int K, int) {
     l.w = reinterpret_cast<const char*>(a.W + (int64_t)n * (K >> 3));
     l.sz = reinterpret_cast<const char*>(a.SZ + (int64_t)n * a.groups);
     l.ratio = a.ratio;
     l.inv = a.inv;
   }
-  __device__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
-  __device__ static const char* s_addr(const Lane& l, int k0) {
+  __device__ __forceinline__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
+  __device__ __forceinline__ static const char* s_addr(const Lane& l, int k0) {
     const uint32_t g32 = (uint32_t)k0 >> 5;
     return l.sz + (l.ratio == 1 ? g32 : __umulhi(g32, l.inv)) * 4;
   }
-  __device__ static const char* s_pair_addr(const Lane& l, int k0) { return s_addr(l, k0); }
+  __device__ __forceinline__ static const char* s_pair_addr(const Lane& l, int k0) { return s_addr(l, k0); }
   static bool pair_aligned(const Args&) { return true; }
-  __device__ static Scale pick_scale(const Lane&, half2_t pair, int) { return pair; }
-  __device__ static Scale const_scale(const Lane&) { return Scale{}; }
-  __device__ static Scale null_scale() { return Scale{(half_t)0.0f, (half_t)0.0f}; }
-  __device__ static void dequant(const uint4_t* pieces, Scale sz, half8_t out[4]) {
+  __device__ __forceinline__ static Scale pick_scale(const Lane&, half2_t pair, int) { return pair; }
+  __device__ __forceinline__ static Scale const_scale(const Lane&) { return Scale{}; }
+  __device__ __forceinline__ static Scale null_scale() { return Scale{(half_t)0.0f, (half_t)0.0f}; }
+  __device__ __forceinline__ static void dequant(const uint4_t* pieces, Scale sz, half8_t out[4]) {
     const half2_t s2 = {sz.x, sz.x};
     const half_t o = sz.y + (half_t)1024.0f;
     const half2_t off = {o, o};
@@ -272,33 +272,33 @@ struct GptqLdsPolicy {
     half2_t s2;   // scale, twice
     half2_t off;  // 1024 + zero point, twice
   };
-  __device__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
+  __device__ __forceinline__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
     const int n = q >> 1, h = q & 1;
     return reinterpret_cast<const char*>(a.W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
   }
-  __device__ static const char* s_src(const Args& a, int n, int) {
+  __device__ __forceinline__ static const char* s_src(const Args& a, int n, int) {
     return reinterpret_cast<const char*>(a.SZ + (int64_t)n * a.groups);
   }
   // ks / steps_per_group by multiplication: exact for ks * steps_per_group < 2^32
-  __device__ static int64_t s_offset(const Args& a, int ks) {
+  __device__ __forceinline__ static int64_t s_offset(const Args& a, int ks) {
     const uint32_t g = a.steps_per_group == 1 ? (uint32_t)ks : __umulhi((uint32_t)ks, a.inv);
     return (int64_t)g * 4;
   }
-  __device__ static Scale read_scale(const unsigned char* p, int) {
+  __device__ __forceinline__ static Scale read_scale(const unsigned char* p, int) {
     const half2_t sz = *reinterpret_cast<const half2_t*>(p);
     const half_t o = sz.y + (half_t)1024.0f;
     return Scale{half2_t{sz.x, sz.x}, half2_t{o, o}};
   }
-  __device__ static Scale const_scale(const Args&, int) { return Scale{}; }
-  __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
+  __device__ __forceinline__ static Scale const_scale(const Args&, int) { return Scale{}; }
+  __device__ __forceinline__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
     f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
   }
-  __device__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
+  __device__ __forceinline__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
     const uint32_t word = kk == 0 ? f.w.x : kk == 1 ? f.w.y : kk == 2 ? f.w.z : f.w.w;
     return q4_pair_bits_natural(word, j);
   }
-  __device__ static half2_t pair_finish(uint32_t bits, const Scale& sc) { return (as_half2(bits) - sc.off) * sc.s2; }
-  __device__ static half2_t pair(const Frag& f, int kk, int j, const Scale& sc) {
+  __device__ __forceinline__ static half2_t pair_finish(uint32_t bits, const Scale& sc) { return (as_half2(bits) - sc.off) * sc.s2; }
+  __device__ __forceinline__ static half2_t pair(const Frag& f, int kk, int j, const Scale& sc) {
     return pair_finish(pair_bits(f, kk, j), sc);
   }
 };

@@ -34,18 +34,18 @@ struct IntbLoader {
     uint4_t w[kPieces];
     half_t s;
   };
-  __device__ static void init(Lane& l, const Args& a, int n, int lh, int K, int N) {
+  __device__ __forceinline__ static void init(Lane& l, const Args& a, int n, int lh, int K, int N) {
     constexpr int I = NBIT == 8 ? 2 : 4;
     l.w = a.B + ((int64_t)(n / I) * (K >> 6)) * 8 + (n % I) * (8 / I) + lh * kPieces;
     l.s = a.scales + n;
     l.N = N;
   }
-  __device__ static void load(Frag& f, const Lane& l, const Args& a, int ks, int, int, bool) {
+  __device__ __forceinline__ static void load(Frag& f, const Lane& l, const Args& a, int ks, int, int, bool) {
 #pragma unroll
     for (int p = 0; p < kPieces; ++p) f.w[p] = l.w[(int64_t)ks * 8 + p];
     f.s = a.group ? l.s[(int64_t)ks * l.N] : l.s[0];
   }
-  __device__ static void dequant(const Frag& f, half8_t out[4]) {
+  __device__ __forceinline__ static void dequant(const Frag& f, half8_t out[4]) {
     const half2_t s2 = {f.s, f.s};
     if (NBIT == 8) {
 #pragma unroll
@@ -98,27 +98,27 @@ struct IntbLdsPolicy {
   struct Frag {
     uint4_t w[NBIT == 8 ? 2 : 1];
   };
-  __device__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
+  __device__ __forceinline__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
     const int group = min(n0 / I + (q >> 3), N / I - 1);  // columns past N re-read the last group
     return reinterpret_cast<const char*>(a.B) + ((int64_t)group * (K >> 6)) * 128 + (q & 7) * 16;
   }
   using Scale = half2_t;  // the column's scale, twice
-  __device__ static const char* s_src(const Args& a, int n, int) {
+  __device__ __forceinline__ static const char* s_src(const Args& a, int n, int) {
     return reinterpret_cast<const char*>(a.scales + (n & ~1));  // the aligned pair of columns (N is even)
   }
-  __device__ static int64_t s_offset(const Args& a, int ks) { return (int64_t)ks * a.N * 2; }
+  __device__ __forceinline__ static int64_t s_offset(const Args& a, int ks) { return (int64_t)ks * a.N * 2; }
   // p = the 4 staged bytes of the lane's column; columns are staged 4 bytes apart from an 8-byte
   // aligned base, so bit 2 of the address is the parity of the column
-  __device__ static Scale read_scale(const unsigned char* p, int) {
+  __device__ __forceinline__ static Scale read_scale(const unsigned char* p, int) {
     const half2_t pair = *reinterpret_cast<const half2_t*>(p);
     const half_t s = (reinterpret_cast<uintptr_t>(p) & 4) ? pair.y : pair.x;
     return Scale{s, s};
   }
-  __device__ static Scale const_scale(const Args& a, int n) {
+  __device__ __forceinline__ static Scale const_scale(const Args& a, int n) {
     const half_t s = a.scales[n];
     return Scale{s, s};
   }
-  __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
+  __device__ __forceinline__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
     if (NBIT == 8) {
       const unsigned char* p = bslot + ((n_local >> 1) * 8 + (n_local & 1) * 4 + 2 * lh) * 16;
       f.w[0] = *reinterpret_cast<const uint4_t*>(p);
@@ -129,7 +129,7 @@ struct IntbLdsPolicy {
   }
   // int8: piece kk/2 holds 16 k; word j of it holds k = 2j, 2j+1 (bytes 0, 2) and 2j+8, 2j+9 (bytes 1, 3).
   // int4: word j holds k = 2j + 8i, 2j + 8i + 1 in nibbles i, i + 4.
-  __device__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
+  __device__ __forceinline__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
     if (NBIT == 8) {
       const uint4_t& p = f.w[NBIT == 8 ? (kk >> 1) : 0];
       const uint32_t word = j == 0 ? p.x : j == 1 ? p.y : j == 2 ? p.z : p.w;
@@ -138,11 +138,11 @@ struct IntbLdsPolicy {
     const uint32_t word = j == 0 ? f.w[0].x : j == 1 ? f.w[0].y : j == 2 ? f.w[0].z : f.w[0].w;
     return and_or(word >> (4 * kk), 0x000F000Fu, 0x64006400u);                                // 1024 + u4
   }
-  __device__ static half2_t pair_finish(uint32_t bits, half2_t s2) {
+  __device__ __forceinline__ static half2_t pair_finish(uint32_t bits, half2_t s2) {
     const half_t o = (half_t)(NBIT == 8 ? 1152.0f : 1032.0f);  // 1024 + the bias of the stored codes
     return (as_half2(bits) - half2_t{o, o}) * s2;
   }
-  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) { return pair_finish(pair_bits(f, kk, j), s2); }
+  __device__ __forceinline__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) { return pair_finish(pair_bits(f, kk, j), s2); }
 };
 
 template <int NBIT, bool GROUPED>

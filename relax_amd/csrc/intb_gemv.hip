@@ -334,8 +334,16 @@ int intb_gemv_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scale
                      : launch_intb_gemv<4, 2, 2>(a, B, scales, c, n, k, group, ep, stream);
       m0 += 2;
     } else {
-      rc = nbit == 8 ? launch_intb_gemv<8, 2, 1>(a, B, scales, c, n, k, group, ep, stream)
-                     : launch_intb_gemv<4, 2, 1>(a, B, scales, c, n, k, group, ep, stream);
+      // column groups per wavefront: one with per-channel scales (K = 8192, N = 28672: int8 40.4 -> 37.9 us, int4
+      // 27.2 -> 26.3 us), two with group scales, whose 8- or 16-byte scale vectors then serve both (int8 45.4
+      // against 48.1 us)
+      const int R = tuning().gemv_rows ? tuning().gemv_rows : (group > 0 ? 2 : 1);
+      if (R == 1)
+        rc = nbit == 8 ? launch_intb_gemv<8, 1, 1>(a, B, scales, c, n, k, group, ep, stream)
+                       : launch_intb_gemv<4, 1, 1>(a, B, scales, c, n, k, group, ep, stream);
+      else
+        rc = nbit == 8 ? launch_intb_gemv<8, 2, 1>(a, B, scales, c, n, k, group, ep, stream)
+                       : launch_intb_gemv<4, 2, 1>(a, B, scales, c, n, k, group, ep, stream);
       m0 += 1;
     }
     if (rc != WQ_OK) return rc;

@@ -26,30 +26,30 @@ struct IntbSkinnyPolicy {
     int N;
     int odd;
   };
-  __device__ static void init(Lane& l, const Args& a, int n, int K, int N) {
+  __device__ __forceinline__ static void init(Lane& l, const Args& a, int n, int K, int N) {
     constexpr int I = NBIT == 8 ? 2 : 4;
     l.w = a.B + ((int64_t)(n / I) * (K >> 6)) * 8 + (n % I) * (8 / I);
     l.s = a.scales + (GROUPED ? (n & ~1) : n);
     l.N = N;
     l.odd = n & 1;
   }
-  __device__ static const char* w_addr(const Lane& l, int k0, int p) {
+  __device__ __forceinline__ static const char* w_addr(const Lane& l, int k0, int p) {
     return reinterpret_cast<const char*>(l.w + (int64_t)(k0 >> 6) * 8 + ((k0 >> 5) & 1) * kPieces + p);
   }
   // fine-grained scales are [K/64, N]: the pair (n & ~1, n | 1) of the lane's K-tile
-  __device__ static const char* s_addr(const Lane& l, int k0) {
+  __device__ __forceinline__ static const char* s_addr(const Lane& l, int k0) {
     return reinterpret_cast<const char*>(l.s + (int64_t)(k0 >> 6) * l.N);
   }
-  __device__ static const char* s_pair_addr(const Lane& l, int k0) {
+  __device__ __forceinline__ static const char* s_pair_addr(const Lane& l, int k0) {
     if (GROUPED) return s_addr(l, k0);
     return reinterpret_cast<const char*>(reinterpret_cast<uintptr_t>(l.s) & ~(uintptr_t)3);  // &scales[n & ~1]
   }
   static bool pair_aligned(const Args& a) { return (reinterpret_cast<uintptr_t>(a.scales) & 3u) == 0; }
-  __device__ static half_t pick_scale(const Lane& l, half2_t pair, int) { return l.odd ? pair.y : pair.x; }
+  __device__ __forceinline__ static half_t pick_scale(const Lane& l, half2_t pair, int) { return l.odd ? pair.y : pair.x; }
   using Scale = half_t;
-  __device__ static half_t const_scale(const Lane& l) { return l.s[0]; }
-  __device__ static half_t null_scale() { return (half_t)0.0f; }
-  __device__ static void dequant(const uint4_t* pieces, half_t s, half8_t out[4]) {
+  __device__ __forceinline__ static half_t const_scale(const Lane& l) { return l.s[0]; }
+  __device__ __forceinline__ static half_t null_scale() { return (half_t)0.0f; }
+  __device__ __forceinline__ static void dequant(const uint4_t* pieces, half_t s, half8_t out[4]) {
     const half2_t s2 = {s, s};
     if (NBIT == 8) {
 #pragma unroll

@@ -25,11 +25,11 @@ struct Q4G32Loader {
     uint4_t w;
     half_t s;
   };
-  __device__ static void init(Lane& l, const Args& a, int n, int lh, int K, int) {
+  __device__ __forceinline__ static void init(Lane& l, const Args& a, int n, int lh, int K, int) {
     l.w = reinterpret_cast<const uint4_t*>(a.W + (int64_t)n * (K >> 3)) + lh;
     l.s = a.S + (int64_t)n * (K >> 5) + lh;
   }
-  __device__ static void load(Frag& f, const Lane& l, const Args&, int ks, int lh, int K,
+  __device__ __forceinline__ static void load(Frag& f, const Lane& l, const Args&, int ks, int lh, int K,
                               bool ktail) {
     if (ktail && (ks * 2 + lh) >= (K >> 5)) {  // the last step may hold a single group
       f.w = uint4_t{0x77777777u, 0x77777777u, 0x77777777u, 0x77777777u};  // code 7 -> weight 0
@@ -39,7 +39,7 @@ struct Q4G32Loader {
       f.s = l.s[ks * 2];
     }
   }
-  __device__ static void dequant(const Frag& f, half8_t out[4]) {
+  __device__ __forceinline__ static void dequant(const Frag& f, half8_t out[4]) {
     const half2_t s2 = {f.s, f.s};
     const uint32_t ws[4] = {f.w.x, f.w.y, f.w.z, f.w.w};
 #pragma unroll
@@ -68,31 +68,31 @@ struct Q4G32LdsPolicy {
     uint4_t w;
   };
   using Scale = half2_t;  // the group's scale, twice
-  __device__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
+  __device__ __forceinline__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
     const int n = q >> 1, h = q & 1;
     return reinterpret_cast<const char*>(a.W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
   }
-  __device__ static const char* s_src(const Args& a, int n, int K) {
+  __device__ __forceinline__ static const char* s_src(const Args& a, int n, int K) {
     return reinterpret_cast<const char*>(a.S + (int64_t)n * (K >> 5));
   }
-  __device__ static int64_t s_offset(const Args&, int ks) { return (int64_t)ks * 4; }
-  __device__ static Scale read_scale(const unsigned char* p, int lh) {
+  __device__ __forceinline__ static int64_t s_offset(const Args&, int ks) { return (int64_t)ks * 4; }
+  __device__ __forceinline__ static Scale read_scale(const unsigned char* p, int lh) {
     const half_t s = *reinterpret_cast<const half_t*>(p + lh * 2);
     return Scale{s, s};
   }
-  __device__ static Scale const_scale(const Args&, int) { return Scale{(half_t)0.0f, (half_t)0.0f}; }
-  __device__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
+  __device__ __forceinline__ static Scale const_scale(const Args&, int) { return Scale{(half_t)0.0f, (half_t)0.0f}; }
+  __device__ __forceinline__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
     f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
   }
-  __device__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
+  __device__ __forceinline__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
     const uint32_t word = kk == 0 ? f.w.x : kk == 1 ? f.w.y : kk == 2 ? f.w.z : f.w.w;
     return q4_pair_bits_natural(word, j);
   }
-  __device__ static half2_t pair_finish(uint32_t bits, half2_t s2) {
+  __device__ __forceinline__ static half2_t pair_finish(uint32_t bits, half2_t s2) {
     const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
     return (as_half2(bits) - off) * s2;
   }
-  __device__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) { return pair_finish(pair_bits(f, kk, j), s2); }
+  __device__ __forceinline__ static half2_t pair(const Frag& f, int kk, int j, half2_t s2) { return pair_finish(pair_bits(f, kk, j), s2); }
 };
 
 }  // namespace wq

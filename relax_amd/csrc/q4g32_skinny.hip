@@ -19,24 +19,24 @@ struct Q4G32SkinnyPolicy {
     const char* w;
     const char* s;
   };
-  __device__ static void init(Lane& l, const Args& a, int n, int K, int) {
+  __device__ __forceinline__ static void init(Lane& l, const Args& a, int n, int K, int) {
     l.w = reinterpret_cast<const char*>(a.W + (int64_t)n * (K >> 3));
     l.s = reinterpret_cast<const char*>(a.S + (int64_t)n * (K >> 5));
   }
-  __device__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
-  __device__ static const char* s_addr(const Lane& l, int k0) { return l.s + ((k0 >> 5) & ~1) * 2; }
-  __device__ static const char* s_pair_addr(const Lane& l, int k0) { return s_addr(l, k0); }
-  __device__ static const char* sblock_addr(const Lane& l, int g) { return l.s + g * 2; }
+  __device__ __forceinline__ static const char* w_addr(const Lane& l, int k0, int) { return l.w + (k0 >> 1); }
+  __device__ __forceinline__ static const char* s_addr(const Lane& l, int k0) { return l.s + ((k0 >> 5) & ~1) * 2; }
+  __device__ __forceinline__ static const char* s_pair_addr(const Lane& l, int k0) { return s_addr(l, k0); }
+  __device__ __forceinline__ static const char* sblock_addr(const Lane& l, int g) { return l.s + g * 2; }
   // rows of K/16 bytes: every 8 scales are 16 aligned bytes when K % 256 == 0 and S is aligned
   static bool scale_block_ok(const Args& a, int64_t K) {
     return K % 256 == 0 && (reinterpret_cast<uintptr_t>(a.S) & 15u) == 0;
   }
   static bool pair_aligned(const Args& a) { return (reinterpret_cast<uintptr_t>(a.S) & 3u) == 0; }
-  __device__ static half_t pick_scale(const Lane&, half2_t pair, int kq) { return (kq & 1) ? pair.y : pair.x; }
+  __device__ __forceinline__ static half_t pick_scale(const Lane&, half2_t pair, int kq) { return (kq & 1) ? pair.y : pair.x; }
   using Scale = half_t;
-  __device__ static half_t const_scale(const Lane&) { return (half_t)0.0f; }
-  __device__ static half_t null_scale() { return (half_t)0.0f; }
-  __device__ static void dequant(const uint4_t* pieces, half_t s, half8_t out[4]) {
+  __device__ __forceinline__ static half_t const_scale(const Lane&) { return (half_t)0.0f; }
+  __device__ __forceinline__ static half_t null_scale() { return (half_t)0.0f; }
+  __device__ __forceinline__ static void dequant(const uint4_t* pieces, half_t s, half8_t out[4]) {
     const half2_t s2 = {s, s};
     const uint32_t words[4] = {pieces[0].x, pieces[0].y, pieces[0].z, pieces[0].w};
 #pragma unroll
