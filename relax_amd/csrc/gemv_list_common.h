@@ -88,6 +88,7 @@ struct wq_gemv_list {
   int batch_ring = 0;      // items the compute wavefronts may spread over (slots of scales and of partial sums)
   int batch_acc_tiles = 0; // tiles whose sums LDS keeps between the panels of a linear: a chunk of the workgroup's tiles
   bool batch_chunked = false;  // some linear is walked in several chunks
+  bool batch_rows = false;     // more than 16 rows: the kernel whose wavefronts own rows of W (q4g32_batch_rows_kernel)
 };
 
 namespace wq {

@@ -5,16 +5,19 @@
 // the matrix cores so that all M rows share one pass over the weights, and the weights go from
 // memory straight into the registers that feed them.
 //
+// Two kernels: up to 16 rows of activations the one described here (q4g32_batch_list_kernel), beyond that
+// q4g32_batch_rows_kernel further down, which shares the unpack, the lane exchange and the staging of activations.
+//
 // Work.  The unit is a TILE of rows of W times a PANEL of K: 16 rows x 4096 k for M <= 8, 32 rows x 2048 k for
-// M <= 16, 32 rows x 1024 k beyond (a panel of activations is at most 64 KiB; an item is 32, 32 or 16 KiB of codes:
-// what a workgroup spends per item on hand-overs does not depend on its size).  A linear is run by one GROUP of
+// M <= 16 (an item is 32 KiB of codes: what a workgroup spends per item on hand-overs does not depend on its
+// size).  A linear is run by one GROUP of
 // workgroups (see batch_assign_groups), its tiles dealt to them round-robin, with a rotation that continues
 // from linear to linear.  Inside a workgroup the 8 compute wavefronts split a tile: 16 rows x an eighth of the
 // panel each, or, with tiles of 32 rows, wavefronts 0 .. 3 a quarter of the panel of rows 0 .. 15 each and
-// wavefronts 4 .. 7 of rows 16 .. 31.  A wavefront's share is U chunks (U = 4 or 2); a chunk is
+// wavefronts 4 .. 7 of rows 16 .. 31.  A wavefront's share is U = 4 chunks; a chunk is
 // one 16-byte load per lane: lane (i, kq) takes scale group 4u + kq of row i, the 32 codes that the four
-// v_mfma_f32_16x16x32_f16 of the chunk consume as A operands (one dword, 8 codes, each).  With more than
-// 16 activation rows every unpacked A operand feeds R = 2 MFMAs, one per set of 16 rows.
+// v_mfma_f32_16x16x32_f16 of the chunk consume as A operands (one dword, 8 codes, each).  (The template
+// parameter R, sets of 16 activation rows per unpacked A operand, is 1 in every instantiation.)
 // Unpacking is exact: OR the code into 0x6400 (1024 + q, or 1024 + 16 q), subtract 1031 (1136),
 // multiply by the scale, all in packed fp16: 13 VALU instructions per 8 weights and lane, whatever M.
 // The B operands (the activations of the wavefront's K slice, in the k order of the unpack, the
@@ -676,6 +679,540 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
   }
 }
 
+// ====================================================================================================
+// More than 16 activation rows: the wavefront that owns rows of W keeps their sums.
+//
+// With 17 .. 32 rows of activations a panel of 1024 k fills 64 KiB of LDS, the kernel above then hands over
+// items of 16 KiB, and what an item costs in hand-overs (partial sums through LDS, the y wavefront's
+// epilogue, the sums kept between panels) is paid four times per 4096 k.  Here nothing is handed over but the
+// operands: a compute wavefront owns up to TR = 4 ROW TILES (16 rows each) of W for ALL of K, its accumulators
+// (TR x R x 4 registers) stay in registers from the first panel to the last, and it writes its own outputs.
+// The 8 compute wavefronts of a workgroup walk the panels of activations together (a PASS of the workgroup:
+// up to 8 x 64 rows; the activations are loaded once per pass, which is why TR is as large as the registers
+// allow: 167 of the 168 that 11 wavefronts leave each other).
+//   * The activations of a panel (512 k: M x 1 KiB) lie in LDS in B-operand order; every compute wavefront
+//     reads the operand of a (step, dword) pair once and uses it for its TR row tiles (LDS reads: 2 bytes per
+//     byte of codes).  Two x wavefronts stage panels by turns into `nxb` buffers; a buffer is free again when
+//     all 8 compute wavefronts have left it.
+//   * One scale wavefront stages the scales of the rows of a pass, 1024 k (64 bytes per row) at a time, into
+//     2 buffers.
+//   * The unit of the weight stream is a PAIR of chunks of a wavefront's rows: 256 k, per row tile two loads of
+//     8 rows x 128 bytes (whole lines; a lane exchange puts the halves where the MFMA wants them), 2 TR loads
+//     in all, waited for by hand.  A pair is first exchanged into registers of its own and its ring slot
+//     refilled at once, so two pairs (32 KiB per wavefront) are in flight while one is multiplied.  The loads
+//     are buffer loads on the wavefront's rows of the pass: rows past them (a short last pass, the end of W)
+//     read zeros without touching memory and are never stored; a wavefront without rows in a pass loads from
+//     an empty buffer and only takes part in the hand-overs.
+//   * A linear's completion counter is raised by the last of the 8 compute wavefronts to have its stores
+//     written through.
+// What bounds it: bytes through the CU.  Codes, scales and the activations of every pass (M x K x 2 bytes per
+// 512 rows: 22 % of the codes at M = 32) together arrive at the rate the one-row list kernel reaches with
+// codes and scales alone.
+constexpr int kRW = 8;      // compute wavefronts
+constexpr int kRXW = 2;     // wavefronts that stage activations
+constexpr int kRThreads = 64 * (kRW + kRXW + 1);
+constexpr int kRPairGroups = 8;   // scale groups per pair of chunks (256 k)
+constexpr int kRPG = 16;          // scale groups per panel of activations
+constexpr int kRSPG = 32;         // scale groups per panel of scales
+constexpr int kRSRow = kRSPG * 2 + 16;  // LDS bytes per row of a panel of scales (+ 16: the 16 rows of a row tile on different banks)
+constexpr int kRMaxXBuf = 4;
+
+struct RowsFlags {
+  int x_ready[kRMaxXBuf];  // [panel mod buffers] = panel + 1 once staged (panels counted over the whole launch)
+  int x_taken[kRMaxXBuf];  // += 1 by each compute wavefront that has left the panel
+  int s_ready[2], s_taken[2];  // the same for the panels of scales
+  int lin_done[8];         // [linear mod 8] += 1 by each compute wavefront whose stores of the linear are written through
+                           // (a wavefront is at most `nxb` <= 4 panels, hence linears, ahead of another)
+  int exited;              // compute wavefronts that have finished the list
+  int abort;               // a wait of this workgroup ran into the spin limit: nobody waits any more
+  int pad[10];
+};
+static_assert(sizeof(RowsFlags) == 128, "flags layout");
+
+struct RowsWait {
+  int* abort;
+  int* error;
+  long long limit;
+  __device__ __forceinline__ void until(const int* flag, int target, int code) const {
+    if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= target) {
+      asm volatile("" ::: "memory");
+      return;
+    }
+    const long long t0 = wall_clock64();
+    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
+      if (__hip_atomic_load(abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) break;
+      if (wall_clock64() - t0 > limit) {
+        __hip_atomic_store(abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_store(error, kBatchInternalWait + code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    asm volatile("" ::: "memory");
+  }
+};
+
+// The walk of a workgroup over (linear, pass, pair of chunks).  All fields are wavefront-uniform.  A workgroup's
+// share of a linear is a run of consecutive ROW TILES (16 rows); a pass takes up to 8 TR of them, `tr` per
+// wavefront: TR while there are that many, and in the last pass as few as cover what is left with all 8
+// wavefronts (three wave tiles of 64 rows left over: 6 wavefronts with 32 rows each, half the time).
+struct RowsCursor {
+  int lin;         // nlin: past the end
+  int q, Q;        // pair of chunks within K
+  int pos, left;   // first row tile of the pass; row tiles of the workgroup from there on (> 0)
+  int tr;          // row tiles per wavefront in this pass (1 .. TR)
+  int N, G, row_w;
+  const char* W;
+  const char* S;
+  // row tiles of wavefront w in this pass, and the first of them
+  __device__ __forceinline__ int tiles_of(int w, int TR) const { return max(0, min(tr, min(left, kRW * TR) - w * tr)); }
+  __device__ __forceinline__ int first_of(int w) const { return pos + w * tr; }
+};
+
+template <int TR>
+__device__ __forceinline__ void rows_begin_pass(RowsCursor& c) {
+  c.q = 0;
+  c.tr = (min(c.left, kRW * TR) + kRW - 1) / kRW;
+}
+
+// positions the cursor on the first linear >= c.lin in which this workgroup holds a row tile.  SIGNAL (the
+// cursor that the first compute wavefront consumes with): a linear of this workgroup's group in which it
+// holds none is signalled as complete on the way.
+template <int TR, bool SIGNAL>
+__device__ __forceinline__ void rows_seek(RowsCursor& c, gemv_desc_ptr descs, int nlin, int b, int nwg, int* sync, int lane) {
+  typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
+  while (c.lin < nlin) {
+    const words_ptr p = (words_ptr)(descs + c.lin);
+    const uint32_t grp = p[16];
+    const int gl = (int)(grp & 0xffu);
+    if ((b & ((1 << gl) - 1)) == (int)((grp >> 8) & 0xffu)) {  // this workgroup's group runs the linear
+      const int ncu = nwg >> gl;
+      const uint32_t w15 = p[15];
+      int rb = (b >> gl) - (int)(w15 >> 16);
+      if (rb < 0) rb += ncu;
+      const int q = (int)p[13], rem = (int)(w15 & 0xffffu);
+      const int cnt = q + (rb < rem ? 1 : 0);
+      if (cnt > 0) {
+        const uint32_t w14 = p[14];
+        const int G = (int)(w14 & 0xffffu);
+        c.left = cnt;
+        c.pos = rb * q + min(rb, rem);
+        c.G = G;
+        c.Q = G / kRPairGroups;
+        c.N = (int)p[12];
+        c.row_w = G << 4;
+        c.W = reinterpret_cast<const char*>(((uint64_t)p[1] << 32) | p[0]);
+        c.S = reinterpret_cast<const char*>(((uint64_t)p[3] << 32) | p[2]);
+        rows_begin_pass<TR>(c);
+        return;
+      }
+      if (SIGNAL && (p[14] & kSignal) && lane == 0)
+        __hip_atomic_fetch_add(sync + sync_counter_index(c.lin, b & (kCountersPerLinear - 1)), 1, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    }
+    ++c.lin;
+  }
+}
+
+template <int TR, bool SIGNAL>
+__device__ __forceinline__ void rows_advance(RowsCursor& c, int step, gemv_desc_ptr descs, int nlin, int b, int nwg, int* sync, int lane) {
+  c.q += step;
+  if (c.q < c.Q) return;
+  const int took = min(c.left, kRW * TR);
+  c.pos += took;
+  c.left -= took;
+  if (c.left > 0) {
+    rows_begin_pass<TR>(c);
+    return;
+  }
+  ++c.lin;
+  rows_seek<TR, SIGNAL>(c, descs, nlin, b, nwg, sync, lane);
+}
+
+template <int TR, int R>
+__global__ __launch_bounds__(kRThreads) void q4g32_batch_rows_kernel(const GemvListDesc* __restrict__ descs_, int nlin,
+                                                                     int* __restrict__ sync, long long spin_limit,
+                                                                     int M, int nxb, int use_sync) {
+  constexpr int TROWS = 16 * TR;                 // rows of a wave tile
+  constexpr int SBUF = kRW * TROWS * kRSRow;     // bytes of a buffer of scales
+  extern __shared__ uint4_t smem[];
+  const gemv_desc_ptr descs = (gemv_desc_ptr)descs_;
+  char* lds = reinterpret_cast<char*>(smem);
+  // flags | nxb panels of activations, M x 1 KiB each | 2 panels of scales
+  RowsFlags* flags = reinterpret_cast<RowsFlags*>(lds);
+  char* const xbuf = lds + sizeof(RowsFlags);
+  const int xbuf_bytes = M * (kRPG * 64);
+  char* const sbuf = xbuf + nxb * xbuf_bytes;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nwg = gridDim.x;
+  const int b = blockIdx.x;
+  const RowsWait wait{&flags->abort, sync + sync_error_index(nlin), spin_limit > 0 ? spin_limit : 1000000};
+
+  if (tid < (int)(sizeof(RowsFlags) / sizeof(int))) reinterpret_cast<int*>(flags)[tid] = 0;
+  lds_done_then_barrier();
+
+  if (wave < kRW) {
+    // =========================== compute wavefront ===========================
+    const int i = lane & 15, kq = lane >> 4;
+    constexpr int NT = 2;        // ring slots: both in flight while a pair is multiplied (out of registers of its own)
+    constexpr int LPI = 2 * TR;  // loads per pair
+    // The ring is loaded in assembly and waited for by hand, as in the kernel above: `magic` orders the first
+    // read of every ring register behind the wait.
+    uint4_t tb[NT][TR][2];
+    uint32_t magic = 0x64006400u;
+    int ahead = 0;
+    RowsCursor ic, cc;
+    ic.lin = 0;
+    rows_seek<TR, false>(ic, descs, nlin, b, nwg, sync, lane);
+    cc.lin = 0;
+    if (wave == 0) rows_seek<TR, true>(cc, descs, nlin, b, nwg, sync, lane);
+    else rows_seek<TR, false>(cc, descs, nlin, b, nwg, sync, lane);
+
+    // the buffer of this wavefront's rows in the pass the cursor is in: rows past it read zeros
+    auto tile_rsrc = [&](const RowsCursor& c) {
+      const int nt = c.tiles_of(wave, TR);
+      const int row0 = c.first_of(wave) * 16;
+      const int rows = nt > 0 ? min(nt * 16, c.N - row0) : 0;
+      const uint64_t a = reinterpret_cast<uint64_t>(c.W + (int64_t)(nt > 0 ? row0 : 0) * c.row_w);
+      return uint4_t{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, (uint32_t)(rows * c.row_w), (uint32_t)kBufferFlags};
+    };
+
+    uint4_t i_rsrc = uint4_t{0, 0, 0, (uint32_t)kBufferFlags};
+    uint32_t i_voff = 0;
+    auto issue = [&](uint4_t (&buf)[TR][2]) {
+      if (ic.lin >= nlin) return;
+      if (ic.q == 0) {
+        i_rsrc = tile_rsrc(ic);
+        // lane (i, kq): row i mod 8 of the half tile, scale group 4 (i / 8) + kq of the pair
+        i_voff = __umul24((uint32_t)(i & 7), (uint32_t)ic.row_w) + (uint32_t)(((i >> 3) * 4 + kq) * 16);
+      }
+      const uint32_t rw8 = (uint32_t)ic.row_w * 8u;
+      uint32_t soff = (uint32_t)ic.q * (kRPairGroups * 16);
+#pragma unroll
+      for (int t = 0; t < TR; ++t) {
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen nt" : "=&v"(buf[t][0]) : "v"(i_voff), "s"(i_rsrc), "s"(soff));
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen nt" : "=&v"(buf[t][1]) : "v"(i_voff), "s"(i_rsrc), "s"(soff + rw8));
+        soff += 2 * rw8;
+      }
+      ++ahead;
+      rows_advance<TR, false>(ic, 1, descs, nlin, b, nwg, sync, lane);
+    };
+
+    const half2_t k1031 = {(half_t)-1031.0f, (half_t)-1031.0f};
+    const half2_t k1136 = {(half_t)-1136.0f, (half_t)-1136.0f};
+    auto unpack = [&](uint32_t t, half2_t c, half2_t s2) { return as_u32((as_half2(t) + c) * s2); };
+
+    float4_t acc[TR][R];
+    int pk = -1, sk = -1;  // panels of activations / of scales taken (counted over the launch)
+    int c_tr = 0;    // row tiles of this wavefront in the pass being multiplied
+    int c_row0 = 0;
+
+    auto epilogue = [&]() {
+      const int lin = cc.lin;
+      const int j16 = lane & 15, rq = lane >> 4;
+      const half_t* bias = descs[lin].bias;
+      const half_t* residual = descs[lin].residual;
+      const int N = cc.N;
+      const int yrows = (int)((desc_group_word(descs, lin) >> 16) & 0xffu);
+      const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(descs[lin].y, 0, yrows * N * 2, kBufferFlags);
+      const bool wide = (N & 3) == 0 && (((uintptr_t)descs[lin].y | (uintptr_t)bias | (uintptr_t)residual) & 7) == 0;
+#pragma unroll
+      for (int t = 0; t < TR; ++t) {
+        if (t >= c_tr) break;
+        // lane (j, rq) holds rows n0 .. n0 + 3 of activation rows j, j + 16
+        const int n0 = c_row0 + 16 * t + 4 * rq;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int j = j16 + 16 * r;
+          if (j < yrows && wide) {
+            if (n0 < N) {
+              float4_t v = acc[t][r];
+              if (bias) {
+                const half4_t bv = *reinterpret_cast<const half4_t*>(bias + n0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += (float)bv[e];
+              }
+              half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+              if (residual) h = h + *reinterpret_cast<const half4_t*>(residual + (int64_t)j * N + n0);
+              // device-scope store: written through, so that a counter update after it publishes it
+              __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uint2_t, h), yr, (j * N + n0) * 2, 0, kDeviceScope);
+            }
+          } else if (j < yrows) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int n = n0 + e;
+              if (n < N) {
+                float v = acc[t][r][e];
+                if (bias) v += (float)bias[n];
+                half_t h = (half_t)v;
+                if (residual) h = h + residual[(int64_t)j * N + n];
+                __builtin_amdgcn_raw_buffer_store_b16(as_u16(h), yr, (j * N + n) * 2, 0, kDeviceScope);
+              }
+            }
+          }
+        }
+      }
+    };
+
+    auto consume = [&](uint4_t (&buf)[TR][2]) {
+      if (cc.q == 0) {
+        c_tr = cc.tiles_of(wave, TR);
+        c_row0 = cc.first_of(wave) * 16;
+#pragma unroll
+        for (int t = 0; t < TR; ++t)
+#pragma unroll
+          for (int r = 0; r < R; ++r) acc[t][r] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+      if ((cc.q & 1) == 0) {
+        ++pk;
+        wait.until(&flags->x_ready[pk % nxb], pk + 1, 1);
+      }
+      if ((cc.q & 3) == 0) {
+        ++sk;
+        wait.until(&flags->s_ready[sk & 1], sk + 1, 2);
+      }
+      if (ahead == NT) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"((NT - 1) * LPI));
+      else asm volatile("s_waitcnt vmcnt(0)" : "+v"(magic));
+      // Both loads of every row tile have landed.  The chunks of the pair, put where the MFMA wants them: lanes 8 .. 15
+      // of every 16 take their half of chunk 0 from the second load 8 lanes below (row_ror:8 turns a row of 16 lanes
+      // by 8), lanes 0 .. 7 their half of chunk 1 from the first load 8 lanes above.  The statements depend on the wait
+      // through `magic`; they are volatile so that they stay in front of the loads that refill the slot.
+      uint32_t cw[TR][2][4];
+#pragma unroll
+      for (int t = 0; t < TR; ++t)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t lo_in = d == 0 ? buf[t][0].x : d == 1 ? buf[t][0].y : d == 2 ? buf[t][0].z : buf[t][0].w;
+          const uint32_t hi_in = d == 0 ? buf[t][1].x : d == 1 ? buf[t][1].y : d == 2 ? buf[t][1].z : buf[t][1].w;
+          asm volatile("v_mov_b32_dpp %0, %2 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf\n\t"
+                       "v_mov_b32_dpp %1, %3 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf\n\t"
+                       "s_nop 1\n\t"
+                       "v_mov_b32_dpp %0, %3 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+                       "v_mov_b32_dpp %1, %2 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+                       "s_nop 1 ; %4"
+                       : "=&v"(cw[t][0][d]), "=&v"(cw[t][1][d])
+                       : "v"(lo_in), "v"(hi_in), "v"(magic));
+        }
+      // the slot is free: the pair after the next one goes into it, so that two pairs are in flight while this one
+      // is multiplied
+      --ahead;
+      issue(buf);
+      if (c_tr > 0) {
+        const char* const xs = xbuf + (pk % nxb) * xbuf_bytes + (kq * M + min(i, M - 1)) * 16;
+        const int xr1 = (min(i + 16, M - 1) - min(i, M - 1)) * 16;  // second set of 16 activation rows
+        const char* const ss = sbuf + (sk & 1) * SBUF + (wave * TROWS + i) * kRSRow + ((cc.q & 3) * kRPairGroups + kq) * 2;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          half2_t s16[TR];
+#pragma unroll
+          for (int t = 0; t < TR; ++t) {
+            const half_t sh = *reinterpret_cast<const half_t*>(ss + t * 16 * kRSRow + u * 8);
+            s16[t] = half2_t{sh, sh};
+          }
+          const int step = (cc.q & 1) * 2 + u;  // 128 k each within the panel
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            half8_t xb[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+              xb[r] = *reinterpret_cast<const half8_t*>(xs + ((step * 4 + d) * 4 * M) * 16 + r * xr1);
+#pragma unroll
+            for (int t = 0; t < TR; ++t) {
+              const uint32_t word = cw[t][u][d];  // (row tiles past the wavefront's share of a short pass: zeros)
+              const uint32_t w8 = word >> 8;
+              const uint32_t a0 = unpack(and_or(word, 0x000F000Fu, magic), k1031, s16[t]);  // (q0, q4)
+              const uint32_t a1 = unpack(and_or(word, 0x00F000F0u, magic), k1136, s16[t]);  // 16 (q1, q5)
+              const uint32_t a2 = unpack(and_or(w8, 0x000F000Fu, magic), k1031, s16[t]);    // (q2, q6)
+              const uint32_t a3 = unpack(and_or(w8, 0x00F000F0u, magic), k1136, s16[t]);    // 16 (q3, q7)
+              const half8_t aop = __builtin_bit_cast(half8_t, uint4_t{a0, a1, a2, a3});
+#pragma unroll
+              for (int r = 0; r < R; ++r) acc[t][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop, xb[r], acc[t][r], 0, 0, 0);
+            }
+          }
+        }
+      }
+      const bool last = cc.q == cc.Q - 1;
+      if ((cc.q & 1) == 1 || last) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wavefront's reads of the panel have returned
+        if (lane == 0) __hip_atomic_fetch_add(&flags->x_taken[pk % nxb], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (((cc.q & 3) == 3 || last) && lane == 0)
+          __hip_atomic_fetch_add(&flags->s_taken[sk & 1], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      if (last) {
+        if (c_tr > 0) epilogue();
+        if (cc.left <= kRW * TR && (descs[cc.lin].g_dep & kSignal)) {
+          // the linear is complete once the stores of all 8 compute wavefronts are written through
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          int old = 0;
+          int* const cnt = &flags->lin_done[cc.lin & 7];
+          if (lane == 0) old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if (__builtin_amdgcn_readfirstlane(old) == kRW - 1 && lane == 0) {
+            __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(sync + sync_counter_index(cc.lin, b & (kCountersPerLinear - 1)), 1, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+      }
+      if (wave == 0) rows_advance<TR, true>(cc, 1, descs, nlin, b, nwg, sync, lane);
+      else rows_advance<TR, false>(cc, 1, descs, nlin, b, nwg, sync, lane);
+    };
+
+#pragma unroll
+    for (int t = 0; t < NT; ++t) issue(tb[t]);
+    while (cc.lin < nlin) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        if (cc.lin < nlin) consume(tb[t]);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing of the ring (or of the signals) is in flight any more
+    if (!use_sync) return;
+    // the last compute wavefront of the last workgroup to get here clears the counters for the next launch
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(&flags->exited, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (__builtin_amdgcn_readfirstlane(old) != kRW - 1) return;
+    int lastwg = 0;
+    if (lane == 0)
+      lastwg = __hip_atomic_fetch_add(sync + sync_finished_index(nlin), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nwg - 1;
+    if (__builtin_amdgcn_readfirstlane(lastwg)) {
+      for (int k = lane; k < nlin * kCountersPerLinear; k += 64)
+        __hip_atomic_store(sync + k * kCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0)
+        __hip_atomic_store(sync + sync_finished_index(nlin), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return;
+  }
+
+  if (wave < kRW + kRXW) {
+    // ====================== x wavefronts: a panel of activations -> LDS ======================
+    const int xw = wave - kRW;
+    bool aborted = false;
+    auto wait_for = [&](int dep) {
+      if (aborted) return;
+      const long long t0 = wall_clock64();
+      while (true) {
+        int v = 0;
+        if (lane < kCountersPerLinear)
+          v = __hip_atomic_fetch_add(sync + sync_counter_index(dep, lane), 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 4, 64);
+        if (__builtin_amdgcn_readfirstlane(v) >= (nwg >> (desc_group_word(descs, dep) & 0xffu))) break;  // every member of its group
+        if (wall_clock64() - t0 > spin_limit) {
+          aborted = true;
+          if (lane == 0)
+            __hip_atomic_store(sync + sync_error_index(nlin), dep + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    };
+    const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+    constexpr int PPR = kRPG * 4;  // 16-byte pieces (8 activations) per row and panel
+    constexpr int UX = 32;         // loads in flight per lane: a whole panel of 32 rows
+    RowsCursor xc;
+    xc.lin = 0;
+    rows_seek<TR, false>(xc, descs, nlin, b, nwg, sync, lane);
+    int pk = 0;
+    int confirmed = -1;
+    while (xc.lin < nlin) {
+      if (pk % kRXW == xw) {
+        const int xslot = pk % nxb;
+        if (pk >= nxb) wait.until(&flags->x_taken[xslot], kRW * (pk / nxb), 4);
+        const int j = xc.lin;
+        const int dep = (int)((descs[j].g_dep >> 16) & 0x7fffu) - 1;
+        if (dep >= 0 && dep != confirmed) {
+          wait_for(dep);
+          confirmed = dep;
+        }
+        const int K8 = xc.G << 2;
+        const int xrows = (int)((desc_group_word(descs, j) >> 16) & 0xffu);
+        const __amdgpu_buffer_rsrc_t xr =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(descs[j].x), 0, xrows * K8 * 16, kBufferFlags);
+        char* const xdst = xbuf + xslot * xbuf_bytes;
+        const int p0 = xc.q * (kRPairGroups * 4);  // the panel's first piece within a row
+        const int total = M * PPR;
+        for (int base = 0; base < total; base += 64 * UX) {
+          uint4_t v[UX];
+#pragma unroll
+          for (int t = 0; t < UX; ++t) {
+            const int idx = base + t * 64 + lane;
+            const int row = idx / PPR, o = idx & (PPR - 1);
+            const int go = p0 + o;
+            v[t] = uint4_t{0, 0, 0, 0};
+            const int src = min(row, xrows - 1);
+            if (idx < total && go < K8)
+              v[t] = dep >= 0 ? __builtin_amdgcn_raw_buffer_load_b128(xr, (src * K8 + go) * 16, 0, kDeviceScope)
+                              : __builtin_amdgcn_raw_buffer_load_b128(xr, (src * K8 + go) * 16, 0, 0);
+          }
+#pragma unroll
+          for (int t = 0; t < UX; ++t) {
+            const int idx = base + t * 64 + lane;
+            if (idx < total) {
+              const int row = idx / PPR, o = idx & (PPR - 1);
+              const uint32_t in[4] = {v[t].x, v[t].y, v[t].z, v[t].w};
+              uint32_t p[4];
+              pair_i_i4(in, p);  // p[e] = (x_e, x_{e+4})
+              // piece o: scale group g = o / 4 of the panel, dword d = o % 4 of it; step g / 4, lane quarter g % 4
+              const int g = o >> 2, d = o & 3;
+              char* dst = xdst + ((((g >> 2) * 4 + d) * 4 + (g & 3)) * M + row) * 16;
+              *reinterpret_cast<uint4_t*>(dst) =
+                  uint4_t{p[0], as_u32(as_half2(p[1]) * sixteenth), p[2], as_u32(as_half2(p[3]) * sixteenth)};
+            }
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) __hip_atomic_store(&flags->x_ready[xslot], pk + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      ++pk;
+      rows_advance<TR, false>(xc, kRPG / kRPairGroups, descs, nlin, b, nwg, sync, lane);
+    }
+    return;
+  }
+
+  // ====================== scale wavefront: the scales of a pass, 1024 k at a time -> LDS ======================
+  {
+    constexpr int PPR = kRSPG / 8;              // 16-byte pieces (8 scales) per row and panel
+    constexpr int LP = kRW * TROWS * PPR / 64;  // pieces per lane and panel
+    RowsCursor sc;
+    sc.lin = 0;
+    rows_seek<TR, false>(sc, descs, nlin, b, nwg, sync, lane);
+    int sk = 0;
+    while (sc.lin < nlin) {
+      const int sslot = sk & 1;
+      const int g0 = sc.q * kRPairGroups;  // first scale group of the panel
+      const __amdgpu_buffer_rsrc_t sr = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<char*>(sc.S), 0, (int)min((int64_t)sc.N * sc.G * 2, (int64_t)0x7fffffff), kBufferFlags);
+      uint4_t v[LP];
+#pragma unroll
+      for (int t = 0; t < LP; ++t) {
+        const int idx = t * 64 + lane;
+        const int rr = idx / PPR, pc = idx % PPR;
+        const int w = rr / TROWS, r = rr % TROWS;
+        const int row = sc.first_of(w) * 16 + r;
+        v[t] = uint4_t{0, 0, 0, 0};  // rows past the wavefront's or past N, groups past K: a zero scale
+        if (r < sc.tiles_of(w, TR) * 16 && row < sc.N && g0 + pc * 8 < sc.G)
+          v[t] = __builtin_amdgcn_raw_buffer_load_b128(sr, (row * sc.G + g0 + pc * 8) * 2, 0, 0);
+      }
+      // the buffer is free once every compute wavefront has left the panel that used it before
+      if (sk >= 2) wait.until(&flags->s_taken[sslot], kRW * (sk / 2), 5);
+#pragma unroll
+      for (int t = 0; t < LP; ++t) {
+        const int idx = t * 64 + lane;
+        const int rr = idx / PPR, pc = idx % PPR;
+        *reinterpret_cast<uint4_t*>(sbuf + sslot * SBUF + rr * kRSRow + pc * 16) = v[t];
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      ++sk;
+      if (lane == 0) __hip_atomic_store(&flags->s_ready[sslot], sk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      rows_advance<TR, false>(sc, kRSPG / kRPairGroups, descs, nlin, b, nwg, sync, lane);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ host side
 // the kernel a list of M activation rows runs: chunks per wavefront and tile, sets of 16 activation rows, tile rows / 16
 struct BatchShape {
@@ -683,9 +1220,8 @@ struct BatchShape {
 };
 static BatchShape batch_shape(int M) {
   if (M <= 8) return {4, 1, 1};   // tiles of 16 rows, panels of 4096 k (tiles of 32 rows x 2048 k: the same time at M = 8, slower at M = 4)
-  if (M <= 16) return {4, 1, 2};  // 32 rows, 2048 k (16 rows x 2048 k, chunks of 2: 0.90 instead of 0.81 ms for the Llama-2-7B stack)
-  return {2, 2, 2};               // 32 rows, 1024 k: a panel of activations is 64 KiB at most (16 rows x 1024 k: 1.36 instead of 1.11 ms)
-}
+  return {4, 1, 2};               // 32 rows, 2048 k (16 rows x 2048 k, chunks of 2: 0.90 instead of 0.81 ms for the Llama-2-7B stack)
+}                                 // (more than 16 rows: q4g32_batch_rows_kernel)
 
 static size_t batch_lds_bytes(BatchShape s, int M, int nxb, int ring, int acc_tiles) {
   return sizeof(BatchFlags) + (size_t)nxb * M * batch_panel_groups(s.U, s.TW) * 64 + (size_t)ring * batch_scale_slot_bytes(s.U, s.TW) +
@@ -740,16 +1276,108 @@ static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, BatchSh
 
 // the kernel that walks the tiles of a linear in chunks carries more loop state: only where a list needs it
 typedef void (*batch_kernel_t)(const GemvListDesc*, int, int*, long long, int, int, int, int, int);
-static int batch_kernel_index(BatchShape s) { return s.R == 2 ? 2 : s.TW == 2 ? 1 : 0; }
+static int batch_kernel_index(BatchShape s) { return s.TW == 2 ? 1 : 0; }
 static batch_kernel_t batch_kernel(BatchShape s, bool chunked) {
   switch (batch_kernel_index(s)) {
-    case 2: return chunked ? q4g32_batch_list_kernel<2, 2, 2, true> : q4g32_batch_list_kernel<2, 2, 2, false>;
     case 1: return chunked ? q4g32_batch_list_kernel<4, 1, 2, true> : q4g32_batch_list_kernel<4, 1, 2, false>;
     default: return chunked ? q4g32_batch_list_kernel<4, 1, 1, true> : q4g32_batch_list_kernel<4, 1, 1, false>;
   }
 }
 
+// ---- lists of more than 16 activation rows: q4g32_batch_rows_kernel
+constexpr int kRowsTR = 4;  // row tiles of a wave tile: 64 rows
+static size_t rows_lds_bytes(int M, int nxb) {
+  return sizeof(RowsFlags) + (size_t)nxb * M * kRPG * 64 + 2 * (size_t)kRW * 16 * kRowsTR * kRSRow;
+}
+
+// as batch_assign_groups, with the duration of a linear from the passes a workgroup makes over its wave tiles
+// (every pass loads all activations; a pass of fewer than 8 wave tiles takes as long as a full one)
+static BatchGroupPlan rows_assign_groups(const wq_gemv_list* l, int gl) {
+  const int groups = 1 << gl, ncu = l->blocks >> gl;
+  BatchGroupPlan plan;
+  plan.group.resize(l->n);
+  std::vector<double> free_at(groups, 0.0), end(l->n, 0.0);
+  for (int i = 0; i < l->n; ++i) {
+    const GemvListDesc& g = l->descs[i];
+    const double K = (double)(g.g_dep & 0xffffu) * 32.0;
+    const int64_t tiles = ((int64_t)g.N + 15) / 16;   // row tiles
+    int64_t left = (tiles + ncu - 1) / ncu;             // of the workgroup with most
+    double dur = 4096.0;
+    while (left > 0) {  // pass by pass: 8 wavefronts x tr row tiles, and all activations
+      const int64_t take = std::min<int64_t>(left, kRW * kRowsTR);
+      const double tr = (double)((take + kRW - 1) / kRW);
+      dur += kRW * tr * 16.0 * K * (0.5 + 1.0 / 16.0) + l->M * K * 2.0;
+      left -= take;
+    }
+    const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
+    const double ready = dep >= 0 ? end[dep] : 0.0;
+    int best = 0;
+    for (int c = 1; c < groups; ++c) {
+      const double sb = std::max(free_at[best], ready), sc = std::max(free_at[c], ready);
+      if (sc < sb || (sc == sb && free_at[c] > free_at[best])) best = c;
+    }
+    plan.group[i] = best;
+    end[i] = std::max(free_at[best], ready) + dur;
+    free_at[best] = end[i];
+  }
+  for (double f : free_at) plan.makespan = std::max(plan.makespan, f);
+  return plan;
+}
+
+static int rows_list_plan(wq_gemv_list* l) {
+  for (int i = 0; i < l->n; ++i)  // the scales are addressed with 32-bit offsets
+    if ((int64_t)l->descs[i].N * (l->descs[i].g_dep & 0xffffu) * 2 >= (1ll << 31))
+      return fail(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d: with more than 16 rows of activations the scales must stay below 2 GiB", i);
+  l->batch_rows = true;
+  l->batch_u = 2;
+  l->threads = kRThreads;
+  l->blocks = std::min(cu_count(), 32768);
+  const size_t budget = 160 * 1024;
+  int nxb = kRMaxXBuf;
+  while (nxb > 1 && rows_lds_bytes(l->M, nxb) > budget) --nxb;
+  if (rows_lds_bytes(l->M, nxb) > budget)
+    return fail(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: %d rows of activations do not fit the LDS", l->M);
+  int best_gl = -1;
+  BatchGroupPlan best;
+  for (int gl = 0; gl <= 6; ++gl) {
+    if (l->blocks % (1 << gl) != 0 || (l->blocks >> gl) < 1) break;
+    BatchGroupPlan p = rows_assign_groups(l, gl);
+    if (best_gl < 0 || p.makespan < best.makespan * 0.98) {
+      best_gl = gl;
+      best = std::move(p);
+    }
+  }
+  const int groups = 1 << best_gl, ncu = l->blocks >> best_gl;
+  std::vector<int64_t> off(groups, 0);
+  for (int i = 0; i < l->n; ++i) {
+    GemvListDesc& g = l->descs[i];
+    const int c = best.group[i];
+    const int64_t tiles = ((int64_t)g.N + 15) / 16;  // row tiles
+    g.q = (int32_t)(tiles / ncu);
+    g.rem = (uint16_t)(tiles % ncu);
+    g.off = (uint16_t)off[c];
+    off[c] = (off[c] + tiles) % ncu;
+    g.gmod_log2 = (uint8_t)best_gl;
+    g.gidx = (uint8_t)c;
+  }
+  l->batch_groups = groups;
+  l->batch_nxb = nxb;
+  l->batch_ring = 2;
+  l->batch_acc_tiles = 0;
+  l->batch_chunked = false;
+  l->lds = rows_lds_bytes(l->M, nxb);
+  const void* kern = reinterpret_cast<const void*>(q4g32_batch_rows_kernel<kRowsTR, 2>);
+  static DynamicLdsLimit limit;
+  if (limit.ensure(kern, (int)l->lds) != hipSuccess)
+    return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
+  int resident = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
+    return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: the workgroup does not fit a CU (%zu bytes of LDS)", l->lds);
+  return WQ_OK;
+}
+
 int batch_list_plan(wq_gemv_list* l) {
+  if (l->M > 16) return rows_list_plan(l);
   const BatchShape s = batch_shape(l->M);
   const int U = s.U;
   const int trows = 16 * s.TW;
@@ -812,7 +1440,7 @@ int batch_list_plan(wq_gemv_list* l) {
   l->lds = batch_lds_bytes(s, l->M, l->batch_nxb, l->batch_ring, best_acc);
   const void* kern = reinterpret_cast<const void*>(batch_kernel(s, best_chunked));
   // several lists share a kernel: the limit only ever grows
-  static DynamicLdsLimit limits[3][2];
+  static DynamicLdsLimit limits[2][2];
   if (limits[batch_kernel_index(s)][best_chunked ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
     return fail(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
   int resident = 0;
@@ -824,6 +1452,11 @@ int batch_list_plan(wq_gemv_list* l) {
 int batch_list_launch(wq_gemv_list* l, hipStream_t stream) {
   const GemvListDesc* table = (const GemvListDesc*)l->table;
   const int use_sync = l->deps > 0 ? 1 : 0;
+  if (l->batch_rows) {
+    WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_batch_rows_kernel<kRowsTR, 2>), dim3((unsigned)l->blocks), dim3((unsigned)l->threads), l->lds,
+              stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, use_sync);
+    return WQ_OK;
+  }
   // chunk: at least 1 (a list without a linear of several panels keeps no sums)
   WQ_LAUNCH("wq_q4g32_gemv_list_run", batch_kernel(batch_shape(l->M), l->batch_chunked), dim3((unsigned)l->blocks), dim3((unsigned)l->threads), l->lds,
             stream, table, l->n, l->sync, l->spin_limit, l->M, l->batch_nxb, l->batch_ring, std::max(l->batch_acc_tiles, 1),

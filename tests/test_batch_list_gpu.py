@@ -1,5 +1,6 @@
 """wq_q4g32_gemv_list_create_batched: a list of linears with 2 .. 32 rows of activations in one launch (matrix
-cores; more than 16 rows as two sets of 16 per weight tile), against the CPU oracle, through the C ABI."""
+cores; up to 16 rows: tiles split along K among the wavefronts; more: wavefronts that own rows of W and keep their
+sums in registers), against the CPU oracle, through the C ABI."""
 import numpy as np
 import pytest
 
@@ -113,10 +114,10 @@ def test_epilogue_and_one_hot(env, oracle, M, N, shift):
         assert np.array_equal(got[m].view(np.uint16), B[:, c].view(np.uint16)), (m, c)
 
 
-def test_tiles_walked_in_chunks_with_a_ragged_end(env, oracle):
-    """One linear of two panels (M = 20: panels of 1024 k) with more tiles per workgroup than LDS keeps sums for: the
-    tiles are walked in chunks.  N is odd (2-byte stores) and ends 7 rows into a 32-row tile (its second 16 rows
-    lie past N)."""
+def test_many_passes_with_a_ragged_end(env, oracle):
+    """One long linear at M = 20 (the kernel whose wavefronts own rows of W): every workgroup makes several passes
+    over its rows, the last one short (fewer row tiles per wavefront, some wavefronts without any).  N is odd
+    (2-byte stores) and ends 7 rows into a row tile."""
     ops, u, torch = env
     M, N, K = 20, 150007, 2048
     l = _linear(oracle, u, N, K, M, seed=77)
@@ -124,10 +125,31 @@ def test_tiles_walked_in_chunks_with_a_ragged_end(env, oracle):
     bias = rng.standard_normal(N).astype(np.float16)
     y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
     gl = ops.Q4G32GemvList([(l["dW"], l["dS"], u.dev(l["x"]), y, u.dev(bias))], M=M)
-    print("batch list: chunks", flush=True)
+    print("batch list: many passes", flush=True)
     gl.run()
     gl.status()
-    u.assert_close(u.host(y), oracle.q4g32_linear(l["W"], l["S"], l["x"], bias=bias, nthreads=8), "batch list in chunks")
+    u.assert_close(u.host(y), oracle.q4g32_linear(l["W"], l["S"], l["x"], bias=bias, nthreads=8), "batch list, many passes")
+
+
+@pytest.mark.parametrize("M,N,K", [(19, 16 * 37 + 5, 512), (32, 8 * 64 * 3 + 16 * 11, 768), (25, 33, 256), (17, 4096, 11008)])
+def test_short_passes_of_the_row_owner_kernel(env, oracle, M, N, K):
+    """M > 16, a list of ONE linear (every workgroup takes part): N chosen so that workgroups hold a few row tiles
+    only (one per wavefront, some wavefronts idle), a last row tile that ends past N, and K of 1, 1.5, 0.5 and 21.5
+    panels of activations (an odd number of 256-k pairs ends a panel after one pair); with bias and residual."""
+    ops, u, torch = env
+    l = _linear(oracle, u, N, K, M, seed=N + K)
+    rng = np.random.default_rng(N)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    gl = ops.Q4G32GemvList([(l["dW"], l["dS"], u.dev(l["x"]), y, u.dev(bias), u.dev(res))], M=M)
+    print(f"batch list: short passes M={M} N={N} K={K}", flush=True)
+    for _ in range(2):
+        y.zero_()
+        gl.run()
+        gl.status()
+        u.assert_close(u.host(y), oracle.q4g32_linear(l["W"], l["S"], l["x"], bias=bias, residual=res, nthreads=8),
+                       f"batch list short passes {M}x{N}x{K}")
 
 
 @pytest.mark.parametrize("M", [4, 12, 27])
