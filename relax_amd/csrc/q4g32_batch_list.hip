@@ -705,9 +705,16 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
 //     an empty buffer and only takes part in the hand-overs.
 //   * A linear's completion counter is raised by the last of the 8 compute wavefronts to have its stores
 //     written through.
-// What bounds it: bytes through the CU.  Codes, scales and the activations of every pass (M x K x 2 bytes per
-// 512 rows: 22 % of the codes at M = 32) together arrive at the rate the one-row list kernel reaches with
-// codes and scales alone.
+// What bounds it (cycle counters around the phases of a compute wavefront, an instrumented copy): not memory.  A
+// compute wavefront waits for its weights 1 % of the time; 43 .. 58 % goes into unpacking and multiplying a pair
+// (about 1100 instructions, 6 .. 8 cycles each with two such wavefronts per SIMD), 13 .. 19 % into the lane
+// exchange and the refill, and the wavefronts that share a SIMD with an older one are slower, so the older ones
+// wait for them at the hand-over of the panels (35 % of their time).  Measured and not kept: B operands and
+// scales requested from LDS one step ahead (no change), the refill spread over the multiplication (no change),
+// a raised priority for the service wavefronts (M = 17 slower), 12 compute wavefronts of 48 rows (128 registers:
+// 5 % slower), branches around the row tiles a short pass does not have (5 % slower: the unrolled code no longer
+// interleaves).  The activations of every pass (M x K x 2 bytes per 512 rows: 22 % of the codes at M = 32)
+// cost what their bytes cost: the stack step grows by 4.5 us per row of activations.
 constexpr int kRW = 8;      // compute wavefronts
 constexpr int kRXW = 2;     // wavefronts that stage activations
 constexpr int kRThreads = 64 * (kRW + kRXW + 1);
@@ -989,10 +996,8 @@ __global__ __launch_bounds__(kRThreads) void q4g32_batch_rows_kernel(const GemvL
           const uint32_t hi_in = d == 0 ? buf[t][1].x : d == 1 ? buf[t][1].y : d == 2 ? buf[t][1].z : buf[t][1].w;
           asm volatile("v_mov_b32_dpp %0, %2 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf\n\t"
                        "v_mov_b32_dpp %1, %3 quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0xf\n\t"
-                       "s_nop 1\n\t"
                        "v_mov_b32_dpp %0, %3 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-                       "v_mov_b32_dpp %1, %2 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-                       "s_nop 1 ; %4"
+                       "v_mov_b32_dpp %1, %2 row_ror:8 row_mask:0xf bank_mask:0x3 ; %4"
                        : "=&v"(cw[t][0][d]), "=&v"(cw[t][1][d])
                        : "v"(lo_in), "v"(hi_in), "v"(magic));
         }
@@ -1303,12 +1308,8 @@ static BatchGroupPlan rows_assign_groups(const wq_gemv_list* l, int gl) {
     const int64_t tiles = ((int64_t)g.N + 15) / 16;   // row tiles
     int64_t left = (tiles + ncu - 1) / ncu;             // of the workgroup with most
     double dur = 4096.0;
-    while (left > 0) {  // pass by pass: 8 wavefronts x tr row tiles, and all activations
-      const int64_t take = std::min<int64_t>(left, kRW * kRowsTR);
-      const double tr = (double)((take + kRW - 1) / kRW);
-      dur += kRW * tr * 16.0 * K * (0.5 + 1.0 / 16.0) + l->M * K * 2.0;
-      left -= take;
-    }
+    const double passes = (double)((left + kRW * kRowsTR - 1) / (kRW * kRowsTR));
+    dur += passes * (kRW * kRowsTR * 16.0 * K * (0.5 + 1.0 / 16.0) + l->M * K * 2.0);
     const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
     const double ready = dep >= 0 ? end[dep] : 0.0;
     int best = 0;
