@@ -321,6 +321,8 @@ static std::vector<int> schedule_group(const std::vector<DecodeLinear>& lin) {
 // short one cannot: four Llama-2-7B linears (one decoder layer) take 48 / 78 / 100 us as a list against
 // 43 / 52 / 71 us call by call at M = 8 / 16 / 32; eight linears 40 / 61 / 56 against 45 / 52 / 71; sixteen
 // 37 / 39 / 54 against 44 / 52 / 71.  At M <= 4 the list wins from the first layer on (30 against 42 us).
+// (M = 32 with the kernel whose wavefronts own rows of W: 111 / 73 / 53 us per layer for lists of 4 / 8 / 32
+// linears against 71.)
 static size_t min_fused_run(int64_t M) { return M <= 4 ? 2 : M <= 8 ? 8 : M <= 16 ? 16 : 8; }
 
 static void find_groups(wq_program* p) {
