@@ -88,14 +88,13 @@ __device__ __forceinline__ half_t intb_finish(float v, int m, int n, int N, cons
 }
 
 // R column groups per wavefront, MB rows of A, U pieces per lane in flight per group.
-template <int NBIT, int R, int MB>
+template <int NBIT, int R, int MB, int U>
 __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
     const uint4_t* __restrict__ B, const half_t* __restrict__ scales, const half_t* __restrict__ A,
     half_t* __restrict__ C, int N, int K, int group, int ngroups, IntbEpilogue ep) {
   constexpr int I = NBIT == 8 ? 2 : 4;      // interleaved columns per group
   constexpr int PPT = NBIT == 8 ? 4 : 2;    // pieces per column per tile
   constexpr int XQ = NBIT == 8 ? 2 : 4;     // 16-byte chunks of x per piece
-  constexpr int U = 4;                      // pieces per lane per round
   extern __shared__ uint4_t smem[];
   uint4_t* xs = smem;                                        // [MB][K/8] chunks of 8 halves
   float* cs = reinterpret_cast<float*>(smem + MB * (K >> 3));  // [MB][K/16 or K/32] folded offsets
@@ -297,7 +296,7 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
   }
 }
 
-template <int NBIT, int R, int MB>
+template <int NBIT, int R, int MB, int U = (NBIT == 8 ? 4 : 1)>
 static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* scales, uint16_t* C,
                             int64_t N, int64_t K, int64_t group, const IntbEpilogue& ep,
                             hipStream_t stream) {
@@ -306,7 +305,7 @@ static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* 
   const int waves = kIntbGemvThreads / 64;
   const int64_t blocks = (ngroups + waves * R - 1) / (waves * R);
   const size_t lds = (size_t)MB * K * 2 + (size_t)MB * (K / (NBIT == 8 ? 16 : 32)) * 4;
-  auto kern = intb_gemv_kernel<NBIT, R, MB>;
+  auto kern = intb_gemv_kernel<NBIT, R, MB, U>;
   if (lds > 60 * 1024) {
     static DynamicLdsLimit limit;  // per instantiation
     WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), (int)lds));
@@ -334,10 +333,12 @@ int intb_gemv_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scale
                      : launch_intb_gemv<4, 2, 2>(a, B, scales, c, n, k, group, ep, stream);
       m0 += 2;
     } else {
-      // column groups per wavefront: one with per-channel scales (K = 8192, N = 28672: int8 40.4 -> 37.9 us, int4
-      // 27.2 -> 26.3 us), two with group scales, whose 8- or 16-byte scale vectors then serve both (int8 45.4
-      // against 48.1 us)
-      const int R = tuning().gemv_rows ? tuning().gemv_rows : (group > 0 ? 2 : 1);
+      // column groups per wavefront and pieces per lane in flight per group (K = 8192, N = 28672, M = 1).  int8: one
+      // group with per-channel scales (40.4 -> 37.9 us), two with group scales, whose 8- or 16-byte scale vectors
+      // then serve both (45.4 against 48.1 us), four pieces (66 registers).  int4: two groups, ONE piece: with four
+      // pieces the compiler keeps 16 LDS operands per piece in registers (154: three wavefronts per SIMD); one piece
+      // needs 68 (seven per SIMD): per-channel 27.2 -> 22.2 us, group-64 27.1 -> 23.2 us.
+      const int R = tuning().gemv_rows ? tuning().gemv_rows : (group > 0 || nbit == 4 ? 2 : 1);
       if (R == 1)
         rc = nbit == 8 ? launch_intb_gemv<8, 1, 1>(a, B, scales, c, n, k, group, ep, stream)
                        : launch_intb_gemv<4, 1, 1>(a, B, scales, c, n, k, group, ep, stream);
