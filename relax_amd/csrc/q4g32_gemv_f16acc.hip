@@ -42,32 +42,49 @@ __global__ __launch_bounds__(256) void q4g32_gemv_f16acc_kernel(const uint4_t* _
   half2_t acc[ROWS];
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) acc[r] = half2_t{(half_t)0.0f, (half_t)0.0f};
-  for (int g = lane; g < G; g += 64) {
-    // the group's 32 activations in the (i, i+4) pairing of the unpack
-    uint32_t xp[4][4];
+  // UNR scale groups per lane and row are requested before the first is multiplied (the order of the sums is
+  // that of one group after the other)
+  constexpr int UNR = 4;
+  for (int g0 = lane; g0 < G; g0 += 64 * UNR) {
+    uint4_t w4[UNR][ROWS];
+    half_t sc[UNR][ROWS];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint4_t v = reinterpret_cast<const uint4_t*>(x)[g * 4 + c];
-      const uint32_t in[4] = {v.x, v.y, v.z, v.w};
-      pair_i_i4(in, xp[c]);
+    for (int j = 0; j < UNR; ++j) {
+      const int g = min(g0 + 64 * j, G - 1);
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        const int n = min(n0 + r, N - 1);
+        w4[j][r] = __builtin_nontemporal_load(&W[(int64_t)n * G + g]);
+        sc[j][r] = S[(int64_t)n * G + g];
+      }
     }
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int n = min(n0 + r, N - 1);
-      const uint4_t w4 = __builtin_nontemporal_load(&W[(int64_t)n * G + g]);
-      const half_t s = S[(int64_t)n * G + g];
-      const half2_t s2 = {s, s};
-      const uint32_t words[4] = {w4.x, w4.y, w4.z, w4.w};
+    for (int j = 0; j < UNR; ++j) {
+      const int g = g0 + 64 * j;
+      if (g >= G) break;
+      // the group's 32 activations in the (i, i+4) pairing of the unpack
+      uint32_t xp[4][4];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        half2_t d[4];
-        q4_word_dequant(words[c], s2, d);
+        const uint4_t v = reinterpret_cast<const uint4_t*>(x)[g * 4 + c];
+        const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+        pair_i_i4(in, xp[c]);
+      }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          // product rounded to fp16, then the sum rounded to fp16: two instructions on purpose
-          half2_t p;
-          asm("v_pk_mul_f16 %0, %1, %2" : "=v"(p) : "v"(d[i]), "v"(as_half2(xp[c][i])));
-          asm("v_pk_add_f16 %0, %1, %2" : "=v"(acc[r]) : "v"(acc[r]), "v"(p));
+      for (int r = 0; r < ROWS; ++r) {
+        const half2_t s2 = {sc[j][r], sc[j][r]};
+        const uint32_t words[4] = {w4[j][r].x, w4[j][r].y, w4[j][r].z, w4[j][r].w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          half2_t d[4];
+          q4_word_dequant(words[c], s2, d);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            // product rounded to fp16, then the sum rounded to fp16: two instructions on purpose
+            half2_t p;
+            asm("v_pk_mul_f16 %0, %1, %2" : "=v"(p) : "v"(d[i]), "v"(as_half2(xp[c][i])));
+            asm("v_pk_add_f16 %0, %1, %2" : "=v"(acc[r]) : "v"(acc[r]), "v"(p));
+          }
         }
       }
     }
