@@ -37,6 +37,10 @@ void wq_debug_set_gemv_blocks_per_cu(int n);
 /* Small-batch kernel: wavefronts side by side (1, 2, 4, 8), ring slots, and which kernel
  * (waves 1: ring, 2: activations in registers); 0 = from the shape. */
 void wq_debug_set_skinny_config(int nw, int stages, int waves);
+/* How a list of 2 .. 32 activation rows was planned: the number of equal groups of workgroups that run
+ * different linears side by side, or 0 if the linears of the (short) list share the 8 XCDs in sets sized by
+ * their cost; -1 for a list of one activation row. */
+int wq_debug_gemv_list_groups(const wq_gemv_list_t* list);
 
 /* ---- librelax_amd_wq_calibrate.so ---- */
 /* Issues `iters` x 8 independent v_mfma_f32_32x32x16_f16 per wavefront, four wavefronts

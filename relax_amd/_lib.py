@@ -81,13 +81,14 @@ _RESTYPES = {"wq_program_unfused_reason": ctypes.c_char_p, "wq_last_error": ctyp
              "wq_gptq_workspace_bytes": _sz, "wq_q4g32_kn_gemv_workspace_bytes": _sz, "wq_gptq_padded_workspace_bytes": _sz, "wq_gptq_padded_k_bound": _i64, "wq_q4g32_gemv_list_workspace_bytes": _sz,
              "wq_q4g32_gemv_list_create": _vp, "wq_q4g32_gemv_list_create_batched": _vp, "wq_q4g32_gemv_list_destroy": None}
 
-# include/relax_amd_wq_testing.h: the work-split overrides of the calling thread (all return void)
+# include/relax_amd_wq_testing.h: the work-split overrides of the calling thread (void) and one query (int)
 TESTING_SIGNATURES = {
     "wq_debug_set_gemm_config": [_int],
     "wq_debug_set_gemm_tail_split": [_int],
     "wq_debug_set_gemv_config": [_int, _int],
     "wq_debug_set_gemv_blocks_per_cu": [_int],
     "wq_debug_set_skinny_config": [_int, _int, _int],
+    "wq_debug_gemv_list_groups": [_vp],
 }
 # ... and the calibration kernels of librelax_amd_wq_calibrate.so
 CALIBRATE_LIB_PATH = os.path.join(HERE, "librelax_amd_wq_calibrate.so")
@@ -125,7 +126,7 @@ def lib() -> ctypes.CDLL:
         for name, argtypes in TESTING_SIGNATURES.items():
             fn = getattr(l, name)
             fn.argtypes = argtypes
-            fn.restype = None
+            fn.restype = ctypes.c_int if name == "wq_debug_gemv_list_groups" else None
         _lib = l
     return _lib
 

@@ -318,12 +318,13 @@ static std::vector<int> schedule_group(const std::vector<DecodeLinear>& lin) {
 
 // Shortest run worth one launch of the list kernel, by rows of x.  With several rows every workgroup of a
 // linear's group loads all of that linear's activations, which a long list spreads over many small groups and a
-// short one cannot: four Llama-2-7B linears (one decoder layer) take 48 / 78 / 100 us as a list against
-// 43 / 52 / 71 us call by call at M = 8 / 16 / 32; eight linears 40 / 61 / 56 against 45 / 52 / 71; sixteen
-// 37 / 39 / 54 against 44 / 52 / 71.  At M <= 4 the list wins from the first layer on (30 against 42 us).
-// (M = 32 with the kernel whose wavefronts own rows of W: 111 / 73 / 53 us per layer for lists of 4 / 8 / 32
-// linears against 71.)
-static size_t min_fused_run(int64_t M) { return M <= 4 ? 2 : M <= 8 ? 8 : M <= 16 ? 16 : 8; }
+// short one cannot (its linears share the 8 XCDs in proportion to their cost instead).  Llama-2-7B linears,
+// us per decoder layer (4 linears), list against call by call:
+//   M = 8:  one layer 41.5 / 44.4, two 40.2 / 44.3, four 37.0 / 44.5
+//   M = 16: one layer 62.4 / 52.0, two 61.8 / 51.8, four 39.2 / 51.9
+//   M = 32: one layer 111 / 70.6, two 73.8 / 70.7, four 44.2 / 70.7
+// At M <= 4 the list wins from the first layer on (30 against 42 us).
+static size_t min_fused_run(int64_t M) { return M <= 4 ? 2 : M <= 8 ? 4 : M <= 16 ? 16 : 12; }
 
 static void find_groups(wq_program* p) {
   drop_lists(p);

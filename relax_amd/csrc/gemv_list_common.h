@@ -24,8 +24,9 @@ struct GemvListDesc {  // 128 bytes, device memory
                        // bit 31: a later linear reads y
   uint16_t rem;        // row groups % workgroups
   uint16_t off;        // rotation: workgroup b owns the row groups local * workgroups + ((b - off) mod workgroups)
-  // words 16 ..: the batch kernel only.  A linear is run by ONE group of workgroups, those with
-  // b mod 2^gmod_log2 == gidx (member c = b >> gmod_log2 of workgroups >> gmod_log2); q, rem and off
+  // words 16 ..: the batch kernels only.  A linear is run by ONE group of workgroups: those with
+  // b mod 2^gmod_log2 == gidx (member c = b >> gmod_log2 of workgroups >> gmod_log2), or, with gmod_log2 = 0x80,
+  // those whose XCD (b mod 8) is in the mask gidx (members counted in order of b); q, rem and off
   // then count within the group.
   uint8_t gmod_log2, gidx;
   uint8_t rows;  // rows of x and y of this entry (the M of the launch)
@@ -83,7 +84,7 @@ struct wq_gemv_list {
   long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
   int M = 1;               // activation rows of the launch; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
   int batch_u = 0;         // chunks per tile and wavefront (4: M <= 16; 2: beyond)
-  int batch_groups = 1;    // groups of workgroups that run different linears side by side
+  int batch_groups = 1;    // groups of workgroups that run different linears side by side (0: sets of XCDs per linear)
   int batch_nxb = 0;       // panels of activations in LDS
   int batch_ring = 0;      // items the compute wavefronts may spread over (slots of scales and of partial sums)
   int batch_acc_tiles = 0; // tiles whose sums LDS keeps between the panels of a linear: a chunk of the workgroup's tiles

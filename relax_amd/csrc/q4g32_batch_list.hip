@@ -121,6 +121,37 @@ struct ItemCursor {
 
 // word 16 of a descriptor: gmod_log2 | gidx << 8 | rows << 16 (read as one word: a scalar load; single
 // bytes would come through a vector load and end up in vector registers)
+// Which workgroups run a linear (bits 0 .. 15 of that word), in two forms:
+//   * gmod_log2 = g < 0x80: the workgroups with b mod 2^g == gidx (for g = 3 one XCD: workgroup b runs on XCD
+//     b mod 8, so the activations stay in that XCD's L2);
+//   * gmod_log2 = 0x80: gidx is a MASK of XCDs, the group is every workgroup whose b mod 8 is in the mask.  This is
+//     what a short list uses: its few linears share the 8 XCDs in proportion to their bytes.
+// A member's index counts the members in order of b.
+struct GroupOf {
+  bool member;
+  int index, size;
+};
+__device__ __forceinline__ int group_size(uint32_t grp, int nwg) {
+  if (grp & 0x80u) return (nwg >> 3) * __builtin_popcount((grp >> 8) & 0xffu);
+  return nwg >> (grp & 0x7fu);
+}
+__device__ __forceinline__ GroupOf group_of(uint32_t grp, int b, int nwg) {
+  GroupOf r;
+  if (grp & 0x80u) {
+    const uint32_t mask = (grp >> 8) & 0xffu;
+    const int pc = __builtin_popcount(mask);
+    r.member = (mask >> (b & 7)) & 1u;
+    r.index = (b >> 3) * pc + __builtin_popcount(mask & ((1u << (b & 7)) - 1u));
+    r.size = (nwg >> 3) * pc;
+  } else {
+    const int gl = (int)(grp & 0x7fu);
+    r.member = (b & ((1 << gl) - 1)) == (int)((grp >> 8) & 0xffu);
+    r.index = b >> gl;
+    r.size = nwg >> gl;
+  }
+  return r;
+}
+
 __device__ __forceinline__ uint32_t desc_group_word(gemv_desc_ptr descs, int lin) {
   typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
   return ((words_ptr)(descs + lin))[16];
@@ -133,13 +164,13 @@ __device__ __forceinline__ void item_seek(ItemCursor& c, gemv_desc_ptr descs, in
   while (c.lin < nlin) {
     const words_ptr p = (words_ptr)(descs + c.lin);
     const uint32_t grp = p[16];
-    const int gl = (int)(grp & 0xffu);
-    if ((b & ((1 << gl) - 1)) == (int)((grp >> 8) & 0xffu)) {  // this workgroup's group runs the linear
+    const GroupOf go = group_of(grp, b, nwg);
+    if (go.member) {  // this workgroup's group runs the linear
       uint32_t w[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) w[i] = p[i];
-      const int ncu = nwg >> gl;
-      int rb = (b >> gl) - (int)(w[15] >> 16);
+      const int ncu = go.size;
+      int rb = go.index - (int)(w[15] >> 16);
       if (rb < 0) rb += ncu;
       const int T = (int)w[13] + (rb < (int)(w[15] & 0xffffu) ? 1 : 0);
       if (T > 0) {
@@ -418,7 +449,7 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
         v += __shfl_xor(v, 1, 64);
         v += __shfl_xor(v, 2, 64);
         v += __shfl_xor(v, 4, 64);
-        if (__builtin_amdgcn_readfirstlane(v) >= (nwg >> (desc_group_word(descs, dep) & 0xffu))) break;  // every member of its group
+        if (__builtin_amdgcn_readfirstlane(v) >= group_size(desc_group_word(descs, dep), nwg)) break;  // every member of its group
         if (wall_clock64() - t0 > spin_limit) {
           aborted = true;
           if (lane == 0)
@@ -562,10 +593,10 @@ __global__ __launch_bounds__(kBThreads) void q4g32_batch_list_kernel(const GemvL
     for (int lin = 0; lin < nlin; ++lin) {
       const uint32_t g_dep = descs[lin].g_dep;
       const uint32_t grp = desc_group_word(descs, lin);
-      const int gl = (int)(grp & 0xffu);
-      if ((b & ((1 << gl) - 1)) != (int)((grp >> 8) & 0xffu)) continue;  // another group's linear
-      const int ncu = nwg >> gl;
-      int rb = (b >> gl) - (int)descs[lin].off;
+      const GroupOf go = group_of(grp, b, nwg);
+      if (!go.member) continue;  // another group's linear
+      const int ncu = go.size;
+      int rb = go.index - (int)descs[lin].off;
       if (rb < 0) rb += ncu;
       const int T = descs[lin].q + (rb < (int)descs[lin].rem ? 1 : 0);
       const int N = descs[lin].N;
@@ -791,11 +822,11 @@ __device__ __forceinline__ void rows_seek(RowsCursor& c, gemv_desc_ptr descs, in
   while (c.lin < nlin) {
     const words_ptr p = (words_ptr)(descs + c.lin);
     const uint32_t grp = p[16];
-    const int gl = (int)(grp & 0xffu);
-    if ((b & ((1 << gl) - 1)) == (int)((grp >> 8) & 0xffu)) {  // this workgroup's group runs the linear
-      const int ncu = nwg >> gl;
+    const GroupOf go = group_of(grp, b, nwg);
+    if (go.member) {  // this workgroup's group runs the linear
+      const int ncu = go.size;
       const uint32_t w15 = p[15];
-      int rb = (b >> gl) - (int)(w15 >> 16);
+      int rb = go.index - (int)(w15 >> 16);
       if (rb < 0) rb += ncu;
       const int q = (int)p[13], rem = (int)(w15 & 0xffffu);
       const int cnt = q + (rb < rem ? 1 : 0);
@@ -1104,7 +1135,7 @@ __global__ __launch_bounds__(kRThreads) void q4g32_batch_rows_kernel(const GemvL
         v += __shfl_xor(v, 1, 64);
         v += __shfl_xor(v, 2, 64);
         v += __shfl_xor(v, 4, 64);
-        if (__builtin_amdgcn_readfirstlane(v) >= (nwg >> (desc_group_word(descs, dep) & 0xffu))) break;  // every member of its group
+        if (__builtin_amdgcn_readfirstlane(v) >= group_size(desc_group_word(descs, dep), nwg)) break;  // every member of its group
         if (wall_clock64() - t0 > spin_limit) {
           aborted = true;
           if (lane == 0)
@@ -1250,6 +1281,65 @@ struct BatchGroupPlan {
 // chunks a workgroup with `tiles` tiles of a linear walks them in (each chunk loads every panel of activations again)
 static int batch_chunks(int tiles, int panels, int chunk) { return panels > 1 && tiles > chunk ? (tiles + chunk - 1) / chunk : 1; }
 
+// bytes through one workgroup of a group of `ncu` for linear i: its tiles' codes and scales, and all activations
+// once per chunk
+static double batch_linear_cost(const wq_gemv_list* l, int i, int ncu, BatchShape s, int chunk) {
+  const GemvListDesc& g = l->descs[i];
+  const int G = (int)(g.g_dep & 0xffffu);
+  const double K = (double)G * 32.0;
+  const int trows = 16 * s.TW;
+  const double tiles = (double)((((int64_t)g.N + trows - 1) / trows + ncu - 1) / ncu);  // of one workgroup
+  const int panels = (G + batch_panel_groups(s.U, s.TW) - 1) / batch_panel_groups(s.U, s.TW);
+  return tiles * trows * K * (0.5 + 1.0 / 16.0) + batch_chunks((int)tiles, panels, chunk) * l->M * K * 2.0 + 4096.0;
+}
+
+// A SHORT list has too few linears for equal groups to be both many (so that few workgroups load a linear's
+// activations) and busy.  Its linears share the 8 XCDs instead, level by level: the linears of a dependency
+// level (level = 1 + the level of the producer) run side by side, each on a set of XCDs in proportion to what
+// it costs, every set at least one XCD; levels follow each other.  cost(i, workgroups of the group) as above.
+struct MaskPlan {
+  bool ok = false;
+  std::vector<uint8_t> mask;  // XCDs of linear i
+  double makespan = 0.0;
+};
+template <class Cost>
+static MaskPlan plan_xcd_masks(const wq_gemv_list* l, Cost cost) {
+  MaskPlan plan;
+  if (l->blocks % 8 != 0 || l->n > 64) return plan;
+  const int per_xcd = l->blocks / 8;
+  std::vector<int> level(l->n, 0);
+  int levels = 0;
+  for (int i = 0; i < l->n; ++i) {
+    const int dep = (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1;
+    level[i] = dep >= 0 ? level[dep] + 1 : 0;
+    levels = std::max(levels, level[i] + 1);
+  }
+  plan.mask.assign(l->n, 0);
+  for (int lv = 0; lv < levels; ++lv) {
+    std::vector<int> who;
+    for (int i = 0; i < l->n; ++i)
+      if (level[i] == lv) who.push_back(i);
+    if (who.size() > 8) return plan;  // a long list: equal groups
+    std::vector<int> k(who.size(), 1);
+    for (int left = 8 - (int)who.size(); left > 0; --left) {  // one more XCD to whoever takes longest
+      size_t worst = 0;
+      for (size_t a = 1; a < who.size(); ++a)
+        if (cost(who[a], per_xcd * k[a]) > cost(who[worst], per_xcd * k[worst])) worst = a;
+      ++k[worst];
+    }
+    double t = 0.0;
+    int next = 0;
+    for (size_t a = 0; a < who.size(); ++a) {
+      plan.mask[who[a]] = (uint8_t)(((1u << k[a]) - 1u) << next);
+      next += k[a];
+      t = std::max(t, cost(who[a], per_xcd * k[a]));
+    }
+    plan.makespan += t;
+  }
+  plan.ok = true;
+  return plan;
+}
+
 static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, BatchShape s, int chunk) {
   const int groups = 1 << gl, ncu = l->blocks >> gl;
   BatchGroupPlan plan;
@@ -1257,13 +1347,7 @@ static BatchGroupPlan batch_assign_groups(const wq_gemv_list* l, int gl, BatchSh
   std::vector<double> free_at(groups, 0.0), end(l->n, 0.0);
   for (int i = 0; i < l->n; ++i) {
     const GemvListDesc& g = l->descs[i];
-    const int G = (int)(g.g_dep & 0xffffu);
-    const double K = (double)G * 32.0;
-    const int trows = 16 * s.TW;
-    const double tiles = (double)((((int64_t)g.N + trows - 1) / trows + ncu - 1) / ncu);  // of one workgroup
-    const int panels = (G + batch_panel_groups(s.U, s.TW) - 1) / batch_panel_groups(s.U, s.TW);
-    // bytes through one workgroup: its tiles' codes and scales, and all activations once per chunk
-    const double dur = tiles * trows * K * (0.5 + 1.0 / 16.0) + batch_chunks((int)tiles, panels, chunk) * l->M * K * 2.0 + 4096.0;
+    const double dur = batch_linear_cost(l, i, ncu, s, chunk);
     const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
     const double ready = dep >= 0 ? end[dep] : 0.0;
     int best = 0;
@@ -1297,6 +1381,18 @@ static size_t rows_lds_bytes(int M, int nxb) {
 
 // as batch_assign_groups, with the duration of a linear from the passes a workgroup makes over its wave tiles
 // (every pass loads all activations; a pass of fewer than 8 wave tiles takes as long as a full one)
+// pass by pass: all activations, and the time of 8 wavefronts x TR row tiles however few rows the pass holds (a
+// wavefront unpacks and multiplies TR row tiles per pair either way; measured on the 32-layer Llama-2-7B stack,
+// M = 32: 16 groups, where the 4096-row linears make one pass of 32 rows per wavefront, 1.19 ms; 32 groups 0.945 ms)
+static double rows_linear_cost(const wq_gemv_list* l, int i, int ncu) {
+  const GemvListDesc& g = l->descs[i];
+  const double K = (double)(g.g_dep & 0xffffu) * 32.0;
+  const int64_t tiles = ((int64_t)g.N + 15) / 16;   // row tiles
+  const int64_t left = (tiles + ncu - 1) / ncu;      // of the workgroup with most
+  const double passes = (double)((left + kRW * kRowsTR - 1) / (kRW * kRowsTR));
+  return 4096.0 + passes * (kRW * kRowsTR * 16.0 * K * (0.5 + 1.0 / 16.0) + l->M * K * 2.0);
+}
+
 static BatchGroupPlan rows_assign_groups(const wq_gemv_list* l, int gl) {
   const int groups = 1 << gl, ncu = l->blocks >> gl;
   BatchGroupPlan plan;
@@ -1304,12 +1400,7 @@ static BatchGroupPlan rows_assign_groups(const wq_gemv_list* l, int gl) {
   std::vector<double> free_at(groups, 0.0), end(l->n, 0.0);
   for (int i = 0; i < l->n; ++i) {
     const GemvListDesc& g = l->descs[i];
-    const double K = (double)(g.g_dep & 0xffffu) * 32.0;
-    const int64_t tiles = ((int64_t)g.N + 15) / 16;   // row tiles
-    int64_t left = (tiles + ncu - 1) / ncu;             // of the workgroup with most
-    double dur = 4096.0;
-    const double passes = (double)((left + kRW * kRowsTR - 1) / (kRW * kRowsTR));
-    dur += passes * (kRW * kRowsTR * 16.0 * K * (0.5 + 1.0 / 16.0) + l->M * K * 2.0);
+    const double dur = rows_linear_cost(l, i, ncu);
     const int dep = (int)((g.g_dep >> 16) & 0x7fffu) - 1;
     const double ready = dep >= 0 ? end[dep] : 0.0;
     int best = 0;
@@ -1348,18 +1439,34 @@ static int rows_list_plan(wq_gemv_list* l) {
       best = std::move(p);
     }
   }
-  const int groups = 1 << best_gl, ncu = l->blocks >> best_gl;
-  std::vector<int64_t> off(groups, 0);
-  for (int i = 0; i < l->n; ++i) {
-    GemvListDesc& g = l->descs[i];
-    const int c = best.group[i];
-    const int64_t tiles = ((int64_t)g.N + 15) / 16;  // row tiles
-    g.q = (int32_t)(tiles / ncu);
-    g.rem = (uint16_t)(tiles % ncu);
-    g.off = (uint16_t)off[c];
-    off[c] = (off[c] + tiles) % ncu;
-    g.gmod_log2 = (uint8_t)best_gl;
-    g.gidx = (uint8_t)c;
+  int groups = 1 << best_gl;
+  const MaskPlan mp = plan_xcd_masks(l, [&](int i, int ncu) { return rows_linear_cost(l, i, ncu); });
+  if (mp.ok && mp.makespan < best.makespan * 0.98) {
+    for (int i = 0; i < l->n; ++i) {
+      GemvListDesc& g = l->descs[i];
+      const int ncu = (l->blocks / 8) * __builtin_popcount(mp.mask[i]);
+      const int64_t tiles = ((int64_t)g.N + 15) / 16;  // row tiles
+      g.q = (int32_t)(tiles / ncu);
+      g.rem = (uint16_t)(tiles % ncu);
+      g.off = 0;
+      g.gmod_log2 = 0x80;
+      g.gidx = mp.mask[i];
+    }
+    groups = 0;  // (sets of XCDs)
+  } else {
+    const int ncu = l->blocks >> best_gl;
+    std::vector<int64_t> off(groups, 0);
+    for (int i = 0; i < l->n; ++i) {
+      GemvListDesc& g = l->descs[i];
+      const int c = best.group[i];
+      const int64_t tiles = ((int64_t)g.N + 15) / 16;  // row tiles
+      g.q = (int32_t)(tiles / ncu);
+      g.rem = (uint16_t)(tiles % ncu);
+      g.off = (uint16_t)off[c];
+      off[c] = (off[c] + tiles) % ncu;
+      g.gmod_log2 = (uint8_t)best_gl;
+      g.gidx = (uint8_t)c;
+    }
   }
   l->batch_groups = groups;
   l->batch_nxb = nxb;
@@ -1415,18 +1522,41 @@ int batch_list_plan(wq_gemv_list* l) {
   }
   if (best_gl < 0)
     return fail(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: %d rows of activations do not fit the LDS", l->M);
-  const int groups = 1 << best_gl, ncu = l->blocks >> best_gl;
-  std::vector<int64_t> off(groups, 0);
-  for (int i = 0; i < l->n; ++i) {
-    GemvListDesc& g = l->descs[i];
-    const int c = best.group[i];
-    const int64_t tiles = ((int64_t)g.N + trows - 1) / trows;
-    g.q = (int32_t)(tiles / ncu);
-    g.rem = (uint16_t)(tiles % ncu);
-    g.off = (uint16_t)off[c];
-    off[c] = (off[c] + tiles) % ncu;
-    g.gmod_log2 = (uint8_t)best_gl;
-    g.gidx = (uint8_t)c;
+  int groups = 1 << best_gl;
+  // a short list: sets of XCDs in proportion to the linears' cost (plan_xcd_masks), if the estimate says so
+  const size_t mbase = batch_lds_bytes(s, l->M, 1, 2, 0);
+  const int mfit = (int)((budget - mbase) / (size_t)batch_kept_bytes(s.R, s.TW));
+  const MaskPlan mp = plan_xcd_masks(l, [&](int i, int ncu) { return batch_linear_cost(l, i, ncu, s, std::max(mfit, 1)); });
+  if (mp.ok && mp.makespan < best.makespan * 0.98) {
+    int acc_tiles = 0;
+    for (int i = 0; i < l->n; ++i) {
+      GemvListDesc& g = l->descs[i];
+      const int ncu = (l->blocks / 8) * __builtin_popcount(mp.mask[i]);
+      const int64_t tiles = ((int64_t)g.N + trows - 1) / trows;
+      if ((int)(g.g_dep & 0xffffu) > batch_panel_groups(s.U, s.TW)) acc_tiles = std::max<int>(acc_tiles, (int)((tiles + ncu - 1) / ncu));
+      g.q = (int32_t)(tiles / ncu);
+      g.rem = (uint16_t)(tiles % ncu);
+      g.off = 0;
+      g.gmod_log2 = 0x80;
+      g.gidx = mp.mask[i];
+    }
+    best_acc = std::min(acc_tiles, mfit);
+    best_chunked = best_acc < acc_tiles;
+    groups = 0;  // (sets of XCDs)
+  } else {
+    const int ncu = l->blocks >> best_gl;
+    std::vector<int64_t> off(groups, 0);
+    for (int i = 0; i < l->n; ++i) {
+      GemvListDesc& g = l->descs[i];
+      const int c = best.group[i];
+      const int64_t tiles = ((int64_t)g.N + trows - 1) / trows;
+      g.q = (int32_t)(tiles / ncu);
+      g.rem = (uint16_t)(tiles % ncu);
+      g.off = (uint16_t)off[c];
+      off[c] = (off[c] + tiles) % ncu;
+      g.gmod_log2 = (uint8_t)best_gl;
+      g.gidx = (uint8_t)c;
+    }
   }
   l->batch_groups = groups;
   l->batch_acc_tiles = best_acc;

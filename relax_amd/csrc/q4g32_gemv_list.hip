@@ -48,6 +48,7 @@
 #include <memory>
 #include <vector>
 
+#include "../../include/relax_amd_wq_testing.h"
 #include "gemv_list_common.h"
 #include "tuning.h"
 #include "wq_device.h"
@@ -730,6 +731,8 @@ extern "C" int wq_q4g32_gemv_list_info(const wq_gemv_list_t* l, int* dependencie
   if (adjacent) *adjacent = l->late;
   return WQ_OK;
 }
+
+extern "C" int wq_debug_gemv_list_groups(const wq_gemv_list_t* l) { return l && l->M > 1 ? l->batch_groups : -1; }
 
 extern "C" int wq_q4g32_gemv_list_set_spin_limit(wq_gemv_list_t* l, long long ticks) {
   using namespace wq;

@@ -152,6 +152,36 @@ def test_short_passes_of_the_row_owner_kernel(env, oracle, M, N, K):
                        f"batch list short passes {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M", [8, 16, 20])
+def test_a_short_list_shares_the_xcds_by_cost(env, oracle, M):
+    """Four linears of a decoder layer's proportions (rows 3 : 1 : 5.4 : 1 with a long K for the last), the last
+    one reading what the third wrote: up to 16 rows the planner gives every linear a SET of XCDs (reported as 0 equal
+    groups) instead of equal groups, two dependency levels; results against the oracle, twice."""
+    ops, u, torch = env
+    from relax_amd import _lib
+
+    shapes = [(1536, 1024), (512, 1024), (2816, 1024), (512, 2816)]
+    lins = [_linear(oracle, u, N, K, M, seed=300 + i) for i, (N, K) in enumerate(shapes)]
+    ys = [torch.zeros((M, N), dtype=torch.float16, device="cuda") for N, _ in shapes]
+    xs = [u.dev(l["x"]) for l in lins]
+    entries = [(l["dW"], l["dS"], x, y) for l, x, y in zip(lins, xs, ys)]
+    entries[3] = (lins[3]["dW"], lins[3]["dS"], ys[2], ys[3])  # the last linear reads what the third wrote
+    gl = ops.Q4G32GemvList(entries, M=M)
+    assert gl.info()[0] == 1
+    if M <= 16:  # (beyond, a pass costs the same however few rows it holds, and equal groups do as well)
+        assert _lib.lib().wq_debug_gemv_list_groups(gl._h) == 0, "expected sets of XCDs for a list of four linears"
+    print(f"batch list: short list, M = {M}", flush=True)
+    for _ in range(2):
+        for y in ys:
+            y.zero_()
+        gl.run()
+        gl.status()
+        for i in range(3):
+            u.assert_close(u.host(ys[i]), oracle.q4g32_linear(lins[i]["W"], lins[i]["S"], lins[i]["x"], nthreads=8), f"short list {i}")
+        # the consumer against the oracle on the producer's DEVICE output (its actual input)
+        u.assert_close(u.host(ys[3]), oracle.q4g32_linear(lins[3]["W"], lins[3]["S"], u.host(ys[2]), nthreads=8), "short list consumer")
+
+
 @pytest.mark.parametrize("M", [4, 12, 27])
 def test_dependent_chain_matches_oracle(env, oracle, M):
     """x of a linear is the y of an earlier one: directly in front, one apart, two consumers of one producer; a

@@ -143,8 +143,8 @@ def test_fused_group_order_keeps_dependences_and_separates_producers_from_consum
         l.wq_program_destroy(p)
 
 
-@pytest.mark.parametrize("M,n,fused", [(1, 2, 1), (4, 2, 1), (4, 1, 0), (8, 4, 0), (8, 8, 1), (16, 8, 0), (16, 16, 1),
-                                       (32, 4, 0), (32, 8, 1)])
+@pytest.mark.parametrize("M,n,fused", [(1, 2, 1), (4, 2, 1), (4, 1, 0), (8, 3, 0), (8, 4, 1), (16, 8, 0), (16, 16, 1),
+                                       (32, 8, 0), (32, 12, 1)])
 def test_short_runs_of_batched_linears_are_not_fused(M, n, fused):
     """Planning alone (no GPU): with several rows of x a run only becomes one launch of the list kernel from the
     length at which that launch is faster than the calls one by one."""
