@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void intb_dequant_kernel(const uint4_t* __rest
 }
 
 // ------------------------------------------------------------------------ GEMV
-constexpr int kIntbGemvThreads = 256;
+constexpr int kIntbGemvThreads = 512;  // at most: 4 .. 8 wavefronts per workgroup, chosen at launch
 
 __device__ __forceinline__ half_t intb_finish(float v, int m, int n, int N, const IntbEpilogue& ep) {
   if (ep.bias) v += (float)ep.bias[ep.bias_stride ? (int64_t)m * ep.bias_stride + n : n];
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ncs = K / (NBIT == 8 ? 16 : 32);
   const int pieces = (K / 64) * I * PPT;    // 16-byte pieces per column group
-  const int gset = (blockIdx.x * (kIntbGemvThreads / 64) + wave) * R;  // first group of this wave
+  const int gset = (blockIdx.x * ((int)blockDim.x >> 6) + wave) * R;  // first group of this wave
 
   // ---- stage x (natural order) and the per-piece offset constants ----
   {
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
     const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
     const int nchunks = K >> 3;
     for (int m = 0; m < MB; ++m)
-      for (int ci = tid; ci < nchunks; ci += kIntbGemvThreads) {
+      for (int ci = tid; ci < nchunks; ci += (int)blockDim.x) {
         uint4_t v = reinterpret_cast<const uint4_t*>(A + (int64_t)m * K)[ci];
         // chunk ci covers k = 8ci..8ci+7; (k % 16) >= 8 for odd ci
         const bool upper = ci & 1;
@@ -302,15 +302,32 @@ static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* 
                             hipStream_t stream) {
   constexpr int I = NBIT == 8 ? 2 : 4;
   const int ngroups = (int)(N / I);
-  const int waves = kIntbGemvThreads / 64;
-  const int64_t blocks = (ngroups + waves * R - 1) / (waves * R);
+  // Wavefronts per workgroup: every workgroup stages x for itself (the more wavefronts, the less of that), and all
+  // workgroups are resident at once, so the launch is as long as the CU with most of them: 4 .. 8 wavefronts,
+  // whichever leaves the fullest last round (K = 8192, N = 28672, int4, two groups per wavefront: 3584 wavefronts
+  // are 896 workgroups of 4, i.e. 3.5 per CU, or 512 of 7, i.e. 2 per CU).
+  const int64_t total_waves = (ngroups + R - 1) / R;
+  // (measured at M = 1: int4 per-channel 22.7 us with 4, 21.6 with 7; int8 group-64 46.0 with 4, 40.9 with 7, 48.8 with 8;
+  // int8 per-channel, 7168 wavefronts: 37.9 .. 38.3 us with any of them)
+  int waves = 4;
+  double best = -1.0;
+  for (int w = 4; w <= 8; ++w) {
+    const int64_t b = (total_waves + w - 1) / w;
+    const int64_t rounds = (b + cu_count() - 1) / cu_count();
+    const double fill = (double)b / (double)(rounds * cu_count());  // 1: every CU has the same number
+    if (fill > best - 1e-9) {  // the fullest last round; among equals the most wavefronts
+      best = std::max(best, fill);
+      waves = w;
+    }
+  }
+  const int64_t blocks = (total_waves + waves - 1) / waves;
   const size_t lds = (size_t)MB * K * 2 + (size_t)MB * (K / (NBIT == 8 ? 16 : 32)) * 4;
   auto kern = intb_gemv_kernel<NBIT, R, MB, U>;
   if (lds > 60 * 1024) {
     static DynamicLdsLimit limit;  // per instantiation
     WQ_HIP(limit.ensure(reinterpret_cast<const void*>(kern), (int)lds));
   }
-  WQ_LAUNCH("wq_fpA_intB_gemm(gemv)", kern, dim3((unsigned)blocks), dim3(kIntbGemvThreads), lds,
+  WQ_LAUNCH("wq_fpA_intB_gemm(gemv)", kern, dim3((unsigned)blocks), dim3((unsigned)(64 * waves)), lds,
             stream, (const uint4_t*)B, (const half_t*)scales, (const half_t*)A, (half_t*)C, (int)N,
             (int)K, (int)group, ngroups, ep);
   return WQ_OK;
