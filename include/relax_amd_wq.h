@@ -154,8 +154,10 @@ wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* descs, int n
 /* The same for M rows of activations per linear, 1 <= M <= WQ_GEMV_LIST_MAX_M (a small decode batch): x is
  * fp16 [M, K], y and residual fp16 [M, N], all contiguous; one launch runs the list on the matrix cores, one pass
  * over the weights for every M (more than 16 rows: each unpacked weight feeds two matrix-core tiles of 16
- * rows).  M > 1 needs K % 256 == 0 and S 16-byte aligned (WQ_EUNSUPPORTED otherwise: run such a list linear by
- * linear with wq_q4g32_linear). */
+ * rows, in a kernel whose wavefronts own rows of W and keep their sums in registers over all of K).  M > 1 needs
+ * K % 256 == 0 and S 16-byte aligned, M > 16 also N * K < 2^35 per linear (WQ_EUNSUPPORTED otherwise: run such a
+ * list linear by linear with wq_q4g32_linear).  A short list (at most 8 independent linears at a time) gives
+ * every linear a set of the 8 XCDs sized by its cost; a long one runs on equal groups of workgroups. */
 #define WQ_GEMV_LIST_MAX_M 32
 wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv_desc* descs, int n, int M, void* workspace,
                                                   size_t workspace_bytes, wq_stream_t stream);
