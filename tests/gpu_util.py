@@ -58,10 +58,11 @@ def assert_close(got: np.ndarray, ref: np.ndarray, what: str = ""):
     assert not bad.any(), f"{what}: {bad.sum()} elements outside rtol={RTOL} atol={ATOL}; max err {err.max()}"
     # An output is rounded to fp16 once, or twice where a residual is added to the rounded
     # y + bias: two results of the same arithmetic in another summation order can then lie
-    # two fp16 steps apart, which near the largest output is 1.0e-3..1.9e-3 of it.  Such an
-    # element passes; anything further off must meet the normalised bound.
+    # two fp16 steps apart, three where the residual takes the sum down one binade (a step of
+    # the binade above and one of its own), which near the largest output is 1.0e-3..1.5e-3
+    # of it.  Such an element passes; anything further off must meet the normalised bound.
     scale = max(np.abs(r).max(), 1e-6)
     ulp = np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64)
-    far = err > 2.0 * ulp
+    far = err > 3.0 * ulp
     worst = float((err * far).max()) if far.any() else 0.0
     assert worst / scale <= NORM_TOL, f"{what}: normalised max error {worst / scale:.3e} > {NORM_TOL}"
