@@ -30,7 +30,9 @@ extern "C" {
 void wq_debug_set_gemm_config(int cfg);
 /* Split the tiles of the last, partly filled round into row slices (default 1). */
 void wq_debug_set_gemm_tail_split(int on);
-/* Decode GEMV: rows per wavefront (1, 2, 4) and scale groups per lane; 0 = from the shape. */
+/* Decode GEMV: rows per wavefront (1, 2, 4) and scale groups per lane; 0 = from the shape.  Format B: column
+ * groups per wavefront (1, 2) at one row; a value other than 0 also keeps one or two rows of a narrow matrix
+ * on the streaming kernel, which the dispatch otherwise hands to the small-batch kernel. */
 void wq_debug_set_gemv_config(int rows, int gpl);
 /* Decode GEMV: persistent workgroups per CU; 0 = from the shape. */
 void wq_debug_set_gemv_blocks_per_cu(int n);

@@ -556,7 +556,9 @@ static int wq::gptq_linear_impl(const uint32_t* W_nk, const uint16_t* SZ, const 
   const int ratio = (int)(gs / 32);
   const uint32_t inv32 = ratio > 1 ? (uint32_t)(((1ull << 32) + ratio - 1) / ratio) : 0u;
   const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
-  if (M <= 2) return gemv_dispatch<true>("wq_gptq_linear", W_nk, SZ, GemvZp{ratio, (int)G}, x, bias, residual, y, M, N, K, stream);
+  // (two rows of more than 8192 columns go to the small-batch kernel, as in wq_q4g32_linear)
+  if (M <= 2 && !(M == 2 && K > 8192 && K % 64 == 0))
+    return gemv_dispatch<true>("wq_gptq_linear", W_nk, SZ, GemvZp{ratio, (int)G}, x, bias, residual, y, M, N, K, stream);
   if (M <= WQ_SMALL_BATCH_MAX_M && K % 64 == 0) {
     const GptqSkinnyPolicy::Args pargs{W_nk, (const half2_t*)SZ, (int)G, ratio, inv32};
     return launch_skinny_auto<GptqSkinnyPolicy, Q4G32Epilogue>("wq_gptq_linear", pargs, x, y, ep, M, N, K, stream);

@@ -22,7 +22,11 @@ int intb_gemv_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scale
                        int64_t m, int64_t n, int64_t k, int64_t group, int nbit,
                        const IntbEpilogue& ep, hipStream_t stream);
 
-// Matrix-core streaming kernel for 2 <= m <= 64 (intb_skinny.hip).
+// Wavefronts that kernel's launch for one or two rows would have: it gives a wavefront whole columns, so a
+// narrow matrix leaves the machine short of them.
+int64_t intb_gemv_wavefronts(int64_t m, int64_t n, int64_t group, int nbit);
+
+// Matrix-core streaming kernel for 1 <= m <= 64 (intb_skinny.hip).
 int intb_small_batch_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scales, uint16_t* C,
                               int64_t m, int64_t n, int64_t k, int64_t group, int nbit,
                               const IntbEpilogue& ep, hipStream_t stream);

@@ -187,11 +187,18 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
   const IntbEpilogue ep{(const half_t*)bias, binary_op ? (const half_t*)residual : nullptr,
                         bias_stride, activation, binary_op, unary_op};
   if (wq_gemm_cfg_override() == 0) {
-    // one or two rows: the VALU streaming kernel; up to 64 rows: still one pass over the
-    // weights, products on the matrix cores; beyond that the tiled GEMM
-    if (m <= 2) return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
+    // one or two rows of a wide matrix: the VALU streaming kernel; up to 64 rows: still one pass over
+    // the weights, products on the matrix cores; beyond that the tiled GEMM
     // fine-grained scales whose pairs are not 4-byte aligned go to the register-staged GEMM below
-    if (m <= WQ_SMALL_BATCH_MAX_M && (!group || (reinterpret_cast<uintptr_t>(scales) & 3u) == 0))
+    const bool small_ok = !group || (reinterpret_cast<uintptr_t>(scales) & 3u) == 0;
+    // The streaming kernel gives a wavefront whole columns: with fewer than 8 wavefronts per CU (int4: N < 16384,
+    // int8 with group scales or two rows: N < 8192) the small-batch kernel, which also splits K, is the faster one
+    // (M = 1, int4: K = 4096, N = 4096: 8.9 -> 5.3 us; K = 11008, N = 4096: 20.2 -> 10.5 us; K = 28672, N = 8192:
+    // 48.9 -> 36 us; at N = 28672 the streaming kernel wins, 22.9 against 32.8 us).
+    // (rows per wavefront forced by a test: the streaming kernel is what is asked for)
+    const bool narrow = intb_gemv_wavefronts(m, n, group, nbit) < 8 * (int64_t)cu_count() && small_ok && !tuning().gemv_rows;
+    if (m <= 2 && !narrow) return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
+    if (m <= WQ_SMALL_BATCH_MAX_M && small_ok)
       return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
   }
   const IntbGemmEpilogue gep{ep, (int)n};

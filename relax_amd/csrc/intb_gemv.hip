@@ -333,6 +333,17 @@ static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* 
   return WQ_OK;
 }
 
+// column groups per wavefront at one row (two rows: always 2)
+static int intb_gemv_groups_per_wave(int64_t group, int nbit) {
+  return tuning().gemv_rows ? tuning().gemv_rows : (group > 0 || nbit == 4 ? 2 : 1);
+}
+
+int64_t intb_gemv_wavefronts(int64_t m, int64_t n, int64_t group, int nbit) {
+  const int I = nbit == 8 ? 2 : 4;
+  const int R = m >= 2 ? 2 : intb_gemv_groups_per_wave(group, nbit);
+  return (n / I + R - 1) / R;
+}
+
 // Called by the dispatcher in intb_gemm.hip for m <= 4.
 int intb_gemv_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scales, uint16_t* C,
                        int64_t m, int64_t n, int64_t k, int64_t group, int nbit,
@@ -355,7 +366,7 @@ int intb_gemv_dispatch(const uint16_t* A, const int8_t* B, const uint16_t* scale
       // then serve both (45.4 against 48.1 us), four pieces (66 registers).  int4: two groups, ONE piece: with four
       // pieces the compiler keeps 16 LDS operands per piece in registers (154: three wavefronts per SIMD); one piece
       // needs 68 (seven per SIMD): per-channel 27.2 -> 22.2 us, group-64 27.1 -> 23.2 us.
-      const int R = tuning().gemv_rows ? tuning().gemv_rows : (group > 0 || nbit == 4 ? 2 : 1);
+      const int R = intb_gemv_groups_per_wave(group, nbit);
       if (R == 1)
         rc = nbit == 8 ? launch_intb_gemv<8, 1, 1>(a, B, scales, c, n, k, group, ep, stream)
                        : launch_intb_gemv<4, 1, 1>(a, B, scales, c, n, k, group, ep, stream);

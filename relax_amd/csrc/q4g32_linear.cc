@@ -12,7 +12,10 @@ extern "C" int wq_q4g32_linear(const uint32_t* W, const uint16_t* S, const uint1
   // for the next one that serves the call.
   const bool gemv_ok = K <= 32768;
   const bool small_ok = K % 64 == 0 && (reinterpret_cast<uintptr_t>(S) & 3u) == 0;
-  if (M <= 2 && gemv_ok) return wq_q4g32_gemv(W, S, x, bias, residual, y, M, N, K, stream);
+  // (two rows of more than 8192 columns: the streaming kernel's two-row form is the slower one there; N = 4096,
+  // K = 11008: 15.5 against 10.9 us, N = 8192, K = 28672: 56 against 37 us)
+  const bool two_long_rows = M == 2 && K > 8192 && small_ok;
+  if (M <= 2 && gemv_ok && !two_long_rows) return wq_q4g32_gemv(W, S, x, bias, residual, y, M, N, K, stream);
   if (M <= WQ_SMALL_BATCH_MAX_M && small_ok)
     return wq_q4g32_small_batch(W, S, x, bias, residual, y, M, N, K, stream);
   // up to 128 rows of a small matrix: the tiled GEMM would have too few tiles for 256

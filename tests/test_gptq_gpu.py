@@ -101,6 +101,8 @@ LINEAR_CASES = [  # (M, N, K, group size, act_order)
     (1, 12288, 4096, 128, True),
     (1, 4096, 11008, 128, True),
     (2, 4096, 4096, 64, True),
+    (2, 520, 11008, 128, True),    # two long rows: the small-batch kernel
+    (2, 72, 8224, 32, False),      # two long rows, K not a multiple of 64: the streaming kernel
     (3, 520, 1024, 32, True),
     (4, 1000, 2048, 1024, False),
     (5, 264, 4096, 4096, True),    # one group

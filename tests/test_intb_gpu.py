@@ -144,6 +144,25 @@ def test_small_batch_work_splits(ops, u, oracle, nbit, group_size, nw, stages, w
         _lib.lib().wq_debug_set_skinny_config(0, 0, 0)
 
 
+@pytest.mark.parametrize("rows", [0, 1, 2])
+@pytest.mark.parametrize("nbit", [8, 4])
+@pytest.mark.parametrize("group_size", [-1, 64])
+def test_one_and_two_rows_on_either_kernel(ops, u, oracle, nbit, group_size, rows):
+    """M <= 2: the automatic choice (the streaming kernel for wide matrices, the small-batch kernel for narrow
+    ones, where whole columns per wavefront leave the machine short of wavefronts) and the streaming kernel asked
+    for by the test hook, with one and two column groups per wavefront."""
+    from relax_amd import _lib
+
+    _lib.lib().wq_debug_set_gemv_config(rows, 0)
+    try:
+        for M, N, K in [(1, 64, 64), (2, 64, 128), (1, 320, 448), (2, 320, 4096), (1, 4096, 1024), (2, 4096, 1024),
+                        (1, 16384, 256), (2, 16384, 256), (1, 1024, 11008)]:
+            print(f"intb rows={rows} nbit={nbit} g={group_size} M={M} N={N} K={K}", flush=True)
+            _run(ops, u, oracle, M, N, K, nbit, seed=M + N + rows, group_size=group_size, bias="row")
+    finally:
+        _lib.lib().wq_debug_set_gemv_config(0, 0)
+
+
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 17, 18])
 @pytest.mark.parametrize("nbit", [8, 4])
 def test_gemm_tile_configurations(ops, u, oracle, nbit, cfg):

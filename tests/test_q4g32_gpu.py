@@ -61,7 +61,7 @@ GEMV_SHAPES = [  # (M, N, K)
     (1, 22016, 4096),   # fused gate/up
     (1, 4096, 11008),   # down
     (1, 1, 32), (1, 7, 64), (1, 1001, 2080), (1, 8, 32768),
-    (2, 515, 4096), (3, 64, 256), (4, 4096, 4096), (5, 130, 11008), (8, 4096, 4096),
+    (2, 515, 4096), (2, 300, 11008), (3, 64, 256), (4, 4096, 4096), (5, 130, 11008), (8, 4096, 4096),
 ]
 
 
@@ -202,7 +202,7 @@ def test_small_batch_vs_oracle(ops, u, oracle, nw, waves, stages, M, N, K):
     u.assert_close(got, ref, f"small batch nw{nw} waves{waves} {M}x{N}x{K}")
 
 
-@pytest.mark.parametrize("M", [1, 4, 5, 8])
+@pytest.mark.parametrize("M", [1, 2, 4, 5, 8])
 def test_low_batch_fixture_shape(ops, u, oracle, M):
     """The shape of the reference's low-batch fixture (tests/python/dlight/test_gpu_low_batch_gemv.py:29-34:
     N = 4096, K = 28672, a dynamic batch) at full size: the automatic dispatch and every kernel that serves it."""
