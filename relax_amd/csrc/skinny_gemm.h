@@ -500,9 +500,26 @@ static int launch_skinny_auto(const char* who, const typename Policy::Args& parg
   // workgroup, each wavefront the whole K), which halves the re-reads of x again, as long as
   // most CUs still get a workgroup (int8, K = 8192, N = 28672, M = 64: 80 -> 62 us)
   if (M > 16 && N / 128 >= (cu_count() * 5) / 8) nw = 8;
+  // ... corrected for how the workgroups fill the machine.  A workgroup of nw wavefronts takes nw column tiles
+  // and stages the activations once, which costs about as much as one tile (two from 33 rows on): the launch
+  // lasts about (rounds of the CUs) x (nw + that).  Fewer wavefronts side by side where that is shorter
+  // (N = 8192 with 4: 128 workgroups on 256 CUs; K = 28672, M = 32: 102 -> 62 us), two instead of one where
+  // one leaves a second, partly filled round (N = 5120, K = 13824, M = 32: 43 -> 31 us; N = 6144, K = 4096,
+  // M = 64: 22 -> 14 us).  Up to 8 rows the choice above stands (measured either way).
+  if (M > 8 && !t.nw) {
+    const int64_t tiles = (N + 15) / 16, cus = cu_count();
+    const double cx = M > 32 ? 2.0 : 1.0;
+    auto cost = [&](int w) { return (double)((tiles + w * cus - 1) / (w * cus)) * (w + cx); };
+    while (nw > 1 && cost(nw / 2) < cost(nw) - 1e-9) nw /= 2;
+    if (nw == 1 && cost(2) < cost(1) - 1e-9) nw = 2;
+  }
   if (t.nw) nw = t.nw;
   if (M <= 8 && nw >= 4) nw = 2;  // 8 rows are two slab loads: at most two wavefronts share them
-  const int stages = t.stages ? t.stages : (nw >= 4 ? 3 : 2);
+  // three ring slots for four or more wavefronts side by side, and for two when every workgroup has a CU of
+  // its own anyway (N = 8192, K = 28672, M = 16: 67 -> 46 us; with more workgroups than CUs the third slot
+  // costs a resident workgroup: N = 10240, K = 8192, M = 16: 20.9 -> 27.4 us)
+  const int64_t wgs = ((N + 15) / 16 + nw - 1) / nw;
+  const int stages = t.stages ? t.stages : (nw >= 4 || (nw == 2 && M > 8 && wgs <= cu_count()) ? 3 : 2);
   // eight wavefronts where two ring slots of that arrangement fit LDS, else four
 #define WQ_SK_GO(TH, NW, WAVES)                                                                        \
   do {                                                                                                 \
