@@ -339,8 +339,9 @@ inline int lds_tail_split(int rest, int slots, int cus, int TM, int a_loads, boo
 // tiles), 17 (128 x 128, two workgroups per CU) or 18 (256 x 128): rounds of the machine times tile
 // area over the rate one CU sustains on such tiles.  The rates are tile areas per microsecond measured
 // at K = 8192, N = 28672 with int8 weights (128 x 128 alone on its CU 193, two per CU 243 together;
-// 256 x 128: 254; 256 x 256: 294); row slices of a cut tile run at 0.85 (halves) and 0.75 (quarters) of
-// them.  The model reproduces the measured times at M = 65 .. 2048 within 6 %.
+// 256 x 128: 254; 256 x 256: 294); row slices of a cut tile run at 0.74 (halves) and 0.56 (quarters) of
+// them (a slice unpacks all columns of its tile whatever its height; fitted to launches that are one cut round:
+// N = 4096 .. 12288, M = 192 .. 1024, where 0.85 / 0.75 chose 256 x 256 tiles 10 .. 15 % too slow).  The model reproduces the measured times at M = 65 .. 2048 within 6 %.
 inline double lds_cfg_cost(int cfg, int64_t M, int64_t N, int cus) {
   const int BM = cfg == 17 ? 128 : 256, BN = cfg == 11 ? 256 : 128, per_cu = cfg == 17 ? 2 : 1;
   const double rate_alone = cfg == 17 ? 193.0 : cfg == 18 ? 254.0 : 294.0;
@@ -353,7 +354,7 @@ inline double lds_cfg_cost(int cfg, int64_t M, int64_t N, int cus) {
   if (rest) {
     const int split = lds_tail_split(rest, slots, cus, BM / 32, BM / 32);
     const bool alone = rest * split <= cus;
-    const double slice = split == 4 ? 0.75 : split == 2 ? 0.85 : 1.0;
+    const double slice = split == 4 ? 0.56 : split == 2 ? 0.74 : 1.0;
     t += area / split * (alone ? 1 : per_cu) / ((alone ? rate_alone : rate_full) * slice);
   }
   return t;
