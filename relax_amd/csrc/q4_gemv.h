@@ -358,8 +358,8 @@ static int launch_gemv(const char* who, const uint32_t* W, const uint16_t* S, co
 // rows == 0 chooses the rows per wavefront from the shape (timings of the Llama-7B layers):
 // what costs most at these kernel lengths (4 .. 12 us) is a second, partly filled round of
 // workgroups, so take the most rows per wavefront (4, 2, 1) for which all workgroups are
-// resident at once and every CU still has at least two; if nothing fits (tall matrices), one
-// row per wavefront and four persistent workgroups per CU, each taking several turns.
+// resident at once and every CU still has at least two; if nothing fits (tall matrices, long rows),
+// persistent workgroups that take several turns each.
 template <int MB, int GPL, bool ZP>
 static int launch_gemv_rows(const char* who, int rows, const uint32_t* W, const uint16_t* S, const GemvZp& zp, const uint16_t* x,
                             const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t N,
@@ -376,8 +376,14 @@ static int launch_gemv_rows(const char* who, int rows, const uint32_t* W, const 
     } else if (gemv_geometry<1, MB, GPL, ZP>(N, K, &nb, &per_cu) && nb <= (int64_t)cus * per_cu) {
       rows = 1;
     } else {
-      rows = 1;
-      bpc = 4;
+      // tall or long: persistent workgroups, as many per CU as are resident at once and at most four (rows of
+      // more than 8192 columns need workgroups of 7 .. 16 wavefronts and up to 60 KB of LDS, of which two or three
+      // fit: N = 8192, K = 28672 with four per CU 31.0 us, with two, two rows per wavefront, 25.0 us; N = 4096,
+      // K = 14336: 10.1 -> 8.8 us)
+      rows = K > 8192 ? 2 : 1;
+      const bool fits = rows == 2 ? gemv_geometry<2, MB, GPL, ZP>(N, K, &nb, &per_cu)
+                                  : gemv_geometry<1, MB, GPL, ZP>(N, K, &nb, &per_cu);
+      bpc = fits && per_cu >= 1 ? std::min(4, per_cu) : 4;
     }
   }
   switch (rows) {
