@@ -34,6 +34,9 @@ void wq_debug_set_gemm_tail_split(int on);
  * groups per wavefront (1, 2) at one row; a value other than 0 also keeps one or two rows of a narrow matrix
  * on the streaming kernel, which the dispatch otherwise hands to the small-batch kernel. */
 void wq_debug_set_gemv_config(int rows, int gpl);
+/* Format B decode GEMV: wavefronts that share a column group and split K between them (1, 2, 4, 8); 0 = from
+ * the shape (int4 at one row of a narrow matrix; otherwise 1). */
+void wq_debug_set_intb_gemv_k_split(int ways);
 /* Decode GEMV: persistent workgroups per CU; 0 = from the shape. */
 void wq_debug_set_gemv_blocks_per_cu(int n);
 /* Small-batch kernel: wavefronts side by side (1, 2, 4, 8), ring slots, and which kernel

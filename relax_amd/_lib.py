@@ -88,6 +88,7 @@ TESTING_SIGNATURES = {
     "wq_debug_set_gemv_config": [_int, _int],
     "wq_debug_set_gemv_blocks_per_cu": [_int],
     "wq_debug_set_skinny_config": [_int, _int, _int],
+    "wq_debug_set_intb_gemv_k_split": [_int],
     "wq_debug_gemv_list_groups": [_vp],
 }
 # ... and the calibration kernels of librelax_amd_wq_calibrate.so

@@ -191,12 +191,13 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
     // the weights, products on the matrix cores; beyond that the tiled GEMM
     // fine-grained scales whose pairs are not 4-byte aligned go to the register-staged GEMM below
     const bool small_ok = !group || (reinterpret_cast<uintptr_t>(scales) & 3u) == 0;
-    // The streaming kernel gives a wavefront whole columns: with fewer than 8 wavefronts per CU (int4: N < 16384,
-    // int8 with group scales or two rows: N < 8192) the small-batch kernel, which also splits K, is the faster one
-    // (M = 1, int4: K = 4096, N = 4096: 8.9 -> 5.3 us; K = 11008, N = 4096: 20.2 -> 10.5 us; K = 28672, N = 8192:
-    // 48.9 -> 36 us; at N = 28672 the streaming kernel wins, 22.9 against 32.8 us).
+    // The streaming kernel gives a wavefront whole columns: with fewer than 8 wavefronts per CU (int8 with group
+    // scales, or two rows: N < 8192; two rows of int4: N < 16384) the small-batch kernel, which also splits K, is
+    // the faster one (int8 group-64, M = 1, K = 4096, N = 4096: 6.7 -> 5.7 us; int4, M = 2, K = 28672, N = 8192:
+    // 56 -> 32 us).  One row of int4 stays: there the streaming kernel splits K itself (intb_gemv.hip).
     // (rows per wavefront forced by a test: the streaming kernel is what is asked for)
-    const bool narrow = intb_gemv_wavefronts(m, n, group, nbit) < 8 * (int64_t)cu_count() && small_ok && !tuning().gemv_rows;
+    const bool narrow = intb_gemv_wavefronts(m, n, group, nbit) < 8 * (int64_t)cu_count() && small_ok &&
+                        !tuning().gemv_rows && !(nbit == 4 && m == 1);
     if (m <= 2 && !narrow) return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
     if (m <= WQ_SMALL_BATCH_MAX_M && small_ok)
       return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);

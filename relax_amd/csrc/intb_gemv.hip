@@ -91,7 +91,7 @@ __device__ __forceinline__ half_t intb_finish(float v, int m, int n, int N, cons
 template <int NBIT, int R, int MB, int U>
 __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
     const uint4_t* __restrict__ B, const half_t* __restrict__ scales, const half_t* __restrict__ A,
-    half_t* __restrict__ C, int N, int K, int group, int ngroups, IntbEpilogue ep) {
+    half_t* __restrict__ C, int N, int K, int group, int ngroups, int ks_log2, IntbEpilogue ep) {
   constexpr int I = NBIT == 8 ? 2 : 4;      // interleaved columns per group
   constexpr int PPT = NBIT == 8 ? 4 : 2;    // pieces per column per tile
   constexpr int XQ = NBIT == 8 ? 2 : 4;     // 16-byte chunks of x per piece
@@ -103,7 +103,12 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ncs = K / (NBIT == 8 ? 16 : 32);
   const int pieces = (K / 64) * I * PPT;    // 16-byte pieces per column group
-  const int gset = (blockIdx.x * ((int)blockDim.x >> 6) + wave) * R;  // first group of this wave
+  // 2^ks_log2 neighbouring wavefronts of a workgroup share the groups of one and split K (a narrow
+  // matrix has too few column groups to give every SIMD its wavefronts otherwise)
+  const int gwave = blockIdx.x * ((int)blockDim.x >> 6) + wave;
+  const int kpart = gwave & ((1 << ks_log2) - 1);
+  const int gset = (gwave >> ks_log2) * R;  // first group of this wave
+  float* red = cs + MB * ncs;               // [wavefronts][R][I][MB] partial sums of the K parts
 
   // ---- stage x (natural order) and the per-piece offset constants ----
   {
@@ -134,7 +139,7 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
       }
   }
   __syncthreads();
-  if (gset >= ngroups) return;
+  if (gset >= ngroups && ks_log2 == 0) return;  // (with a split of K every wavefront goes on to the barrier below)
 
   // lane geometry: piece index p = lane + 64*it; column and k-position follow from p % 8
   const int col_in_group = (lane & 7) / PPT;
@@ -152,7 +157,12 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
   // R and N / I of 16: the load stays inside the row); needs 16-byte aligned scales
   constexpr bool kVecFits = R * I * 2 == 8 || R * I * 2 == 16;
   const bool vec_scales = kVecFits && group > 0 && (reinterpret_cast<uintptr_t>(scales) & 15u) == 0;
-  for (int p0 = 0; p0 < pieces; p0 += 64 * U) {
+  // this wavefront's part of K: whole rounds of 64 U pieces
+  const int rounds = (pieces + 64 * U - 1) / (64 * U);
+  const int rounds_part = (rounds + (1 << ks_log2) - 1) >> ks_log2;
+  const int p_begin = gset < ngroups ? min(kpart * rounds_part * 64 * U, pieces) : 0;
+  const int p_end = gset < ngroups ? min(p_begin + rounds_part * 64 * U, pieces) : 0;
+  for (int p0 = p_begin; p0 < p_end; p0 += 64 * U) {
     uint4_t wv[R][U];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -280,7 +290,26 @@ __global__ __launch_bounds__(kIntbGemvThreads) void intb_gemv_kernel(
       v += __shfl_xor(v, 32, 64);
       acc[r][m] = v;
     }
-  if (lane < 8 && (lane & (PPT - 1)) == 0) {
+  const bool holder = lane < 8 && (lane & (PPT - 1)) == 0;  // one lane per column of a group
+  if (ks_log2) {
+    // the parts of K meet in LDS; the wavefront of part 0 adds them in order of K
+    if (holder) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) red[((wave * R + r) * I + col_in_group) * MB + m] = acc[r][m];
+    }
+    __syncthreads();
+    if (kpart != 0 || gset >= ngroups) return;
+    if (holder) {
+      for (int k = 1; k < (1 << ks_log2); ++k)
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int m = 0; m < MB; ++m) acc[r][m] += red[(((wave + k) * R + r) * I + col_in_group) * MB + m];
+    }
+  }
+  if (holder) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int g = gset + r;
@@ -306,12 +335,34 @@ static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* 
   // workgroups are resident at once, so the launch is as long as the CU with most of them: 4 .. 8 wavefronts,
   // whichever leaves the fullest last round (K = 8192, N = 28672, int4, two groups per wavefront: 3584 wavefronts
   // are 896 workgroups of 4, i.e. 3.5 per CU, or 512 of 7, i.e. 2 per CU).
-  const int64_t total_waves = (ngroups + R - 1) / R;
+  // A narrow matrix has too few column groups for that.  int4 at one row (one piece per lane in flight, the most
+  // arithmetic per byte) then lets 2, 4 or 8 neighbouring wavefronts share a group and split K, whichever brings
+  // the launch closest to 18 wavefronts per CU (K = 28672, N = 8192: 47 us unsplit, 37 us through the small-batch
+  // kernel, 22.5 us split 4 ways; K = 13824, N = 5120: 17.4 -> 10.4 us split 8 ways; N = 22016: 2 ways, N = 28672:
+  // none).  int8 keeps whole columns: its wavefronts have four pieces per lane in flight, and a split measured
+  // 5 .. 10 % slower on most shapes.
+  const int64_t group_waves = (ngroups + R - 1) / R;
+  constexpr int PPT = NBIT == 8 ? 4 : 2;
+  const int64_t k_rounds = ((K / 64) * I * PPT + 64 * U - 1) / (64 * U);
+  int ks_log2 = 0;
+  if (tuning().intb_k_split) {
+    while ((1 << ks_log2) < tuning().intb_k_split && ks_log2 < 3) ++ks_log2;
+  } else if (NBIT == 4 && MB == 1) {
+    const double want = 18.0 * cu_count();
+    double best_d = -1.0;
+    for (int s = 0; s <= 3 && (k_rounds >> s) >= 1; ++s) {
+      const double ratio = (double)(group_waves << s) / want;
+      const double d = ratio > 1.0 ? ratio : 1.0 / ratio;  // distance on a logarithmic scale
+      if (best_d < 0.0 || d < best_d) best_d = d, ks_log2 = s;
+    }
+  }
+  const int64_t total_waves = group_waves << ks_log2;
   // (measured at M = 1: int4 per-channel 22.7 us with 4, 21.6 with 7; int8 group-64 46.0 with 4, 40.9 with 7, 48.8 with 8;
   // int8 per-channel, 7168 wavefronts: 37.9 .. 38.3 us with any of them)
   int waves = 4;
   double best = -1.0;
   for (int w = 4; w <= 8; ++w) {
+    if (w & ((1 << ks_log2) - 1)) continue;  // the wavefronts of a group sit in one workgroup
     const int64_t b = (total_waves + w - 1) / w;
     const int64_t rounds = (b + cu_count() - 1) / cu_count();
     const double fill = (double)b / (double)(rounds * cu_count());  // 1: every CU has the same number
@@ -321,7 +372,8 @@ static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* 
     }
   }
   const int64_t blocks = (total_waves + waves - 1) / waves;
-  const size_t lds = (size_t)MB * K * 2 + (size_t)MB * (K / (NBIT == 8 ? 16 : 32)) * 4;
+  const size_t lds = (size_t)MB * K * 2 + (size_t)MB * (K / (NBIT == 8 ? 16 : 32)) * 4 +
+                     (ks_log2 ? (size_t)waves * R * I * MB * 4 : 0);
   auto kern = intb_gemv_kernel<NBIT, R, MB, U>;
   if (lds > 60 * 1024) {
     static DynamicLdsLimit limit;  // per instantiation
@@ -329,7 +381,7 @@ static int launch_intb_gemv(const uint16_t* A, const int8_t* B, const uint16_t* 
   }
   WQ_LAUNCH("wq_fpA_intB_gemm(gemv)", kern, dim3((unsigned)blocks), dim3((unsigned)(64 * waves)), lds,
             stream, (const uint4_t*)B, (const half_t*)scales, (const half_t*)A, (half_t*)C, (int)N,
-            (int)K, (int)group, ngroups, ep);
+            (int)K, (int)group, ngroups, ks_log2, ep);
   return WQ_OK;
 }
 

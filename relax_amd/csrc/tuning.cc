@@ -24,3 +24,4 @@ extern "C" void wq_debug_set_skinny_config(int nw, int stages, int waves) {
   wq::tuning().skinny_stages = stages;
   wq::tuning().skinny_waves = waves;
 }
+extern "C" void wq_debug_set_intb_gemv_k_split(int ways) { wq::tuning().intb_k_split = ways; }

@@ -16,6 +16,7 @@ struct Tuning {
   int gemm_tail_split = 1;   // split the tiles of the last, partial round (on by default)
   int gemv_rows = 0, gemv_gpl = 0, gemv_blocks_per_cu = 0;
   int skinny_nw = 0, skinny_stages = 0, skinny_waves = 0;
+  int intb_k_split = 0;      // Format B decode GEMV: wavefronts that share a column group and split K (1, 2, 4, 8)
 };
 Tuning& tuning();
 

@@ -163,6 +163,39 @@ def test_one_and_two_rows_on_either_kernel(ops, u, oracle, nbit, group_size, row
         _lib.lib().wq_debug_set_gemv_config(0, 0)
 
 
+@pytest.mark.parametrize("ways", [2, 4, 8])
+@pytest.mark.parametrize("nbit", [8, 4])
+@pytest.mark.parametrize("group_size", [-1, 64])
+def test_streaming_kernel_with_k_split(ops, u, oracle, nbit, group_size, ways):
+    """2, 4 or 8 wavefronts share a column group and split K (what one row of a narrow int4 matrix gets by itself):
+    K shorter than the split, K that does not divide by it, one and two rows, ragged last workgroup."""
+    from relax_amd import _lib
+
+    L = _lib.lib()
+    L.wq_debug_set_intb_gemv_k_split(ways)
+    L.wq_debug_set_gemv_config(2, 0)
+    try:
+        for M, N, K in [(1, 64, 64), (2, 64, 128), (1, 320, 448), (1, 4096, 1024), (2, 1024, 4096), (1, 8192, 2112),
+                        (1, 5120, 13824)]:
+            print(f"intb k split {ways} nbit={nbit} g={group_size} M={M} N={N} K={K}", flush=True)
+            _run(ops, u, oracle, M, N, K, nbit, seed=M + N + ways, group_size=group_size, bias="row", residual=True)
+        L.wq_debug_set_gemv_config(1, 0)
+        _run(ops, u, oracle, 1, 1024, 4096, nbit, seed=ways, group_size=group_size)
+    finally:
+        L.wq_debug_set_gemv_config(0, 0)
+        L.wq_debug_set_intb_gemv_k_split(0)
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_one_row_of_a_narrow_matrix(ops, u, oracle, nbit):
+    """The automatic choice at M = 1 over widths on both sides of every threshold (int4: the streaming kernel with
+    its own split of K; int8: the small-batch kernel below 8 wavefronts per CU)."""
+    for N, K in [(1024, 4096), (4096, 4096), (5120, 13824), (8192, 8192), (12288, 4096), (22016, 4096)]:
+        for g in (-1, 64):
+            print(f"intb narrow nbit={nbit} g={g} N={N} K={K}", flush=True)
+            _run(ops, u, oracle, 1, N, K, nbit, seed=N + K, group_size=g)
+
+
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 11, 12, 17, 18])
 @pytest.mark.parametrize("nbit", [8, 4])
 def test_gemm_tile_configurations(ops, u, oracle, nbit, cfg):
