@@ -19,6 +19,7 @@
 #include <mutex>
 #include <vector>
 
+#include "mfma_gemm.h"
 #include "mfma_gemm_lds.h"
 #include "q4_gemv.h"
 #include "q4g32_common.h"
@@ -563,14 +564,25 @@ static int wq::gptq_linear_impl(const uint32_t* W_nk, const uint16_t* SZ, const 
     const GptqSkinnyPolicy::Args pargs{W_nk, (const half2_t*)SZ, (int)G, ratio, inv32};
     return launch_skinny_auto<GptqSkinnyPolicy, Q4G32Epilogue>("wq_gptq_linear", pargs, x, y, ep, M, N, K, stream);
   }
+  // up to 128 rows of a small matrix: two passes of the small-batch kernel, as in wq_q4g32_linear (the tiled
+  // GEMM would have too few tiles for 256 CUs: N = K = 4096, M = 128: 35.6 us)
+  if (M <= 2 * WQ_SMALL_BATCH_MAX_M && K % 64 == 0 && N <= 8192) {
+    const GptqSkinnyPolicy::Args pargs{W_nk, (const half2_t*)SZ, (int)G, ratio, inv32};
+    const int64_t m0 = WQ_SMALL_BATCH_MAX_M;
+    if (int rc = launch_skinny_auto<GptqSkinnyPolicy, Q4G32Epilogue>("wq_gptq_linear", pargs, x, y, ep, m0, N, K, stream)) return rc;
+    const Q4G32Epilogue ep2{(const half_t*)bias, residual ? (const half_t*)residual + m0 * N : nullptr, (int)N};
+    return launch_skinny_auto<GptqSkinnyPolicy, Q4G32Epilogue>("wq_gptq_linear", pargs, x + m0 * K, y + m0 * N, ep2, M - m0, N, K, stream);
+  }
   if (gs % 64 != 0)  // a K-step of the GEMM would straddle two groups: repeat the streaming kernel
     return gemv_dispatch<true>("wq_gptq_linear", W_nk, SZ, GemvZp{ratio, (int)G}, x, bias, residual, y, M, N, K, stream);
   const int spg = (int)(gs / 64);
   const GptqLdsPolicy::Args largs{W_nk, (const half2_t*)SZ, (int)G, spg,
                                   spg > 1 ? (uint32_t)(((1ull << 32) + spg - 1) / spg) : 0u};
-  if (M <= 384)
-    return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 4, 1, 1, 4, 2>("wq_gptq_linear", largs, x, y, ep, M, N, K,
-                                                                        stream);
-  return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 8, 2, 1, 4, 1>("wq_gptq_linear", largs, x, y, ep, M, N, K,
-                                                                      stream);
+  // tile shape as for q4f16_1 (N = K = 4096, M = 512 with 256 x 256 tiles: 47 us, with 256 x 128: 33 us)
+  switch (choose_q4_lds_cfg(M, N, cu_count())) {
+    case 17: return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 4, 1, 1, 4, 2>("wq_gptq_linear", largs, x, y, ep, M, N, K, stream);
+    case 18: return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 8, 1, 1, 4, 1>("wq_gptq_linear", largs, x, y, ep, M, N, K, stream);
+    case 13: return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 4, 2, 2, 2, 2>("wq_gptq_linear", largs, x, y, ep, M, N, K, stream);
+    default: return launch_gemm_lds<GptqLdsPolicy, Q4G32Epilogue, 8, 2, 1, 4, 1>("wq_gptq_linear", largs, x, y, ep, M, N, K, stream);
+  }
 }

@@ -246,5 +246,18 @@ inline int choose_gemm_cfg(int64_t M, int64_t N, bool lds_staged) {
   return (N <= 4096 && M <= 1536) ? 13 : 11;
 }
 
+// The fully LDS-staged kernel's tile shape for the 4-bit row-major formats (q4f16_1, AutoGPTQ after its
+// load-time conversion): the choice above, then 256 x 128 tiles, one workgroup per CU and a four-slot ring (18)
+// where they make at most one round of the machine (M = 2048, N = 4096, K = 11008: 208 -> 193 us; M = 1024:
+// 141 -> 116 us; M = 256, N = 12288, K = 4096: 42 -> 39 us); up to 128 rows only for narrow matrices, where
+// 128 x 128 tiles (17) are too few (N = 4096: 35 -> 30 us; N = 12288: 33 against 38 us).
+inline int choose_q4_lds_cfg(int64_t M, int64_t N, int cus) {
+  int cfg = choose_gemm_cfg(M, N, true);
+  if ((cfg == 11 || cfg == 13 || (cfg == 17 && (M > 128 || N <= 6144))) &&
+      ((M + 255) / 256) * ((N + 127) / 128) <= cus)
+    cfg = 18;
+  return cfg;
+}
+
 }  // namespace wq
 #endif  // RELAX_AMD_CSRC_MFMA_GEMM_H_

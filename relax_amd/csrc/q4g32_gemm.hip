@@ -113,14 +113,7 @@ extern "C" int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_
   WQ_REQUIRE(W && S && x && y, "wq_q4g32_gemm: null pointer");
   WQ_REQUIRE(aligned16(W) && aligned16(x), "wq_q4g32_gemm: W and x must be 16-byte aligned");
   WQ_REQUIRE(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), "wq_q4g32_gemm: too large");
-  int cfg = tuning().gemm_cfg ? tuning().gemm_cfg : choose_gemm_cfg(M, N, true);
-  // 256 x 128 tiles, one workgroup per CU and a four-slot ring (18) where they make at most one round of the
-  // machine (M = 2048, N = 4096, K = 11008: 208 -> 193 us; M = 1024: 141 -> 116 us; M = 256, N = 12288,
-  // K = 4096: 42 -> 39 us); up to 128 rows only for narrow matrices, where 128 x 128 tiles (17) are too few
-  // (N = 4096: 35 -> 30 us; N = 12288: 33 against 38 us)
-  if (!tuning().gemm_cfg && (cfg == 11 || cfg == 13 || (cfg == 17 && (M > 128 || N <= 6144))) &&
-      ((M + 255) / 256) * ((N + 127) / 128) <= cu_count())
-    cfg = 18;
+  int cfg = tuning().gemm_cfg ? tuning().gemm_cfg : choose_q4_lds_cfg(M, N, cu_count());
   const Q4G32Loader::Args bargs{W, (const half_t*)S};
   const Q4G32LdsPolicy::Args largs{W, (const half_t*)S};
   const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};

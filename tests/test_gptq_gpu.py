@@ -112,7 +112,9 @@ LINEAR_CASES = [  # (M, N, K, group size, act_order)
     (33, 1032, 4096, 128, True),
     (64, 4096, 4096, 128, False),
     (64, 264, 384, 96, True),      # three 32-code groups per scale group
-    (65, 512, 1024, 128, True),    # MFMA GEMM from here
+    (65, 512, 1024, 128, True),    # two passes of the small-batch kernel up to 128 rows of a matrix with N <= 8192
+    (128, 264, 2048, 64, True),
+    (100, 8200, 256, 128, False),  # wider: the MFMA GEMM
     (16, 512, 1024, 128, False),
     (40, 264, 1152, 192, True),
     (130, 1096, 2048, 64, True),
