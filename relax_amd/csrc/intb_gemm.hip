@@ -201,6 +201,18 @@ static int intb_gemm_common(const char* who, const uint16_t* A, const int8_t* B,
     if (m <= 2 && !narrow) return intb_gemv_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
     if (m <= WQ_SMALL_BATCH_MAX_M && small_ok)
       return intb_small_batch_dispatch(A, B, scales, C, m, n, k, group, nbit, ep, stream);
+    // up to 128 rows of a small matrix: the tiled GEMM has too few tiles for 256 CUs, two passes of the
+    // small-batch kernel (64 rows, then the rest) are faster: n <= 4096 (int8, k = 11008, m = 128: 70 -> 55 us;
+    // k = 4096: 28.4 -> 26.9 us), and up to 96 rows of a long, moderately wide one (k = 13824, n = 5120, m = 96:
+    // 88 -> 75 us; k = n = 8192: 54 -> 50 us).  Wider matrices keep the GEMM (n = 11008, k = 4096: 31 against 36 us).
+    if (m <= 2 * WQ_SMALL_BATCH_MAX_M && small_ok && (n <= 4096 || (m <= 96 && n <= 8192 && k >= 8192))) {
+      const int64_t m0 = WQ_SMALL_BATCH_MAX_M;
+      if (int rc = intb_small_batch_dispatch(A, B, scales, C, m0, n, k, group, nbit, ep, stream)) return rc;
+      IntbEpilogue ep2 = ep;
+      if (ep2.bias && ep2.bias_stride) ep2.bias += m0 * ep2.bias_stride;
+      if (ep2.residual) ep2.residual += m0 * n;
+      return intb_small_batch_dispatch(A + m0 * k, B, scales, C + m0 * n, m - m0, n, k, group, nbit, ep2, stream);
+    }
   }
   const IntbGemmEpilogue gep{ep, (int)n};
   // the fully LDS-staged kernel under the tile shape (11, 17 or 18) whose rounds of the machine come out

@@ -115,7 +115,7 @@ def test_gemm_finegrained(ops, u, oracle, nbit, M):
 
 
 @pytest.mark.parametrize("nbit", [8, 4])
-@pytest.mark.parametrize("M", [2, 48, 130])
+@pytest.mark.parametrize("M", [2, 48, 100, 130])
 @pytest.mark.parametrize("ep", [
     dict(bias="row"), dict(bias="full"), dict(bias="row", activation="relu"), dict(bias="row", activation="silu"),
     dict(bias="row", activation="gelu"), dict(residual=True), dict(bias="row", residual=True, binary_op="plus"),
@@ -161,6 +161,17 @@ def test_one_and_two_rows_on_either_kernel(ops, u, oracle, nbit, group_size, row
             _run(ops, u, oracle, M, N, K, nbit, seed=M + N + rows, group_size=group_size, bias="row")
     finally:
         _lib.lib().wq_debug_set_gemv_config(0, 0)
+
+
+@pytest.mark.parametrize("nbit", [8, 4])
+def test_65_to_128_rows_in_two_small_batch_passes(ops, u, oracle, nbit):
+    """65 .. 128 rows of a small matrix run as two passes of the small-batch kernel (64 rows, then the rest), wider
+    ones as a tiled GEMM: both sides of the rule, with an epilogue that reads per-row operands."""
+    for M, N, K, g in [(65, 4096, 256, -1), (128, 1024, 1024, 64), (96, 5120, 8192, -1), (97, 5120, 8192, -1),
+                       (128, 4160, 512, 64)]:
+        print(f"intb two passes nbit={nbit} M={M} N={N} K={K} g={g}", flush=True)
+        _run(ops, u, oracle, M, N, K, nbit, seed=M + N, group_size=g, bias="full")
+        _run(ops, u, oracle, M, N, K, nbit, seed=M + N + 1, group_size=g, bias="row", residual=True, binary_op="multiply")
 
 
 @pytest.mark.parametrize("ways", [2, 4, 8])
