@@ -147,7 +147,7 @@ typedef struct wq_q4g32_gemv_desc {
 } wq_q4g32_gemv_desc;
 typedef struct wq_gemv_list wq_gemv_list_t;
 #define WQ_GEMV_LIST_MAX 4096
-#define WQ_GEMV_LIST_MAX_K 16384
+#define WQ_GEMV_LIST_MAX_K 32768
 size_t wq_q4g32_gemv_list_workspace_bytes(int n);
 wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* descs, int n, void* workspace,
                                           size_t workspace_bytes, wq_stream_t stream);

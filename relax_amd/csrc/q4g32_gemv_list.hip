@@ -386,6 +386,17 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       // its part of the ring (and its flags and row-sum buffer) is free once the linears that used them
       // before have been flushed: all their rows have been consumed by then
       lds_spin_until(&flags->flushed, descs[j].free_after);
+      // A linear of which this workgroup has no row is not staged.  (It must not be: the y wavefront declares such
+      // a linear flushed at once, so a later linear may already be given the same part of the ring while this
+      // wavefront still waits for a producer or writes: two consecutive rows of more than 40 KB, or a wait for a
+      // producer that outlasts the staging of the linears behind it, then left a mixture of two linears'
+      // activations there.)
+      int rb = (int)blockIdx.x - (int)descs[j].off;
+      if (rb < 0) rb += nwg;
+      if (descs[j].q + (rb < (int)descs[j].rem ? 1 : 0) == 0) {
+        if (lane == 0) __hip_atomic_store(&flags->x_ready[j & (kYSlots - 1)], j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        continue;
+      }
       const int dep = (int)((descs[j].g_dep >> 16) & 0x7fffu) - 1;
       if (dep >= 0) wait_for(dep);
       const int K = (int)(descs[j].g_dep & 0xffffu) << 5;

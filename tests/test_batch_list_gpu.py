@@ -26,7 +26,7 @@ def _linear(oracle, u, N, K, M, seed):
 # K = 256: one short panel; 4096: exactly one panel at M <= 8, two at M > 8; 11008: three panels, the last one short;
 # N = 1, 7, 130: fewer rows than a tile / a partial last tile; 40000: ten tiles per workgroup
 SHAPES = [(4096, 4096), (12288, 4096), (22016, 4096), (4096, 11008), (1, 256), (7, 512), (130, 11008), (1001, 2304),
-          (40000, 256), (48, 16384)]
+          (40000, 256), (48, 16384), (600, 28672), (70, 32768)]
 
 
 @pytest.mark.parametrize("M", [2, 5, 8, 9, 16, 17, 32])
@@ -230,6 +230,32 @@ def test_dependent_chain_matches_oracle(env, oracle, M):
         for y, k in zip(t, keep):
             assert torch.equal(y, k), rep
     gl.status()
+
+
+@pytest.mark.parametrize("M", [3, 16, 32])
+def test_a_long_row_behind_its_producer(env, oracle, M):
+    """The longest rows (K = 28672: seven or fourteen panels, 56 of the row-owner kernel) fed by a linear of the same
+    list, beside a second long linear."""
+    ops, u, torch = env
+    rng = np.random.default_rng(5)
+    up = _linear(oracle, u, 28672, 256, M, seed=21)     # 0: x0 -> t0 [M, 28672]
+    down = _linear(oracle, u, 300, 28672, M, seed=22)   # 1: t0 -> t1
+    other = _linear(oracle, u, 64, 32768, M, seed=23)   # 2: independent
+    x0 = rng.standard_normal((M, 256)).astype(np.float16)
+    t = [torch.zeros((M, n), dtype=torch.float16, device="cuda") for n in (28672, 300, 64)]
+    gl = ops.Q4G32GemvList([(up["dW"], up["dS"], u.dev(x0), t[0]), (down["dW"], down["dS"], t[0], t[1]),
+                            (other["dW"], other["dS"], u.dev(other["x"]), t[2])], M=M)
+    print(f"batch list: long rows, M = {M}", flush=True)
+    r0 = oracle.q4g32_linear(up["W"], up["S"], x0, nthreads=8)
+    refs = (r0, oracle.q4g32_linear(down["W"], down["S"], r0, nthreads=8),
+            oracle.q4g32_linear(other["W"], other["S"], other["x"], nthreads=8))
+    for rep in range(2):
+        for y in t:
+            y.zero_()
+        gl.run()
+        gl.status()
+        for got, ref, name in zip(t, refs, ("up", "down", "other")):
+            u.assert_close(u.host(got), ref, f"batch long rows M={M} {name} rep {rep}")
 
 
 def test_argument_errors(env, oracle):

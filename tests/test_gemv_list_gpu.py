@@ -24,7 +24,7 @@ def _linear(oracle, u, torch, N, K, seed, x=None):
 # ragged shapes: one group, one group more than a chunk of 64, a partial last chunk (K = 11008: 344 groups),
 # fewer rows than wavefronts, more rows than one turn of the grid
 SHAPES = [(4096, 4096), (12288, 4096), (22016, 4096), (4096, 11008), (1, 32), (7, 64), (1001, 2080), (130, 11008),
-          (5000, 8192), (40000, 256), (64, 16384)]
+          (5000, 8192), (40000, 256), (64, 16384), (600, 28672), (9, 32736), (70, 32768)]
 
 
 def test_independent_linears_match_oracle(env, oracle):
@@ -122,6 +122,59 @@ def test_dependent_chain_matches_oracle(env, oracle):
         for y, k in zip(t, keep):
             assert torch.equal(y, k), rep
     gl.status()
+
+
+def test_a_long_row_behind_its_producer(env, oracle):
+    """The longest rows (K = 28672: 72 KB of staged activations) fed by a linear of the same list, next to a
+    second long linear whose activations share the LDS ring with them."""
+    ops, u, torch = env
+    rng = np.random.default_rng(5)
+    up = _linear(oracle, u, torch, 28672, 256, seed=21)     # 0: x0 -> t0 [28672]
+    down = _linear(oracle, u, torch, 300, 28672, seed=22)   # 1: t0 -> t1
+    other = _linear(oracle, u, torch, 64, 32768, seed=23)   # 2: independent
+    x0 = rng.standard_normal((1, 256)).astype(np.float16)
+    t = [torch.zeros((1, n), dtype=torch.float16, device="cuda") for n in (28672, 300, 64)]
+    gl = ops.Q4G32GemvList([(up["dW"], up["dS"], u.dev(x0), t[0]), (down["dW"], down["dS"], t[0], t[1]),
+                            (other["dW"], other["dS"], u.dev(other["x"]), t[2])])
+    print("gemv list: long rows", flush=True)
+    r0 = oracle.q4g32_linear(up["W"], up["S"], x0, nthreads=8)
+    refs = (r0, oracle.q4g32_linear(down["W"], down["S"], r0, nthreads=8),
+            oracle.q4g32_linear(other["W"], other["S"], other["x"], nthreads=8))
+    for rep in range(2):
+        for y in t:
+            y.zero_()
+        gl.run()
+        gl.status()
+        for got, ref, name in zip(t, refs, ("up", "down", "other")):
+            u.assert_close(u.host(got), ref, f"long rows {name} rep {rep}")
+
+
+def test_a_linear_without_rows_in_a_workgroup_does_not_disturb_the_ring(env, oracle):
+    """A narrow linear (most workgroups hold no row of it) that waits for a large producer, followed by enough long
+    linears that the last one is given the narrow one's part of the LDS ring: a workgroup without rows of the narrow
+    linear must leave that part alone (it used to stage the narrow linear's activations there late, over the
+    activations of the last one)."""
+    ops, u, torch = env
+    rng = np.random.default_rng(9)
+    prod = _linear(oracle, u, torch, 16384, 4096, seed=31)    # 0: x0 -> t0 [16384]
+    narrow = _linear(oracle, u, torch, 5, 16384, seed=32)     # 1: t0 -> t1, five rows
+    fill = [_linear(oracle, u, torch, 4096, 16384, seed=33 + i) for i in range(4)]  # 2 .. 5: independent
+    x0 = rng.standard_normal((1, 4096)).astype(np.float16)
+    t = [torch.zeros((1, n), dtype=torch.float16, device="cuda") for n in (16384, 5, 4096, 4096, 4096, 4096)]
+    ent = [(prod["dW"], prod["dS"], u.dev(x0), t[0]), (narrow["dW"], narrow["dS"], t[0], t[1])]
+    ent += [(f["dW"], f["dS"], u.dev(f["x"]), t[2 + i]) for i, f in enumerate(fill)]
+    gl = ops.Q4G32GemvList(ent)
+    print("gemv list: a narrow dependent linear in front of long ones", flush=True)
+    r0 = oracle.q4g32_linear(prod["W"], prod["S"], x0, nthreads=8)
+    refs = [r0, oracle.q4g32_linear(narrow["W"], narrow["S"], r0, nthreads=8)]
+    refs += [oracle.q4g32_linear(f["W"], f["S"], f["x"], nthreads=8) for f in fill]
+    for rep in range(6):
+        for y in t:
+            y.zero_()
+        gl.run()
+        gl.status()
+        for i, (got, ref) in enumerate(zip(t, refs)):
+            u.assert_close(u.host(got), ref, f"narrow dependent linear: linear {i} rep {rep}")
 
 
 def test_a_wait_that_runs_out_is_reported_and_every_wavefront_exits(env, oracle):
