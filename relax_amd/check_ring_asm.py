@@ -20,6 +20,8 @@ sources therefore wait for all loads (``s_waitcnt vmcnt(0)``) where the ring's l
 Registers that the compiler also uses for short-lived temporaries while a slot is empty are
 recognised by being written by another instruction first.
 
+Kernels with such a ring must also be free of register spills (no ``scratch_*`` instruction).
+
 A second check (``check_asm_results``) covers what inline assembly costs besides: the compiler does
 not keep the hardware's wait states between an inline-assembly VALU result and an MFMA or DPP
 instruction that reads it.
@@ -148,6 +150,12 @@ def check(asm_text: str) -> list[str]:
         if any(_is_ring_load(l) for l in body):
             with_ring += 1
             errors += _check_function(body)
+            # These kernels are written to fit their register budget.  A spill anywhere in them (also in a service
+            # wavefront's path: one extra branch there once sent 64 load registers through scratch memory and
+            # cost the 4-linear step 3 of 21 us) is a regression the tests do not show.
+            spills = [l for l in body if l.startswith(("scratch_load", "scratch_store"))]
+            if spills:
+                errors.append(f"{len(spills)} scratch accesses (register spills), the first: `{spills[0]}`")
     if with_ring == 0:
         return ["no ring loads found (expected global_load_* / buffer_load_* ... nt in the kernel)"]
     return errors

@@ -29,6 +29,13 @@ def test_ring_registers_may_only_be_read_by_the_unpack_instructions():
     assert _errors("\tv_mov_b32_e32 v2, 0\n\tv_add_u32_e32 v9, v2, v2") == []
 
 
+def test_a_kernel_with_a_ring_must_not_spill_any_register():
+    spill = "\tscratch_store_dword off, v40, off offset:84\n\tscratch_load_dword v40, off, off offset:84"
+    errs = _errors(spill)
+    assert errs and "scratch accesses" in errs[0]
+    assert _errors("\tv_add_u32_e32 v40, v41, v42") == []
+
+
 def test_a_file_without_ring_loads_is_refused():
     assert c.check("_ZN2wq4testEv:\n\tv_mov_b32_e32 v0, 0\n\ts_endpgm\n.Lfunc_end0:\n")
 
