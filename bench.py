@@ -19,7 +19,8 @@ GEMM of the same quantization scheme, `cpu_baseline` the CPU restatement of the
 reference's path timed on this machine's host cores.  Further objects on the same
 line: `stack` (32 decoder layers' linears run as one captured instruction list at
 M = 1, 8, 16, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
-128, 512), `autogptq` and `kn_gemv` (the neighbouring checkpoint layouts at decode) and
+128, 512), `autogptq` (N = K = 4096, and under `larger_shapes` 4096 -> 22016 and 11008 -> 4096) and `kn_gemv` (the
+neighbouring checkpoint layouts at decode) and
 `calibration` (measured pure-read and MFMA-only ceilings); `single_gemv_4096x4096` (one linear per launch, with
 its own roofline), `list_steady_state` (the list kernel over 906 MB in one launch) and `f16acc` (the
 fp16-accumulate decode entry point).
@@ -646,6 +647,9 @@ def main():
         torch.cuda.empty_cache()
     if not args.no_autogptq:
         out["autogptq"] = bench_autogptq(torch, ops)
+        # the same layer type at the two large decoder shapes (the 4096 x 4096 matrix is 8.9 MB: launch-bound)
+        out["autogptq"]["larger_shapes"] = [bench_autogptq(torch, ops, K=4096, N=22016, batches=(1,), copies=12),
+                                            bench_autogptq(torch, ops, K=11008, N=4096, batches=(1,), copies=24)]
         out["kn_gemv"] = bench_kn_gemv(torch, ops)
     if not args.no_calibration:
         out["calibration"] = bench_calibration(torch)
