@@ -322,6 +322,25 @@ int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm
                    const uint16_t* bias, const uint16_t* residual, uint16_t* y, int64_t M, int64_t N,
                    int64_t K, int64_t G, void* workspace, size_t workspace_bytes, wq_stream_t stream);
 
+/* A list of prepared AutoGPTQ layers at M = 1 as ONE launch: wq_q4g32_gemv_list_create for the layers of
+ * tests/python/dlight/test_gpu_gemv.py:636-665, which the reference's GEMV rule leaves unscheduled (:667-672).
+ * Same kernel design, same workspace (wq_q4g32_gemv_list_workspace_bytes), and the list is run, checked and
+ * destroyed with the wq_q4g32_gemv_list_* calls above; arithmetic as wq_gptq_linear at M = 1.  W_nk / SZ from
+ * wq_gptq_prepare, in the prepared row order: a layer whose preparation reported *needs_perm = 1 cannot be a
+ * member (its activations would have to be gathered between two linears of the launch); x fp16 [K], y fp16 [N].
+ * The group size K / G must be 32 << t, t = 0 .. 6 (WQ_EUNSUPPORTED otherwise). */
+typedef struct wq_gptq_gemv_desc {
+  const uint32_t* W_nk;     /* uint32 [N, K/8] */
+  const uint16_t* SZ;       /* fp16 [N, G, 2] */
+  const uint16_t* x;        /* fp16 [K] */
+  const uint16_t* bias;     /* fp16 [N] or NULL */
+  const uint16_t* residual; /* fp16 [N] or NULL */
+  uint16_t* y;              /* fp16 [N] */
+  int64_t N, K, G;          /* K % 32 == 0, K <= WQ_GEMV_LIST_MAX_K */
+} wq_gptq_gemv_desc;
+wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* descs, int n, void* workspace,
+                                         size_t workspace_bytes, wq_stream_t stream);
+
 /* wq_gptq_linear for callers that cannot allocate device memory and have no workspace to
  * pass (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It has
  * no counterpart in the reference.  Same arguments and results as wq_gptq_linear without the

@@ -8,7 +8,7 @@ spill of a ring register inserted between load and wait would read it too early)
 compiles the file to assembly and verifies, in the kernel's text, that
 
 * every ring register (destination of a ``global_load_* ... nt`` or ``buffer_load_* ... nt`` instruction) is read only by the
-  instructions the source uses for it (``v_and_or_b32``, ``v_lshrrev_b32 .., 8, ..``, ``v_cvt_f32_f16``,
+  instructions the source uses for it (``v_and_or_b32``, ``v_lshrrev_b32 .., 8 | 16, ..``, ``v_cvt_f32_f16``,
   and the cross-lane ``v_mov_b32_dpp`` of the batch kernel's lane exchange, which the compiler never
   generates by itself), never by a plain move, a store or anything else, and
 * each ring slot keeps one register in the prologue and in the loop (no renaming copies).
@@ -81,7 +81,7 @@ def _check_function(body: list[str]) -> list[str]:
         hit = reads & loaded
         if hit and not op.startswith(ALLOWED_READERS):
             errors.append(f"ring register(s) {sorted(hit)} read by `{l}`")
-        if op.startswith("v_lshrrev_b32") and hit and ops[1] != "8":
+        if op.startswith("v_lshrrev_b32") and hit and ops[1] not in ("8", "16"):
             errors.append(f"unexpected shift of a ring register: `{l}`")
         loaded -= writes  # now a temporary of the compiler
     return errors

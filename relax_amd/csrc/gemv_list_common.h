@@ -34,7 +34,8 @@ struct GemvListDesc {  // 128 bytes, device memory
   uint8_t ts;          // log2 of the rows a compute wavefront takes at a time (0 .. gs)
   uint32_t x_off;      // LDS byte offset of the linear's activations (the workgroup's LDS is dealt as a ring)
   int32_t free_after;  // ... which may be written once this many linears of the list have been flushed
-  uint8_t pad[52];
+  uint8_t szl;         // lists of AutoGPTQ layers: log2 of (group size / 32); S then holds (scale, zero point + 1) pairs
+  uint8_t pad[51];
 };
 static_assert(sizeof(GemvListDesc) == 128, "descriptor layout");
 constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y
@@ -82,6 +83,7 @@ struct wq_gemv_list {
   int nb = 2;
   int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
   long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
+  bool zp = false;         // AutoGPTQ layers: a (scale, zero point + 1) pair per group instead of a scale per 32 columns
   int M = 1;               // activation rows of the launch; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
   int batch_u = 0;         // chunks per tile and wavefront (4: M <= 16; 2: beyond)
   int batch_groups = 1;    // groups of workgroups that run different linears side by side (0: sets of XCDs per linear)

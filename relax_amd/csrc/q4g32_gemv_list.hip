@@ -72,10 +72,12 @@ struct GroupCursor {
   int xoff;         // LDS offset of the linear's activations
   int C;            // chunks per row
   int row_w, row_s; // bytes per row of W and S
+  int szl;          // ZP: log2 of the 32-column groups that share one (scale, zero point) pair
   const char* W;
   const char* S;
 };
 
+template <bool ZP>
 __device__ __forceinline__ void group_cursor_load(GroupCursor& cu, gemv_desc_ptr descs, int nlin, int b, int nwg, int gs) {
   if (cu.lin >= nlin) {
     cu.R = 0x7fffffff;  // every position from here on is "past the end"
@@ -84,9 +86,10 @@ __device__ __forceinline__ void group_cursor_load(GroupCursor& cu, gemv_desc_ptr
   // (W, S: words 0..3; N, q, g_dep, rem | off << 16: 12..15)
   typedef const uint32_t __attribute__((address_space(4)))* words_ptr;
   const words_ptr p = (words_ptr)(descs + cu.lin);
-  uint32_t w[19];
+  constexpr int kWords = ZP ? 20 : 19;
+  uint32_t w[kWords];
 #pragma unroll
-  for (int i = 0; i < 19; ++i) w[i] = p[i];  // (16: groups of the batch kernel, ts; 17: x_off)
+  for (int i = 0; i < kWords; ++i) w[i] = p[i];  // (16: groups of the batch kernel, ts; 17: x_off; 19: szl)
   const int G = (int)(w[14] & 0xffffu);
   int rb = b - (int)(w[15] >> 16);
   if (rb < 0) rb += nwg;
@@ -97,7 +100,13 @@ __device__ __forceinline__ void group_cursor_load(GroupCursor& cu, gemv_desc_ptr
   cu.R = ((int)w[13] + (rb < (int)(w[15] & 0xffffu) ? 1 : 0)) << (gs - cu.ts);
   cu.C = (G + 63) >> 6;
   cu.row_w = G << 4;
-  cu.row_s = G << 1;
+  if constexpr (ZP) {
+    cu.szl = (int)(w[19] & 0xffu);
+    cu.row_s = (G >> cu.szl) << 2;  // a pair of fp16 per group
+  } else {
+    cu.szl = 0;
+    cu.row_s = G << 1;
+  }
   cu.W = reinterpret_cast<const char*>(((uint64_t)w[1] << 32) | w[0]);
   cu.S = reinterpret_cast<const char*>(((uint64_t)w[3] << 32) | w[2]);
 }
@@ -119,7 +128,11 @@ struct ListFlags {
   int pad[13];
 };
 
-template <int NC, int XW, int D>
+// ZP: the linears are prepared AutoGPTQ layers.  S holds a (scale, zero point + 1) pair of fp16 per column and
+// group of 32 << szl columns; a lane loads the 4 bytes of its group's pair instead of a scale, and the constant
+// that starts a group's sum becomes -(1024 A + 64 B) - zp (A + B) from the two sums the x wavefronts leave in LDS
+// (A, B: the activations under the codes that are unpacked as 1024 + q and as 1024 + 16 q).
+template <int NC, int XW, int D, bool ZP>
 __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(const GemvListDesc* __restrict__ descs_,
                                                                         int nlin, int* __restrict__ sync,
                                                                         long long spin_limit, int ybuf0,
@@ -179,7 +192,7 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
     GroupCursor ic;
     ic.lin = 0;
     ic.base = 0;
-    group_cursor_load(ic, descs, nlin, b, nwg, gs);
+    group_cursor_load<ZP>(ic, descs, nlin, b, nwg, gs);
     int i_rows = 0;       // rows of the group still to start
     int i_left = 0;       // chunks of the row still to issue
     int i_off = 0;        // byte offset of the next chunk in the row of codes
@@ -188,6 +201,8 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
     int i_x0 = 0;         // ... of the row's first chunk
     int i_yl = 0;         // slot_yl of the row
     int i_first = 0;      // kFirst until the group's first chunk has been issued
+    int i_sinc = 128;     // bytes of a row of S per chunk (64 scales; ZP: 64 >> szl pairs)
+    uint32_t s_lane = lane16 >> 3;  // this lane's byte offset in a chunk's piece of S
     // buffer resources of the row: base address, size in bytes, flags (an empty one: every lane reads zero, no memory access)
     auto row_rsrc = [](const char* p, int bytes) {
       const uint64_t a = reinterpret_cast<uint64_t>(p);
@@ -202,7 +217,7 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         while (ic.lin < nlin && pos >= ic.base + ic.R) {
           ic.base += ic.R;
           ++ic.lin;
-          group_cursor_load(ic, descs, nlin, b, nwg, gs);
+          group_cursor_load<ZP>(ic, descs, nlin, b, nwg, gs);
         }
         if (ic.lin >= nlin) {  // the list has run out: the slots drain
           i_left = -1;
@@ -218,7 +233,13 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       i_rows = min(1 << ic.ts, ic.N - (int)row) - 1;
       const uint64_t woff = (uint64_t)row * (uint32_t)ic.row_w;  // a row of scales is an eighth of a row of codes
       i_w = row_rsrc(ic.W + woff, ic.row_w);
-      i_s = row_rsrc(ic.S + (woff >> 3), ic.row_s);
+      if constexpr (ZP) {
+        i_s = row_rsrc(ic.S + (uint64_t)row * (uint32_t)ic.row_s, ic.row_s);
+        i_sinc = 256 >> ic.szl;
+        s_lane = ((uint32_t)lane >> ic.szl) << 2;
+      } else {
+        i_s = row_rsrc(ic.S + (woff >> 3), ic.row_s);
+      }
       i_left = ic.C;
       i_off = i_soff = 0;
       i_x = i_x0 = ic.xoff;
@@ -244,11 +265,18 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
         if (i_rows > 0) next_row();
         else next_group();
       }
-      asm volatile(
-          "buffer_load_dwordx4 %0, %2, %3, %4 offen nt\n\t"
-          "buffer_load_ushort %1, %5, %6, %7 offen nt"
-          : "=&v"(w), "=&v"(s)
-          : "v"(lane16), "s"(i_w), "s"(i_off), "v"(lane16 >> 3), "s"(i_s), "s"(i_soff));
+      if constexpr (ZP)
+        asm volatile(
+            "buffer_load_dwordx4 %0, %2, %3, %4 offen nt\n\t"
+            "buffer_load_dword %1, %5, %6, %7 offen nt"
+            : "=&v"(w), "=&v"(s)
+            : "v"(lane16), "s"(i_w), "s"(i_off), "v"(s_lane), "s"(i_s), "s"(i_soff));
+      else
+        asm volatile(
+            "buffer_load_dwordx4 %0, %2, %3, %4 offen nt\n\t"
+            "buffer_load_ushort %1, %5, %6, %7 offen nt"
+            : "=&v"(w), "=&v"(s)
+            : "v"(lane16), "s"(i_w), "s"(i_off), "v"(lane16 >> 3), "s"(i_s), "s"(i_soff));
       if (i_left < 0) {
         meta = kDead;
         return;
@@ -258,7 +286,7 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       yl = i_yl;
       i_first = 0;
       i_off += 1024;
-      i_soff += 128;
+      i_soff += ZP ? i_sinc : 128;
       i_x += kChunkBytes;
     };
 
@@ -272,6 +300,11 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
     auto ring_shr8 = [&](uint32_t word) {
       uint32_t r;
       asm("v_lshrrev_b32 %0, 8, %1 ; %2" : "=v"(r) : "v"(word), "v"(magic));
+      return r;
+    };
+    auto ring_shr16 = [&](uint32_t word) {
+      uint32_t r;
+      asm("v_lshrrev_b32 %0, 16, %1 ; %2" : "=v"(r) : "v"(word), "v"(magic));
       return r;
     };
     auto ring_scale = [&](uint32_t s16) {
@@ -288,9 +321,17 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       uint4_t xv[4];
 #pragma unroll
       for (int ch = 0; ch < 4; ++ch) xv[ch] = *reinterpret_cast<const uint4_t*>(xb + ch * 1024);
-      float grp = *reinterpret_cast<const float*>(xb + 4096);
+      float grp, zsum = 0.0f;
+      if constexpr (ZP) {
+        const float2 cz = *reinterpret_cast<const float2*>(xb + 4096);
+        grp = cz.x;
+        zsum = cz.y;
+      } else {
+        grp = *reinterpret_cast<const float*>(xb + 4096);
+      }
       // every slot is always in flight (the drained ones with loads that fetch nothing): this one is the oldest
       asm volatile("s_waitcnt vmcnt(%1)" : "+v"(magic) : "n"(2 * (D - 1)));
+      if constexpr (ZP) grp = fmaf((float)as_half((uint16_t)ring_shr16(s16)), zsum, grp);
 #pragma unroll
       for (int ch = 0; ch < 4; ++ch) {
         const uint32_t word = ch == 0 ? w4.x : ch == 1 ? w4.y : ch == 2 ? w4.z : w4.w;
@@ -373,8 +414,10 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     };
 
-    const half2_t k1031 = {(half_t)1031.0f, (half_t)1031.0f};
-    const half2_t k71 = {(half_t)71.0f, (half_t)71.0f};
+    // without zero points the constant 7 is folded here: 1024 + 7 and 64 + 7
+    const half2_t k1031 = {(half_t)(ZP ? 1024.0f : 1031.0f), (half_t)(ZP ? 1024.0f : 1031.0f)};
+    const half2_t k71 = {(half_t)(ZP ? 64.0f : 71.0f), (half_t)(ZP ? 64.0f : 71.0f)};
+    const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
     const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
     while (true) {
       // whichever x wavefront is free takes the next linear, so that one slow wait does not hold up
@@ -443,7 +486,17 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
             char* cb = xb + (grp >> 6) * kChunkBytes;
             *reinterpret_cast<uint4_t*>(cb + ch * 1024 + (grp & 63) * 16) =
                 uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
-            if (ch == 0) *reinterpret_cast<float*>(cb + 4096 + (grp & 63) * 16) = -c;
+            if constexpr (ZP) {  // the zero point multiplies the plain sum of the group's activations
+              float t = dot2(as_half2(o[0]), ones, 0.0f);
+              t = dot2(as_half2(o[1]), ones, t);
+              t = dot2(as_half2(o[2]), ones, t);
+              t = dot2(as_half2(o[3]), ones, t);
+              t += dpp_shift<0xb1, 0xf>(t);
+              t += dpp_shift<0x4e, 0xf>(t);
+              if (ch == 0) *reinterpret_cast<float2*>(cb + 4096 + (grp & 63) * 16) = float2{-c, -t};
+            } else {
+              if (ch == 0) *reinterpret_cast<float*>(cb + 4096 + (grp & 63) * 16) = -c;
+            }
           }
         }
       }
@@ -544,10 +597,47 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
   return wq_q4g32_gemv_list_create_batched(d, n, 1, workspace, workspace_bytes, stream);
 }
 
+namespace wq {
+// szl == nullptr: format A.  Else the linears are prepared AutoGPTQ layers: d[i].S is SZ and szl[i] the log2 of
+// the 32-column groups per (scale, zero point) pair.
+static wq_gemv_list_t* gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, int n, int M, void* workspace,
+                                        size_t workspace_bytes, hipStream_t stream);
+}  // namespace wq
+
 extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv_desc* d, int n, int M, void* workspace,
-                                                             size_t workspace_bytes, wq_stream_t stream_) {
+                                                             size_t workspace_bytes, wq_stream_t stream) {
+  return wq::gemv_list_create(d, nullptr, n, M, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* d, int n, void* workspace,
+                                                    size_t workspace_bytes, wq_stream_t stream) {
   using namespace wq;
-  hipStream_t stream = (hipStream_t)stream_;
+#define bad(code, ...) ((void)fail(code, __VA_ARGS__), (wq_gemv_list_t*)nullptr)
+  if (!d || n <= 0 || n > WQ_GEMV_LIST_MAX)
+    return bad(WQ_EINVAL, "wq_gptq_gemv_list_create: need 1 .. %d linears, got %d", WQ_GEMV_LIST_MAX, n);
+  std::vector<wq_q4g32_gemv_desc> e(n);
+  std::vector<uint8_t> szl(n);
+  for (int i = 0; i < n; ++i) {
+    const wq_gptq_gemv_desc& s = d[i];
+    // a pair serves 32 << szl columns of a row; a chunk of 64 x 32 columns must hold whole pairs' worth of lanes
+    int lg = -1;
+    if (s.K > 0 && s.G > 0 && s.K % s.G == 0)
+      for (int t = 0; t <= 6; ++t)
+        if (s.K / s.G == (32ll << t)) lg = t;
+    if (lg < 0)
+      return bad(WQ_EUNSUPPORTED, "wq_gptq_gemv_list_create: linear %d: K=%lld G=%lld (the group size K / G must be 32, 64, ... or 2048)",
+                 i, (long long)s.K, (long long)s.G);
+    if (!s.SZ || (reinterpret_cast<uintptr_t>(s.SZ) & 3))
+      return bad(WQ_EINVAL, "wq_gptq_gemv_list_create: linear %d: SZ must be 4-byte aligned", i);
+    e[i] = wq_q4g32_gemv_desc{s.W_nk, s.SZ, s.x, s.bias, s.residual, s.y, s.N, s.K};
+    szl[i] = (uint8_t)lg;
+  }
+  return gemv_list_create(e.data(), szl.data(), n, 1, workspace, workspace_bytes, (hipStream_t)stream);
+#undef bad
+}
+
+static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, int n, int M, void* workspace,
+                                            size_t workspace_bytes, hipStream_t stream) {
 #define bad(code, ...) ((void)fail(code, __VA_ARGS__), (wq_gemv_list_t*)nullptr)
   if (M < 1 || M > WQ_GEMV_LIST_MAX_M)
     return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: 1 .. %d rows of activations, got %d", WQ_GEMV_LIST_MAX_M, M);
@@ -576,6 +666,7 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
   std::unique_ptr<wq_gemv_list> l(new wq_gemv_list());
   l->n = ne;
   l->M = M;
+  l->zp = szl != nullptr;
   l->descs.resize(ne);
   int cmax = 1;
   for (int i = 0; i < ne; ++i) {
@@ -593,6 +684,7 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
     g.rem = 0;
     g.off = 0;
     g.rows = (uint8_t)rows[i];
+    g.szl = szl ? szl[i] : 0;
     cmax = std::max(cmax, (int)((s.K / 32 + 63) / 64));
   }
   // Who reads what an earlier linear of the list wrote.  Writing over something an earlier linear
@@ -687,9 +779,10 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv
       l->descs[i].ts = (uint8_t)ts;
     }
   }
-  auto kern = q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>;
-  static DynamicLdsLimit limit;  // several lists share the kernel: the limit only ever grows
-  if (l->lds > 48 * 1024 && limit.ensure(reinterpret_cast<const void*>(kern), (int)l->lds) != hipSuccess)
+  const void* kern = l->zp ? reinterpret_cast<const void*>(q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth, true>)
+                           : reinterpret_cast<const void*>(q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth, false>);
+  static DynamicLdsLimit limit[2];  // several lists share a kernel: its limit only ever grows
+  if (l->lds > 48 * 1024 && limit[l->zp ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
     return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
@@ -709,7 +802,13 @@ extern "C" int wq_q4g32_gemv_list_run(wq_gemv_list_t* l, wq_stream_t stream) {
   using namespace wq;
   WQ_REQUIRE(l && l->table, "wq_q4g32_gemv_list_run: null list");
   if (l->M > 1) return batch_list_launch(l, (hipStream_t)stream);
-  WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth>), dim3((unsigned)l->blocks),
+  if (l->zp) {
+    WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth, true>), dim3((unsigned)l->blocks),
+              dim3((unsigned)l->threads), l->lds, (hipStream_t)stream, (const GemvListDesc*)l->table, l->n, l->sync,
+              l->spin_limit, l->ybuf0, l->ybuf_floats, l->gs, l->deps > 0 ? 1 : 0);
+    return WQ_OK;
+  }
+  WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth, false>), dim3((unsigned)l->blocks),
             dim3((unsigned)l->threads), l->lds, (hipStream_t)stream, (const GemvListDesc*)l->table, l->n, l->sync,
             l->spin_limit, l->ybuf0, l->ybuf_floats, l->gs, l->deps > 0 ? 1 : 0);
   return WQ_OK;
