@@ -19,7 +19,8 @@ GEMM of the same quantization scheme, `cpu_baseline` the CPU restatement of the
 reference's path timed on this machine's host cores.  Further objects on the same
 line: `stack` (32 decoder layers' linears run as one captured instruction list at
 M = 1, 8, 16, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
-128, 512), `autogptq` (N = K = 4096, and under `larger_shapes` 4096 -> 22016 and 11008 -> 4096) and `kn_gemv` (the
+128, 512), `autogptq` (N = K = 4096; under `larger_shapes` 4096 -> 22016 and 11008 -> 4096; under `decode_step_as_list`
+the four decoder linears as one launch against four) and `kn_gemv` (the
 neighbouring checkpoint layouts at decode) and
 `calibration` (measured pure-read and MFMA-only ceilings); `single_gemv_4096x4096` (one linear per launch, with
 its own roofline), `list_steady_state` (the list kernel over 906 MB in one launch) and `f16acc` (the
@@ -337,6 +338,57 @@ def bench_autogptq(torch, ops, K=4096, N=4096, group=128, batches=(1, 8), copies
     return res
 
 
+def bench_autogptq_list(torch, ops, copies=6, group=128):
+    """The decode step of the four Llama-2-7B-shaped linears as prepared AutoGPTQ layers (group 128, rows in
+    group order) at M = 1: ONE launch of the list kernel per step (`wq_gptq_gemv_list_create`) against four
+    calls of `wq_gptq_linear`; `copies` weight sets (more than the last-level cache) are cycled inside one
+    captured graph.  Bytes = codes + (scale, zero point) pairs + x + y."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(13)
+    sets = []
+    for _ in range(copies):
+        layers = []
+        for N, K in DECODE_SHAPES:
+            G = K // group
+            qw = torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device="cuda", generator=g)
+            qz = torch.randint(-2**31, 2**31 - 1, (G, N // 8), dtype=torch.int32, device="cuda", generator=g)
+            sc = (torch.rand((G, N), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+            gi = (torch.arange(K, device="cuda") // group).to(torch.int32)
+            layers.append(ops.gptq_prepare(qw, qz, sc, gi))
+            del qw, qz, sc
+        sets.append(layers)
+    xs = [torch.randn((1, K), device="cuda", dtype=torch.float16) for _, K in DECODE_SHAPES]
+    ys = [torch.empty((1, N), device="cuda", dtype=torch.float16) for N, _ in DECODE_SHAPES]
+    lists = [ops.GptqGemvList([(w, x, y) for w, x, y in zip(layers, xs, ys)]) for layers in sets]
+    nbytes = sum(N * K // 2 + N * (K // group) * 4 + K * 2 + N * 2 for N, K in DECODE_SHAPES)
+    res = {"group_size": group, "weight": "int4 + zero points", "linears": [list(s) for s in DECODE_SHAPES],
+           "bytes_per_step": nbytes, "weight_sets": copies}
+
+    def as_list():
+        for l in lists:
+            l.run()
+
+    def call_by_call():
+        for layers in sets:
+            for w, x, y in zip(layers, xs, ys):
+                ops.gptq_linear(w, x, out=y)
+
+    for name, fn in (("one_launch", as_list), ("four_launches", call_by_call)):
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(4):
+                fn()
+        graph.replay()
+        ms, _ = _measure(torch, torch.cuda.current_stream(), graph.replay, min_ms=MIN_SAMPLE_MS / 4, samples=3)
+        ms /= 4 * copies
+        res[name] = {"us_per_step": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    lists[0].status()
+    return res
+
+
 def bench_kn_gemv(torch, ops, copies=24):
     """The decode linear over K-major (KN) q4f16_1 weights used in place (`wq_q4g32_kn_gemv`), M = 1, the
     four Llama-2-7B shapes; `copies` weight copies (more than the last-level cache) are cycled inside one
@@ -648,6 +700,7 @@ def main():
     if not args.no_autogptq:
         out["autogptq"] = bench_autogptq(torch, ops)
         # the same layer type at the two large decoder shapes (the 4096 x 4096 matrix is 8.9 MB: launch-bound)
+        out["autogptq"]["decode_step_as_list"] = bench_autogptq_list(torch, ops)
         out["autogptq"]["larger_shapes"] = [bench_autogptq(torch, ops, K=4096, N=22016, batches=(1,), copies=12),
                                             bench_autogptq(torch, ops, K=11008, N=4096, batches=(1,), copies=24)]
         out["kn_gemv"] = bench_kn_gemv(torch, ops)
