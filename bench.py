@@ -339,53 +339,63 @@ def bench_autogptq(torch, ops, K=4096, N=4096, group=128, batches=(1, 8), copies
 
 
 def bench_autogptq_list(torch, ops, copies=6, group=128):
-    """The decode step of the four Llama-2-7B-shaped linears as prepared AutoGPTQ layers (group 128, rows in
-    group order) at M = 1: ONE launch of the list kernel per step (`wq_gptq_gemv_list_create`) against four
-    calls of `wq_gptq_linear`; `copies` weight sets (more than the last-level cache) are cycled inside one
-    captured graph.  Bytes = codes + (scale, zero point) pairs + x + y."""
+    """The decode step of the four Llama-2-7B-shaped linears as prepared AutoGPTQ layers (group 128) at M = 1,
+    without and with a row order (desc_act): ONE launch of the list kernel per step (`wq_gptq_gemv_list_create`;
+    a row order is applied while the activations are staged) against four calls of `wq_gptq_linear` (each
+    preceded by a gather kernel when there is a row order); `copies` weight sets (more than the last-level
+    cache) are cycled inside one captured graph.  Bytes = codes + (scale, zero point) pairs + x + y."""
     g = torch.Generator(device="cuda")
     g.manual_seed(13)
-    sets = []
-    for _ in range(copies):
-        layers = []
-        for N, K in DECODE_SHAPES:
-            G = K // group
-            qw = torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device="cuda", generator=g)
-            qz = torch.randint(-2**31, 2**31 - 1, (G, N // 8), dtype=torch.int32, device="cuda", generator=g)
-            sc = (torch.rand((G, N), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
-            gi = (torch.arange(K, device="cuda") // group).to(torch.int32)
-            layers.append(ops.gptq_prepare(qw, qz, sc, gi))
-            del qw, qz, sc
-        sets.append(layers)
-    xs = [torch.randn((1, K), device="cuda", dtype=torch.float16) for _, K in DECODE_SHAPES]
-    ys = [torch.empty((1, N), device="cuda", dtype=torch.float16) for N, _ in DECODE_SHAPES]
-    lists = [ops.GptqGemvList([(w, x, y) for w, x, y in zip(layers, xs, ys)]) for layers in sets]
     nbytes = sum(N * K // 2 + N * (K // group) * 4 + K * 2 + N * 2 for N, K in DECODE_SHAPES)
     res = {"group_size": group, "weight": "int4 + zero points", "linears": [list(s) for s in DECODE_SHAPES],
-           "bytes_per_step": nbytes, "weight_sets": copies}
+           "bytes_per_step": nbytes, "weight_sets": copies, "cases": []}
+    xs = [torch.randn((1, K), device="cuda", dtype=torch.float16) for _, K in DECODE_SHAPES]
+    ys = [torch.empty((1, N), device="cuda", dtype=torch.float16) for N, _ in DECODE_SHAPES]
+    wss = [torch.empty((max(1, ops.gptq_workspace_bytes(1, K, True)),), dtype=torch.uint8, device="cuda")
+           for _, K in DECODE_SHAPES]
+    for act in (False, True):
+        sets = []
+        for _ in range(copies):
+            layers = []
+            for N, K in DECODE_SHAPES:
+                G = K // group
+                qw = torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device="cuda", generator=g)
+                qz = torch.randint(-2**31, 2**31 - 1, (G, N // 8), dtype=torch.int32, device="cuda", generator=g)
+                sc = (torch.rand((G, N), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+                gi = (torch.arange(K, device="cuda") // group).to(torch.int32)
+                if act:
+                    gi = gi[torch.randperm(K, device="cuda", generator=g)].contiguous()
+                layers.append(ops.gptq_prepare(qw, qz, sc, gi))
+                del qw, qz, sc
+            sets.append(layers)
+        lists = [ops.GptqGemvList([(w, x, y) for w, x, y in zip(layers, xs, ys)]) for layers in sets]
 
-    def as_list():
-        for l in lists:
-            l.run()
+        def as_list():
+            for l in lists:
+                l.run()
 
-    def call_by_call():
-        for layers in sets:
-            for w, x, y in zip(layers, xs, ys):
-                ops.gptq_linear(w, x, out=y)
+        def call_by_call():
+            for layers in sets:
+                for w, x, y, ws in zip(layers, xs, ys, wss):
+                    ops.gptq_linear(w, x, out=y, workspace=ws)
 
-    for name, fn in (("one_launch", as_list), ("four_launches", call_by_call)):
-        fn()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            for _ in range(4):
-                fn()
-        graph.replay()
-        ms, _ = _measure(torch, torch.cuda.current_stream(), graph.replay, min_ms=MIN_SAMPLE_MS / 4, samples=3)
-        ms /= 4 * copies
-        res[name] = {"us_per_step": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
-                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
-    lists[0].status()
+        case = {"row_order": act}
+        for name, fn in (("one_launch", as_list), ("four_calls", call_by_call)):
+            fn()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(4):
+                    fn()
+            graph.replay()
+            ms, _ = _measure(torch, torch.cuda.current_stream(), graph.replay, min_ms=MIN_SAMPLE_MS / 4, samples=3)
+            ms /= 4 * copies
+            case[name] = {"us_per_step": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+                          "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            del graph
+        lists[0].status()
+        res["cases"].append(case)
+        del lists, sets
     return res
 
 

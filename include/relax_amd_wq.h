@@ -326,12 +326,14 @@ int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm
  * tests/python/dlight/test_gpu_gemv.py:636-665, which the reference's GEMV rule leaves unscheduled (:667-672).
  * Same kernel design, same workspace (wq_q4g32_gemv_list_workspace_bytes), and the list is run, checked and
  * destroyed with the wq_q4g32_gemv_list_* calls above; arithmetic as wq_gptq_linear at M = 1.  W_nk / SZ from
- * wq_gptq_prepare, in the prepared row order: a layer whose preparation reported *needs_perm = 1 cannot be a
- * member (its activations would have to be gathered between two linears of the launch); x fp16 [K], y fp16 [N].
- * The group size K / G must be 32 << t, t = 0 .. 6 (WQ_EUNSUPPORTED otherwise). */
+ * wq_gptq_prepare; perm is the row order it wrote when it reported *needs_perm = 1 (16-byte aligned), else NULL:
+ * the activations of such a layer are gathered through it while they are staged, inside the launch, so x is always
+ * the layer's input in checkpoint order, fp16 [K]; y fp16 [N].  The group size K / G must be 32 << t, t = 0 .. 6
+ * (WQ_EUNSUPPORTED otherwise); operands of wq_gptq_prepare_padded are not accepted. */
 typedef struct wq_gptq_gemv_desc {
   const uint32_t* W_nk;     /* uint32 [N, K/8] */
   const uint16_t* SZ;       /* fp16 [N, G, 2] */
+  const int32_t* perm;      /* int32 [K] or NULL */
   const uint16_t* x;        /* fp16 [K] */
   const uint16_t* bias;     /* fp16 [N] or NULL */
   const uint16_t* residual; /* fp16 [N] or NULL */

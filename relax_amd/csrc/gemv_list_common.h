@@ -35,7 +35,9 @@ struct GemvListDesc {  // 128 bytes, device memory
   uint32_t x_off;      // LDS byte offset of the linear's activations (the workgroup's LDS is dealt as a ring)
   int32_t free_after;  // ... which may be written once this many linears of the list have been flushed
   uint8_t szl;         // lists of AutoGPTQ layers: log2 of (group size / 32); S then holds (scale, zero point + 1) pairs
-  uint8_t pad[51];
+  uint8_t pad0[3];
+  const int32_t* perm; // ... and the row order of the layer, int32 [K], or null: position k' of a row of W multiplies x[perm[k']]
+  uint8_t pad[40];
 };
 static_assert(sizeof(GemvListDesc) == 128, "descriptor layout");
 constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y

@@ -434,7 +434,9 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       const half_t* const x_src = descs[j].x;
       const uint32_t x_off = descs[j].x_off;
       const int d_off = (int)descs[j].off, d_q = descs[j].q, d_rem = (int)descs[j].rem;
-      asm volatile("" ::"s"(free_after), "s"(g_dep), "s"(x_src), "s"(x_off), "s"(d_off), "s"(d_q), "s"(d_rem));
+      const int32_t* perm = nullptr;
+      if constexpr (ZP) perm = descs[j].perm;
+      asm volatile("" ::"s"(free_after), "s"(g_dep), "s"(x_src), "s"(x_off), "s"(d_off), "s"(d_q), "s"(d_rem), "s"(perm));
       // its part of the ring (and its flags and row-sum buffer) is free once the linears that used them
       // before have been flushed: all their rows have been consumed by then
       lds_spin_until(&flags->flushed, free_after);
@@ -459,6 +461,76 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
       // none without rows (the same path, so that the loop keeps its shape: a `continue` above made the compiler
       // spill this wavefront's 64 load registers)
       const int nwords = has_rows ? (((K >> 5) + 63) & ~63) << 2 : 0;
+      // one 16-byte word of 8 activations (natural order) -> the pairing of the unpack and the group constants, to LDS
+      auto stage = [&](int wi, const uint4_t& w8) {
+        const uint32_t in[4] = {w8.x, w8.y, w8.z, w8.w};
+        uint32_t o[4];
+        pair_i_i4(in, o);  // o[i] = (x_i, x_{i+4})
+        float c = dot2(as_half2(o[0]), k1031, 0.0f);
+        c = dot2(as_half2(o[1]), k71, c);
+        c = dot2(as_half2(o[2]), k1031, c);
+        c = dot2(as_half2(o[3]), k71, c);
+        c += dpp_shift<0xb1, 0xf>(c);  // the 4 words of a group sit in 4 adjacent lanes
+        c += dpp_shift<0x4e, 0xf>(c);
+        const int grp = wi >> 2, ch = wi & 3;
+        char* cb = xb + (grp >> 6) * kChunkBytes;
+        *reinterpret_cast<uint4_t*>(cb + ch * 1024 + (grp & 63) * 16) =
+            uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
+        if constexpr (ZP) {  // the zero point multiplies the plain sum of the group's activations
+          float t = dot2(as_half2(o[0]), ones, 0.0f);
+          t = dot2(as_half2(o[1]), ones, t);
+          t = dot2(as_half2(o[2]), ones, t);
+          t = dot2(as_half2(o[3]), ones, t);
+          t += dpp_shift<0xb1, 0xf>(t);
+          t += dpp_shift<0x4e, 0xf>(t);
+          if (ch == 0) *reinterpret_cast<float2*>(cb + 4096 + (grp & 63) * 16) = float2{-c, -t};
+        } else {
+          if (ch == 0) *reinterpret_cast<float*>(cb + 4096 + (grp & 63) * 16) = -c;
+        }
+      };
+      if (ZP && perm != nullptr) {
+        // a layer with a row order: position k' takes x[perm[k']]; positions beyond K (the rest of the last chunk)
+        // are zeros.  Per round of 4 words a lane: the order (2 x 16 bytes per word), then 8 two-byte loads per
+        // word: two round trips.  (8 words a round, or the next round's order requested ahead, need more
+        // registers than the kernel's budget of 128 leaves: the compiler spilled 31 .. 158 of them.)
+        const __amdgpu_buffer_rsrc_t pr =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(perm), 0, K * 4, kBufferFlags);
+        constexpr int UP = 4;
+        uint4_t pa[UP], pb[UP];
+        auto load_order = [&](int base) {
+#pragma unroll
+          for (int u = 0; u < UP; ++u) {
+            const int wi = base + u * 64 + lane;
+            pa[u] = __builtin_amdgcn_raw_buffer_load_b128(pr, wi * 32, 0, 0);  // (beyond K: zeros)
+            pb[u] = __builtin_amdgcn_raw_buffer_load_b128(pr, wi * 32 + 16, 0, 0);
+          }
+        };
+        for (int base = 0; base < nwords; base += 64 * UP) {
+          load_order(base);
+          half2_t h[UP][4];
+#pragma unroll
+          for (int u = 0; u < UP; ++u) {
+            const uint32_t idx[8] = {pa[u].x, pa[u].y, pa[u].z, pa[u].w, pb[u].x, pb[u].y, pb[u].z, pb[u].w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const uint16_t bits = dep >= 0 ? (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(xr, (int)(idx[e] * 2u), 0, kDeviceScope)
+                                             : (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(xr, (int)(idx[e] * 2u), 0, 0);
+              if (e & 1) h[u][e >> 1].y = as_half(bits);
+              else h[u][e >> 1].x = as_half(bits);
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < UP; ++u) {
+            const int wi = base + u * 64 + lane;
+            if (wi < nwords) {  // a quad of lanes (one group) is in or out together
+              const bool in_row = wi * 8 < K;
+              const uint4_t w8 = {in_row ? as_u32(h[u][0]) : 0u, in_row ? as_u32(h[u][1]) : 0u,
+                                  in_row ? as_u32(h[u][2]) : 0u, in_row ? as_u32(h[u][3]) : 0u};
+              stage(wi, w8);
+            }
+          }
+        }
+      } else {
       constexpr int U = 16;       // loads in flight per lane: one round trip per 16 KiB of x
       for (int base = 0; base < nwords; base += 64 * U) {
         uint4_t v[U];
@@ -472,33 +544,9 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const int wi = base + u * 64 + lane;
-          if (wi < nwords) {  // a quad of lanes (one group) is in or out together
-            const uint32_t in[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
-            uint32_t o[4];
-            pair_i_i4(in, o);  // o[i] = (x_i, x_{i+4})
-            float c = dot2(as_half2(o[0]), k1031, 0.0f);
-            c = dot2(as_half2(o[1]), k71, c);
-            c = dot2(as_half2(o[2]), k1031, c);
-            c = dot2(as_half2(o[3]), k71, c);
-            c += dpp_shift<0xb1, 0xf>(c);  // the 4 words of a group sit in 4 adjacent lanes
-            c += dpp_shift<0x4e, 0xf>(c);
-            const int grp = wi >> 2, ch = wi & 3;
-            char* cb = xb + (grp >> 6) * kChunkBytes;
-            *reinterpret_cast<uint4_t*>(cb + ch * 1024 + (grp & 63) * 16) =
-                uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
-            if constexpr (ZP) {  // the zero point multiplies the plain sum of the group's activations
-              float t = dot2(as_half2(o[0]), ones, 0.0f);
-              t = dot2(as_half2(o[1]), ones, t);
-              t = dot2(as_half2(o[2]), ones, t);
-              t = dot2(as_half2(o[3]), ones, t);
-              t += dpp_shift<0xb1, 0xf>(t);
-              t += dpp_shift<0x4e, 0xf>(t);
-              if (ch == 0) *reinterpret_cast<float2*>(cb + 4096 + (grp & 63) * 16) = float2{-c, -t};
-            } else {
-              if (ch == 0) *reinterpret_cast<float*>(cb + 4096 + (grp & 63) * 16) = -c;
-            }
-          }
+          if (wi < nwords) stage(wi, v[u]);  // a quad of lanes (one group) is in or out together
         }
+      }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       if (lane == 0) __hip_atomic_store(&flags->x_ready[j & (kYSlots - 1)], j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -600,13 +648,13 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
 namespace wq {
 // szl == nullptr: format A.  Else the linears are prepared AutoGPTQ layers: d[i].S is SZ and szl[i] the log2 of
 // the 32-column groups per (scale, zero point) pair.
-static wq_gemv_list_t* gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, int n, int M, void* workspace,
-                                        size_t workspace_bytes, hipStream_t stream);
+static wq_gemv_list_t* gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, const int32_t* const* perm, int n,
+                                        int M, void* workspace, size_t workspace_bytes, hipStream_t stream);
 }  // namespace wq
 
 extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv_desc* d, int n, int M, void* workspace,
                                                              size_t workspace_bytes, wq_stream_t stream) {
-  return wq::gemv_list_create(d, nullptr, n, M, workspace, workspace_bytes, (hipStream_t)stream);
+  return wq::gemv_list_create(d, nullptr, nullptr, n, M, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* d, int n, void* workspace,
@@ -617,6 +665,7 @@ extern "C" wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* d, 
     return bad(WQ_EINVAL, "wq_gptq_gemv_list_create: need 1 .. %d linears, got %d", WQ_GEMV_LIST_MAX, n);
   std::vector<wq_q4g32_gemv_desc> e(n);
   std::vector<uint8_t> szl(n);
+  std::vector<const int32_t*> perm(n);
   for (int i = 0; i < n; ++i) {
     const wq_gptq_gemv_desc& s = d[i];
     // a pair serves 32 << szl columns of a row; a chunk of 64 x 32 columns must hold whole pairs' worth of lanes
@@ -631,13 +680,16 @@ extern "C" wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* d, 
       return bad(WQ_EINVAL, "wq_gptq_gemv_list_create: linear %d: SZ must be 4-byte aligned", i);
     e[i] = wq_q4g32_gemv_desc{s.W_nk, s.SZ, s.x, s.bias, s.residual, s.y, s.N, s.K};
     szl[i] = (uint8_t)lg;
+    if (s.perm && !aligned16(s.perm))
+      return bad(WQ_EINVAL, "wq_gptq_gemv_list_create: linear %d: perm must be 16-byte aligned", i);
+    perm[i] = s.perm;
   }
-  return gemv_list_create(e.data(), szl.data(), n, 1, workspace, workspace_bytes, (hipStream_t)stream);
+  return gemv_list_create(e.data(), szl.data(), perm.data(), n, 1, workspace, workspace_bytes, (hipStream_t)stream);
 #undef bad
 }
 
-static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, int n, int M, void* workspace,
-                                            size_t workspace_bytes, hipStream_t stream) {
+static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, const int32_t* const* perm,
+                                            int n, int M, void* workspace, size_t workspace_bytes, hipStream_t stream) {
 #define bad(code, ...) ((void)fail(code, __VA_ARGS__), (wq_gemv_list_t*)nullptr)
   if (M < 1 || M > WQ_GEMV_LIST_MAX_M)
     return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: 1 .. %d rows of activations, got %d", WQ_GEMV_LIST_MAX_M, M);
@@ -685,6 +737,7 @@ static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const u
     g.off = 0;
     g.rows = (uint8_t)rows[i];
     g.szl = szl ? szl[i] : 0;
+    g.perm = perm ? perm[i] : nullptr;
     cmax = std::max(cmax, (int)((s.K / 32 + 63) / 64));
   }
   // Who reads what an earlier linear of the list wrote.  Writing over something an earlier linear

@@ -520,7 +520,7 @@ def gptq_workspace_bytes(M: int, K: int, has_perm: bool) -> int:
 
 class GptqGemvDesc(ctypes.Structure):
     """``wq_gptq_gemv_desc`` of include/relax_amd_wq.h."""
-    _fields_ = [("W_nk", ctypes.c_void_p), ("SZ", ctypes.c_void_p), ("x", ctypes.c_void_p), ("bias", ctypes.c_void_p),
+    _fields_ = [("W_nk", ctypes.c_void_p), ("SZ", ctypes.c_void_p), ("perm", ctypes.c_void_p), ("x", ctypes.c_void_p), ("bias", ctypes.c_void_p),
                 ("residual", ctypes.c_void_p), ("y", ctypes.c_void_p), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
                 ("G", ctypes.c_int64)]
 
@@ -530,7 +530,7 @@ class GptqGemvList(Q4G32GemvList):
     poll, info as :class:`Q4G32GemvList`).
 
     ``linears``: sequence of ``(w, x, y)`` or ``(w, x, y, bias, residual)`` with ``w`` a :class:`GptqWeight` from
-    :func:`gptq_prepare` whose rows were already in group order (``w.perm is None``)."""
+    :func:`gptq_prepare` (with or without a row order; not :func:`gptq_prepare_padded`)."""
 
     def __init__(self, linears):
         self._l = _lib.lib()
@@ -541,8 +541,8 @@ class GptqGemvList(Q4G32GemvList):
             w, x, y = lin[:3]
             bias = lin[3] if len(lin) > 3 else None
             residual = lin[4] if len(lin) > 4 else None
-            if w.perm is not None or getattr(w, "K_padded", 0):
-                raise ValueError(f"linear {i}: a layer whose activations must be gathered cannot be a member of a list")
+            if getattr(w, "K_padded", 0):
+                raise ValueError(f"linear {i}: a layer prepared with padded groups cannot be a member of a list")
             x = _dev(x, torch.float16, "x")
             y = _dev(y, torch.float16, "y")
             if x.numel() != w.K or y.numel() != w.N:
@@ -550,7 +550,7 @@ class GptqGemvList(Q4G32GemvList):
             for t, name in ((bias, "bias"), (residual, "residual")):
                 if t is not None and _dev(t, torch.float16, name).numel() != w.N:
                     raise ValueError(f"linear {i}: {name} must hold {w.N} elements")
-            arr[i] = GptqGemvDesc(_ptr(w.W_nk), _ptr(w.SZ), _ptr(x), _ptr(bias), _ptr(residual), _ptr(y), w.N, w.K, w.G)
+            arr[i] = GptqGemvDesc(_ptr(w.W_nk), _ptr(w.SZ), _ptr(w.perm), _ptr(x), _ptr(bias), _ptr(residual), _ptr(y), w.N, w.K, w.G)
             self._keep.append((w, x, y, bias, residual))
         need = self._l.wq_q4g32_gemv_list_workspace_bytes(n)
         self._workspace = torch.zeros(max(int(need), 256), dtype=torch.uint8, device="cuda")

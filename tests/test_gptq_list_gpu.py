@@ -17,11 +17,11 @@ def env():
     return ops, gpu_util, torch
 
 
-def _layer(oracle, ops, u, N, K, gs, seed, shrink=1.0):
-    x, qw, qz, s, g_idx = oracle.make_gptq_inputs(1, N, K, gs, seed=seed)
+def _layer(oracle, ops, u, N, K, gs, seed, shrink=1.0, act_order=False):
+    x, qw, qz, s, g_idx = oracle.make_gptq_inputs(1, N, K, gs, seed=seed, act_order=act_order)
     s = (s.astype(np.float32) * shrink).astype(np.float16)
     w = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
-    assert w.perm is None
+    assert (w.perm is not None) == act_order
     B = oracle.gptq_dequant(qw, qz, s, g_idx)  # fp16 [K, N]
     return dict(w=w, x=x, Bt=np.ascontiguousarray(B.T), N=N, K=K, gs=gs)
 
@@ -37,11 +37,14 @@ SHAPES = [(4096, 4096, 128), (12288, 4096, 128), (4096, 11008, 128), (8, 32, 32)
           (520, 4096, 2048), (96, 2048, 2048), (600, 28672, 128), (16, 32768, 32), (200, 4224, 128), (88, 1024, 1024)]
 
 
-def test_independent_layers_match_oracle_and_call_by_call(env, oracle):
+@pytest.mark.parametrize("act_order", [False, True])
+def test_independent_layers_match_oracle_and_call_by_call(env, oracle, act_order):
+    """With ``act_order`` every layer but each third has a row order (a random assignment of the rows to the groups,
+    what AutoGPTQ's desc_act leaves): its activations are gathered while they are staged."""
     ops, u, torch = env
     lins = []
     for i, (N, K, gs) in enumerate(SHAPES):
-        l = _layer(oracle, ops, u, N, K, gs, seed=300 + i)
+        l = _layer(oracle, ops, u, N, K, gs, seed=300 + i, act_order=act_order and i % 3 != 2 and K > gs)
         l["dx"] = u.dev(l["x"])
         l["y"] = torch.zeros((1, N), dtype=torch.float16, device="cuda")
         lins.append(l)
@@ -67,8 +70,8 @@ def test_independent_layers_match_oracle_and_call_by_call(env, oracle):
 def test_epilogue_and_one_hot(env, oracle):
     ops, u, torch = env
     rng = np.random.default_rng(3)
-    for N, K, gs in [(520, 1024, 128), (264, 4224, 64)]:
-        l = _layer(oracle, ops, u, N, K, gs, seed=7)
+    for N, K, gs, act in [(520, 1024, 128, False), (264, 4224, 64, False), (264, 4224, 64, True), (72, 2048, 32, True)]:
+        l = _layer(oracle, ops, u, N, K, gs, seed=7, act_order=act)
         bias = rng.standard_normal(N).astype(np.float16)
         res = rng.standard_normal((1, N)).astype(np.float16)
         y = torch.zeros((1, N), dtype=torch.float16, device="cuda")
@@ -83,20 +86,21 @@ def test_epilogue_and_one_hot(env, oracle):
         u.assert_close(u.host(y), _ref(oracle, l, l["x"], bias, res), "gptq list epilogue")
         # a one-hot x selects a dequantized row of the [K, N] weight exactly
         for k, _, yh in hot:
-            assert np.array_equal(u.host(yh)[0].view(np.uint16), l["Bt"][:, k].view(np.uint16)), (N, K, gs, k)
+            assert np.array_equal(u.host(yh)[0].view(np.uint16), l["Bt"][:, k].view(np.uint16)), (N, K, gs, act, k)
 
 
-def test_decoder_layer_chain(env, oracle):
+@pytest.mark.parametrize("act_order", [False, True])
+def test_decoder_layer_chain(env, oracle, act_order):
     """The four linears of a Llama-2-7B decoder layer at group size 128, each fed by the one in front (qkv -> o
     takes the first 4096 of qkv's outputs, gate/up -> down the first 11008), eager and as a replayed HIP graph.
     (Scales a twentieth of the generator's: its weights have mean -scale, which a chain of four would amplify
-    beyond fp16.)"""
+    beyond fp16.)  With ``act_order`` the consumers gather what their producers wrote."""
     ops, u, torch = env
     rng = np.random.default_rng(11)
-    qkv = _layer(oracle, ops, u, 12288, 4096, 128, seed=1, shrink=0.05)
-    o = _layer(oracle, ops, u, 4096, 4096, 128, seed=2, shrink=0.05)
-    gu = _layer(oracle, ops, u, 22016, 4096, 128, seed=3, shrink=0.05)
-    down = _layer(oracle, ops, u, 4096, 11008, 128, seed=4, shrink=0.05)
+    qkv = _layer(oracle, ops, u, 12288, 4096, 128, seed=1, shrink=0.05, act_order=act_order)
+    o = _layer(oracle, ops, u, 4096, 4096, 128, seed=2, shrink=0.05, act_order=act_order)
+    gu = _layer(oracle, ops, u, 22016, 4096, 128, seed=3, shrink=0.05, act_order=act_order)
+    down = _layer(oracle, ops, u, 4096, 11008, 128, seed=4, shrink=0.05, act_order=act_order)
     x0 = rng.standard_normal((1, 4096)).astype(np.float16)
     res = rng.standard_normal((1, 4096)).astype(np.float16)
     t = [torch.zeros((1, n), dtype=torch.float16, device="cuda") for n in (12288, 4096, 22016, 4096)]
@@ -144,8 +148,7 @@ def test_what_the_list_refuses(env, oracle):
     y = torch.zeros((1, 64), dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.WqError, match="group size"):
         ops.GptqGemvList([(w, u.dev(x), y)])
-    x, qw, qz, s, g_idx = oracle.make_gptq_inputs(1, 64, 256, 64, seed=6, act_order=True)
-    w = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
-    assert w.perm is not None
-    with pytest.raises(ValueError, match="gathered"):
+    g_idx = np.random.default_rng(1).integers(0, 2, size=192).astype(np.int32)  # groups of unequal size
+    w = ops.gptq_prepare_padded(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
+    with pytest.raises(ValueError, match="padded"):
         ops.GptqGemvList([(w, u.dev(x), y)])
