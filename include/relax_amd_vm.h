@@ -84,7 +84,10 @@ int wq_program_num_instructions(const wq_program_t* p);
  * linears; K % 256 == 0 where M > 1) is executed as ONE launch of the list kernel if it is long
  * enough for that to be the faster way: 2 instructions at M <= 4, 8 at M <= 8, 16 at M <= 16, 8 beyond
  * (a short list with several rows of x cannot spread the loads of the activations over small groups
- * of workgroups).  The list kernel is wq_q4g32_gemv_list_* of relax_amd_wq.h; one kernel per
+ * of workgroups).  A run of relax_amd.autogptq_matmul instructions with one row of x and a group size of
+ * 32 << t (t = 0 .. 6), with or without a row order, is fused the same way from 2 instructions on
+ * (wq_gptq_gemv_list_create; a gather workspace argument is then not used); the two kinds do not share a run.
+ * The list kernel is wq_q4g32_gemv_list_* of relax_amd_wq.h; one kernel per
  * instruction is what the reference's VM does with the generated kernels
  * of python/tvm/dlight/gpu/gemv.py.  Inside such a run, independent linears are moved between a
  * producer and its consumer (results are unchanged: every true, anti and output dependence

@@ -39,8 +39,9 @@ struct Instr {
   std::vector<int> regs;  // register per argument, -1 for an immediate
 };
 
-// A run of consecutive decode linears (relax_amd.q4f16_1_matmul*, one row of x each) that is
-// executed as ONE launch of the list kernel (wq_q4g32_gemv_list_*).
+// A run of consecutive decode linears (relax_amd.q4f16_1_matmul*, a few rows of x each, or
+// relax_amd.autogptq_matmul with one row) that is executed as ONE launch of the list kernel
+// (wq_q4g32_gemv_list_* / wq_gptq_gemv_list_create).
 struct FusedGroup {
   int first = 0, last = 0;     // instruction indices, inclusive
   std::vector<int> order;      // the order the list kernel walks them in
@@ -50,11 +51,14 @@ struct FusedGroup {
   std::string why;             // ... and what wq_q4g32_gemv_list_create said
 };
 
-// What a q4f16_1_matmul* instruction reads and writes, if it qualifies for a fused group.
+// What a q4f16_1_matmul* or autogptq_matmul instruction reads and writes, if it qualifies for a fused group.
 struct DecodeLinear {
   int W, S, x, bias, residual, y;  // registers; bias / residual -1 when absent
   int64_t N, K;
   int64_t M;  // rows of x: 1 .. WQ_GEMV_LIST_MAX_M
+  bool gptq = false;  // a prepared AutoGPTQ layer: S is SZ [N, G, 2], perm its row order (-1: none)
+  int perm = -1;
+  int64_t G = 0;
 };
 
 }  // namespace
@@ -225,12 +229,8 @@ static bool as_decode_linear(const wq_program* p, const Instr& in, DecodeLinear*
   int kind = -1;
   for (int k = 0; k < 3; ++k)
     if (in.name == names[k][0] || in.name == names[k][1]) kind = k;
-  if (kind < 0 || (int)in.regs.size() != 4 + kind) return false;
   for (size_t i = 0; i < in.regs.size(); ++i)
     if (in.regs[i] < 0 && !(in.codes[i] == kTVMNullptr)) return false;
-  DecodeLinear d{in.regs[0], in.regs[1], in.regs[2], kind >= 1 ? in.regs[3] : -1, kind >= 2 ? in.regs[4] : -1,
-                 in.regs[3 + kind], 0, 0, 0};
-  if (d.W < 0 || d.S < 0 || d.x < 0 || d.y < 0 || (kind >= 1 && d.bias < 0) || (kind >= 2 && d.residual < 0)) return false;
   auto numel = [&](int r) {
     int64_t n = 1;
     for (int64_t e : p->regs[r].shape) n *= e;
@@ -240,6 +240,33 @@ static bool as_decode_linear(const wq_program* p, const Instr& in, DecodeLinear*
     const DLTensor& t = p->regs[r].dl;
     return t.dtype.code == code && t.dtype.bits == bits && t.device.device_type == kDLROCM;
   };
+  if (in.name == "relax_amd.autogptq_matmul" || in.name == "relax_amd_autogptq_matmul") {
+    // (W_nk, SZ, perm | null, x, residual | null, out [, workspace]); one row of x, group size 32 << t
+    if (in.regs.size() != 6 && in.regs.size() != 7) return false;
+    DecodeLinear d{in.regs[0], in.regs[1], in.regs[3], -1, in.regs[4], in.regs[5], 0, 0, 1};
+    d.gptq = true;
+    d.perm = in.regs[2];
+    if (d.W < 0 || d.S < 0 || d.x < 0 || d.y < 0) return false;
+    const Reg &W = p->regs[d.W], &SZ = p->regs[d.S];
+    if (!is(d.W, kDLUInt, 32) || !is(d.S, kDLFloat, 16) || !is(d.x, kDLFloat, 16) || !is(d.y, kDLFloat, 16)) return false;
+    if (W.shape.size() != 2 || SZ.shape.size() != 3 || SZ.shape[2] != 2 || SZ.shape[0] != W.shape[0]) return false;
+    d.N = W.shape[0];
+    d.K = W.shape[1] * 8;
+    d.G = SZ.shape[1];
+    if (d.N <= 0 || d.K <= 0 || d.K > WQ_GEMV_LIST_MAX_K || d.G <= 0 || d.K % d.G != 0) return false;
+    bool size_ok = false;
+    for (int t = 0; t <= 6; ++t) size_ok = size_ok || d.K / d.G == (32ll << t);
+    if (!size_ok) return false;
+    if (numel(d.x) != d.K || numel(d.y) != d.N) return false;
+    if (d.perm >= 0 && (!is(d.perm, kDLInt, 32) || numel(d.perm) != d.K)) return false;
+    if (d.residual >= 0 && (!is(d.residual, kDLFloat, 16) || numel(d.residual) != d.N)) return false;
+    *out = d;
+    return true;
+  }
+  if (kind < 0 || (int)in.regs.size() != 4 + kind) return false;
+  DecodeLinear d{in.regs[0], in.regs[1], in.regs[2], kind >= 1 ? in.regs[3] : -1, kind >= 2 ? in.regs[4] : -1,
+                 in.regs[3 + kind], 0, 0, 0};
+  if (d.W < 0 || d.S < 0 || d.x < 0 || d.y < 0 || (kind >= 1 && d.bias < 0) || (kind >= 2 && d.residual < 0)) return false;
   const Reg &W = p->regs[d.W], &S = p->regs[d.S];
   if (!is(d.W, kDLUInt, 32) || !is(d.S, kDLFloat, 16) || !is(d.x, kDLFloat, 16) || !is(d.y, kDLFloat, 16)) return false;
   if (W.shape.size() != 2 || S.shape.size() != 2) return false;
@@ -336,7 +363,7 @@ static void find_groups(wq_program* p) {
     DecodeLinear d;
     int j = i;
     while (j < n && (int)lin.size() < WQ_GEMV_LIST_MAX && as_decode_linear(p, p->instrs[j], &d) &&
-           (lin.empty() || d.M == lin[0].M)) {  // one list, one batch size
+           (lin.empty() || (d.M == lin[0].M && d.gptq == lin[0].gptq))) {  // one list, one batch size, one weight format
       // The list kernel orders a linear behind ONE earlier linear, through its x.  A bias or a residual that an
       // earlier linear of the run writes (the residual stream: down_proj adds what o_proj produced) is refused
       // by wq_q4g32_gemv_list_create: the run ends in front of such an instruction, which starts the next one.
@@ -462,18 +489,27 @@ static int build_lists(wq_program* p, hipStream_t stream) {
   for (FusedGroup& g : p->groups) {
     if (g.list || g.failed) continue;
     std::vector<wq_q4g32_gemv_desc> descs;
+    std::vector<wq_gptq_gemv_desc> gptq_descs;
     int64_t rows = 1;
     for (int k : g.order) {
       DecodeLinear d;
       if (!as_decode_linear(p, p->instrs[k], &d)) return wq::fail(WQ_EINVAL, "instruction %d no longer qualifies for its fused group", k);
       auto ptr = [&](int r) { return r < 0 ? nullptr : static_cast<char*>(p->regs[r].dl.data) + p->regs[r].dl.byte_offset; };
-      descs.push_back({(const uint32_t*)ptr(d.W), (const uint16_t*)ptr(d.S), (const uint16_t*)ptr(d.x),
-                       (const uint16_t*)ptr(d.bias), (const uint16_t*)ptr(d.residual), (uint16_t*)ptr(d.y), d.N, d.K});
+      if (d.gptq)
+        gptq_descs.push_back({(const uint32_t*)ptr(d.W), (const uint16_t*)ptr(d.S), (const int32_t*)ptr(d.perm),
+                              (const uint16_t*)ptr(d.x), nullptr, (const uint16_t*)ptr(d.residual), (uint16_t*)ptr(d.y),
+                              d.N, d.K, d.G});
+      else
+        descs.push_back({(const uint32_t*)ptr(d.W), (const uint16_t*)ptr(d.S), (const uint16_t*)ptr(d.x),
+                         (const uint16_t*)ptr(d.bias), (const uint16_t*)ptr(d.residual), (uint16_t*)ptr(d.y), d.N, d.K});
       rows = d.M;
     }
     char* ws = static_cast<char*>(p->workspace) + g.ws_offset;
-    g.list = wq_q4g32_gemv_list_create_batched(descs.data(), (int)descs.size(), (int)rows, ws,
-                                               wq_q4g32_gemv_list_workspace_bytes((int)descs.size()), stream);
+    const int count = (int)(descs.size() + gptq_descs.size());
+    g.list = !gptq_descs.empty()
+                 ? wq_gptq_gemv_list_create(gptq_descs.data(), count, ws, wq_q4g32_gemv_list_workspace_bytes(count), stream)
+                 : wq_q4g32_gemv_list_create_batched(descs.data(), count, (int)rows, ws,
+                                                     wq_q4g32_gemv_list_workspace_bytes(count), stream);
     // operands that alias in a way the list kernel cannot order (or pointers it cannot take): the
     // group runs instruction by instruction, which is always valid
     if (!g.list) {

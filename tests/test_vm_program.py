@@ -201,6 +201,55 @@ def test_a_residual_from_the_run_ends_the_fused_run():
         l.wq_program_destroy(p)
 
 
+def test_runs_of_autogptq_decode_linears_are_fused_apart_from_q4f16_1_runs():
+    """Planning alone: relax_amd.autogptq_matmul with one row of x and a group size of 32 << t joins a run of its
+    own kind (with or without a row order, with or without the gather workspace argument); a q4f16_1 linear, a
+    group size of 96 or a second row of x ends the run."""
+    l = _lib()
+    p = l.wq_program_create()
+    try:
+        addr = [0x100000]
+
+        def ext(code, bits, *shape):
+            addr[0] += 0x100000
+            return l.wq_program_add_external(p, code, bits, len(shape), _shape(*shape), addr[0], 10)
+
+        def call(name, args):  # None: a null handle
+            n = len(args)
+            vals = (ctypes.c_int64 * n)(*[0 if a is None else a for a in args])
+            kinds = (ctypes.c_int * n)(*[2 if a is None else 1 for a in args])
+            return l.wq_program_add_call(p, name.encode(), n, vals, kinds)
+
+        K, N = 768, 64
+        x, x2, ws = ext(2, 16, 1, K), ext(2, 16, 2, K), ext(1, 8, 2 * K)
+        perm = ext(0, 32, K)
+
+        def gptq(G, xr=None, with_perm=False, with_ws=False, rows=1):
+            W, SZ, y = ext(1, 32, N, K // 8), ext(2, 16, N, G, 2), ext(2, 16, rows, N)
+            args = [W, SZ, perm if with_perm else None, x if xr is None else xr, None, y] + ([ws] if with_ws else [])
+            assert call("relax_amd.autogptq_matmul", args) == 0
+
+        gptq(6)                                   # 0: group size 128
+        gptq(24, with_perm=True, with_ws=True)    # 1: group size 32, a row order
+        gptq(3, with_ws=True)                     # 2: group size 256
+        W, S, y = ext(1, 32, N, K // 8), ext(2, 16, N, K // 32), ext(2, 16, 1, N)
+        assert call("relax_amd.q4f16_1_matmul", [W, S, x, y]) == 0   # 3
+        W, S, y = ext(1, 32, N, K // 8), ext(2, 16, N, K // 32), ext(2, 16, 1, N)
+        assert call("relax_amd.q4f16_1_matmul", [W, S, x, y]) == 0   # 4
+        gptq(6)                                   # 5
+        gptq(8)                                   # 6: group size 96: call by call
+        gptq(6)                                   # 7
+        gptq(6, xr=x2, rows=2)                    # 8: two rows: call by call
+        gptq(6)                                   # 9 (a run of one is not fused)
+        assert l.wq_program_plan(p) > 0
+        buf = (ctypes.c_int * 8)()
+        assert l.wq_program_fused_order(p, 0, buf, 8) == 3 and sorted(buf[:3]) == [0, 1, 2]
+        assert l.wq_program_fused_order(p, 1, buf, 8) == 2 and sorted(buf[:2]) == [3, 4]
+        assert l.wq_program_fused_order(p, 2, buf, 8) < 0  # no third run
+    finally:
+        l.wq_program_destroy(p)
+
+
 def test_options_and_a_program_of_external_tensors_only_needs_its_workspace():
     l = _lib()
     p = l.wq_program_create()
@@ -540,3 +589,75 @@ def test_autogptq_layer_in_a_program(oracle):
         p.replay(stream)
         torch.cuda.synchronize()
         assert torch.equal(y2, keep)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("act_order", [False, True])
+def test_autogptq_decoder_layer_is_one_launch(oracle, act_order):
+    """The four linears of a decoder layer as AutoGPTQ layers at M = 1 (o and down add the residual stream, which
+    comes from outside the run): the program runs them as ONE launch of the list kernel, with the same results as
+    the calls one by one, eager and replayed; the gather workspaces of the calls are simply not used."""
+    import torch
+
+    from relax_amd import ops, vm
+    from tests import gpu_util as u
+
+    shapes = [(1536, 512), (512, 512), (2752, 512), (512, 1376 + 32)]  # (N, K); the last K: a partial chunk
+    gs = 32
+    rng = np.random.default_rng(9)
+    layers = []
+    for i, (N, K) in enumerate(shapes):
+        _, qw, qz, s, g_idx = oracle.make_gptq_inputs(1, N, K, gs, seed=40 + i, act_order=act_order)
+        s = (s.astype(np.float32) * 0.2).astype(np.float16)
+        w = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
+        layers.append((w, np.ascontiguousarray(oracle.gptq_dequant(qw, qz, s, g_idx).T)))
+    x0 = rng.standard_normal((1, 512)).astype(np.float16)
+    res = rng.standard_normal((1, 512)).astype(np.float16)
+    attn = rng.standard_normal((1, 512)).astype(np.float16)
+    act = rng.standard_normal((1, 1408)).astype(np.float16)
+
+    def build(fuse):
+        p = vm.DpsProgram()
+        p.set_option("fuse_decode", fuse)
+        regs = []
+        for w, _ in layers:
+            regs.append((p.external(w.W_nk, as_uint32=True), p.external(w.SZ),
+                         p.external(w.perm) if w.perm is not None else None))
+        X0, R, A, C = p.external(u.dev(x0)), p.external(u.dev(res)), p.external(u.dev(attn)), p.external(u.dev(act))
+        outs = [torch.zeros((1, n), dtype=torch.float16, device="cuda") for n, _ in shapes]
+        O = [p.external(o) for o in outs]
+        ws = [p.planned((max(16, ops.gptq_workspace_bytes(1, k, True)),), torch.uint8) for _, k in shapes]
+        p.call("relax_amd.autogptq_matmul", *regs[0], X0, None, O[0], ws[0])   # qkv
+        p.call("relax_amd.autogptq_matmul", *regs[1], A, R, O[1], ws[1])       # o + residual
+        p.call("relax_amd.autogptq_matmul", *regs[2], O[1], None, O[2], ws[2])  # gate/up, fed by o
+        p.call("relax_amd.autogptq_matmul", *regs[3], C, R, O[3], ws[3])       # down + residual
+        p.plan()
+        return p, outs
+
+    fused, got = build(1)
+    assert sorted(fused.fused_order(0)) == [0, 1, 2, 3]
+    plain, want = build(0)
+    print("autogptq decoder layer as one launch", flush=True)
+    fused.run()
+    plain.run()
+    torch.cuda.synchronize()
+    assert fused.num_fused_groups == 1 and plain.num_fused_groups == 0  # (lists are built by the first run)
+    fused.status()
+    r1 = oracle.nt_matmul_f32acc(layers[1][1], attn, None, res)
+    refs = [oracle.nt_matmul_f32acc(layers[0][1], x0), r1, oracle.nt_matmul_f32acc(layers[2][1], r1),
+            oracle.nt_matmul_f32acc(layers[3][1], act, None, res)]
+    for g, w, r, name in zip(got, want, refs, ("qkv", "o", "gate_up", "down")):
+        u.assert_close(u.host(g), r, f"fused autogptq {name}")
+        u.assert_close(u.host(g), u.host(w), f"fused against call by call, {name}")
+    keep = [g.clone() for g in got]
+    stream = torch.cuda.Stream()
+    fused.capture(stream)
+    for _ in range(3):
+        for g in got:
+            g.zero_()
+        torch.cuda.synchronize()
+        fused.replay(stream)
+        torch.cuda.synchronize()
+        for g, k in zip(got, keep):
+            assert torch.equal(g, k)
+    fused.status()
