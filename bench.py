@@ -208,7 +208,29 @@ def bench_f16acc(torch, ops, stream, copies, xs):
                     "us_min": round(sp1["min"] * 1e3 / (4 * len(copies)), 3),
                     "us_max": round(sp1["max"] * 1e3 / (4 * len(copies)), 3)})
         del g1
-    return {"kernel": "q4g32_gemv_f16acc_kernel (wq_q4g32_gemv_f16acc)", "bound": "hbm", "M": 1, "shapes": res}
+    # four rows of x in one pass over the weights (the low-batch case), on the largest of the four linears
+    N, K = DECODE_SHAPES[2]
+    x4 = torch.randn((4, K), device="cuda", dtype=torch.float16)
+
+    def four(i):
+        W, S = copies[i % len(copies)][2]
+        ops.q4g32_gemv_f16acc(W, S, x4)
+
+    for i in range(len(copies)):
+        four(i)
+    stream.synchronize()
+    g4 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g4, stream=stream):
+        for i in range(4 * len(copies)):
+            four(i)
+    ms4, _ = _measure(torch, stream, g4.replay, min_ms=MIN_SAMPLE_MS / 4)
+    us4 = ms4 * 1e3 / (4 * len(copies))
+    nb4 = gemv_bytes(4, N, K)
+    batch = {"M": 4, "N": N, "K": K, "us": round(us4, 3), "GB/s": round(nb4 / us4 / 1e3, 1),
+             "frac_of_hbm_peak": round(nb4 / us4 / 1e3 / HBM_PEAK_GBS, 4), "bytes": nb4}
+    del g4
+    return {"kernel": "q4g32_gemv_f16acc_kernel (wq_q4g32_gemv_f16acc)", "bound": "hbm", "M": 1, "shapes": res,
+            "four_rows_one_pass": batch}
 
 
 def bench_stack(torch, layers=32, batches=(1, 8, 16, 32)):

@@ -100,8 +100,10 @@ int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x, const
 /* The decode GEMV with the reference's fp16 accumulation (tests/python/dlight/test_gpu_reduction.py:44-51,
  * test_gpu_gemv.py:199-206: `NT_matmul += x * decode`, everything fp16): every product and every partial
  * sum is rounded to fp16.  The order of the sum is free in the reference (its schedules reorder it) and a
- * tree here, so results agree with a sequential fp16 sum only within fp16 accumulation error.  x fp16 [M, K]
- * (rows one launch each), y fp16 [M, N]; no epilogue.  wq_q4g32_linear accumulates in fp32 instead. */
+ * tree here, so results agree with a sequential fp16 sum only within fp16 accumulation error.  x fp16 [M, K],
+ * y fp16 [M, N]; no epilogue.  Up to 4 rows of x share one pass over the weights (the dynamic batch of
+ * tests/python/dlight/test_gpu_low_batch_gemv.py:29-57); every row is summed in the order it has alone, so the
+ * result of a row does not depend on M.  wq_q4g32_linear accumulates in fp32 instead. */
 int wq_q4g32_gemv_f16acc(const uint32_t* W, const uint16_t* S, const uint16_t* x, uint16_t* y, int64_t M,
                          int64_t N, int64_t K, wq_stream_t stream);
 

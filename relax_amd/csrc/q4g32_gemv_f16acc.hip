@@ -28,8 +28,10 @@ __device__ __forceinline__ half_t wave_sum_f16_to_lane63(half_t v) {
   return v;
 }
 
-// One wavefront per ROWS consecutive rows; lane l takes the scale groups l, l + 64, ...
-template <int ROWS>
+// One wavefront per ROWS consecutive rows of W; lane l takes the scale groups l, l + 64, ...  MB rows of x
+// (K apart; their outputs N apart) share one pass over the weights: every row of x keeps sums of its own, added
+// in the order of a launch with that row alone, so batching changes no bit of the result.
+template <int ROWS, int MB>
 __global__ __launch_bounds__(256) void q4g32_gemv_f16acc_kernel(const uint4_t* __restrict__ W,
                                                                 const half_t* __restrict__ S,
                                                                 const half_t* __restrict__ x,
@@ -39,9 +41,11 @@ __global__ __launch_bounds__(256) void q4g32_gemv_f16acc_kernel(const uint4_t* _
   const int n0 = wave * ROWS;
   if (n0 >= N) return;
   const int G = K >> 5;
-  half2_t acc[ROWS];
+  half2_t acc[MB][ROWS];
 #pragma unroll
-  for (int r = 0; r < ROWS; ++r) acc[r] = half2_t{(half_t)0.0f, (half_t)0.0f};
+  for (int m = 0; m < MB; ++m)
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) acc[m][r] = half2_t{(half_t)0.0f, (half_t)0.0f};
   // UNR scale groups per lane and row are requested before the first is multiplied (the order of the sums is
   // that of one group after the other)
   constexpr int UNR = 4;
@@ -63,13 +67,15 @@ __global__ __launch_bounds__(256) void q4g32_gemv_f16acc_kernel(const uint4_t* _
       const int g = g0 + 64 * j;
       if (g >= G) break;
       // the group's 32 activations in the (i, i+4) pairing of the unpack
-      uint32_t xp[4][4];
+      uint32_t xp[MB][4][4];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const uint4_t v = reinterpret_cast<const uint4_t*>(x)[g * 4 + c];
-        const uint32_t in[4] = {v.x, v.y, v.z, v.w};
-        pair_i_i4(in, xp[c]);
-      }
+      for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint4_t v = reinterpret_cast<const uint4_t*>(x + (int64_t)m * K)[g * 4 + c];
+          const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+          pair_i_i4(in, xp[m][c]);
+        }
 #pragma unroll
       for (int r = 0; r < ROWS; ++r) {
         const half2_t s2 = {sc[j][r], sc[j][r]};
@@ -79,21 +85,36 @@ __global__ __launch_bounds__(256) void q4g32_gemv_f16acc_kernel(const uint4_t* _
           half2_t d[4];
           q4_word_dequant(words[c], s2, d);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            // product rounded to fp16, then the sum rounded to fp16: two instructions on purpose
-            half2_t p;
-            asm("v_pk_mul_f16 %0, %1, %2" : "=v"(p) : "v"(d[i]), "v"(as_half2(xp[c][i])));
-            asm("v_pk_add_f16 %0, %1, %2" : "=v"(acc[r]) : "v"(acc[r]), "v"(p));
-          }
+          for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              // product rounded to fp16, then the sum rounded to fp16: two instructions on purpose
+              half2_t p;
+              asm("v_pk_mul_f16 %0, %1, %2" : "=v"(p) : "v"(d[i]), "v"(as_half2(xp[m][c][i])));
+              asm("v_pk_add_f16 %0, %1, %2" : "=v"(acc[m][r]) : "v"(acc[m][r]), "v"(p));
+            }
         }
       }
     }
   }
 #pragma unroll
-  for (int r = 0; r < ROWS; ++r) {
-    const half_t t = wave_sum_f16_to_lane63(acc[r].x + acc[r].y);
-    if (lane == 63 && n0 + r < N) y[n0 + r] = t;
-  }
+  for (int m = 0; m < MB; ++m)
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const half_t t = wave_sum_f16_to_lane63(acc[m][r].x + acc[m][r].y);
+      if (lane == 63 && n0 + r < N) y[(int64_t)m * N + n0 + r] = t;
+    }
+}
+
+template <int MB>
+static int launch_f16acc(const uint32_t* W, const uint16_t* S, const uint16_t* x, uint16_t* y, int64_t N, int64_t K,
+                         hipStream_t stream) {
+  constexpr int kRows = 2;
+  const int64_t waves = (N + kRows - 1) / kRows;
+  const unsigned blocks = (unsigned)((waves + 3) / 4);
+  WQ_LAUNCH("wq_q4g32_gemv_f16acc", (q4g32_gemv_f16acc_kernel<kRows, MB>), dim3(blocks), dim3(256), 0, stream,
+            (const uint4_t*)W, (const half_t*)S, (const half_t*)x, (half_t*)y, (int)N, (int)K);
+  return WQ_OK;
 }
 
 }  // namespace wq
@@ -109,11 +130,15 @@ extern "C" int wq_q4g32_gemv_f16acc(const uint32_t* W, const uint16_t* S, const 
   WQ_REQUIRE(W && S && x && y, "wq_q4g32_gemv_f16acc: null pointer");
   WQ_REQUIRE(aligned16(W) && aligned16(x), "wq_q4g32_gemv_f16acc: W and x must be 16-byte aligned");
   WQ_REQUIRE(N < (1ll << 30) && K < (1ll << 30) && M <= 65536, "wq_q4g32_gemv_f16acc: too large");
-  constexpr int kRows = 2;
-  const int64_t waves = (N + kRows - 1) / kRows;
-  const unsigned blocks = (unsigned)((waves + 3) / 4);
-  for (int64_t m = 0; m < M; ++m)  // rows of x one after the other: a decode entry point
-    WQ_LAUNCH("wq_q4g32_gemv_f16acc", q4g32_gemv_f16acc_kernel<kRows>, dim3(blocks), dim3(256), 0, stream,
-              (const uint4_t*)W, (const half_t*)S, (const half_t*)(x + m * K), (half_t*)(y + m * N), (int)N, (int)K);
+  // up to 4 rows of x per pass over the weights (the low-batch case of
+  // tests/python/dlight/test_gpu_low_batch_gemv.py:29-57); more rows: more passes
+  for (int64_t m = 0; m < M;) {
+    const int64_t mb = M - m >= 4 ? 4 : M - m >= 2 ? 2 : 1;
+    const int rc = mb == 4   ? launch_f16acc<4>(W, S, x + m * K, y + m * N, N, K, stream)
+                   : mb == 2 ? launch_f16acc<2>(W, S, x + m * K, y + m * N, N, K, stream)
+                             : launch_f16acc<1>(W, S, x + m * K, y + m * N, N, K, stream);
+    if (rc != WQ_OK) return rc;
+    m += mb;
+  }
   return WQ_OK;
 }

@@ -59,7 +59,9 @@ def kernel_order_model(B: np.ndarray, x: np.ndarray) -> np.ndarray:
 
 SHAPES = [(1, 8, 32), (1, 37, 64), (1, 64, 4096), (2, 129, 2048 + 32), (1, 256, 11008), (3, 5, 160),
           # the reference's low-batch fixture (test_gpu_low_batch_gemv.py:29-34: N = 4096, K = 28672, fp16 accumulation)
-          (1, 4096, 28672), (5, 64, 28672)]
+          (1, 4096, 28672), (5, 64, 28672),
+          # several rows of x in one pass over the weights (4, 4 + 2 + 1, 4 + 4): every row as if alone
+          (4, 300, 11008), (7, 37, 2048 + 32), (8, 64, 4096)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
