@@ -57,10 +57,10 @@ const char* wq_target_arch(void);
  *   tests/python/dlight/test_gpu_low_batch_gemv.py:30-57         (small batch)
  *   tests/python/dlight/test_gpu_matmul.py:378-401               (prefill: the EPILOGUE chain only, see below)
  * which the reference schedules with python/tvm/dlight/gpu/{gemv,low_batch_gemv,matmul}.py.
- * Not served: the weight layout of that prefill fixture itself.  Its decode block (test_gpu_matmul.py:366-377)
- * reads W[k, n/8] and S[k, n/32]: the codes are packed along N and a scale covers 32 consecutive n of one k, a
- * third scheme next to the two of the decode fixtures (rows of 32 k here, K-major words in wq_q4g32_kn_*).  Its
- * square 4096 x 4096 shape hides the difference; no entry point of this library takes it.
+ * The weight layout of that prefill fixture itself is a third scheme: its decode block
+ * (test_gpu_matmul.py:366-377) reads W[k, n/8] and S[k, n/32], i.e. the codes are packed along N and a scale
+ * covers 32 consecutive n of one k (rows of 32 k here, K-major words in wq_q4g32_kn_*); the square 4096 x 4096
+ * shape hides the difference.  The entry points below do not take it: wq_q4n32_prepare / wq_q4n32_linear do.
  * Requirements: K % 32 == 0; W, S rows 16-byte aligned (true for K % 32 == 0
  * and 16-byte aligned bases).
  * ------------------------------------------------------------------------- */
@@ -96,6 +96,23 @@ int wq_q4g32_gemv(const uint32_t* W, const uint16_t* S, const uint16_t* x, const
 int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x, const uint16_t* bias,
                   const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
                   wq_stream_t stream);
+
+/* q4f16_1 weights packed along N, the scheme of tests/python/dlight/test_gpu_matmul.py:352-401 (which the
+ * reference schedules with python/tvm/dlight/gpu/matmul.py):
+ *   W uint32 [K, N/8], S fp16 [K, N/32],  w[k, n] = (fp16((W[k, n/8] >> 4 (n % 8)) & 15) - 7) * S[k, n/32]
+ *   y[m, n] = residual[m, n] + fp16(sum_k x[m, k] w[k, n] + bias[n])     (:378-401; fp32 accumulation)
+ * prepare  a load-time rearrangement (no arithmetic): W_nk uint32 [N, K/8] holds the same codes with 8 consecutive k
+ *          of one column per word, ST fp16 [N/32, K] the same scales with those of a group of 32 columns contiguous
+ *          along k.  K % 8 == 0, N % 32 == 0.
+ * linear   the matrix-core GEMM over the prepared operands for any M (the fixture's dynamic n): every weight is
+ *          the reference's fp16 value bit for bit ((code - 7) is exact, the product rounds once).  K % 64 == 0,
+ *          N % 32 == 0; bias fp16 [N] / residual fp16 [M, N] may be NULL.
+ * The fp16 weight itself, [K, N], is what wq_q4g32_dequantize(W, S, out, K, N) returns for these operands (the
+ * decode of format A with the two dimensions exchanged). */
+int wq_q4n32_prepare(const uint32_t* W, const uint16_t* S, uint32_t* W_nk, uint16_t* ST, int64_t K, int64_t N,
+                     wq_stream_t stream);
+int wq_q4n32_linear(const uint32_t* W_nk, const uint16_t* ST, const uint16_t* x, const uint16_t* bias,
+                    const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K, wq_stream_t stream);
 
 /* The decode GEMV with the reference's fp16 accumulation (tests/python/dlight/test_gpu_reduction.py:44-51,
  * test_gpu_gemv.py:199-206: `NT_matmul += x * decode`, everything fp16): every product and every partial

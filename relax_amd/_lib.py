@@ -43,6 +43,8 @@ SIGNATURES = {
     "wq_q4g32_kn_to_nk": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
     "wq_q4g32_kn_gemv_workspace_bytes": [_i64, _i64, _i64],
     "wq_q4g32_kn_gemv": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _sz, _vp],
+    "wq_q4n32_prepare": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
+    "wq_q4n32_linear": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_gptq_dequantize": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "wq_gptq_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(ctypes.c_int), _i64, _i64, _i64, _vp],
     "wq_gptq_workspace_bytes": [_i64, _i64, _int],

@@ -42,6 +42,10 @@
 //                              as a bit pattern, then (integer - offset) * scale.  The K loop runs the two
 //                              halves in different MFMA slots: a chain of four dependent VALU operations
 //                              does not fit behind one MFMA, two do.
+// and, only where the scale of a weight depends on its k inside the step (scales along N):
+//   phase_begin(scale, kk)     called once per column sub-tile in front of the phase that unpacks the weights
+//                              of MFMA kk: fetches what pair_finish_at needs for them
+//   pair_finish_at(bits, scale, j)   pair_finish for pair j of that MFMA
 #ifndef RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 #define RELAX_AMD_CSRC_MFMA_GEMM_LDS_H_
 
@@ -84,6 +88,11 @@ struct LdsGemmCfg {
 #define WQ_WAITCNT_VM(n) __builtin_amdgcn_s_waitcnt(((n)&0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
 // the same with lgkmcnt(0): this wavefront's LDS reads have returned as well
 #define WQ_WAITCNT_VM_LGKM0(n) __builtin_amdgcn_s_waitcnt(((n)&0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0x0 << 8))
+
+template <class P, class = void>
+struct ScalePerK : std::false_type {};
+template <class P>
+struct ScalePerK<P, std::void_t<decltype(&P::phase_begin)>> : std::true_type {};
 
 typedef const void __attribute__((address_space(1))) * wq_gptr_t;
 typedef void __attribute__((address_space(3))) * wq_lptr_t;
@@ -262,6 +271,10 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
       // arithmetic in the second half; in phase 3 the packed weights were requested from LDS
       // just above, so the first slots stay free.
       const int first = kk < 3 ? 0 : NSLOT * 3 / 8, usable = NSLOT - first, half = usable / 2;
+      if constexpr (ScalePerK<Policy>::value) {
+#pragma unroll
+        for (int t = 0; t < TN; ++t) Policy::phase_begin(bs[t], (kk + 1) & 3);
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int sl = 0; sl < NSLOT; ++sl) {
@@ -277,7 +290,10 @@ __device__ __forceinline__ void gemm_lds_tile(const typename Policy::Args& wargs
         for (int p = 0; p < NPAIR; ++p) {
           const int tt = p >> 2, j = p & 3;
           if (sl == first + p * half / NPAIR) pb[p] = Policy::pair_bits(bw[tt], (kk + 1) & 3, j);
-          if (sl == first + half + p * (usable - half) / NPAIR) dq[tt][j] = Policy::pair_finish(pb[p], bs[tt]);
+          if (sl == first + half + p * (usable - half) / NPAIR) {
+            if constexpr (ScalePerK<Policy>::value) dq[tt][j] = Policy::pair_finish_at(pb[p], bs[tt], j);
+            else dq[tt][j] = Policy::pair_finish(pb[p], bs[tt]);
+          }
         }
         // direct loads of step ks+AHEAD, all in phase 0 (into the slot of step ks-1, free since the
         // barrier of its phase 3): timed on the GPU, one phase with loads and three without beat

@@ -1,0 +1,143 @@
+// q4f16_1 weights whose codes are packed along N (the decode block of
+// tests/python/dlight/test_gpu_matmul.py:366-377):
+//   W uint32 [K, N/8], S fp16 [K, N/32]
+//   w[k, n] = (fp16((W[k, n/8] >> 4 (n % 8)) & 15) - 7) * S[k, n/32],   y = epilogue(x . w)
+// A scale covers 32 consecutive n of ONE k, so this is not a transposed format A: no rearrangement
+// turns its scales into scales per 32 consecutive k.  What a rearrangement does give is the weight
+// stream of the MFMA GEMM (mfma_gemm_lds.h): at load time the codes are transposed to [N, K/8]
+// (8 consecutive k of one column per word, as every kernel of this library reads them) and the scales
+// to ST [N/32, K] (the scales of a group of 32 columns contiguous along k).  The GEMM then stages, per
+// K-step of 64 k and group of 32 columns, the group's 64 scales (128 bytes: the 4 bytes per column that
+// format A stages, laid out differently) and multiplies every pair of weights by its own pair of
+// scales: (code - 7) is exact and the product rounds once, the reference's fp16 weight bit for bit.
+#include "../../include/relax_amd_wq.h"
+#include "mfma_gemm.h"
+#include "mfma_gemm_lds.h"
+#include "q4g32_common.h"
+#include "tuning.h"
+#include "wq_device.h"
+#include "wq_host.h"
+
+namespace wq {
+
+// W_nk[n][kw] = the codes of column n at rows 8 kw .. 8 kw + 7; one thread per output word, kw fastest
+__global__ __launch_bounds__(256) void q4n32_repack_kernel(const uint32_t* __restrict__ W_kn, uint32_t* __restrict__ W_nk,
+                                                           int K, int N) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int K8 = K >> 3, N8 = N >> 3;
+  if (idx >= (int64_t)N * K8) return;
+  const int n = (int)(idx / K8), kw = (int)(idx % K8);
+  const int shift = 4 * (n & 7);
+  uint32_t out = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) out |= ((W_kn[(int64_t)(8 * kw + j) * N8 + (n >> 3)] >> shift) & 15u) << (4 * j);
+  W_nk[idx] = out;
+}
+
+// ST[g][k] = S[k][g]
+__global__ __launch_bounds__(256) void q4n32_scales_kernel(const half_t* __restrict__ S, half_t* __restrict__ ST, int K,
+                                                           int G) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)G * K) return;
+  const int g = (int)(idx / K), k = (int)(idx % K);
+  ST[idx] = S[(int64_t)k * G + g];
+}
+
+// Weight policy of gemm_lds_kernel: the code stream of format A, scales per (k, group of 32 columns).
+struct Q4N32LdsPolicy {
+  static constexpr int kColBytes = 32;
+  static constexpr int kScaleBytes = 4;
+  static constexpr int kStepStride = 32;
+  struct Args {
+    const uint32_t* W;  // [N, K/8]
+    const half_t* ST;   // [N/32, K]
+  };
+  struct Frag {
+    uint4_t w;
+  };
+  // where the 32 scales of the lane's half of the step lie in LDS, and the 8 of the MFMA being unpacked
+  struct Scale {
+    const unsigned char* p;
+    uint4_t cur;
+  };
+  __device__ __forceinline__ static const char* b_src(const Args& a, int n0, int q, int N, int K) {
+    const int n = q >> 1, h = q & 1;
+    return reinterpret_cast<const char*>(a.W + (int64_t)min(n0 + n, N - 1) * (K >> 3)) + h * 16;
+  }
+  // "the 4 scale bytes of column n" of a step: bytes 4 (n % 32) .. + 3 of the 128 bytes of its group, so that
+  // the 32 columns of a group stage the group's 64 scales in order
+  __device__ __forceinline__ static const char* s_src(const Args& a, int n, int K) {
+    return reinterpret_cast<const char*>(a.ST + (int64_t)(n >> 5) * K) + (n & 31) * 4;
+  }
+  __device__ __forceinline__ static int64_t s_offset(const Args&, int ks) { return (int64_t)ks * 128; }
+  // p: the staged bytes of the lane's column; a sub-tile of 32 columns is one group (tiles start at multiples of 128)
+  __device__ __forceinline__ static Scale read_scale(const unsigned char* p, int lh) {
+    return Scale{p - ((threadIdx.x & 31) << 2) + lh * 64, uint4_t{0, 0, 0, 0}};
+  }
+  __device__ __forceinline__ static Scale const_scale(const Args&, int) { return Scale{nullptr, uint4_t{0, 0, 0, 0}}; }
+  __device__ __forceinline__ static void read(Frag& f, const unsigned char* bslot, int n_local, int lh) {
+    f.w = *reinterpret_cast<const uint4_t*>(bslot + (n_local * 2 + lh) * 16);
+  }
+  __device__ __forceinline__ static uint32_t pair_bits(const Frag& f, int kk, int j) {
+    const uint32_t word = kk == 0 ? f.w.x : kk == 1 ? f.w.y : kk == 2 ? f.w.z : f.w.w;
+    return q4_pair_bits_natural(word, j);
+  }
+  __device__ __forceinline__ static void phase_begin(Scale& s, int kk) {
+    s.cur = *reinterpret_cast<const uint4_t*>(s.p + kk * 16);
+  }
+  __device__ __forceinline__ static half2_t pair_finish_at(uint32_t bits, const Scale& s, int j) {
+    const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+    const uint32_t s2 = j == 0 ? s.cur.x : j == 1 ? s.cur.y : j == 2 ? s.cur.z : s.cur.w;
+    return (as_half2(bits) - off) * as_half2(s2);
+  }
+  __device__ __forceinline__ static half2_t pair_finish(uint32_t, const Scale&) { return half2_t{}; }  // (not used)
+  __device__ __forceinline__ static half2_t pair(const Frag& f, int kk, int j, const Scale& s) {
+    const half2_t off = {(half_t)1031.0f, (half_t)1031.0f};
+    return (as_half2(pair_bits(f, kk, j)) - off) * *reinterpret_cast<const half2_t*>(s.p + kk * 16 + j * 4);
+  }
+};
+
+}  // namespace wq
+
+extern "C" int wq_q4n32_prepare(const uint32_t* W, const uint16_t* S, uint32_t* W_nk, uint16_t* ST, int64_t K, int64_t N,
+                                wq_stream_t stream_) {
+  using namespace wq;
+  hipStream_t stream = (hipStream_t)stream_;
+  WQ_REQUIRE(K >= 0 && N >= 0, "wq_q4n32_prepare: negative dimension");
+  WQ_REQUIRE(K % 8 == 0 && N % 32 == 0, "wq_q4n32_prepare: K=%lld must be a multiple of 8 and N=%lld of the group size 32",
+             (long long)K, (long long)N);
+  if (K == 0 || N == 0) return WQ_OK;
+  WQ_REQUIRE(W && S && W_nk && ST, "wq_q4n32_prepare: null pointer");
+  WQ_REQUIRE(K < (1ll << 30) && N < (1ll << 30), "wq_q4n32_prepare: too large");
+  const int64_t words = N * (K / 8), scales = (N / 32) * K;
+  WQ_LAUNCH("wq_q4n32_prepare", q4n32_repack_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, W, W_nk,
+            (int)K, (int)N);
+  WQ_LAUNCH("wq_q4n32_prepare", q4n32_scales_kernel, dim3((unsigned)((scales + 255) / 256)), dim3(256), 0, stream,
+            (const half_t*)S, (half_t*)ST, (int)K, (int)(N / 32));
+  return WQ_OK;
+}
+
+extern "C" int wq_q4n32_linear(const uint32_t* W_nk, const uint16_t* ST, const uint16_t* x, const uint16_t* bias,
+                               const uint16_t* residual, uint16_t* y, int64_t M, int64_t N, int64_t K,
+                               wq_stream_t stream_) {
+  using namespace wq;
+  hipStream_t stream = (hipStream_t)stream_;
+  WQ_REQUIRE(M >= 0 && N >= 0 && K >= 0, "wq_q4n32_linear: negative dimension");
+  WQ_REQUIRE(K % 64 == 0 && N % 32 == 0,
+             "wq_q4n32_linear: K=%lld must be a multiple of 64 (a step of the matrix-core kernel) and N=%lld of the group size 32",
+             (long long)K, (long long)N);
+  if (M == 0 || N == 0) return WQ_OK;
+  WQ_REQUIRE(K > 0, "wq_q4n32_linear: K must be positive");
+  WQ_REQUIRE(W_nk && ST && x && y, "wq_q4n32_linear: null pointer");
+  WQ_REQUIRE(aligned16(W_nk) && aligned16(x) && (reinterpret_cast<uintptr_t>(ST) & 3u) == 0,
+             "wq_q4n32_linear: W_nk and x must be 16-byte aligned, ST 4-byte aligned");
+  WQ_REQUIRE(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), "wq_q4n32_linear: too large");
+  const Q4N32LdsPolicy::Args args{W_nk, (const half_t*)ST};
+  const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
+  // the tile shapes of format A's GEMM (same code stream, same bytes per step)
+  switch (tuning().gemm_cfg ? tuning().gemm_cfg : choose_q4_lds_cfg(M, N, cu_count())) {
+    case 11: return launch_gemm_lds<Q4N32LdsPolicy, Q4G32Epilogue, 8, 2, 1, 4, 1>("wq_q4n32_linear", args, x, y, ep, M, N, K, stream);
+    case 18: return launch_gemm_lds<Q4N32LdsPolicy, Q4G32Epilogue, 8, 1, 1, 4, 1>("wq_q4n32_linear", args, x, y, ep, M, N, K, stream);
+    default: return launch_gemm_lds<Q4N32LdsPolicy, Q4G32Epilogue, 4, 1, 1, 4, 2>("wq_q4n32_linear", args, x, y, ep, M, N, K, stream);
+  }
+}

@@ -404,6 +404,49 @@ def q4g32_kn_gemv(W_kn: torch.Tensor, S_kn: torch.Tensor, x: torch.Tensor, bias:
     return out
 
 
+# ------------------------------------------------------------------ q4f16_1 packed along N
+
+
+def q4n32_prepare(W: torch.Tensor, S: torch.Tensor):
+    """Load-time rearrangement of q4f16_1 weights packed along N (``W`` uint32 ``[K, N/8]``, ``S`` fp16
+    ``[K, N/32]``; tests/python/dlight/test_gpu_matmul.py:366-377) for :func:`q4n32_linear`: returns
+    ``(W_nk [N, K/8], ST [N/32, K])``."""
+    W = _w32(W)
+    S = _dev(S, torch.float16, "S")
+    K, n8 = W.shape
+    N = n8 * 8
+    if N % 32 or tuple(S.shape) != (K, N // 32):
+        raise ValueError(f"S must be [K, N/32] = [{K}, {N // 32}], got {tuple(S.shape)}")
+    W_nk = torch.empty((N, K // 8), dtype=W.dtype, device=W.device)
+    ST = torch.empty((N // 32, K), dtype=torch.float16, device=W.device)
+    check(_lib.lib().wq_q4n32_prepare(_ptr(W), _ptr(S), _ptr(W_nk), _ptr(ST), K, N, _stream()), "wq_q4n32_prepare")
+    return W_nk, ST
+
+
+def q4n32_linear(W_nk: torch.Tensor, ST: torch.Tensor, x: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                 residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y = residual + fp16(x . w + bias)`` over operands of :func:`q4n32_prepare` (test_gpu_matmul.py:352-401);
+    ``x`` fp16 ``[..., K]``."""
+    W_nk = _w32(W_nk)
+    ST = _dev(ST, torch.float16, "ST")
+    x = _dev(x, torch.float16, "x")
+    N, K = W_nk.shape[0], W_nk.shape[1] * 8
+    if tuple(ST.shape) != (N // 32, K) or x.shape[-1] != K:
+        raise ValueError(f"expected ST [N/32, K] = [{N // 32}, {K}] and x [..., {K}]; got {tuple(ST.shape)}, {tuple(x.shape)}")
+    M = x.numel() // K if K else 0
+    if bias is not None and _dev(bias, torch.float16, "bias").numel() != N:
+        raise ValueError("bias must have N elements")
+    if residual is not None and _dev(residual, torch.float16, "residual").numel() != M * N:
+        raise ValueError("residual must have M*N elements")
+    if out is None:
+        out = torch.empty((*x.shape[:-1], N), dtype=torch.float16, device=x.device)
+    elif not out.is_contiguous() or out.numel() != M * N or out.dtype != torch.float16:
+        raise ValueError("out must be a contiguous fp16 tensor of M*N elements")
+    check(_lib.lib().wq_q4n32_linear(_ptr(W_nk), _ptr(ST), _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), M, N, K,
+                                     _stream()), "wq_q4n32_linear")
+    return out
+
+
 # ------------------------------------------------------------------ AutoGPTQ checkpoints
 
 
