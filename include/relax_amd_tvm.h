@@ -43,7 +43,7 @@ WQ_PACKED(relax_amd_ft_preprocess_weight_dps);
 
 /* Format A (q4f16_1).  Buffer order of the reference's PrimFuncs
  * (tests/python/dlight/test_gpu_gemv.py:189, test_gpu_matmul.py:352; of the latter the argument order and the
- * epilogue chain :378-401 only: its weights are packed along N, W[k, n/8], which no entry point takes):
+ * epilogue chain :378-401 only: its weights are packed along N, W[k, n/8], which the q4f16_1_ngroup pair below takes):
  * "relax_amd.q4f16_1_matmul"(W u32[N,K/8], S f16[N,K/32], x f16[..,K], out f16[..,N])
  * "relax_amd.q4f16_1_matmul_bias"(W, S, x, bias f16[N], out)
  * "relax_amd.q4f16_1_matmul_bias_residual"(W, S, x, bias f16[N], residual f16[..,N], out) */
@@ -60,6 +60,12 @@ WQ_PACKED(relax_amd_q4f16_1_decode);
  *                                (tests/python/relax/test_codegen_cutlass.py:1392-1457, 1631-1676, 2044-2109) */
 WQ_PACKED(relax_amd_q4f16_1_encode);
 WQ_PACKED(relax_amd_q4f16_1_kn_to_nk);
+/* q4f16_1 packed along N, the operands of tests/python/dlight/test_gpu_matmul.py:352-401 (W u32[K,N/8], S f16[K,N/32]):
+ * "relax_amd.q4f16_1_ngroup_prepare"(W, S, W_out u32[N,K/8], ST_out f16[N/32,K]): load-time rearrangement;
+ * "relax_amd.q4f16_1_ngroup_matmul_bias_residual"(W_nk, ST, x f16[..,K], bias f16[N] | null, residual f16[..,N] | null,
+ * out f16[..,N]): the matmul and the fixture's epilogue chain, buffer order as there. */
+WQ_PACKED(relax_amd_q4f16_1_ngroup_prepare);
+WQ_PACKED(relax_amd_q4f16_1_ngroup_matmul_bias_residual);
 /* "relax_amd.q4f16_1_kn_matmul"(W_kn u32[K/8,N], S_kn f16[K/32,N], x f16[..,K], out f16[..,N][, workspace u8]):
  * the decode linear over a K-major checkpoint in place (tests/python/dlight/test_gpu_reduction.py:102-165), up to
  * WQ_KN_GEMV_MAX_M rows; workspace >= wq_q4g32_kn_gemv_workspace_bytes(M, N, K) bytes where that is not 0. */

@@ -487,6 +487,67 @@ WQ_PACKED(relax_amd_q4f16_1_kn_to_nk) {
   return rc == WQ_OK ? 0 : packed_fail();
 }
 
+// ---- q4f16_1 packed along N (tests/python/dlight/test_gpu_matmul.py:352-401) ----
+// (W uint32 [K, N/8], S fp16 [K, N/32], W_out uint32 [N, K/8], ST_out fp16 [N/32, K]): the load-time rearrangement
+WQ_PACKED(relax_amd_q4f16_1_ngroup_prepare) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.q4f16_1_ngroup_prepare";
+  Tensor Wi, Si, Wo, So;
+  if (num_args != 4) {
+    fail(WQ_EINVAL, "%s: expected (W, S, W_out, ST_out)", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W", &Wi) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "S", &Si) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLUInt, 32, "W_out", &Wo) ||
+      !get_tensor(who, args, type_codes, num_args, 3, kDLFloat, 16, "ST_out", &So))
+    return packed_fail();
+  if (Wi.t->ndim != 2 || Si.t->ndim != 2 || Wo.t->ndim != 2 || So.t->ndim != 2 || Si.t->shape[0] != Wi.t->shape[0] ||
+      Si.t->shape[1] * 4 != Wi.t->shape[1] || Wo.t->shape[0] != Wi.t->shape[1] * 8 || Wo.t->shape[1] * 8 != Wi.t->shape[0] ||
+      So.t->shape[0] != Si.t->shape[1] || So.t->shape[1] != Si.t->shape[0]) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (W [K,N/8], S [K,N/32], W_out [N,K/8], ST_out [N/32,K])", who);
+    return packed_fail();
+  }
+  const int rc = wq_q4n32_prepare((const uint32_t*)Wi.ptr, (const uint16_t*)Si.ptr, (uint32_t*)Wo.ptr, (uint16_t*)So.ptr,
+                                  Wi.t->shape[0], Wi.t->shape[1] * 8, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
+// (W_nk, ST, x fp16 [.., K], bias fp16 [N] | null, residual fp16 [.., N] | null, out fp16 [.., N]): the matmul and the
+// epilogue chain of the fixture (:378-401) over the prepared operands, buffer order as there.
+WQ_PACKED(relax_amd_q4f16_1_ngroup_matmul_bias_residual) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.q4f16_1_ngroup_matmul_bias_residual";
+  Tensor W, ST, x, bias, res, y;
+  if (num_args != 6) {
+    fail(WQ_EINVAL, "%s: expected (W_nk, ST, x, bias|null, residual|null, out)", who);
+    return packed_fail();
+  }
+  const bool has_bias = type_codes[3] != kTVMNullptr, has_res = type_codes[4] != kTVMNullptr;
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W_nk", &W) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "ST", &ST) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLFloat, 16, "x", &x) ||
+      (has_bias && !get_tensor(who, args, type_codes, num_args, 3, kDLFloat, 16, "bias", &bias)) ||
+      (has_res && !get_tensor(who, args, type_codes, num_args, 4, kDLFloat, 16, "residual", &res)) ||
+      !get_tensor(who, args, type_codes, num_args, 5, kDLFloat, 16, "out", &y))
+    return packed_fail();
+  if (W.t->ndim != 2 || ST.t->ndim != 2 || x.t->ndim < 1 || y.t->ndim < 1) {
+    fail(WQ_EINVAL, "%s: W_nk and ST must be matrices", who);
+    return packed_fail();
+  }
+  const int64_t N = W.t->shape[0], K = W.t->shape[1] * 8;
+  const int64_t M = leading(x.t);
+  if (ST.t->shape[0] * 32 != N || ST.t->shape[1] != K || x.t->shape[x.t->ndim - 1] != K || y.numel != M * N ||
+      y.t->shape[y.t->ndim - 1] != N || (has_bias && bias.numel != N) || (has_res && res.numel != M * N)) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (N=%lld K=%lld M=%lld)", who, (long long)N, (long long)K, (long long)M);
+    return packed_fail();
+  }
+  const int rc = wq_q4n32_linear((const uint32_t*)W.ptr, (const uint16_t*)ST.ptr, (const uint16_t*)x.ptr,
+                                 (const uint16_t*)bias.ptr, (const uint16_t*)res.ptr, (uint16_t*)y.ptr, M, N, K,
+                                 current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
+
 // ---- AutoGPTQ layers (tests/python/dlight/test_gpu_gemv.py:636-665) ----
 // g_idx is uint32 in the reference's PrimFunc and int32 in AutoGPTQ checkpoints: same bytes.
 static bool get_index_tensor(const char* who, TVMValue* args, int* tcodes, int n, int i, const char* what, Tensor* t) {
@@ -787,6 +848,9 @@ const std::vector<Entry>& table() {
     v.push_back({"relax_amd.q4f16_1_encode", "relax_amd_q4f16_1_encode", relax_amd_q4f16_1_encode});
     v.push_back({"relax_amd.q4f16_1_kn_to_nk", "relax_amd_q4f16_1_kn_to_nk", relax_amd_q4f16_1_kn_to_nk});
     v.push_back({"relax_amd.q4f16_1_kn_matmul", "relax_amd_q4f16_1_kn_matmul", relax_amd_q4f16_1_kn_matmul});
+    v.push_back({"relax_amd.q4f16_1_ngroup_prepare", "relax_amd_q4f16_1_ngroup_prepare", relax_amd_q4f16_1_ngroup_prepare});
+    v.push_back({"relax_amd.q4f16_1_ngroup_matmul_bias_residual", "relax_amd_q4f16_1_ngroup_matmul_bias_residual",
+                 relax_amd_q4f16_1_ngroup_matmul_bias_residual});
     v.push_back({"relax_amd.fpA_intB_encode", "relax_amd_fpA_intB_encode", relax_amd_fpA_intB_encode});
     v.push_back({"relax_amd.autogptq_decode", "relax_amd_autogptq_decode", relax_amd_autogptq_decode});
     v.push_back({"relax_amd.autogptq_prepare", "relax_amd_autogptq_prepare", relax_amd_autogptq_prepare});

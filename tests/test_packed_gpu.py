@@ -268,6 +268,45 @@ def test_q4f16_1_kn_matmul(env, oracle):
     assert rc == -1
 
 
+def test_q4f16_1_ngroup_pair(env, oracle):
+    """relax_amd.q4f16_1_ngroup_prepare / _matmul_bias_residual: the operands and the buffer order of
+    tests/python/dlight/test_gpu_matmul.py:352-401 (codes packed along N; dynamic n rows of x)."""
+    lib, u, T, torch = env
+    n, N, K = 70, 416, 256
+    _, W, S = oracle.make_q4g32_inputs(1, K, N, seed=50)  # W [K, N/8], S [K, N/32]
+    rng = np.random.default_rng(51)
+    x = rng.standard_normal((1, n, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((1, n, N)).astype(np.float16)
+    dW, dS = u.dev(W), u.dev(S)
+    W_nk = torch.empty((N, K // 8), dtype=torch.int32, device="cuda")
+    ST = torch.empty((N // 32, K), dtype=torch.float16, device="cuda")
+    y = torch.empty((1, n, N), dtype=torch.float16, device="cuda")
+    tW, _ = T.from_torch(dW, "uint32")
+    tS, _ = T.from_torch(dS)
+    tWn, _ = T.from_torch(W_nk, "uint32")
+    tST, _ = T.from_torch(ST)
+    tx, _ = T.from_torch(u.dev(x))
+    tb, _ = T.from_torch(u.dev(bias))
+    tr, _ = T.from_torch(u.dev(res))
+    ty, _ = T.from_torch(y)
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_ngroup_prepare, tW, tS, tWn, tST)
+    assert rc == 0, lib.wq_last_error()
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_ngroup_matmul_bias_residual, tWn, tST, tx, tb, tr, ty)
+    assert rc == 0, lib.wq_last_error()
+    Bt = np.ascontiguousarray(oracle.q4g32_dequant(W, S).T)  # [N, K]: the fixture's decode, transposed
+    want = oracle.nt_matmul_f32acc(Bt, x.reshape(n, K), bias, res.reshape(n, N))
+    u.assert_close(u.host(y).reshape(n, N), want, "packed ngroup matmul + bias + residual")
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_ngroup_matmul_bias_residual, tWn, tST, tx, None, None, ty)
+    assert rc == 0, lib.wq_last_error()
+    u.assert_close(u.host(y).reshape(n, N), oracle.nt_matmul_f32acc(Bt, x.reshape(n, K)), "packed ngroup matmul")
+    # the unprepared operands are refused by their shapes; wrong arity
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_ngroup_matmul_bias_residual, tW, tS, tx, None, None, ty)
+    assert rc == -1 and b"inconsistent" in lib.wq_last_error()
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_ngroup_prepare, tW, tS, tWn)
+    assert rc == -1
+
+
 @pytest.mark.parametrize("M", [1, 3, 40])
 def test_autogptq_padded_pair(env, oracle, M):
     """relax_amd.autogptq_prepare_padded / autogptq_matmul_padded: a g_idx whose groups differ in size
