@@ -701,6 +701,24 @@ def main():
             vendor.append({"N": N, "K": K, "us": round(vms * 1e3, 2), "tflops": round(fl / vms / 1e9, 1)})
             vendor_ms += vms
             del W, S, x, y, Wf
+        # the same GEMM over weights packed along N (the layout of the reference's prefill fixture,
+        # tests/python/dlight/test_gpu_matmul.py:352-401, at its own 4096 x 4096 and at the gate/up shape)
+        ngroup = []
+        for N, K in ((4096, 4096), PREFILL_SHAPES[0]):
+            g = torch.Generator(device="cuda")
+            g.manual_seed(N + 1)
+            W = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+            S = (torch.rand((K, N // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+            W_nk, ST = ops.q4n32_prepare(W, S)
+            x = torch.randn((PREFILL_M, K), device="cuda", dtype=torch.float16)
+            y = torch.empty((PREFILL_M, N), device="cuda", dtype=torch.float16)
+            for _ in range(3):
+                ops.q4n32_linear(W_nk, ST, x, out=y)
+            ms, _ = _measure(torch, cur, lambda: ops.q4n32_linear(W_nk, ST, x, out=y), min_ms=MIN_SAMPLE_MS / 4, samples=3)
+            fl = 2.0 * PREFILL_M * N * K
+            ngroup.append({"M": PREFILL_M, "N": N, "K": K, "us": round(ms * 1e3, 2), "tflops": round(fl / ms / 1e9, 1),
+                           "frac_of_mfma_peak": round(fl / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)})
+            del W, S, W_nk, ST, x, y
         tf = tot_flops / tot_ms / 1e9
         gtraffic, gsrc = offline_traffic("gemm_lds_kernel")
         out["gemm"] = {
@@ -715,6 +733,7 @@ def main():
                                              "value": round(tot_flops / vendor_ms / 1e9, 1), "unit": "TFLOP/s",
                                              "frac_of_mfma_peak": round(tot_flops / vendor_ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                                              "shapes": vendor},
+            "packed_along_n": {"kernel": "gemm_lds_kernel<Q4N32LdsPolicy> (wq_q4n32_linear)", "shapes": ngroup},
         }
 
     del lists
