@@ -719,6 +719,36 @@ def main():
             ngroup.append({"M": PREFILL_M, "N": N, "K": K, "us": round(ms * 1e3, 2), "tflops": round(fl / ms / 1e9, 1),
                            "frac_of_mfma_peak": round(fl / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)})
             del W, S, W_nk, ST, x, y
+        # ... and its decode kernel at M = 1, weight copies (more than the last-level cache) cycled inside one graph
+        ngroup_decode = []
+        for (N, K), ncopy in (((4096, 4096), 40), ((11008, 4096), 16)):
+            g = torch.Generator(device="cuda")
+            g.manual_seed(N + 2)
+            prepared = []
+            for _ in range(ncopy):
+                W = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+                S = (torch.rand((K, N // 32), device="cuda", generator=g) * 0.015 + 0.005).to(torch.float16)
+                prepared.append(ops.q4n32_prepare(W, S))
+                del W, S
+            x = torch.randn((1, K), device="cuda", dtype=torch.float16)
+            y = torch.empty((1, N), device="cuda", dtype=torch.float16)
+
+            def cycle():
+                for W_nk, ST in prepared:
+                    ops.q4n32_linear(W_nk, ST, x, out=y)
+
+            cycle()
+            torch.cuda.synchronize()
+            g1 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g1):
+                cycle()
+            g1.replay()
+            ms, _ = _measure(torch, cur, g1.replay, min_ms=MIN_SAMPLE_MS / 4, samples=3)
+            us = ms * 1e3 / ncopy
+            nb = gemv_bytes(1, N, K)  # (codes + scales + x + y: the same bytes as format A)
+            ngroup_decode.append({"M": 1, "N": N, "K": K, "us": round(us, 2), "GB/s": round(nb / us / 1e3, 1),
+                                  "frac_of_hbm_peak": round(nb / us / 1e3 / HBM_PEAK_GBS, 4)})
+            del g1, prepared
         tf = tot_flops / tot_ms / 1e9
         gtraffic, gsrc = offline_traffic("gemm_lds_kernel")
         out["gemm"] = {
@@ -733,7 +763,8 @@ def main():
                                              "value": round(tot_flops / vendor_ms / 1e9, 1), "unit": "TFLOP/s",
                                              "frac_of_mfma_peak": round(tot_flops / vendor_ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                                              "shapes": vendor},
-            "packed_along_n": {"kernel": "gemm_lds_kernel<Q4N32LdsPolicy> (wq_q4n32_linear)", "shapes": ngroup},
+            "packed_along_n": {"kernel": "gemm_lds_kernel<Q4N32LdsPolicy> (wq_q4n32_linear)", "shapes": ngroup,
+                               "decode_kernel": "q4n32_gemv_kernel (wq_q4n32_linear, M <= 4)", "decode": ngroup_decode},
         }
 
     del lists

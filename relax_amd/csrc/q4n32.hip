@@ -43,6 +43,96 @@ __global__ __launch_bounds__(256) void q4n32_scales_kernel(const half_t* __restr
   ST[idx] = S[(int64_t)k * G + g];
 }
 
+// ---- decode: a few rows of x, the weights streamed once per row of x ---------------------------------------
+// y[n] = sum_k x[k] s[k, g] (code[k, n] - 7) with g = n / 32: for the 32 rows of W_nk of one group the scales
+// belong to the ACTIVATIONS, xs[k] = fp16(x[k] * ST[g][k]), and what is left is format A's decode GEMV with every
+// scale 1.  A workgroup takes RPW rows of one group: it stages xs in LDS (in the pairing of the unpack, with the
+// zero-point constant of every 32 k, as q4_gemv.h does), then its four wavefronts stream two rows each at a time,
+// lane l the 16-byte pieces l, l + 64, ... of a row.  One rounding differs from the reference: it rounds
+// (code - 7) * s to fp16 and multiplies by x in fp32, here x * s is rounded and (code - 7) is exact; a one-hot x
+// still returns the reference's weight bit for bit.
+__global__ __launch_bounds__(256) void q4n32_gemv_kernel(const uint4_t* __restrict__ W, const half_t* __restrict__ ST,
+                                                         const half_t* __restrict__ x, const half_t* __restrict__ bias,
+                                                         const half_t* __restrict__ residual, half_t* __restrict__ y,
+                                                         int N, int K, int rpw) {
+  extern __shared__ uint4_t smem[];
+  const int G = K >> 5;                                       // pieces of 32 k per row
+  uint4_t* xs = smem;                                         // [4][G]: word ch of piece g at ch * G + g
+  float* cs = reinterpret_cast<float*>(smem + 4 * (size_t)G);  // [G]: -(1031 A + 71 B) of the piece
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * rpw;
+  const half_t* st = ST + (int64_t)(n0 >> 5) * K;
+  const half2_t k1031 = {(half_t)1031.0f, (half_t)1031.0f};
+  const half2_t k71 = {(half_t)71.0f, (half_t)71.0f};
+  const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+  for (int wi = tid; wi < (K >> 3); wi += 256) {  // K % 32 == 0: the 4 words of a piece sit in 4 adjacent lanes
+    const uint4_t xv = reinterpret_cast<const uint4_t*>(x)[wi];
+    const uint4_t sv = reinterpret_cast<const uint4_t*>(st)[wi];
+    const uint32_t in[4] = {as_u32(as_half2(xv.x) * as_half2(sv.x)), as_u32(as_half2(xv.y) * as_half2(sv.y)),
+                            as_u32(as_half2(xv.z) * as_half2(sv.z)), as_u32(as_half2(xv.w) * as_half2(sv.w))};
+    uint32_t o[4];
+    pair_i_i4(in, o);  // o[i] = (xs_i, xs_{i+4})
+    float c = dot2(as_half2(o[0]), k1031, 0.0f);
+    c = dot2(as_half2(o[1]), k71, c);
+    c = dot2(as_half2(o[2]), k1031, c);
+    c = dot2(as_half2(o[3]), k71, c);
+    c += dpp_shift<0xb1, 0xf>(c);
+    c += dpp_shift<0x4e, 0xf>(c);
+    const int g = wi >> 2, ch = wi & 3;
+    xs[ch * G + g] = uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
+    if (ch == 0) cs[g] = -c;
+  }
+  __syncthreads();
+  const uint32_t magic = 0x64006400u;
+  for (int r = wave * 2; r < rpw; r += 8) {  // two rows at a time share the reads of xs
+    const int na = n0 + r, nb = na + 1;
+    if (na >= N) break;
+    const uint4_t* wa = W + (int64_t)na * G;
+    const uint4_t* wb = W + (int64_t)min(nb, N - 1) * G;
+    float acc_a = 0.0f, acc_b = 0.0f;
+    constexpr int UNR = 2;  // pieces per lane and row requested before the first is multiplied
+    for (int g0 = lane; g0 < G; g0 += 64 * UNR) {
+      uint4_t qa[UNR], qb[UNR];
+#pragma unroll
+      for (int j = 0; j < UNR; ++j) {
+        const int g = min(g0 + 64 * j, G - 1);
+        qa[j] = __builtin_nontemporal_load(&wa[g]);
+        qb[j] = __builtin_nontemporal_load(&wb[g]);
+      }
+#pragma unroll
+      for (int j = 0; j < UNR; ++j) {
+        const int g = g0 + 64 * j;
+        if (g >= G) break;
+        float ga = cs[g], gb = ga;
+#pragma unroll
+        for (int ch = 0; ch < 4; ++ch) {
+          const uint4_t xv = xs[ch * G + g];
+          const uint32_t a = ch == 0 ? qa[j].x : ch == 1 ? qa[j].y : ch == 2 ? qa[j].z : qa[j].w;
+          const uint32_t b = ch == 0 ? qb[j].x : ch == 1 ? qb[j].y : ch == 2 ? qb[j].z : qb[j].w;
+          const uint32_t a8 = a >> 8, b8 = b >> 8;
+          ga = dot2(as_half2(and_or(a, 0x000F000Fu, magic)), as_half2(xv.x), ga);  // 1024 + (q0, q4)
+          ga = dot2(as_half2(and_or(a, 0x00F000F0u, magic)), as_half2(xv.y), ga);  // 1024 + 16 (q1, q5)
+          ga = dot2(as_half2(and_or(a8, 0x000F000Fu, magic)), as_half2(xv.z), ga);
+          ga = dot2(as_half2(and_or(a8, 0x00F000F0u, magic)), as_half2(xv.w), ga);
+          gb = dot2(as_half2(and_or(b, 0x000F000Fu, magic)), as_half2(xv.x), gb);
+          gb = dot2(as_half2(and_or(b, 0x00F000F0u, magic)), as_half2(xv.y), gb);
+          gb = dot2(as_half2(and_or(b8, 0x000F000Fu, magic)), as_half2(xv.z), gb);
+          gb = dot2(as_half2(and_or(b8, 0x00F000F0u, magic)), as_half2(xv.w), gb);
+        }
+        acc_a += ga;
+        acc_b += gb;
+      }
+    }
+    acc_a = wave_sum_to_lane63(acc_a);
+    acc_b = wave_sum_to_lane63(acc_b);
+    if (lane == 63) {
+      const Q4G32Epilogue ep{bias, residual, N};
+      y[na] = ep(acc_a, 0, na);
+      if (nb < N && r + 1 < rpw) y[nb] = ep(acc_b, 0, nb);
+    }
+  }
+}
+
 // Weight policy of gemm_lds_kernel: the code stream of format A, scales per (k, group of 32 columns).
 struct Q4N32LdsPolicy {
   static constexpr int kColBytes = 32;
@@ -132,6 +222,19 @@ extern "C" int wq_q4n32_linear(const uint32_t* W_nk, const uint16_t* ST, const u
   WQ_REQUIRE(aligned16(W_nk) && aligned16(x) && (reinterpret_cast<uintptr_t>(ST) & 3u) == 0,
              "wq_q4n32_linear: W_nk and x must be 16-byte aligned, ST 4-byte aligned");
   WQ_REQUIRE(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), "wq_q4n32_linear: too large");
+  // a few rows of x: the streaming kernel, one launch per row (the GEMM below costs the same from 1 to 128 rows)
+  const size_t gemv_lds = (size_t)K * 2 + (size_t)(K / 32) * 4;
+  if (M <= WQ_Q4N32_GEMV_MAX_M && gemv_lds <= 96 * 1024 && !tuning().gemm_cfg) {
+    const int cus = cu_count();
+    const int rpw = N / 32 >= 4 * cus ? 32 : N / 16 >= 4 * cus ? 16 : 8;
+    static DynamicLdsLimit limit;
+    WQ_HIP(limit.ensure(reinterpret_cast<const void*>(q4n32_gemv_kernel), (int)gemv_lds));
+    for (int64_t m = 0; m < M; ++m)
+      WQ_LAUNCH("wq_q4n32_linear", q4n32_gemv_kernel, dim3((unsigned)((N + rpw - 1) / rpw)), dim3(256), gemv_lds, stream,
+                (const uint4_t*)W_nk, (const half_t*)ST, (const half_t*)(x + m * K), (const half_t*)bias,
+                residual ? (const half_t*)(residual + m * N) : nullptr, (half_t*)(y + m * N), (int)N, (int)K, rpw);
+    return WQ_OK;
+  }
   const Q4N32LdsPolicy::Args args{W_nk, (const half_t*)ST};
   const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
   // the tile shapes of format A's GEMM (same code stream, same bytes per step)

@@ -49,7 +49,10 @@ def test_prepare_is_a_pure_rearrangement(env, oracle):
 
 # the fixture's shape (4096 x 4096, dynamic n) at several n; ragged tiles: N not a multiple of the tile width,
 # M one row, one more than a tile, K of one and of a few steps
-SHAPES = [(1, 4096, 4096), (7, 4096, 4096), (130, 4096, 4096), (513, 4096, 4096), (33, 96, 64), (257, 160, 192),
+# (up to 4 rows of x run the streaming kernel, one pass per row; more, the matrix-core GEMM)
+# (N = 16384 and 32800: the streaming kernel with 16 and with 32 rows per workgroup)
+SHAPES = [(1, 4096, 4096), (2, 16384, 128), (1, 32800, 64), (2, 96, 64), (3, 4128, 320), (4, 11008, 4096), (1, 64, 32768), (4, 32, 28672), (2, 4096, 11008),
+          (5, 4096, 4096), (7, 4096, 4096), (130, 4096, 4096), (513, 4096, 4096), (33, 96, 64), (257, 160, 192),
           (300, 4128, 320), (64, 11008, 4096), (1100, 2048, 1024)]
 
 
@@ -80,6 +83,20 @@ def test_one_hot_rows_select_the_reference_weight_bit_for_bit(env, oracle):
     assert np.array_equal(got.view(np.uint16), D.view(np.uint16))
 
 
+def test_one_hot_rows_through_the_streaming_kernel(env, oracle):
+    """The same with 4 rows of x per call: the decode kernel rounds x * s instead of (code - 7) * s, which for
+    x = 1 is the same number."""
+    ops, u, torch = env
+    N, K = 160, 192
+    _, W, S = _inputs(oracle, 1, N, K, seed=10)
+    D = oracle.q4g32_dequant(W, S)  # [K, N]
+    W_nk, ST = ops.q4n32_prepare(u.dev(W), u.dev(S))
+    eye = np.eye(K, dtype=np.float16)
+    for k0 in range(0, K, 4):
+        got = u.host(ops.q4n32_linear(W_nk, ST, u.dev(eye[k0:k0 + 4])))
+        assert np.array_equal(got.view(np.uint16), D[k0:k0 + 4].view(np.uint16)), k0
+
+
 def test_every_tile_shape_gives_the_same_sums(env, oracle):
     """The tile shape is chosen from M and N; forced through the test hook, the three shapes agree with the oracle."""
     ops, u, torch = env
@@ -93,6 +110,8 @@ def test_every_tile_shape_gives_the_same_sums(env, oracle):
         for cfg in (11, 17, 18):
             _lib.lib().wq_debug_set_gemm_config(cfg)
             u.assert_close(u.host(ops.q4n32_linear(W_nk, ST, u.dev(x))), ref, f"q4n32 tile shape {cfg}")
+            # (a forced tile shape also keeps one or two rows on the GEMM)
+            u.assert_close(u.host(ops.q4n32_linear(W_nk, ST, u.dev(x[:2]))), ref[:2], f"q4n32 tile shape {cfg}, 2 rows")
     finally:
         _lib.lib().wq_debug_set_gemm_config(0)
 
