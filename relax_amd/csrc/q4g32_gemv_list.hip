@@ -648,13 +648,14 @@ extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create(const wq_q4g32_gemv_desc* d
 namespace wq {
 // szl == nullptr: format A.  Else the linears are prepared AutoGPTQ layers: d[i].S is SZ and szl[i] the log2 of
 // the 32-column groups per (scale, zero point) pair.
-static wq_gemv_list_t* gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, const int32_t* const* perm, int n,
-                                        int M, void* workspace, size_t workspace_bytes, hipStream_t stream);
+static wq_gemv_list_t* gemv_list_create(const char* who, const wq_q4g32_gemv_desc* d, const uint8_t* szl,
+                                        const int32_t* const* perm, int n, int M, void* workspace, size_t workspace_bytes,
+                                        hipStream_t stream);
 }  // namespace wq
 
 extern "C" wq_gemv_list_t* wq_q4g32_gemv_list_create_batched(const wq_q4g32_gemv_desc* d, int n, int M, void* workspace,
                                                              size_t workspace_bytes, wq_stream_t stream) {
-  return wq::gemv_list_create(d, nullptr, nullptr, n, M, workspace, workspace_bytes, (hipStream_t)stream);
+  return wq::gemv_list_create("wq_q4g32_gemv_list_create", d, nullptr, nullptr, n, M, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* d, int n, void* workspace,
@@ -684,33 +685,35 @@ extern "C" wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* d, 
       return bad(WQ_EINVAL, "wq_gptq_gemv_list_create: linear %d: perm must be 16-byte aligned", i);
     perm[i] = s.perm;
   }
-  return gemv_list_create(e.data(), szl.data(), perm.data(), n, 1, workspace, workspace_bytes, (hipStream_t)stream);
+  return gemv_list_create("wq_gptq_gemv_list_create", e.data(), szl.data(), perm.data(), n, 1, workspace, workspace_bytes,
+                          (hipStream_t)stream);
 #undef bad
 }
 
-static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const uint8_t* szl, const int32_t* const* perm,
-                                            int n, int M, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+static wq_gemv_list_t* wq::gemv_list_create(const char* who, const wq_q4g32_gemv_desc* d, const uint8_t* szl,
+                                            const int32_t* const* perm, int n, int M, void* workspace,
+                                            size_t workspace_bytes, hipStream_t stream) {
 #define bad(code, ...) ((void)fail(code, __VA_ARGS__), (wq_gemv_list_t*)nullptr)
   if (M < 1 || M > WQ_GEMV_LIST_MAX_M)
-    return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: 1 .. %d rows of activations, got %d", WQ_GEMV_LIST_MAX_M, M);
-  if (!d || n <= 0 || n > WQ_GEMV_LIST_MAX) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: need 1 .. %d linears, got %d", WQ_GEMV_LIST_MAX, n);
+    return bad(WQ_EUNSUPPORTED, "%s: 1 .. %d rows of activations, got %d", who, WQ_GEMV_LIST_MAX_M, M);
+  if (!d || n <= 0 || n > WQ_GEMV_LIST_MAX) return bad(WQ_EINVAL, "%s: need 1 .. %d linears, got %d", who, WQ_GEMV_LIST_MAX, n);
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & (kListAlign - 1)) ||
       workspace_bytes < wq_q4g32_gemv_list_workspace_bytes(n))
-    return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: workspace must be 256-byte aligned device memory of %zu bytes",
+    return bad(WQ_EINVAL, "%s: workspace must be 256-byte aligned device memory of %zu bytes", who,
                wq_q4g32_gemv_list_workspace_bytes(n));
   std::vector<wq_q4g32_gemv_desc> e;
   std::vector<int> rows;
   for (int i = 0; i < n; ++i) {
     const wq_q4g32_gemv_desc& s = d[i];
     if (s.N <= 0 || s.K <= 0 || s.K % 32 != 0 || s.K > WQ_GEMV_LIST_MAX_K || s.N >= (1ll << 30))
-      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: N=%lld K=%lld (K must be a positive multiple of 32, at most %d)",
+      return bad(WQ_EINVAL, "%s: linear %d: N=%lld K=%lld (K must be a positive multiple of 32, at most %d)", who,
                  i, (long long)s.N, (long long)s.K, WQ_GEMV_LIST_MAX_K);
-    if (!s.W || !s.S || !s.x || !s.y) return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: null pointer", i);
+    if (!s.W || !s.S || !s.x || !s.y) return bad(WQ_EINVAL, "%s: linear %d: null pointer", who, i);
     if (!aligned16(s.W) || !aligned16(s.x))
-      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: W and x must be 16-byte aligned", i);
+      return bad(WQ_EINVAL, "%s: linear %d: W and x must be 16-byte aligned", who, i);
     // several rows: the scales travel in 16-byte pieces of 8, and rows of x and y are addressed with 32-bit offsets
     if (M > 1 && (s.K % 256 != 0 || !aligned16(s.S) || (int64_t)M * s.N >= (1ll << 30) || s.K / 32 > 0xffff))
-      return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d: with %d rows of activations K=%lld must be a multiple of 256, S 16-byte aligned and M * N < 2^30", i, M, (long long)s.K);
+      return bad(WQ_EUNSUPPORTED, "%s: linear %d: with %d rows of activations K=%lld must be a multiple of 256, S 16-byte aligned and M * N < 2^30", who, i, M, (long long)s.K);
     e.push_back(s);
     rows.push_back(M);
   }
@@ -751,18 +754,18 @@ static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const u
       if (ranges_overlap(a.x, xa, b.y, yb)) {
         // one producer per linear: the consumer waits for a single counter set
         if (((l->descs[i].g_dep >> 16) & 0x7fffu) != 0)
-          return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations of linear %d are written by more than one linear of the list (%d and %d)",
+          return bad(WQ_EUNSUPPORTED, "%s: the activations of linear %d are written by more than one linear of the list (%d and %d)", who,
                      i, j, (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1);
         l->descs[i].g_dep |= (uint32_t)(j + 1) << 16;
       }
       if (ranges_overlap(a.residual, ya, b.y, yb) || ranges_overlap(a.bias, (size_t)a.N * 2, b.y, yb))
-        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: linear %d takes its bias or residual from linear %d of the same list", i, j);
+        return bad(WQ_EUNSUPPORTED, "%s: linear %d takes its bias or residual from linear %d of the same list", who, i, j);
       if (ranges_overlap(a.y, ya, b.y, yb) || ranges_overlap(a.y, ya, b.x, xb) ||
           ranges_overlap(a.y, ya, b.residual, yb) || ranges_overlap(a.y, ya, b.bias, (size_t)b.N * 2))
-        return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the output of linear %d overlaps an operand of linear %d", i, j);
+        return bad(WQ_EUNSUPPORTED, "%s: the output of linear %d overlaps an operand of linear %d", who, i, j);
     }
     if (ranges_overlap(a.y, ya, a.x, xa))
-      return bad(WQ_EINVAL, "wq_q4g32_gemv_list_create: linear %d: y overlaps x", i);
+      return bad(WQ_EINVAL, "%s: linear %d: y overlaps x", who, i);
     const int dep = (int)((l->descs[i].g_dep >> 16) & 0x7fffu) - 1;
     if (dep >= 0) {
       l->descs[dep].g_dep |= kSignal;
@@ -797,7 +800,7 @@ static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const u
   const size_t ysums = (size_t)kYSlots * l->ybuf_floats * sizeof(float);
   const size_t lds_budget = 150 * 1024;
   if (sizeof(ListFlags) + ysums + (size_t)cmax * kChunkBytes > lds_budget)
-    return bad(WQ_EUNSUPPORTED, "wq_q4g32_gemv_list_create: the activations and row sums do not fit the LDS");
+    return bad(WQ_EUNSUPPORTED, "%s: the activations and row sums do not fit the LDS", who);
   const int ring0 = (int)sizeof(ListFlags), ring1 = (int)(lds_budget - ysums);
   l->ybuf0 = ring1;
   l->lds = lds_budget;
@@ -836,17 +839,17 @@ static wq_gemv_list_t* wq::gemv_list_create(const wq_q4g32_gemv_desc* d, const u
                            : reinterpret_cast<const void*>(q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth, false>);
   static DynamicLdsLimit limit[2];  // several lists share a kernel: its limit only ever grows
   if (l->lds > 48 * 1024 && limit[l->zp ? 1 : 0].ensure(kern, (int)l->lds) != hipSuccess)
-    return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: hipFuncSetAttribute failed");
+    return bad(WQ_EDEVICE, "%s: hipFuncSetAttribute failed", who);
   int resident = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
-    return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: the workgroup does not fit a CU (%zu bytes of LDS)", l->lds);
+    return bad(WQ_EDEVICE, "%s: the workgroup does not fit a CU (%zu bytes of LDS)", who, l->lds);
   }
   l->table = workspace;
   l->sync = reinterpret_cast<int*>(static_cast<char*>(workspace) + list_table_bytes(ne));
   if (hipMemcpyAsync(l->table, l->descs.data(), (size_t)ne * sizeof(GemvListDesc), hipMemcpyHostToDevice, stream) != hipSuccess ||
       hipMemsetAsync(l->sync, 0, (size_t)sync_ints(ne) * sizeof(int), stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
-    return bad(WQ_EDEVICE, "wq_q4g32_gemv_list_create: could not upload the descriptor table");
+    return bad(WQ_EDEVICE, "%s: could not upload the descriptor table", who);
   return l.release();
 #undef bad
 }

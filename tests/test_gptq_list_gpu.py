@@ -148,6 +148,11 @@ def test_what_the_list_refuses(env, oracle):
     y = torch.zeros((1, 64), dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.WqError, match="group size"):
         ops.GptqGemvList([(w, u.dev(x), y)])
+    # an error found by the code shared with the q4f16_1 lists names the entry point that was called
+    x2, qw2, qz2, s2, g2 = oracle.make_gptq_inputs(1, 64, 64, 32, seed=8)
+    w2 = ops.gptq_prepare(u.dev(qw2), u.dev(qz2), u.dev(s2), u.dev(g2))
+    with pytest.raises(_lib.WqError, match="wq_gptq_gemv_list_create: linear 0: y overlaps x"):
+        ops.GptqGemvList([(w2, y, y)])
     g_idx = np.random.default_rng(1).integers(0, 2, size=192).astype(np.int32)  # groups of unequal size
     w = ops.gptq_prepare_padded(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
     with pytest.raises(ValueError, match="padded"):
