@@ -20,7 +20,7 @@ reference's path timed on this machine's host cores.  Further objects on the sam
 line: `stack` (32 decoder layers' linears run as one captured instruction list at
 M = 1, 8, 16, 32), `fpA_intB` (int8 per-channel weights, K=8192, N=28672, M = 1, 16,
 128, 512), `autogptq` (N = K = 4096; under `larger_shapes` 4096 -> 22016 and 11008 -> 4096; under `decode_step_as_list`
-the four decoder linears as one launch against four) and `kn_gemv` (the
+the four decoder linears as one launch against four; under `stack` the 32-layer stack) and `kn_gemv` (the
 neighbouring checkpoint layouts at decode) and
 `calibration` (measured pure-read and MFMA-only ceilings); `single_gemv_4096x4096` (one linear per launch, with
 its own roofline), `list_steady_state` (the list kernel over 906 MB in one launch) and `f16acc` (the
@@ -421,6 +421,48 @@ def bench_autogptq_list(torch, ops, copies=6, group=128):
     return res
 
 
+def bench_autogptq_stack(torch, ops, layers=32, group=128):
+    """The 32-layer stack of `stack` with AutoGPTQ layers (group 128, rows in group order) at M = 1: 128
+    `relax_amd.autogptq_matmul` calls per step, run by the executor as one launch, and call by call."""
+    from relax_amd import vm
+
+    g = torch.Generator(device="cuda")
+    g.manual_seed(14)
+    weights = []
+    for _ in range(layers):
+        layer = {}
+        for name, N, K in vm.LLAMA7B_LINEARS:
+            G = K // group
+            qw = torch.randint(-2**31, 2**31 - 1, (K // 8, N), dtype=torch.int32, device="cuda", generator=g)
+            qz = torch.randint(-2**31, 2**31 - 1, (G, N // 8), dtype=torch.int32, device="cuda", generator=g)
+            sc = (torch.rand((G, N), device="cuda", generator=g) * 0.0015 + 0.0005).to(torch.float16)
+            gi = (torch.arange(K, device="cuda") // group).to(torch.int32)
+            layer[name] = ops.gptq_prepare(qw, qz, sc, gi)
+            del qw, qz, sc
+        weights.append(layer)
+    hidden = torch.randn((1, 4096), device="cuda", dtype=torch.float16)
+    attn = torch.randn((1, 4096), device="cuda", dtype=torch.float16)
+    act = torch.randn((1, 11008), device="cuda", dtype=torch.float16)
+    outp = torch.empty((1, 4096), device="cuda", dtype=torch.float16)
+    nbytes = layers * sum(N * K // 2 + N * (K // group) * 4 + K * 2 + N * 2 for _, N, K in vm.LLAMA7B_LINEARS)
+    res = {"layers": layers, "group_size": group, "M": 1, "bytes_per_step": nbytes}
+    stream = torch.cuda.Stream()
+    for name, fuse in (("one_launch", 1), ("call_by_call", 0)):
+        prog = vm.llama_autogptq_stack(weights, hidden, attn, act, outp)
+        prog.set_option("fuse_decode", fuse)
+        prog.plan()
+        prog.capture(stream)
+        prog.replay(stream)
+        stream.synchronize()
+        ms, _ = _measure(torch, stream, lambda: prog.replay(stream), min_ms=MIN_SAMPLE_MS / 2, samples=3)
+        prog.status(stream)
+        res[name] = {"ms_per_step": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1),
+                     "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                     "launches_per_step": 4 * layers - sum(len(prog.fused_order(i)) - 1 for i in range(prog.num_fused_groups))}
+        del prog
+    return res
+
+
 def bench_kn_gemv(torch, ops, copies=24):
     """The decode linear over K-major (KN) q4f16_1 weights used in place (`wq_q4g32_kn_gemv`), M = 1, the
     four Llama-2-7B shapes; `copies` weight copies (more than the last-level cache) are cycled inside one
@@ -783,6 +825,8 @@ def main():
         out["autogptq"] = bench_autogptq(torch, ops)
         # the same layer type at the two large decoder shapes (the 4096 x 4096 matrix is 8.9 MB: launch-bound)
         out["autogptq"]["decode_step_as_list"] = bench_autogptq_list(torch, ops)
+        out["autogptq"]["stack"] = bench_autogptq_stack(torch, ops)
+        torch.cuda.empty_cache()
         out["autogptq"]["larger_shapes"] = [bench_autogptq(torch, ops, K=4096, N=22016, batches=(1,), copies=12),
                                             bench_autogptq(torch, ops, K=11008, N=4096, batches=(1,), copies=24)]
         out["kn_gemv"] = bench_kn_gemv(torch, ops)

@@ -190,3 +190,38 @@ def llama_linear_stack(weights, M: int, hidden: torch.Tensor, attn_out: torch.Te
         p.call("relax_amd.q4f16_1_matmul", *regs["down_proj"], g, nxt)
         h = nxt
     return p
+
+
+def llama_autogptq_stack(weights, hidden: torch.Tensor, attn_out: torch.Tensor, mlp_act: torch.Tensor,
+                         out: torch.Tensor, linears=LLAMA7B_LINEARS) -> DpsProgram:
+    """:func:`llama_linear_stack` for AutoGPTQ layers at one row of activations: ``weights[l][name]`` is a
+    prepared layer (``ops.GptqWeight`` from ``ops.gptq_prepare``, with or without a row order); every linear is a
+    ``relax_amd.autogptq_matmul`` call without residual, and a layer with a row order gets a planned gather
+    workspace (which a fused run does not use)."""
+    from . import ops
+
+    p = DpsProgram()
+    h = p.external(hidden)
+    a = p.external(attn_out)
+    g = p.external(mlp_act)
+    dims = {name: (n, k) for name, n, k in linears}
+    L = len(weights)
+
+    def call(w, x, y):
+        regs = (p.external(w.W_nk, as_uint32=True), p.external(w.SZ), p.external(w.perm) if w.perm is not None else None)
+        if w.perm is not None:
+            p.call("relax_amd.autogptq_matmul", *regs, x, None, y, p.planned((ops.gptq_workspace_bytes(1, w.K, True),), torch.uint8))
+        else:
+            p.call("relax_amd.autogptq_matmul", *regs, x, None, y)
+
+    for l, layer in enumerate(weights):
+        qkv = p.planned((1, dims["qkv_proj"][0]))
+        call(layer["qkv_proj"], h, qkv)
+        o = p.planned((1, dims["o_proj"][0]))
+        call(layer["o_proj"], a, o)
+        gu = p.planned((1, dims["gate_up_proj"][0]))
+        call(layer["gate_up_proj"], o, gu)
+        nxt = p.external(out) if l == L - 1 else p.planned((1, dims["down_proj"][0]))
+        call(layer["down_proj"], g, nxt)
+        h = nxt
+    return p

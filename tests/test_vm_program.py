@@ -661,3 +661,44 @@ def test_autogptq_decoder_layer_is_one_launch(oracle, act_order):
         for g, k in zip(got, keep):
             assert torch.equal(g, k)
     fused.status()
+
+
+@pytest.mark.gpu
+def test_autogptq_stack_program_fused_against_call_by_call(oracle):
+    """vm.llama_autogptq_stack on a small stack (3 layers, every other layer with a row order): the fused program
+    (one launch) against the same program run call by call, and its last output against the oracle."""
+    import torch
+
+    from relax_amd import ops, vm
+    from tests import gpu_util as u
+
+    linears = (("qkv_proj", 384, 128), ("o_proj", 128, 128), ("gate_up_proj", 704, 128), ("down_proj", 128, 352))
+    rng = np.random.default_rng(3)
+    weights, dense = [], []
+    for l in range(3):
+        layer, dl = {}, {}
+        for name, N, K in linears:
+            _, qw, qz, s, g_idx = oracle.make_gptq_inputs(1, N, K, 32, seed=60 + 7 * l + len(name), act_order=(l % 2 == 1))
+            s = (s.astype(np.float32) * 0.3).astype(np.float16)
+            layer[name] = ops.gptq_prepare(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
+            dl[name] = np.ascontiguousarray(oracle.gptq_dequant(qw, qz, s, g_idx).T)
+        weights.append(layer)
+        dense.append(dl)
+    hidden = rng.standard_normal((1, 128)).astype(np.float16)
+    attn = rng.standard_normal((1, 128)).astype(np.float16)
+    act = rng.standard_normal((1, 352)).astype(np.float16)
+    outs = []
+    for fuse in (1, 0):
+        out = torch.zeros((1, 128), dtype=torch.float16, device="cuda")
+        p = vm.llama_autogptq_stack(weights, u.dev(hidden), u.dev(attn), u.dev(act), out, linears=linears)
+        p.set_option("fuse_decode", fuse)
+        p.plan()
+        p.run()
+        torch.cuda.synchronize()
+        p.status()
+        assert p.num_fused_groups == (1 if fuse else 0)
+        outs.append(u.host(out))
+    # only down_proj of the last layer reaches `out`, and its input is the stand-in activation
+    want = oracle.nt_matmul_f32acc(dense[-1]["down_proj"], act)
+    u.assert_close(outs[0], want, "autogptq stack, fused")
+    u.assert_close(outs[1], want, "autogptq stack, call by call")
