@@ -47,18 +47,19 @@ __global__ __launch_bounds__(256) void q4n32_scales_kernel(const half_t* __restr
 // y[n] = sum_k x[k] s[k, g] (code[k, n] - 7) with g = n / 32: for the 32 rows of W_nk of one group the scales
 // belong to the ACTIVATIONS, xs[k] = fp16(x[k] * ST[g][k]), and what is left is format A's decode GEMV with every
 // scale 1.  A workgroup takes RPW rows of one group: it stages xs in LDS (in the pairing of the unpack, with the
-// zero-point constant of every 32 k, as q4_gemv.h does), then its four wavefronts stream two rows each at a time,
-// lane l the 16-byte pieces l, l + 64, ... of a row.  One rounding differs from the reference: it rounds
+// zero-point constant of every 32 k, as q4_gemv.h does) for MB rows of x, then its four wavefronts stream two rows
+// of W each at a time, lane l the 16-byte pieces l, l + 64, ... of a row, every unpacked word against all MB rows.  One rounding differs from the reference: it rounds
 // (code - 7) * s to fp16 and multiplies by x in fp32, here x * s is rounded and (code - 7) is exact; a one-hot x
 // still returns the reference's weight bit for bit.
+template <int MB>
 __global__ __launch_bounds__(256) void q4n32_gemv_kernel(const uint4_t* __restrict__ W, const half_t* __restrict__ ST,
                                                          const half_t* __restrict__ x, const half_t* __restrict__ bias,
                                                          const half_t* __restrict__ residual, half_t* __restrict__ y,
                                                          int N, int K, int rpw) {
   extern __shared__ uint4_t smem[];
-  const int G = K >> 5;                                       // pieces of 32 k per row
-  uint4_t* xs = smem;                                         // [4][G]: word ch of piece g at ch * G + g
-  float* cs = reinterpret_cast<float*>(smem + 4 * (size_t)G);  // [G]: -(1031 A + 71 B) of the piece
+  const int G = K >> 5;                                             // pieces of 32 k per row
+  uint4_t* xs = smem;                                               // [MB][4][G]: word ch of piece g of row m at (m * 4 + ch) * G + g
+  float* cs = reinterpret_cast<float*>(smem + MB * 4 * (size_t)G);  // [MB][G]: -(1031 A + 71 B) of the piece
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * rpw;
   const half_t* st = ST + (int64_t)(n0 >> 5) * K;
@@ -66,30 +67,35 @@ __global__ __launch_bounds__(256) void q4n32_gemv_kernel(const uint4_t* __restri
   const half2_t k71 = {(half_t)71.0f, (half_t)71.0f};
   const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
   for (int wi = tid; wi < (K >> 3); wi += 256) {  // K % 32 == 0: the 4 words of a piece sit in 4 adjacent lanes
-    const uint4_t xv = reinterpret_cast<const uint4_t*>(x)[wi];
     const uint4_t sv = reinterpret_cast<const uint4_t*>(st)[wi];
-    const uint32_t in[4] = {as_u32(as_half2(xv.x) * as_half2(sv.x)), as_u32(as_half2(xv.y) * as_half2(sv.y)),
-                            as_u32(as_half2(xv.z) * as_half2(sv.z)), as_u32(as_half2(xv.w) * as_half2(sv.w))};
-    uint32_t o[4];
-    pair_i_i4(in, o);  // o[i] = (xs_i, xs_{i+4})
-    float c = dot2(as_half2(o[0]), k1031, 0.0f);
-    c = dot2(as_half2(o[1]), k71, c);
-    c = dot2(as_half2(o[2]), k1031, c);
-    c = dot2(as_half2(o[3]), k71, c);
-    c += dpp_shift<0xb1, 0xf>(c);
-    c += dpp_shift<0x4e, 0xf>(c);
     const int g = wi >> 2, ch = wi & 3;
-    xs[ch * G + g] = uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
-    if (ch == 0) cs[g] = -c;
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const uint4_t xv = reinterpret_cast<const uint4_t*>(x + (int64_t)m * K)[wi];
+      const uint32_t in[4] = {as_u32(as_half2(xv.x) * as_half2(sv.x)), as_u32(as_half2(xv.y) * as_half2(sv.y)),
+                              as_u32(as_half2(xv.z) * as_half2(sv.z)), as_u32(as_half2(xv.w) * as_half2(sv.w))};
+      uint32_t o[4];
+      pair_i_i4(in, o);  // o[i] = (xs_i, xs_{i+4})
+      float c = dot2(as_half2(o[0]), k1031, 0.0f);
+      c = dot2(as_half2(o[1]), k71, c);
+      c = dot2(as_half2(o[2]), k1031, c);
+      c = dot2(as_half2(o[3]), k71, c);
+      c += dpp_shift<0xb1, 0xf>(c);
+      c += dpp_shift<0x4e, 0xf>(c);
+      xs[(m * 4 + ch) * G + g] = uint4_t{o[0], as_u32(as_half2(o[1]) * sixteenth), o[2], as_u32(as_half2(o[3]) * sixteenth)};
+      if (ch == 0) cs[m * G + g] = -c;
+    }
   }
   __syncthreads();
   const uint32_t magic = 0x64006400u;
-  for (int r = wave * 2; r < rpw; r += 8) {  // two rows at a time share the reads of xs
+  for (int r = wave * 2; r < rpw; r += 8) {  // two rows of W at a time share the reads of xs
     const int na = n0 + r, nb = na + 1;
     if (na >= N) break;
     const uint4_t* wa = W + (int64_t)na * G;
     const uint4_t* wb = W + (int64_t)min(nb, N - 1) * G;
-    float acc_a = 0.0f, acc_b = 0.0f;
+    float acc_a[MB], acc_b[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc_a[m] = acc_b[m] = 0.0f;
     constexpr int UNR = 2;  // pieces per lane and row requested before the first is multiplied
     for (int g0 = lane; g0 < G; g0 += 64 * UNR) {
       uint4_t qa[UNR], qb[UNR];
@@ -103,34 +109,62 @@ __global__ __launch_bounds__(256) void q4n32_gemv_kernel(const uint4_t* __restri
       for (int j = 0; j < UNR; ++j) {
         const int g = g0 + 64 * j;
         if (g >= G) break;
-        float ga = cs[g], gb = ga;
+        float ga[MB], gb[MB];
+#pragma unroll
+        for (int m = 0; m < MB; ++m) ga[m] = gb[m] = cs[m * G + g];
 #pragma unroll
         for (int ch = 0; ch < 4; ++ch) {
-          const uint4_t xv = xs[ch * G + g];
           const uint32_t a = ch == 0 ? qa[j].x : ch == 1 ? qa[j].y : ch == 2 ? qa[j].z : qa[j].w;
           const uint32_t b = ch == 0 ? qb[j].x : ch == 1 ? qb[j].y : ch == 2 ? qb[j].z : qb[j].w;
           const uint32_t a8 = a >> 8, b8 = b >> 8;
-          ga = dot2(as_half2(and_or(a, 0x000F000Fu, magic)), as_half2(xv.x), ga);  // 1024 + (q0, q4)
-          ga = dot2(as_half2(and_or(a, 0x00F000F0u, magic)), as_half2(xv.y), ga);  // 1024 + 16 (q1, q5)
-          ga = dot2(as_half2(and_or(a8, 0x000F000Fu, magic)), as_half2(xv.z), ga);
-          ga = dot2(as_half2(and_or(a8, 0x00F000F0u, magic)), as_half2(xv.w), ga);
-          gb = dot2(as_half2(and_or(b, 0x000F000Fu, magic)), as_half2(xv.x), gb);
-          gb = dot2(as_half2(and_or(b, 0x00F000F0u, magic)), as_half2(xv.y), gb);
-          gb = dot2(as_half2(and_or(b8, 0x000F000Fu, magic)), as_half2(xv.z), gb);
-          gb = dot2(as_half2(and_or(b8, 0x00F000F0u, magic)), as_half2(xv.w), gb);
+          const half2_t a0 = as_half2(and_or(a, 0x000F000Fu, magic)), a1 = as_half2(and_or(a, 0x00F000F0u, magic));    // 1024 + (q0, q4), 1024 + 16 (q1, q5)
+          const half2_t a2 = as_half2(and_or(a8, 0x000F000Fu, magic)), a3 = as_half2(and_or(a8, 0x00F000F0u, magic));
+          const half2_t b0 = as_half2(and_or(b, 0x000F000Fu, magic)), b1 = as_half2(and_or(b, 0x00F000F0u, magic));
+          const half2_t b2 = as_half2(and_or(b8, 0x000F000Fu, magic)), b3 = as_half2(and_or(b8, 0x00F000F0u, magic));
+#pragma unroll
+          for (int m = 0; m < MB; ++m) {
+            const uint4_t xv = xs[(m * 4 + ch) * G + g];
+            ga[m] = dot2(a0, as_half2(xv.x), ga[m]);
+            ga[m] = dot2(a1, as_half2(xv.y), ga[m]);
+            ga[m] = dot2(a2, as_half2(xv.z), ga[m]);
+            ga[m] = dot2(a3, as_half2(xv.w), ga[m]);
+            gb[m] = dot2(b0, as_half2(xv.x), gb[m]);
+            gb[m] = dot2(b1, as_half2(xv.y), gb[m]);
+            gb[m] = dot2(b2, as_half2(xv.z), gb[m]);
+            gb[m] = dot2(b3, as_half2(xv.w), gb[m]);
+          }
         }
-        acc_a += ga;
-        acc_b += gb;
+#pragma unroll
+        for (int m = 0; m < MB; ++m) {
+          acc_a[m] += ga[m];
+          acc_b[m] += gb[m];
+        }
       }
     }
-    acc_a = wave_sum_to_lane63(acc_a);
-    acc_b = wave_sum_to_lane63(acc_b);
-    if (lane == 63) {
-      const Q4G32Epilogue ep{bias, residual, N};
-      y[na] = ep(acc_a, 0, na);
-      if (nb < N && r + 1 < rpw) y[nb] = ep(acc_b, 0, nb);
+    const Q4G32Epilogue ep{bias, residual, N};
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const float ta = wave_sum_to_lane63(acc_a[m]), tb = wave_sum_to_lane63(acc_b[m]);
+      if (lane == 63) {
+        y[(int64_t)m * N + na] = ep(ta, m, na);
+        if (nb < N && r + 1 < rpw) y[(int64_t)m * N + nb] = ep(tb, m, nb);
+      }
     }
   }
+}
+
+template <int MB>
+static int launch_q4n32_gemv(const uint32_t* W_nk, const uint16_t* ST, const uint16_t* x, const uint16_t* bias,
+                             const uint16_t* residual, uint16_t* y, int64_t N, int64_t K, hipStream_t stream) {
+  const size_t lds = MB * ((size_t)K * 2 + (size_t)(K / 32) * 4);
+  const int cus = cu_count();
+  const int rpw = N / 32 >= 4 * cus ? 32 : N / 16 >= 4 * cus ? 16 : 8;
+  static DynamicLdsLimit limit;
+  WQ_HIP(limit.ensure(reinterpret_cast<const void*>(q4n32_gemv_kernel<MB>), (int)lds));
+  WQ_LAUNCH("wq_q4n32_linear", q4n32_gemv_kernel<MB>, dim3((unsigned)((N + rpw - 1) / rpw)), dim3(256), lds, stream,
+            (const uint4_t*)W_nk, (const half_t*)ST, (const half_t*)x, (const half_t*)bias, (const half_t*)residual,
+            (half_t*)y, (int)N, (int)K, rpw);
+  return WQ_OK;
 }
 
 // Weight policy of gemm_lds_kernel: the code stream of format A, scales per (k, group of 32 columns).
@@ -222,18 +256,25 @@ extern "C" int wq_q4n32_linear(const uint32_t* W_nk, const uint16_t* ST, const u
   WQ_REQUIRE(aligned16(W_nk) && aligned16(x) && (reinterpret_cast<uintptr_t>(ST) & 3u) == 0,
              "wq_q4n32_linear: W_nk and x must be 16-byte aligned, ST 4-byte aligned");
   WQ_REQUIRE(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), "wq_q4n32_linear: too large");
-  // a few rows of x: the streaming kernel, one launch per row (the GEMM below costs the same from 1 to 128 rows)
-  const size_t gemv_lds = (size_t)K * 2 + (size_t)(K / 32) * 4;
-  if (M <= WQ_Q4N32_GEMV_MAX_M && gemv_lds <= 96 * 1024 && !tuning().gemm_cfg) {
-    const int cus = cu_count();
-    const int rpw = N / 32 >= 4 * cus ? 32 : N / 16 >= 4 * cus ? 16 : 8;
-    static DynamicLdsLimit limit;
-    WQ_HIP(limit.ensure(reinterpret_cast<const void*>(q4n32_gemv_kernel), (int)gemv_lds));
-    for (int64_t m = 0; m < M; ++m)
-      WQ_LAUNCH("wq_q4n32_linear", q4n32_gemv_kernel, dim3((unsigned)((N + rpw - 1) / rpw)), dim3(256), gemv_lds, stream,
-                (const uint4_t*)W_nk, (const half_t*)ST, (const half_t*)(x + m * K), (const half_t*)bias,
-                residual ? (const half_t*)(residual + m * N) : nullptr, (half_t*)(y + m * N), (int)N, (int)K, rpw);
-    return WQ_OK;
+  // a few rows of x: the streaming kernel, as many rows per pass over the weights as their staged activations
+  // fit the LDS (the GEMM below costs the same from 1 to 128 rows)
+  if (M <= WQ_Q4N32_GEMV_MAX_M && !tuning().gemm_cfg) {
+    const size_t per_row = (size_t)K * 2 + (size_t)(K / 32) * 4;
+    // (64 KiB of LDS leave room for two workgroups per CU; a single row may take up to 96 KiB)
+    const int64_t fit = std::min<int64_t>(4, std::max<int64_t>((int64_t)((64 * 1024) / per_row), per_row <= 96 * 1024 ? 1 : 0));
+    if (fit >= 1) {
+      for (int64_t m = 0; m < M;) {
+        const int64_t mb = std::min(fit, M - m);
+        const uint16_t* r = residual ? residual + m * N : nullptr;
+        const int rc = mb >= 4   ? launch_q4n32_gemv<4>(W_nk, ST, x + m * K, bias, r, y + m * N, N, K, stream)
+                       : mb == 3 ? launch_q4n32_gemv<3>(W_nk, ST, x + m * K, bias, r, y + m * N, N, K, stream)
+                       : mb == 2 ? launch_q4n32_gemv<2>(W_nk, ST, x + m * K, bias, r, y + m * N, N, K, stream)
+                                 : launch_q4n32_gemv<1>(W_nk, ST, x + m * K, bias, r, y + m * N, N, K, stream);
+        if (rc != WQ_OK) return rc;
+        m += mb;
+      }
+      return WQ_OK;
+    }
   }
   const Q4N32LdsPolicy::Args args{W_nk, (const half_t*)ST};
   const Q4G32Epilogue ep{(const half_t*)bias, (const half_t*)residual, (int)N};
