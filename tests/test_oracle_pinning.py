@@ -302,3 +302,24 @@ def test_kn_layout_oracle_matches_loops_and_nk_form(oracle):
     y = oracle.q4g32_kn_linear(W_kn, S_kn, x)
     y_nk = oracle.q4g32_linear(np.ascontiguousarray(W_kn.T), np.ascontiguousarray(S_kn.T), x)
     assert np.allclose(y.astype(np.float32), y_nk.astype(np.float32), rtol=2e-3, atol=2e-3)
+
+
+def test_weights_packed_along_n_are_format_a_with_the_dimensions_exchanged(oracle):
+    """The decode block of tests/python/dlight/test_gpu_matmul.py:366-377, written out index by index
+    (D[i, j] from W[i, j // 8] and S[i, j // 32]), and its matmul (:378-383, D[k, n]) in float64: the oracle the GPU
+    tests of that layout use — wqo_q4g32_dequant on the same two arrays, then the NT matmul over the transpose."""
+    K, N, M = 24, 96, 3
+    rng = np.random.default_rng(17)
+    W = rng.integers(0, 2**32, size=(K, N // 8), dtype=np.uint64).astype(np.uint32)
+    S = rng.uniform(0.005, 0.02, size=(K, N // 32)).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    D = np.zeros((K, N), np.float16)
+    for i in range(K):
+        for j in range(N):
+            code = (int(W[i, j // 8]) >> ((j % 8) * 4)) & 15
+            D[i, j] = np.float16(np.float16(code) - np.float16(7)) * S[i, j // 32]
+    got = oracle.q4g32_dequant(W, S)
+    assert got.shape == (K, N) and np.array_equal(got.view(np.uint16), D.view(np.uint16))
+    y = oracle.nt_matmul_f32acc(np.ascontiguousarray(got.T), x)
+    want = x.astype(np.float64) @ D.astype(np.float64)
+    assert np.allclose(y.astype(np.float64), want, rtol=2e-3, atol=2e-3)
