@@ -50,6 +50,10 @@ WQ_PACKED(relax_amd_ft_preprocess_weight_dps);
 WQ_PACKED(relax_amd_q4f16_1_matmul);
 WQ_PACKED(relax_amd_q4f16_1_matmul_bias);
 WQ_PACKED(relax_amd_q4f16_1_matmul_bias_residual);
+/* "relax_amd.q4f16_1_matmul_f16acc"(W, S, x f16[..,K], out f16[..,N]): the matmul with the fp16 accumulation of the
+ * decode fixtures (tests/python/dlight/test_gpu_reduction.py:44-51, test_gpu_low_batch_gemv.py:50-57); a decode /
+ * low-batch entry (wq_q4g32_gemv_f16acc), no epilogue. */
+WQ_PACKED(relax_amd_q4f16_1_matmul_f16acc);
 /* "relax_amd.q4f16_1_decode"(W, S, out f16[N,K]): the decode block alone. */
 WQ_PACKED(relax_amd_q4f16_1_decode);
 /* Weight preparation, destination-passing:

@@ -383,6 +383,36 @@ WQ_PACKED(relax_amd_q4f16_1_matmul_bias_residual) {
   (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
   return q4_matmul("relax_amd.q4f16_1_matmul_bias_residual", args, type_codes, num_args, true, true);
 }
+// (W, S, x fp16 [.., K], out fp16 [.., N]): the matmul with the reference's fp16 accumulation
+// (tests/python/dlight/test_gpu_reduction.py:44-51, test_gpu_low_batch_gemv.py:50-57): a decode / low-batch entry
+WQ_PACKED(relax_amd_q4f16_1_matmul_f16acc) {
+  (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
+  const char* who = "relax_amd.q4f16_1_matmul_f16acc";
+  Tensor W, S, x, y;
+  if (num_args != 4) {
+    fail(WQ_EINVAL, "%s: expected (W, S, x, out)", who);
+    return packed_fail();
+  }
+  if (!get_tensor(who, args, type_codes, num_args, 0, kDLUInt, 32, "W", &W) ||
+      !get_tensor(who, args, type_codes, num_args, 1, kDLFloat, 16, "S", &S) ||
+      !get_tensor(who, args, type_codes, num_args, 2, kDLFloat, 16, "x", &x) ||
+      !get_tensor(who, args, type_codes, num_args, 3, kDLFloat, 16, "out", &y))
+    return packed_fail();
+  if (W.t->ndim != 2 || S.t->ndim != 2 || x.t->ndim < 1 || y.t->ndim < 1) {
+    fail(WQ_EINVAL, "%s: W and S must be matrices", who);
+    return packed_fail();
+  }
+  const int64_t N = W.t->shape[0], K = W.t->shape[1] * 8;
+  const int64_t M = leading(x.t);
+  if (S.t->shape[0] != N || S.t->shape[1] * 32 != K || x.t->shape[x.t->ndim - 1] != K || y.numel != M * N ||
+      y.t->shape[y.t->ndim - 1] != N) {
+    fail(WQ_EINVAL, "%s: inconsistent shapes (N=%lld K=%lld M=%lld)", who, (long long)N, (long long)K, (long long)M);
+    return packed_fail();
+  }
+  const int rc = wq_q4g32_gemv_f16acc((const uint32_t*)W.ptr, (const uint16_t*)S.ptr, (const uint16_t*)x.ptr,
+                                      (uint16_t*)y.ptr, M, N, K, current_stream());
+  return rc == WQ_OK ? 0 : packed_fail();
+}
 WQ_PACKED(relax_amd_q4f16_1_decode) {
   (void)resource_handle; (void)out_ret_value; (void)out_ret_tcode;
   const char* who = "relax_amd.q4f16_1_decode";
@@ -848,6 +878,7 @@ const std::vector<Entry>& table() {
     v.push_back({"relax_amd.q4f16_1_encode", "relax_amd_q4f16_1_encode", relax_amd_q4f16_1_encode});
     v.push_back({"relax_amd.q4f16_1_kn_to_nk", "relax_amd_q4f16_1_kn_to_nk", relax_amd_q4f16_1_kn_to_nk});
     v.push_back({"relax_amd.q4f16_1_kn_matmul", "relax_amd_q4f16_1_kn_matmul", relax_amd_q4f16_1_kn_matmul});
+    v.push_back({"relax_amd.q4f16_1_matmul_f16acc", "relax_amd_q4f16_1_matmul_f16acc", relax_amd_q4f16_1_matmul_f16acc});
     v.push_back({"relax_amd.q4f16_1_ngroup_prepare", "relax_amd_q4f16_1_ngroup_prepare", relax_amd_q4f16_1_ngroup_prepare});
     v.push_back({"relax_amd.q4f16_1_ngroup_matmul_bias_residual", "relax_amd_q4f16_1_ngroup_matmul_bias_residual",
                  relax_amd_q4f16_1_ngroup_matmul_bias_residual});

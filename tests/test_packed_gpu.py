@@ -268,6 +268,33 @@ def test_q4f16_1_kn_matmul(env, oracle):
     assert rc == -1
 
 
+def test_q4f16_1_matmul_f16acc(env, oracle):
+    """relax_amd.q4f16_1_matmul_f16acc: the fp16-accumulate mode of the decode fixtures with a small dynamic batch;
+    the same bits as the C entry point, and within the fp16 accumulation bound of the fp32-accumulate result."""
+    lib, u, T, torch = env
+    from relax_amd import ops
+
+    M, N, K = 5, 264, 2048
+    x, W, S = oracle.make_q4g32_inputs(M, N, K, seed=60)
+    dW, dS, dx = u.dev(W), u.dev(S), u.dev(x.reshape(M, 1, K))
+    y = torch.empty((M, 1, N), dtype=torch.float16, device="cuda")
+    tW, _ = T.from_torch(dW, "uint32")
+    tS, _ = T.from_torch(dS)
+    tx, _ = T.from_torch(dx)
+    ty, _ = T.from_torch(y)
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_matmul_f16acc, tW, tS, tx, ty)
+    assert rc == 0, lib.wq_last_error()
+    direct = ops.q4g32_gemv_f16acc(dW, dS, u.dev(x))
+    assert torch.equal(y.reshape(M, N), direct)
+    ref = oracle.q4g32_linear(W, S, x).astype(np.float64)
+    mag = np.abs(x).astype(np.float64) @ np.abs(oracle.q4g32_dequant(W, S)).astype(np.float64).T
+    assert np.all(np.abs(u.host(y).reshape(M, N) - ref) <= 1.1 * (16 + 8 + 2) * 2.0**-11 * mag + 1e-6)
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_matmul_f16acc, tW, tS, tx)
+    assert rc == -1
+    rc, _, _ = T.call(lib.relax_amd_q4f16_1_matmul_f16acc, tW, tW, tx, ty)
+    assert rc == -1
+
+
 def test_q4f16_1_ngroup_pair(env, oracle):
     """relax_amd.q4f16_1_ngroup_prepare / _matmul_bias_residual: the operands and the buffer order of
     tests/python/dlight/test_gpu_matmul.py:352-401 (codes packed along N; dynamic n rows of x)."""
