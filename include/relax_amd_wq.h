@@ -106,13 +106,14 @@ int wq_q4g32_gemm(const uint32_t* W, const uint16_t* S, const uint16_t* x, const
  *          along k.  K % 8 == 0, N % 32 == 0.
  * linear   over the prepared operands, any M (the fixture's n is dynamic).  More than WQ_Q4N32_GEMV_MAX_M rows: the
  *          matrix-core GEMM; every weight is the reference's fp16 value bit for bit ((code - 7) is exact, the
- *          product rounds once).  Up to that many rows: a streaming kernel, one pass over the weights per 4 rows of
+ *          product rounds once).  Up to 8 rows, and up to WQ_Q4N32_GEMV_MAX_M where that is the faster way (small
+ *          matrices, whose GEMM fills few CUs): a streaming kernel, one pass over the weights per 4 rows of
  *          x (fewer where K > 15000), which rounds x[k] * s[k, n/32] to fp16 instead (the scales of a group of 32 columns belong to the
  *          activations there) and keeps (code - 7) exact.  K % 64 == 0, N % 32 == 0; bias fp16 [N] / residual
  *          fp16 [M, N] may be NULL.
  * The fp16 weight itself, [K, N], is what wq_q4g32_dequantize(W, S, out, K, N) returns for these operands (the
  * decode of format A with the two dimensions exchanged). */
-#define WQ_Q4N32_GEMV_MAX_M 8
+#define WQ_Q4N32_GEMV_MAX_M 64
 int wq_q4n32_prepare(const uint32_t* W, const uint16_t* S, uint32_t* W_nk, uint16_t* ST, int64_t K, int64_t N,
                      wq_stream_t stream);
 int wq_q4n32_linear(const uint32_t* W_nk, const uint16_t* ST, const uint16_t* x, const uint16_t* bias,

@@ -256,13 +256,24 @@ extern "C" int wq_q4n32_linear(const uint32_t* W_nk, const uint16_t* ST, const u
   WQ_REQUIRE(aligned16(W_nk) && aligned16(x) && (reinterpret_cast<uintptr_t>(ST) & 3u) == 0,
              "wq_q4n32_linear: W_nk and x must be 16-byte aligned, ST 4-byte aligned");
   WQ_REQUIRE(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), "wq_q4n32_linear: too large");
-  // a few rows of x: the streaming kernel, as many rows per pass over the weights as their staged activations
-  // fit the LDS (the GEMM below costs the same from 1 to 128 rows)
+  // A few rows of x: the streaming kernel, as many rows per pass over the weights as their staged activations fit
+  // the LDS.  The GEMM below costs the same from 1 to 128 rows (one round of few tiles, about 0.52 us per K-step of
+  // the 128-row tiles it would use), a pass of the streaming kernel about 2 us + 0.5 us per MB of weights (measured
+  // at 4096 x 4096, 11008 x 4096 and 4096 x 11008): up to 8 rows always stream, beyond that whichever is cheaper.
   if (M <= WQ_Q4N32_GEMV_MAX_M && !tuning().gemm_cfg) {
     const size_t per_row = (size_t)K * 2 + (size_t)(K / 32) * 4;
     // (64 KiB of LDS leave room for two workgroups per CU; a single row may take up to 96 KiB)
     const int64_t fit = std::min<int64_t>(4, std::max<int64_t>((int64_t)((64 * 1024) / per_row), per_row <= 96 * 1024 ? 1 : 0));
-    if (fit >= 1) {
+    bool stream_it = fit >= 1;
+    if (stream_it && M > 8) {
+      const double passes = (double)((M + fit - 1) / fit);
+      const double t_stream = passes * (2.0 + 0.5 * ((double)N * (double)K / 2.0) / 1e6);
+      const int64_t tiles = ((N + 127) / 128) * ((M + 127) / 128);
+      const double rounds = (double)((tiles + 2 * cu_count() - 1) / (2 * cu_count()));  // two 128 x 128 tiles per CU
+      const double t_gemm = 0.52 * (double)(K / 64) * rounds;
+      stream_it = t_stream < t_gemm;
+    }
+    if (stream_it) {
       for (int64_t m = 0; m < M;) {
         const int64_t mb = std::min(fit, M - m);
         const uint16_t* r = residual ? residual + m * N : nullptr;

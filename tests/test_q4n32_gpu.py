@@ -49,10 +49,11 @@ def test_prepare_is_a_pure_rearrangement(env, oracle):
 
 # the fixture's shape (4096 x 4096, dynamic n) at several n; ragged tiles: N not a multiple of the tile width,
 # M one row, one more than a tile, K of one and of a few steps
-# (up to 8 rows of x run the streaming kernel, up to 4 rows per pass over the weights; more, the matrix-core GEMM)
+# (up to 8 rows of x run the streaming kernel, up to 4 rows per pass over the weights, and more rows where that is
+# cheaper than a GEMM of few tiles: 17 x 4096 x 4096 streams, 17 x 11008 x 4096 does not; else the matrix-core GEMM)
 # (N = 16384 and 32800: the streaming kernel with 16 and with 32 rows per workgroup)
 SHAPES = [(1, 4096, 4096), (2, 16384, 128), (1, 32800, 64), (2, 96, 64), (3, 4128, 320), (4, 11008, 4096), (1, 64, 32768), (4, 32, 28672), (2, 4096, 11008),
-          (5, 4096, 4096), (7, 4096, 4096), (8, 4128, 320), (6, 160, 11008), (3, 96, 32768), (9, 4096, 4096), (130, 4096, 4096), (513, 4096, 4096), (33, 96, 64), (257, 160, 192),
+          (5, 4096, 4096), (7, 4096, 4096), (8, 4128, 320), (6, 160, 11008), (3, 96, 32768), (9, 4096, 4096), (17, 4096, 4096), (17, 11008, 4096), (13, 256, 8192), (130, 4096, 4096), (513, 4096, 4096), (33, 96, 64), (257, 160, 192),
           (300, 4128, 320), (64, 11008, 4096), (1100, 2048, 1024)]
 
 
