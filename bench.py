@@ -363,8 +363,8 @@ def bench_autogptq(torch, ops, K=4096, N=4096, group=128, batches=(1, 8), copies
 def bench_autogptq_list(torch, ops, copies=6, group=128):
     """The decode step of the four Llama-2-7B-shaped linears as prepared AutoGPTQ layers (group 128) at M = 1,
     without and with a row order (desc_act): ONE launch of the list kernel per step (`wq_gptq_gemv_list_create`;
-    a row order is applied while the activations are staged) against four calls of `wq_gptq_linear` (each
-    preceded by a gather kernel when there is a row order); `copies` weight sets (more than the last-level
+    with a row order one small gather kernel for all four layers runs in front of it, their x coming from outside
+    the list) against four calls of `wq_gptq_linear` (each preceded by a gather kernel when there is a row order); `copies` weight sets (more than the last-level
     cache) are cycled inside one captured graph.  Bytes = codes + (scale, zero point) pairs + x + y."""
     g = torch.Generator(device="cuda")
     g.manual_seed(13)

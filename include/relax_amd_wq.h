@@ -348,7 +348,8 @@ int wq_gptq_linear(const uint32_t* W_nk, const uint16_t* SZ, const int32_t* perm
 
 /* A list of prepared AutoGPTQ layers at M = 1 as ONE launch: wq_q4g32_gemv_list_create for the layers of
  * tests/python/dlight/test_gpu_gemv.py:636-665, which the reference's GEMV rule leaves unscheduled (:667-672).
- * Same kernel design, same workspace (wq_q4g32_gemv_list_workspace_bytes), and the list is run, checked and
+ * Same kernel design, workspace of wq_gptq_gemv_list_workspace_bytes (the plain size of
+ * wq_q4g32_gemv_list_workspace_bytes is accepted as well), and the list is run, checked and
  * destroyed with the wq_q4g32_gemv_list_* calls above; arithmetic as wq_gptq_linear at M = 1.  W_nk / SZ from
  * wq_gptq_prepare; perm is the row order it wrote when it reported *needs_perm = 1 (16-byte aligned), else NULL:
  * the activations of such a layer are gathered through it while they are staged, inside the launch, so x is always
@@ -364,6 +365,12 @@ typedef struct wq_gptq_gemv_desc {
   uint16_t* y;              /* fp16 [N] */
   int64_t N, K, G;          /* K % 32 == 0, K <= WQ_GEMV_LIST_MAX_K */
 } wq_gptq_gemv_desc;
+/* Workspace for a list with row orders: wq_q4g32_gemv_list_workspace_bytes(n) plus room for the gathered activations
+ * of every layer that has one.  With that much workspace a layer with a row order whose x comes from outside the list
+ * has its activations gathered by a small kernel that wq_q4g32_gemv_list_run launches in front of the list kernel
+ * (two launches then, still capturable); with only the plain size, and for a layer fed by another linear of the
+ * list, the gather happens inside the list kernel while the activations are staged (slower by about 3 us a layer). */
+size_t wq_gptq_gemv_list_workspace_bytes(const wq_gptq_gemv_desc* descs, int n);
 wq_gemv_list_t* wq_gptq_gemv_list_create(const wq_gptq_gemv_desc* descs, int n, void* workspace,
                                          size_t workspace_bytes, wq_stream_t stream);
 

@@ -29,6 +29,7 @@ SIGNATURES = {
     "wq_q4g32_gemv_list_create": [_vp, _int, _vp, _sz, _vp],
     "wq_q4g32_gemv_list_create_batched": [_vp, _int, _int, _vp, _sz, _vp],
     "wq_gptq_gemv_list_create": [_vp, _int, _vp, _sz, _vp],
+    "wq_gptq_gemv_list_workspace_bytes": [_vp, _int],
     "wq_q4g32_gemv_list_run": [_vp, _vp],
     "wq_q4g32_gemv_list_status": [_vp, _vp],
     "wq_q4g32_gemv_list_poll": [_vp, _vp, _vp],
@@ -82,7 +83,7 @@ SIGNATURES = {
 _RESTYPES = {"wq_program_unfused_reason": ctypes.c_char_p, "wq_last_error": ctypes.c_char_p, "wq_target_arch": ctypes.c_char_p, "wq_program_create": _vp,
              "wq_program_destroy": None, "wq_program_plan": _i64, "wq_program_unplanned_bytes": _i64,
              "wq_gptq_workspace_bytes": _sz, "wq_q4g32_kn_gemv_workspace_bytes": _sz, "wq_gptq_padded_workspace_bytes": _sz, "wq_gptq_padded_k_bound": _i64, "wq_q4g32_gemv_list_workspace_bytes": _sz,
-             "wq_q4g32_gemv_list_create": _vp, "wq_q4g32_gemv_list_create_batched": _vp, "wq_gptq_gemv_list_create": _vp, "wq_q4g32_gemv_list_destroy": None}
+             "wq_q4g32_gemv_list_create": _vp, "wq_q4g32_gemv_list_create_batched": _vp, "wq_gptq_gemv_list_create": _vp, "wq_gptq_gemv_list_workspace_bytes": _sz, "wq_q4g32_gemv_list_destroy": None}
 
 # include/relax_amd_wq_testing.h: the work-split overrides of the calling thread (void) and one query (int)
 TESTING_SIGNATURES = {

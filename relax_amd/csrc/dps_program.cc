@@ -44,6 +44,7 @@ struct Instr {
 // (wq_q4g32_gemv_list_* / wq_gptq_gemv_list_create).
 struct FusedGroup {
   int first = 0, last = 0;     // instruction indices, inclusive
+  int64_t ws_bytes = 0;        // bytes of workspace of the list (wq_q4g32_gemv_list_workspace_bytes, or the AutoGPTQ size)
   std::vector<int> order;      // the order the list kernel walks them in
   int64_t ws_offset = 0;       // the list's descriptor table and counters inside the workspace
   wq_gemv_list_t* list = nullptr;
@@ -437,7 +438,18 @@ extern "C" int64_t wq_program_plan(wq_program_t* p) {
   // descriptor tables and counters of the fused groups
   for (FusedGroup& g : p->groups) {
     g.ws_offset = top;
-    const int64_t need = (int64_t)wq_q4g32_gemv_list_workspace_bytes(g.last - g.first + 1);
+    int64_t need = (int64_t)wq_q4g32_gemv_list_workspace_bytes(g.last - g.first + 1);
+    // AutoGPTQ layers with a row order: room for their gathered activations (sizes only: the addresses come later)
+    static const int32_t kHasRowOrder = 0;  // (only whether a layer has a row order counts for the size)
+    std::vector<wq_gptq_gemv_desc> shapes;
+    for (int k = g.first; k <= g.last; ++k) {
+      DecodeLinear d;
+      if (as_decode_linear(p, p->instrs[k], &d) && d.gptq)
+        shapes.push_back({nullptr, nullptr, d.perm >= 0 ? &kHasRowOrder : nullptr, nullptr, nullptr,
+                          nullptr, nullptr, d.N, d.K, d.G});
+    }
+    if (!shapes.empty()) need = (int64_t)wq_gptq_gemv_list_workspace_bytes(shapes.data(), (int)shapes.size());
+    g.ws_bytes = need;
     top += (need + kAlign - 1) / kAlign * kAlign;
   }
   p->workspace_bytes = top;
@@ -507,7 +519,7 @@ static int build_lists(wq_program* p, hipStream_t stream) {
     char* ws = static_cast<char*>(p->workspace) + g.ws_offset;
     const int count = (int)(descs.size() + gptq_descs.size());
     g.list = !gptq_descs.empty()
-                 ? wq_gptq_gemv_list_create(gptq_descs.data(), count, ws, wq_q4g32_gemv_list_workspace_bytes(count), stream)
+                 ? wq_gptq_gemv_list_create(gptq_descs.data(), count, ws, (size_t)g.ws_bytes, stream)
                  : wq_q4g32_gemv_list_create_batched(descs.data(), count, (int)rows, ws,
                                                      wq_q4g32_gemv_list_workspace_bytes(count), stream);
     // operands that alias in a way the list kernel cannot order (or pointers it cannot take): the

@@ -44,6 +44,15 @@ constexpr uint32_t kSignal = 1u << 31;  // a later linear reads y
 
 typedef const GemvListDesc __attribute__((address_space(4)))* gemv_desc_ptr;  // scalar loads
 
+// xp[k'] = x[perm[k']], k' < K: the activations of an AutoGPTQ layer with a row order whose x comes from outside the list
+struct GatherJob {
+  const half_t* x;
+  const int32_t* perm;
+  half_t* xp;
+  int64_t K;
+};
+static_assert(sizeof(GatherJob) == 32, "job layout");
+
 constexpr int kCounterStride = 16;   // ints between two counters (64 bytes: one cache line each)
 constexpr int kCountersPerLinear = 8;
 constexpr int kBufferFlags = 0x00020000;  // buffer resource word 3: 32-bit data format, no swizzle
@@ -85,6 +94,8 @@ struct wq_gemv_list {
   int nb = 2;
   int gs = 2;  // log2 of the rows per row group: 4 consecutive rows (8 KiB at K = 4096) per workgroup at a time
   long long spin_limit = 200000000;  // 2 s of the 100 MHz wall clock
+  void* gather_table = nullptr;  // device: jobs of the gather kernel that runs in front of an AutoGPTQ list (GatherJob[gather_jobs])
+  int gather_jobs = 0, gather_blocks = 0;
   bool zp = false;         // AutoGPTQ layers: a (scale, zero point + 1) pair per group instead of a scale per 32 columns
   int M = 1;               // activation rows of the launch; > 1: the batch kernel (q4g32_batch_list.hip) and the fields below
   int batch_u = 0;         // chunks per tile and wavefront (4: M <= 16; 2: beyond)

@@ -610,6 +610,15 @@ __global__ __launch_bounds__(64 * (NC + XW + 1)) void q4g32_gemv_list_kernel(con
   }
 }
 
+// Gathers in front of a list of AutoGPTQ layers: job blockIdx.y, 256 positions per workgroup.
+__global__ __launch_bounds__(256) void gptq_list_gather_kernel(const GatherJob* __restrict__ jobs) {
+  const GatherJob j = jobs[blockIdx.y];
+  for (int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x; k < j.K; k += (int64_t)gridDim.x * 256) {
+    const uint32_t src = (uint32_t)j.perm[k];
+    j.xp[k] = src < (uint32_t)j.K ? j.x[src] : (half_t)0.0f;
+  }
+}
+
 }  // namespace wq
 
 namespace wq {
@@ -636,6 +645,20 @@ constexpr int kListDepth = 4;  // ring slots (KiB of codes in flight) per comput
 extern "C" size_t wq_q4g32_gemv_list_workspace_bytes(int n) {
   if (n <= 0) return 0;
   return wq::list_table_bytes(n) + (size_t)wq::sync_ints(n) * sizeof(int);
+}
+
+// room for the gathered activations of every layer with a row order (whether its x turns out to come from the list
+// or not is only known from the addresses) and for the jobs of the gather kernel
+extern "C" size_t wq_gptq_gemv_list_workspace_bytes(const wq_gptq_gemv_desc* d, int n) {
+  if (!d || n <= 0) return 0;
+  size_t extra = wq::kListAlign * (((size_t)n * sizeof(wq::GatherJob) + wq::kListAlign - 1) / wq::kListAlign);
+  bool any = false;
+  for (int i = 0; i < n; ++i)
+    if (d[i].perm && d[i].K > 0) {
+      any = true;
+      extra += ((size_t)d[i].K * 2 + wq::kListAlign - 1) / wq::kListAlign * wq::kListAlign;
+    }
+  return wq_q4g32_gemv_list_workspace_bytes(n) + (any ? extra : 0);
 }
 
 extern "C" void wq_q4g32_gemv_list_destroy(wq_gemv_list_t* l) { delete l; }
@@ -844,6 +867,37 @@ static wq_gemv_list_t* wq::gemv_list_create(const char* who, const wq_q4g32_gemv
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, kern, l->threads, l->lds) != hipSuccess || resident < 1)
     return bad(WQ_EDEVICE, "%s: the workgroup does not fit a CU (%zu bytes of LDS)", who, l->lds);
   }
+  // Layers with a row order whose x comes from outside the list: if the workspace has room
+  // (wq_gptq_gemv_list_workspace_bytes), a small kernel in front of the list gathers their activations and the list
+  // reads the gathered copy like any other x; the others (and all of them in a workspace of the plain size) gather
+  // while they stage, which costs the step about 3 us per layer.
+  std::vector<GatherJob> jobs;
+  if (perm) {
+    char* const base = static_cast<char*>(workspace);
+    size_t at = wq_q4g32_gemv_list_workspace_bytes(ne);
+    const size_t jobs_bytes = ((size_t)ne * sizeof(GatherJob) + kListAlign - 1) / kListAlign * kListAlign;
+    char* const job_table = base + at;
+    at += jobs_bytes;
+    int64_t kmax = 0;
+    for (int i = 0; i < ne && at <= workspace_bytes; ++i) {
+      GemvListDesc& g = l->descs[i];
+      if (!g.perm || ((g.g_dep >> 16) & 0x7fffu) != 0) continue;
+      const size_t need = ((size_t)e[i].K * 2 + kListAlign - 1) / kListAlign * kListAlign;
+      if (at + need > workspace_bytes) break;
+      jobs.push_back(GatherJob{g.x, g.perm, reinterpret_cast<half_t*>(base + at), e[i].K});
+      g.x = reinterpret_cast<const half_t*>(base + at);
+      g.perm = nullptr;
+      at += need;
+      kmax = std::max(kmax, e[i].K);
+    }
+    if (!jobs.empty()) {
+      l->gather_table = job_table;
+      l->gather_jobs = (int)jobs.size();
+      l->gather_blocks = (int)std::min<int64_t>((kmax + 255) / 256, 64);
+      if (hipMemcpyAsync(job_table, jobs.data(), jobs.size() * sizeof(GatherJob), hipMemcpyHostToDevice, stream) != hipSuccess)
+        return bad(WQ_EDEVICE, "%s: could not upload the gather jobs", who);
+    }
+  }
   l->table = workspace;
   l->sync = reinterpret_cast<int*>(static_cast<char*>(workspace) + list_table_bytes(ne));
   if (hipMemcpyAsync(l->table, l->descs.data(), (size_t)ne * sizeof(GemvListDesc), hipMemcpyHostToDevice, stream) != hipSuccess ||
@@ -859,6 +913,9 @@ extern "C" int wq_q4g32_gemv_list_run(wq_gemv_list_t* l, wq_stream_t stream) {
   WQ_REQUIRE(l && l->table, "wq_q4g32_gemv_list_run: null list");
   if (l->M > 1) return batch_list_launch(l, (hipStream_t)stream);
   if (l->zp) {
+    if (l->gather_jobs > 0)
+      WQ_LAUNCH("wq_q4g32_gemv_list_run", gptq_list_gather_kernel, dim3((unsigned)l->gather_blocks, (unsigned)l->gather_jobs),
+                dim3(256), 0, (hipStream_t)stream, (const GatherJob*)l->gather_table);
     WQ_LAUNCH("wq_q4g32_gemv_list_run", (q4g32_gemv_list_kernel<kListNC, kListXW, kListDepth, true>), dim3((unsigned)l->blocks),
               dim3((unsigned)l->threads), l->lds, (hipStream_t)stream, (const GemvListDesc*)l->table, l->n, l->sync,
               l->spin_limit, l->ybuf0, l->ybuf_floats, l->gs, l->deps > 0 ? 1 : 0);

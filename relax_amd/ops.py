@@ -575,7 +575,10 @@ class GptqGemvList(Q4G32GemvList):
     ``linears``: sequence of ``(w, x, y)`` or ``(w, x, y, bias, residual)`` with ``w`` a :class:`GptqWeight` from
     :func:`gptq_prepare` (with or without a row order; not :func:`gptq_prepare_padded`)."""
 
-    def __init__(self, linears):
+    def __init__(self, linears, gather_in_front: bool = True):
+        """``gather_in_front=False`` gives the list the plain workspace only, so that every row order is applied
+        inside the list kernel (otherwise layers whose x comes from outside the list are gathered by a small kernel
+        launched in front of it)."""
         self._l = _lib.lib()
         n = len(linears)
         arr = (GptqGemvDesc * max(1, n))()
@@ -595,7 +598,8 @@ class GptqGemvList(Q4G32GemvList):
                     raise ValueError(f"linear {i}: {name} must hold {w.N} elements")
             arr[i] = GptqGemvDesc(_ptr(w.W_nk), _ptr(w.SZ), _ptr(w.perm), _ptr(x), _ptr(bias), _ptr(residual), _ptr(y), w.N, w.K, w.G)
             self._keep.append((w, x, y, bias, residual))
-        need = self._l.wq_q4g32_gemv_list_workspace_bytes(n)
+        need = (self._l.wq_gptq_gemv_list_workspace_bytes(arr, n) if gather_in_front
+                else self._l.wq_q4g32_gemv_list_workspace_bytes(n))
         self._workspace = torch.zeros(max(int(need), 256), dtype=torch.uint8, device="cuda")
         self.M = 1
         self._h = self._l.wq_gptq_gemv_list_create(arr, n, self._workspace.data_ptr(), self._workspace.numel(), _stream())

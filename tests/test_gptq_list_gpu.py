@@ -37,10 +37,11 @@ SHAPES = [(4096, 4096, 128), (12288, 4096, 128), (4096, 11008, 128), (8, 32, 32)
           (520, 4096, 2048), (96, 2048, 2048), (600, 28672, 128), (16, 32768, 32), (200, 4224, 128), (88, 1024, 1024)]
 
 
-@pytest.mark.parametrize("act_order", [False, True])
-def test_independent_layers_match_oracle_and_call_by_call(env, oracle, act_order):
+@pytest.mark.parametrize("act_order,gather_in_front", [(False, True), (True, True), (True, False)])
+def test_independent_layers_match_oracle_and_call_by_call(env, oracle, act_order, gather_in_front):
     """With ``act_order`` every layer but each third has a row order (a random assignment of the rows to the groups,
-    what AutoGPTQ's desc_act leaves): its activations are gathered while they are staged."""
+    what AutoGPTQ's desc_act leaves): its activations are gathered by a kernel in front of the list, or, in a
+    workspace of the plain size (``gather_in_front=False``), inside the list kernel while they are staged."""
     ops, u, torch = env
     lins = []
     for i, (N, K, gs) in enumerate(SHAPES):
@@ -48,7 +49,7 @@ def test_independent_layers_match_oracle_and_call_by_call(env, oracle, act_order
         l["dx"] = u.dev(l["x"])
         l["y"] = torch.zeros((1, N), dtype=torch.float16, device="cuda")
         lins.append(l)
-    gl = ops.GptqGemvList([(l["w"], l["dx"], l["y"]) for l in lins])
+    gl = ops.GptqGemvList([(l["w"], l["dx"], l["y"]) for l in lins], gather_in_front=gather_in_front)
     assert gl.info() == (0, 0)
     print("gptq list: independent layers", flush=True)
     gl.run()
@@ -70,7 +71,8 @@ def test_independent_layers_match_oracle_and_call_by_call(env, oracle, act_order
 def test_epilogue_and_one_hot(env, oracle):
     ops, u, torch = env
     rng = np.random.default_rng(3)
-    for N, K, gs, act in [(520, 1024, 128, False), (264, 4224, 64, False), (264, 4224, 64, True), (72, 2048, 32, True)]:
+    for N, K, gs, act, front in [(520, 1024, 128, False, True), (264, 4224, 64, False, True), (264, 4224, 64, True, True),
+                                 (264, 4224, 64, True, False), (72, 2048, 32, True, False)]:
         l = _layer(oracle, ops, u, N, K, gs, seed=7, act_order=act)
         bias = rng.standard_normal(N).astype(np.float16)
         res = rng.standard_normal((1, N)).astype(np.float16)
@@ -80,7 +82,8 @@ def test_epilogue_and_one_hot(env, oracle):
             xh = np.zeros((1, K), np.float16)
             xh[0, k] = 1
             hot.append((k, u.dev(xh), torch.zeros((1, N), dtype=torch.float16, device="cuda")))
-        gl = ops.GptqGemvList([(l["w"], u.dev(l["x"]), y, u.dev(bias), u.dev(res))] + [(l["w"], dx, yh) for _, dx, yh in hot])
+        gl = ops.GptqGemvList([(l["w"], u.dev(l["x"]), y, u.dev(bias), u.dev(res))] + [(l["w"], dx, yh) for _, dx, yh in hot],
+                              gather_in_front=front)
         gl.run()
         gl.status()
         u.assert_close(u.host(y), _ref(oracle, l, l["x"], bias, res), "gptq list epilogue")
@@ -157,3 +160,32 @@ def test_what_the_list_refuses(env, oracle):
     w = ops.gptq_prepare_padded(u.dev(qw), u.dev(qz), u.dev(s), u.dev(g_idx))
     with pytest.raises(ValueError, match="padded"):
         ops.GptqGemvList([(w, u.dev(x), y)])
+
+
+def test_the_gathered_copy_follows_the_input_between_launches(env, oracle):
+    """A layer with a row order fed from outside the list: the gather in front of the list kernel runs at every launch,
+    so new contents of x are seen (eager and in a replayed graph)."""
+    ops, u, torch = env
+    l = _layer(oracle, ops, u, 136, 1024, 128, seed=12, act_order=True)
+    dx = torch.zeros((1, 1024), dtype=torch.float16, device="cuda")
+    y = torch.zeros((1, 136), dtype=torch.float16, device="cuda")
+    gl = ops.GptqGemvList([(l["w"], dx, y)])
+    rng = np.random.default_rng(13)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        gl.run()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            gl.run()
+    for rep in range(4):
+        x = rng.standard_normal((1, 1024)).astype(np.float16)
+        dx.copy_(u.dev(x))
+        torch.cuda.synchronize()
+        if rep % 2:
+            graph.replay()
+        else:
+            gl.run()
+        torch.cuda.synchronize()
+        u.assert_close(u.host(y), _ref(oracle, l, x), f"new x, launch {rep}")
+    gl.status()

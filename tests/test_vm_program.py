@@ -250,6 +250,27 @@ def test_runs_of_autogptq_decode_linears_are_fused_apart_from_q4f16_1_runs():
         l.wq_program_destroy(p)
 
 
+def test_autogptq_list_workspace_size():
+    """wq_gptq_gemv_list_workspace_bytes: the plain size, plus (only if some layer has a row order) a table of jobs
+    and 2 K bytes per such layer, each rounded up to 256."""
+    import ctypes as C
+
+    class Desc(C.Structure):
+        _fields_ = [(n, C.c_void_p) for n in ("W_nk", "SZ", "perm", "x", "bias", "residual", "y")] + \
+                   [(n, C.c_int64) for n in ("N", "K", "G")]
+
+    l = _lib()
+    arr = (Desc * 3)()
+    for i, (K, has) in enumerate(((4096, False), (1000 * 32, True), (96, True))):
+        arr[i] = Desc(None, None, 0x1000 if has else None, None, None, None, None, 64, K, K // 32)
+    plain = l.wq_q4g32_gemv_list_workspace_bytes(3)
+    assert l.wq_gptq_gemv_list_workspace_bytes(arr, 3) == plain + 256 + 64000 + 256
+    arr[1].perm = None
+    arr[2].perm = None
+    assert l.wq_gptq_gemv_list_workspace_bytes(arr, 3) == plain
+    assert l.wq_gptq_gemv_list_workspace_bytes(None, 3) == 0
+
+
 def test_options_and_a_program_of_external_tensors_only_needs_its_workspace():
     l = _lib()
     p = l.wq_program_create()
